@@ -1,0 +1,97 @@
+// Device-side numeric helpers shared by the kernels (gfx950, wave64).
+#ifndef CVCUDA_AMD_DEVICEUTILS_HPP
+#define CVCUDA_AMD_DEVICEUTILS_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <type_traits>
+
+namespace cvamd {
+
+// float -> T with round-half-to-even and saturation; NaN -> 0 for integer targets
+// (semantics of the reference's SaturateCast, cuda_tools/detail/SaturateCastImpl.hpp:41-50, 125).
+template<class T>
+__device__ __forceinline__ T SaturateCast(float v)
+{
+    if constexpr (std::is_same_v<T, float>)
+    {
+        return v;
+    }
+    else if constexpr (std::is_same_v<T, uint8_t>)
+    {
+        float r = rintf(v);
+        r       = fminf(fmaxf(r, 0.f), 255.f); // fmaxf(NaN, 0) == 0
+        return (uint8_t)(int)r;
+    }
+    else if constexpr (std::is_same_v<T, int8_t>)
+    {
+        float r = rintf(v);
+        r       = fminf(fmaxf(r, -128.f), 127.f);
+        return (int8_t)(int)(v != v ? 0.f : r);
+    }
+    else if constexpr (std::is_same_v<T, uint16_t>)
+    {
+        float r = rintf(v);
+        r       = fminf(fmaxf(r, 0.f), 65535.f);
+        return (uint16_t)(int)r;
+    }
+    else if constexpr (std::is_same_v<T, int16_t>)
+    {
+        float r = rintf(v);
+        r       = fminf(fmaxf(r, -32768.f), 32767.f);
+        return (int16_t)(int)(v != v ? 0.f : r);
+    }
+    else if constexpr (std::is_same_v<T, int32_t>)
+    {
+        if (v != v)
+        {
+            return 0;
+        }
+        float r = rintf(v);
+        if (r >= 2147483648.f)
+        {
+            return 2147483647;
+        }
+        if (r <= -2147483648.f)
+        {
+            return (int32_t)(-2147483647 - 1);
+        }
+        return (int32_t)r;
+    }
+    else
+    {
+        return (T)v;
+    }
+}
+
+__device__ __forceinline__ uint8_t SaturateU8(int v)
+{
+    return (uint8_t)min(max(v, 0), 255);
+}
+
+// Loads of 4 / 8 bytes from an address of arbitrary alignment. gfx950 global memory instructions
+// accept unaligned addresses, so these compile to a single global_load_dword / _dwordx2.
+struct __attribute__((packed, aligned(1))) UnalignedU32
+{
+    uint32_t v;
+};
+
+struct __attribute__((packed, aligned(1))) UnalignedU64
+{
+    uint64_t v;
+};
+
+__device__ __forceinline__ uint32_t LoadU32Unaligned(const uint8_t *p)
+{
+    return reinterpret_cast<const UnalignedU32 *>(p)->v;
+}
+
+__device__ __forceinline__ uint64_t LoadU64Unaligned(const uint8_t *p)
+{
+    return reinterpret_cast<const UnalignedU64 *>(p)->v;
+}
+
+} // namespace cvamd
+
+#endif // CVCUDA_AMD_DEVICEUTILS_HPP

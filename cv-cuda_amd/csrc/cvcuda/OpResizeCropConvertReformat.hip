@@ -1,0 +1,437 @@
+// Fused resize -> crop -> scale/offset/convert -> channel reorder -> layout change.
+//
+// Arithmetic follows the reference's kernels (src/cvcuda/priv/OpResizeCropConvertReformat.cu:137-278)
+// expression for expression in float32 without FMA contraction; validation order and status codes
+// follow its operator() (:418-683).
+//
+// Kernel shape (gfx950, wave64): one lane per output column, each wave produces kRowsPerWave output
+// rows, a 256-thread block covers 64 columns x 8 rows. The x-dependent terms (source column, weight)
+// are computed once per lane and reused for all its rows. Source taps are two adjacent u8x3 pixels,
+// i.e. 6 contiguous bytes, fetched with ONE unaligned 8-byte load per source row; consecutive lanes
+// read addresses ~3*scale bytes apart, so a wave touches a dense run of cache lines and the HBM
+// traffic equals the row span the output needs. Output stores are one element per lane per plane
+// (planar: 256 contiguous bytes per wave).
+#include "DeviceUtils.hpp"
+#include "OpCommon.hpp"
+
+#include <cvcuda/OpResizeCropConvertReformat.h>
+
+namespace cvamd {
+
+namespace {
+
+constexpr int kRowsPerWave  = 2;
+constexpr int kWavesPerBlk  = 4;
+constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlk;
+
+struct FusedArgs
+{
+    // source: tensor (base + n*sampleStride) or var-shape descriptor list
+    const uint8_t                *srcBase;
+    int64_t                       srcSampleStride;
+    int32_t                       srcRowStride;
+    int32_t                       srcW, srcH;
+    const NVCVImageBufferStrided *srcList;
+    // destination, strides in elements
+    void   *dstBase;
+    int64_t dstStrideN;
+    int32_t dstStrideY, dstStrideX;
+    int64_t dstOffC[3]; // element offset of source channel c in the destination (mapping applied)
+    int32_t dstW, dstH;
+    // geometry
+    int32_t newW, newH;
+    int32_t cropX, cropY;
+    float   scaleX, scaleY; // tensor path: srcW/newW, srcH/newH
+    float   scale, offset;
+    int32_t srcCast;
+};
+
+struct SrcImage
+{
+    const uint8_t *base;
+    int32_t        rowStride, w, h;
+    float          scaleX, scaleY;
+};
+
+template<bool VARSHAPE>
+__device__ __forceinline__ SrcImage GetSource(const FusedArgs &a, int n)
+{
+    SrcImage s;
+    if constexpr (VARSHAPE)
+    {
+        const NVCVImagePlaneStrided &pl = a.srcList[n].planes[0];
+        s.base                          = pl.basePtr;
+        s.rowStride                     = pl.rowStride;
+        s.w                             = pl.width;
+        s.h                             = pl.height;
+        s.scaleX                        = static_cast<float>(s.w) / a.newW;
+        s.scaleY                        = static_cast<float>(s.h) / a.newH;
+    }
+    else
+    {
+        s.base      = a.srcBase + n * a.srcSampleStride;
+        s.rowStride = a.srcRowStride;
+        s.w         = a.srcW;
+        s.h         = a.srcH;
+        s.scaleX    = a.scaleX;
+        s.scaleY    = a.scaleY;
+    }
+    return s;
+}
+
+template<class DstT>
+__device__ __forceinline__ void StorePixel(const FusedArgs &a, DstT *out, float v0, float v1, float v2)
+{
+    out[a.dstOffC[0]] = SaturateCast<DstT>(a.scale * v0 + a.offset);
+    out[a.dstOffC[1]] = SaturateCast<DstT>(a.scale * v1 + a.offset);
+    out[a.dstOffC[2]] = SaturateCast<DstT>(a.scale * v2 + a.offset);
+}
+
+template<class DstT, bool VARSHAPE>
+__global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
+{
+    const int n    = blockIdx.z;
+    const int dx   = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int wave = threadIdx.x >> 6;
+    const int dy0  = blockIdx.y * kRowsPerBlock + wave * kRowsPerWave;
+    if (dx >= a.dstW)
+    {
+        return;
+    }
+    const SrcImage s   = GetSource<VARSHAPE>(a, n);
+    DstT          *dst = static_cast<DstT *>(a.dstBase) + n * a.dstStrideN;
+
+    int sx = (int)floorf((dx + a.cropX + 0.5f) * s.scaleX);
+    sx     = min(sx, s.w - 1);
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+    {
+        const int dy = dy0 + r;
+        if (dy >= a.dstH)
+        {
+            break;
+        }
+        int sy = (int)floorf((dy + a.cropY + 0.5f) * s.scaleY);
+        sy     = min(sy, s.h - 1);
+        const uint8_t *p = s.base + (int64_t)sy * s.rowStride + sx * 3;
+        StorePixel<DstT>(a, dst + (int64_t)dy * a.dstStrideY + dx * a.dstStrideX, (float)p[0], (float)p[1], (float)p[2]);
+    }
+}
+
+template<class DstT, bool VARSHAPE>
+__global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
+{
+    const int n    = blockIdx.z;
+    const int dx   = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int wave = threadIdx.x >> 6;
+    const int dy0  = blockIdx.y * kRowsPerBlock + wave * kRowsPerWave;
+    if (dx >= a.dstW)
+    {
+        return;
+    }
+    const SrcImage s   = GetSource<VARSHAPE>(a, n);
+    DstT          *dst = static_cast<DstT *>(a.dstBase) + n * a.dstStrideN;
+
+    // x terms, shared by all rows of this lane
+    float fx  = (dx + a.cropX + 0.5f) * s.scaleX - 0.5f;
+    int   sx0 = (int)floorf(fx);
+    int   sx1 = min(sx0 + 1, s.w - 1);
+    fx -= sx0;
+    sx0               = max(0, sx0);
+    const bool twoTap = sx1 > sx0; // second tap is the next pixel, otherwise the same pixel
+    const int  xoff   = sx0 * 3;
+    const float wx0   = 1 - fx;
+
+    // The 8-byte load reads 2 bytes (5 when only one pixel is needed) past the taps. That stays
+    // inside the image for every row but the last one; rows whose load could cross the end of the
+    // image take byte loads instead.
+    const int64_t imgBytes = (int64_t)(s.h - 1) * s.rowStride + (int64_t)s.w * 3;
+
+#pragma unroll
+    for (int r = 0; r < kRowsPerWave; ++r)
+    {
+        const int dy = dy0 + r;
+        if (dy >= a.dstH)
+        {
+            break;
+        }
+        float fy  = (dy + a.cropY + 0.5f) * s.scaleY - 0.5f;
+        int   sy0 = (int)floorf(fy);
+        int   sy1 = min(sy0 + 1, s.h - 1);
+        fy -= sy0;
+        sy0 = max(0, sy0);
+
+        const int64_t off0 = (int64_t)sy0 * s.rowStride + xoff;
+        const int64_t off1 = (int64_t)sy1 * s.rowStride + xoff;
+
+        uint64_t q0, q1;
+        if (off1 + 8 <= imgBytes) // off0 <= off1
+        {
+            q0 = LoadU64Unaligned(s.base + off0);
+            q1 = LoadU64Unaligned(s.base + off1);
+        }
+        else
+        {
+            const int nb = twoTap ? 6 : 3;
+            q0 = q1 = 0;
+            for (int b = 0; b < nb; ++b)
+            {
+                q0 |= (uint64_t)s.base[off0 + b] << (8 * b);
+                q1 |= (uint64_t)s.base[off1 + b] << (8 * b);
+            }
+        }
+        const int sh = twoTap ? 24 : 0; // bit offset of the second tap inside q
+        float     v[3];
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+        {
+            const float p00 = (float)((q0 >> (8 * c)) & 0xFF);
+            const float p01 = (float)((q0 >> (8 * c + sh)) & 0xFF);
+            const float p10 = (float)((q1 >> (8 * c)) & 0xFF);
+            const float p11 = (float)((q1 >> (8 * c + sh)) & 0xFF);
+            float       t   = (1 - fy) * (wx0 * p00 + p01 * fx) + fy * (wx0 * p10 + p11 * fx);
+            if (a.srcCast)
+            {
+                t = (float)SaturateCast<uint8_t>(t);
+            }
+            v[c] = t;
+        }
+        StorePixel<DstT>(a, dst + (int64_t)dy * a.dstStrideY + dx * a.dstStrideX, v[0], v[1], v[2]);
+    }
+}
+
+template<class DstT, bool VARSHAPE>
+void Launch(const FusedArgs &a, int N, NVCVInterpolationType interp, hipStream_t stream)
+{
+    dim3 block(256);
+    dim3 grid(DivUp(a.dstW, 64), DivUp(a.dstH, kRowsPerBlock), N);
+    if (N == 0 || a.dstW == 0 || a.dstH == 0)
+    {
+        return;
+    }
+    if (interp == NVCV_INTERP_NEAREST)
+    {
+        hipLaunchKernelGGL((FusedNearest<DstT, VARSHAPE>), grid, block, 0, stream, a);
+        CheckLaunch("FusedNearest");
+    }
+    else
+    {
+        hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE>), grid, block, 0, stream, a);
+        CheckLaunch("FusedBilinear");
+    }
+}
+
+class ResizeCropConvertReformat final : public IOperator
+{
+public:
+    void submit(hipStream_t stream, NVCVTensorHandle hin, NVCVTensorHandle hout, NVCVSize2D resizeDim,
+                NVCVInterpolationType interp, int2 cropPos, NVCVChannelManip manip, float scale, float offset,
+                bool srcCast) const
+    {
+        NVCVTensorData din, dout;
+        ExportTensor(hin, din, "Input");
+        ExportTensor(hout, dout, "Output");
+        // Layout problems are NOT_COMPATIBLE for this operator; a tensor that is not an image batch
+        // at all is reported the same way.
+        ImageBatchView in  = RequireImageBatchView(din, "Input", NVCV_ERROR_NOT_COMPATIBLE);
+        ImageBatchView out = RequireImageBatchView(dout, "Output", NVCV_ERROR_NOT_COMPATIBLE);
+
+        checkCommon(in.N, in.C, in.elem, /*srcPlanes*/ 1, out);
+        if (in.layout != kLayoutNHWC)
+        {
+            throw OpError(NVCV_ERROR_NOT_COMPATIBLE, "Input tensor must have 'NHWC' or 'HWC' layout: Layout provided %s",
+                          in.layoutName);
+        }
+        if (resizeDim.w <= 1 || resizeDim.h <= 1)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Invalid resize dimensions: width x hight = %d x %d dimensions must be larger than 1.",
+                          resizeDim.w, resizeDim.h);
+        }
+        checkCrop(cropPos, out, resizeDim.w, resizeDim.h);
+        if (in.bytesSpanned() > INT32_MAX)
+        {
+            throw OpError(NVCV_ERROR_OVERFLOW, "Input size exceeds %d. Tensor is too large.", INT32_MAX);
+        }
+        checkInterp(interp);
+
+        FusedArgs a       = makeArgs(out, resizeDim, cropPos, manip, scale, offset, srcCast);
+        a.srcBase         = in.base;
+        a.srcSampleStride = in.strideN;
+        a.srcRowStride    = (int32_t)in.strideH;
+        a.srcW            = in.W;
+        a.srcH            = in.H;
+        a.scaleX          = static_cast<float>(in.W) / resizeDim.w;
+        a.scaleY          = static_cast<float>(in.H) / resizeDim.h;
+        if (out.elem == kU8)
+        {
+            Launch<uint8_t, false>(a, in.N, interp, stream);
+        }
+        else
+        {
+            Launch<float, false>(a, in.N, interp, stream);
+        }
+    }
+
+    void submit(hipStream_t stream, NVCVImageBatchHandle hin, NVCVTensorHandle hout, NVCVSize2D resizeDim,
+                NVCVInterpolationType interp, int2 cropPos, NVCVChannelManip manip, float scale, float offset,
+                bool srcCast) const
+    {
+        VarShapeView   in = ExportVarShape(hin, stream, "Input");
+        NVCVTensorData dout;
+        ExportTensor(hout, dout, "Output");
+        if (in.uniqueFormat == NVCV_IMAGE_FORMAT_NONE)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "All input images in a batch must have the same format (including number of channels)");
+        }
+        ImageBatchView out = RequireImageBatchView(dout, "Output", NVCV_ERROR_NOT_COMPATIBLE);
+        FormatInfo     fi  = DecodeFormat(in.uniqueFormat);
+        checkCommon(in.N, fi.channels, fi.elem, fi.planes, out);
+        checkCrop(cropPos, out, std::abs(resizeDim.w), std::abs(resizeDim.h));
+        checkInterp(interp);
+        if (resizeDim.w <= 0 || resizeDim.h <= 0)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid resize dimensions: %d x %d", resizeDim.w, resizeDim.h);
+        }
+        FusedArgs a = makeArgs(out, resizeDim, cropPos, manip, scale, offset, srcCast);
+        a.srcList   = in.data.buffer.varShapeStrided.imageList;
+        if (out.elem == kU8)
+        {
+            Launch<uint8_t, true>(a, in.N, interp, stream);
+        }
+        else
+        {
+            Launch<float, true>(a, in.N, interp, stream);
+        }
+    }
+
+private:
+    static void checkCommon(int samples, int channels, ElemType srcElem, int srcPlanes, const ImageBatchView &out)
+    {
+        if (samples != out.N)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Input and output must have the same batch size (i.e., same number of images): Provided %d "
+                          "input and %d output images / samples",
+                          samples, out.N);
+        }
+        if (channels != out.C)
+        {
+            throw OpError(NVCV_ERROR_NOT_COMPATIBLE,
+                          "Input and output must have same number of channels: Provided %d input and %d output channels",
+                          channels, out.C);
+        }
+        if (channels != 3)
+        {
+            throw OpError(NVCV_ERROR_NOT_COMPATIBLE,
+                          "Only three-channel input is currently supported: Provided %d input channels", channels);
+        }
+        if (srcElem != kU8)
+        {
+            throw OpError(NVCV_ERROR_NOT_COMPATIBLE, "Input must be of data type uchar.");
+        }
+        if (out.elem != kU8 && out.elem != kF32)
+        {
+            throw OpError(NVCV_ERROR_NOT_COMPATIBLE, "Output must be of data type uchar or float.");
+        }
+        if (srcPlanes > 1)
+        {
+            throw OpError(NVCV_ERROR_NOT_COMPATIBLE, "Input must be non-planar (i.e., interleaved).");
+        }
+    }
+
+    static void checkCrop(int2 cropPos, const ImageBatchView &out, int newW, int newH)
+    {
+        if (cropPos.x < 0 || cropPos.y < 0 || cropPos.x + out.W > newW || cropPos.y + out.H > newH)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Invalid crop region: crop region(x, y, w, h) = (%d, %d, %d, %d) extends beyond bounds of "
+                          "resized tensor",
+                          cropPos.x, cropPos.y, out.W, out.H);
+        }
+    }
+
+    static void checkInterp(NVCVInterpolationType interp)
+    {
+        if (interp != NVCV_INTERP_NEAREST && interp != NVCV_INTERP_LINEAR)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "%s",
+                          interp == NVCV_INTERP_CUBIC  ? "Interpolation not implemented: NVCV_INTERP_CUBIC"
+                          : interp == NVCV_INTERP_AREA ? "Interpolation not implemented: NVCV_INTERP_AREA"
+                                                       : "Invalid interpolation");
+        }
+    }
+
+    static FusedArgs makeArgs(const ImageBatchView &out, NVCVSize2D resizeDim, int2 cropPos, NVCVChannelManip manip,
+                              float scale, float offset, bool srcCast)
+    {
+        const int es = ElemSize(out.elem);
+        if (out.strideN % es || out.strideH % es || out.strideW % es || out.strideC % es)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Output strides must be multiples of the element size");
+        }
+        FusedArgs a  = {};
+        a.dstBase    = out.base;
+        a.dstStrideN = out.strideN / es;
+        a.dstStrideY = (int32_t)(out.strideH / es);
+        a.dstStrideX = (int32_t)(out.strideW / es);
+        for (int c = 0; c < 3; ++c)
+        {
+            int to       = manip == NVCV_CHANNEL_REVERSE ? 2 - c : c;
+            a.dstOffC[c] = to * (out.strideC / es);
+        }
+        a.dstW    = out.W;
+        a.dstH    = out.H;
+        a.newW    = resizeDim.w;
+        a.newH    = resizeDim.h;
+        a.cropX   = cropPos.x;
+        a.cropY   = cropPos.y;
+        a.scale   = scale;
+        a.offset  = offset;
+        a.srcCast = srcCast ? 1 : 0;
+        return a;
+    }
+};
+
+} // namespace
+} // namespace cvamd
+
+using namespace cvamd;
+
+extern "C"
+{
+CVCUDA_PUBLIC NVCVStatus cvcudaResizeCropConvertReformatCreate(NVCVOperatorHandle *handle)
+{
+    return CreateOperator<ResizeCropConvertReformat>(handle);
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaResizeCropConvertReformatSubmit(NVCVOperatorHandle handle, hipStream_t stream,
+                                                               NVCVTensorHandle in, NVCVTensorHandle out,
+                                                               const NVCVSize2D            resizeDim,
+                                                               const NVCVInterpolationType interpolation,
+                                                               const int2 cropPos, const NVCVChannelManip manip,
+                                                               const float scale, const float offset,
+                                                               const bool srcCast)
+{
+    return Protect(
+        [&]
+        {
+            ToOperator<ResizeCropConvertReformat>(handle).submit(stream, in, out, resizeDim, interpolation, cropPos,
+                                                                 manip, scale, offset, srcCast);
+        });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaResizeCropConvertReformatVarShapeSubmit(
+    NVCVOperatorHandle handle, hipStream_t stream, NVCVImageBatchHandle in, NVCVTensorHandle out,
+    const NVCVSize2D resizeDim, const NVCVInterpolationType interpolation, const int2 cropPos,
+    const NVCVChannelManip manip, const float scale, const float offset, const bool srcCast)
+{
+    return Protect(
+        [&]
+        {
+            ToOperator<ResizeCropConvertReformat>(handle).submit(stream, in, out, resizeDim, interpolation, cropPos,
+                                                                 manip, scale, offset, srcCast);
+        });
+}
+}

@@ -1,0 +1,923 @@
+// Decoding and construction of the 64-bit format / data-type words (field map in
+// nvcv/detail/FormatBits.h). Covers the queries the operators and the object layer need; follows
+// the decoding rules of the reference's src/nvcv/src/priv/ImageFormat.cpp:560-860 and
+// DataLayout.cpp:645-667 (channel count = distinct X/Y/Z/W selectors).
+#include "Priv.hpp"
+
+#include <cstring>
+
+namespace nvcvamd {
+
+namespace {
+
+struct PackingRow
+{
+    NVCVPacking packing;
+    int32_t     bits[4];
+};
+
+const PackingRow kPackings[] = {
+#include "PackingTable.inc"
+};
+
+const char *const kSwizzles[] = {
+#include "SwizzleTable.inc"
+};
+constexpr int kNumSwizzles = sizeof(kSwizzles) / sizeof(kSwizzles[0]);
+
+inline uint64_t Get(uint64_t v, int off, int len)
+{
+    return NVCV_DETAIL_BITS_GET(v, off, len);
+}
+
+inline uint64_t Put(uint64_t v, int off, int len)
+{
+    return NVCV_DETAIL_BITS_PUT(v, off, len);
+}
+
+int BppFromCode(int code, int sub, int nch)
+{
+    switch (code)
+    {
+    case 0:
+        return (nch == 1 && sub >= 1 && sub <= 3) ? (sub == 3 ? 4 : sub) : 8;
+    case 1:
+    case 2:
+    case 3:
+        return (code + 1) * 8;
+    case 4:
+    case 5:
+        return (code - 1) * 16;
+    case 6:
+    case 7:
+        return (code - 3) * 32;
+    default:
+        return (code - 5) * 64;
+    }
+}
+
+uint64_t PackSlot(NVCVPacking p, int nsub, int nch, int nbpp)
+{
+    return NVCV_DETAIL_PACKING_SLOT((uint64_t)p, nsub, nch, nbpp);
+}
+
+} // namespace
+
+PackingInfo DecodePacking(NVCVPacking p)
+{
+    PackingInfo info = {};
+    if (p == NVCV_PACKING_0)
+    {
+        info.known = true;
+        return info;
+    }
+    info.numChannels  = (int)Get(p, 4, 2) + 1;
+    info.bitsPerPixel = BppFromCode((int)Get(p, 6, 4), (int)Get(p, 0, 4), info.numChannels);
+    for (const PackingRow &row : kPackings)
+    {
+        if (row.packing == p)
+        {
+            std::memcpy(info.bits, row.bits, sizeof(info.bits));
+            info.known = true;
+            break;
+        }
+    }
+    return info;
+}
+
+NVCVPacking FormatPlanePacking(uint64_t fmt, int plane)
+{
+    if (fmt == 0)
+    {
+        return NVCV_PACKING_0;
+    }
+    uint64_t sub, ch, bpp;
+    switch (plane)
+    {
+    case 0:
+        sub = Get(fmt, 35, 3);
+        ch  = Get(fmt, 38, 2);
+        bpp = Get(fmt, 40, 4);
+        break;
+    case 1:
+    case 2:
+        if (Get(fmt, 7, 1) == 0) // slots 1..3 hold extra-channel info instead
+        {
+            return NVCV_PACKING_0;
+        }
+        sub = Get(fmt, plane == 1 ? 44 : 51, 3);
+        ch  = Get(fmt, plane == 1 ? 47 : 54, 1);
+        bpp = Get(fmt, plane == 1 ? 48 : 55, 3);
+        break;
+    case 3:
+    {
+        if (Get(fmt, 7, 1) == 0)
+        {
+            return NVCV_PACKING_0;
+        }
+        uint64_t code = Get(fmt, 58, 3);
+        if (code == 0)
+        {
+            return NVCV_PACKING_0;
+        }
+        if (code == 7) // an 8-bit fourth plane is stored as all ones
+        {
+            return NVCV_PACKING_X8;
+        }
+        return (NVCVPacking)Put(code, 6, 4);
+    }
+    default:
+        return NVCV_PACKING_0;
+    }
+    return (NVCVPacking)(Put(bpp, 6, 4) | Put(ch, 4, 2) | Put(sub, 0, 4));
+}
+
+int FormatNumPlanes(uint64_t fmt)
+{
+    int n = 0;
+    for (int p = 0; p < 4; ++p)
+    {
+        n += FormatPlanePacking(fmt, p) != NVCV_PACKING_0 ? 1 : 0;
+    }
+    return n;
+}
+
+NVCVSwizzle FormatSwizzle(uint64_t fmt)
+{
+    return (NVCVSwizzle)Get(fmt, 0, 6);
+}
+
+void SwizzleChannels(NVCVSwizzle sw, NVCVChannel out[4])
+{
+    if ((int)sw < 0 || (int)sw >= kNumSwizzles)
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid swizzle code %d", (int)sw);
+    }
+    const char *s = kSwizzles[(int)sw];
+    for (int i = 0; i < 4; ++i)
+    {
+        switch (s[i])
+        {
+        case 'X':
+            out[i] = NVCV_CHANNEL_X;
+            break;
+        case 'Y':
+            out[i] = NVCV_CHANNEL_Y;
+            break;
+        case 'Z':
+            out[i] = NVCV_CHANNEL_Z;
+            break;
+        case 'W':
+            out[i] = NVCV_CHANNEL_W;
+            break;
+        case '1':
+            out[i] = NVCV_CHANNEL_1;
+            break;
+        default:
+            out[i] = NVCV_CHANNEL_0;
+            break;
+        }
+    }
+}
+
+int SwizzleNumChannels(NVCVSwizzle sw)
+{
+    NVCVChannel ch[4];
+    SwizzleChannels(sw, ch);
+    bool seen[4] = {};
+    int  n       = 0;
+    for (NVCVChannel c : ch)
+    {
+        if (c >= NVCV_CHANNEL_X && c <= NVCV_CHANNEL_W && !seen[c - NVCV_CHANNEL_X])
+        {
+            seen[c - NVCV_CHANNEL_X] = true;
+            ++n;
+        }
+    }
+    return n;
+}
+
+int FormatNumChannels(uint64_t fmt)
+{
+    return fmt == 0 ? 0 : SwizzleNumChannels(FormatSwizzle(fmt));
+}
+
+NVCVDataKind FormatDataKind(uint64_t fmt)
+{
+    return (NVCVDataKind)Get(fmt, 61, 3);
+}
+
+NVCVMemLayout FormatMemLayout(uint64_t fmt)
+{
+    return (NVCVMemLayout)Get(fmt, 12, 3);
+}
+
+NVCVColorModel FormatColorModel(uint64_t fmt)
+{
+    if (fmt == 0)
+    {
+        return NVCV_COLOR_MODEL_UNDEFINED;
+    }
+    if (Get(fmt, 16, 1) == 0)
+    {
+        return NVCV_COLOR_MODEL_YCbCr;
+    }
+    if (Get(fmt, 16, 19) == (1u << 19) - 1)
+    {
+        return NVCV_COLOR_MODEL_UNDEFINED;
+    }
+    uint64_t m = Get(fmt, 17, 3);
+    if (m < 7)
+    {
+        return (NVCVColorModel)(m + 2);
+    }
+    if (Get(fmt, 20, 1) == 0)
+    {
+        return NVCV_COLOR_MODEL_RAW;
+    }
+    return (NVCVColorModel)(Get(fmt, 21, 6) + 10);
+}
+
+NVCVColorSpec FormatColorSpec(uint64_t fmt)
+{
+    NVCVColorModel m = FormatColorModel(fmt);
+    if (m != NVCV_COLOR_MODEL_UNDEFINED && (int)m < 7)
+    {
+        return (NVCVColorSpec)Get(fmt, 20, 15);
+    }
+    return NVCV_COLOR_SPEC_UNDEFINED;
+}
+
+NVCVChromaSubsampling FormatCSS(uint64_t fmt)
+{
+    return FormatColorModel(fmt) == NVCV_COLOR_MODEL_YCbCr ? (NVCVChromaSubsampling)Get(fmt, 17, 3) : NVCV_CSS_NONE;
+}
+
+int FormatPlanePixelStrideBytes(uint64_t fmt, int plane)
+{
+    return (DecodePacking(FormatPlanePacking(fmt, plane)).bitsPerPixel + 7) / 8;
+}
+
+uint64_t MakeFormatWord(NVCVColorModel model, uint32_t specOrRaw, NVCVChromaSubsampling css, NVCVMemLayout layout,
+                        NVCVDataKind kind, NVCVSwizzle swizzle, NVCVAlphaType alpha, NVCVPacking p0, NVCVPacking p1,
+                        NVCVPacking p2, NVCVPacking p3)
+{
+    uint64_t color;
+    int      m = (int)model;
+    if (m == NVCV_COLOR_MODEL_YCbCr)
+    {
+        color = Put(specOrRaw, 20, 15) | Put(css, 17, 3);
+    }
+    else if (m == NVCV_COLOR_MODEL_UNDEFINED)
+    {
+        color = Put((1u << 19) - 1, 16, 19);
+    }
+    else if (m - 2 < 7)
+    {
+        color = Put(1, 16, 1) | Put(specOrRaw, 20, 15) | Put(m - 2, 17, 3);
+    }
+    else if (m == NVCV_COLOR_MODEL_RAW)
+    {
+        color = Put(1, 16, 1) | Put(7, 17, 3) | Put(specOrRaw, 21, 6);
+    }
+    else
+    {
+        color = Put(1, 16, 1) | Put(7, 17, 3) | Put(1, 20, 1) | Put(m - 10, 21, 6);
+    }
+    return Put(kind, 61, 3) | Put(swizzle, 0, 6) | Put(alpha, 6, 1) | Put(layout, 12, 3) | color | Put(1, 7, 1)
+         | Put(PackSlot(p0, 3, 2, 4), 35, 9) | Put(PackSlot(p1, 3, 1, 3), 44, 7) | Put(PackSlot(p2, 3, 1, 3), 51, 7)
+         | Put(PackSlot(p3, 0, 0, 3), 58, 3);
+}
+
+NVCVDataType FormatPlaneDataType(uint64_t fmt, int plane)
+{
+    NVCVPacking p = FormatPlanePacking(fmt, plane);
+    if (p == NVCV_PACKING_0)
+    {
+        return NVCV_DATA_TYPE_NONE;
+    }
+    return NVCV_DETAIL_MAKE_DATA_TYPE(FormatDataKind(fmt), (uint64_t)p);
+}
+
+void FormatPlaneSize(uint64_t fmt, int plane, int32_t w, int32_t h, int32_t *pw, int32_t *ph)
+{
+    int sh = 4, sv = 4; // chroma samples per 4 luma samples
+    if (plane >= 1)
+    {
+        switch (FormatCSS(fmt))
+        {
+        case NVCV_CSS_444:
+            break;
+        case NVCV_CSS_422:
+            sh = 2;
+            break;
+        case NVCV_CSS_422R:
+            sv = 2;
+            break;
+        case NVCV_CSS_411:
+            sh = 1;
+            break;
+        case NVCV_CSS_411R:
+            sv = 1;
+            break;
+        case NVCV_CSS_420:
+            sh = sv = 2;
+            break;
+        case NVCV_CSS_410:
+            sh = 1;
+            sv = 2;
+            break;
+        case NVCV_CSS_410R:
+            sh = 2;
+            sv = 1;
+            break;
+        }
+    }
+    *pw = (int32_t)(((int64_t)w * sh + 3) / 4);
+    *ph = (int32_t)(((int64_t)h * sv + 3) / 4);
+}
+
+int DataTypeStrideBytes(NVCVDataType t)
+{
+    return (DecodePacking(DataTypePacking(t)).bitsPerPixel + 7) / 8;
+}
+
+int DataTypeAlignment(NVCVDataType t)
+{
+    // Machine-word size of one stored component group: for the "_"-separated packings this is the
+    // component size, for sub-word packings the whole pixel.
+    PackingInfo pi = DecodePacking(DataTypePacking(t));
+    if (pi.numChannels == 0)
+    {
+        return 1;
+    }
+    bool uniform = pi.known && pi.bits[0] >= 8;
+    for (int i = 1; uniform && i < pi.numChannels; ++i)
+    {
+        uniform = pi.bits[i] == pi.bits[0];
+    }
+    int bytes = uniform && pi.bits[0] * pi.numChannels == pi.bitsPerPixel ? pi.bits[0] / 8 : (pi.bitsPerPixel + 7) / 8;
+    return (int)NextPow2(bytes);
+}
+
+namespace {
+
+const char *ThreadName(const char *fmt, ...)
+{
+    // Small ring so that a name built from other generated names does not overwrite its inputs.
+    static thread_local char ring[4][256];
+    static thread_local int  next = 0;
+    char                    *buf  = ring[next];
+    next                          = (next + 1) % 4;
+    va_list va;
+    va_start(va, fmt);
+    vsnprintf(buf, sizeof(ring[0]), fmt, va);
+    va_end(va);
+    return buf;
+}
+
+const char *KindLetter(NVCVDataKind k)
+{
+    switch (k)
+    {
+    case NVCV_DATA_KIND_UNSIGNED:
+        return "U";
+    case NVCV_DATA_KIND_SIGNED:
+        return "S";
+    case NVCV_DATA_KIND_FLOAT:
+        return "F";
+    case NVCV_DATA_KIND_COMPLEX:
+        return "C";
+    default:
+        return "?";
+    }
+}
+
+void CheckPlane(int plane)
+{
+    if (plane < 0 || plane >= 4)
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Plane index must be in [0,4), not %d", plane);
+    }
+}
+
+NVCVStatus MakeFormat(NVCVImageFormat *out, NVCVColorModel model, uint32_t spec, NVCVChromaSubsampling css,
+                      NVCVMemLayout layout, NVCVDataKind kind, NVCVSwizzle swizzle, NVCVPacking p0, NVCVPacking p1,
+                      NVCVPacking p2, NVCVPacking p3, NVCVAlphaType alpha, const NVCVExtraChannelInfo *ex)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(out, "Pointer to output format");
+            if (ex != nullptr && ex->numChannels > 0)
+            {
+                throw Error(NVCV_ERROR_NOT_IMPLEMENTED, "Formats with extra channels are not supported");
+            }
+            if (p0 == NVCV_PACKING_0 && (p1 != NVCV_PACKING_0 || p2 != NVCV_PACKING_0 || p3 != NVCV_PACKING_0))
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Plane packings must be given without gaps");
+            }
+            *out = MakeFormatWord(model, spec, css, layout, kind, swizzle, alpha, p0, p1, p2, p3);
+        });
+}
+
+} // namespace
+} // namespace nvcvamd
+
+using namespace nvcvamd;
+
+extern "C"
+{
+// ---- swizzle / packing -------------------------------------------------------------------------
+NVCVStatus nvcvSwizzleGetChannels(NVCVSwizzle swizzle, NVCVChannel *channels)
+{
+    return Protect([&] { SwizzleChannels(swizzle, NotNull(channels, "Pointer to output channels")); });
+}
+
+NVCVStatus nvcvSwizzleGetNumChannels(NVCVSwizzle swizzle, int32_t *outNumChannels)
+{
+    return Protect([&] { *NotNull(outNumChannels, "Pointer to output") = SwizzleNumChannels(swizzle); });
+}
+
+NVCVStatus nvcvMakeSwizzle(NVCVSwizzle *outSwizzle, NVCVChannel x, NVCVChannel y, NVCVChannel z, NVCVChannel w)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outSwizzle, "Pointer to output swizzle");
+            NVCVChannel want[4] = {x, y, z, w};
+            for (int i = 0; i < kNumSwizzles; ++i)
+            {
+                NVCVChannel have[4];
+                SwizzleChannels((NVCVSwizzle)i, have);
+                if (std::memcmp(have, want, sizeof(want)) == 0)
+                {
+                    *outSwizzle = (NVCVSwizzle)i;
+                    return;
+                }
+            }
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Channel combination has no swizzle code");
+        });
+}
+
+NVCVStatus nvcvPackingGetNumComponents(NVCVPacking packing, int32_t *outNumComponents)
+{
+    return Protect([&] { *NotNull(outNumComponents, "Pointer to output") = DecodePacking(packing).numChannels; });
+}
+
+NVCVStatus nvcvPackingGetBitsPerComponent(NVCVPacking packing, int32_t *outBits)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outBits, "Pointer to output");
+            PackingInfo pi = DecodePacking(packing);
+            if (!pi.known)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Unknown packing value %d", (int)packing);
+            }
+            std::memcpy(outBits, pi.bits, sizeof(pi.bits));
+        });
+}
+
+NVCVStatus nvcvPackingGetBitsPerPixel(NVCVPacking packing, int32_t *outBPP)
+{
+    return Protect([&] { *NotNull(outBPP, "Pointer to output") = DecodePacking(packing).bitsPerPixel; });
+}
+
+NVCVStatus nvcvPackingGetAlignment(NVCVPacking packing, int32_t *outAlignment)
+{
+    return Protect(
+        [&]
+        {
+            *NotNull(outAlignment, "Pointer to output")
+                = DataTypeAlignment(NVCV_DETAIL_MAKE_DATA_TYPE(NVCV_DATA_KIND_UNSIGNED, (uint64_t)packing));
+        });
+}
+
+const char *nvcvDataKindGetName(NVCVDataKind kind)
+{
+    switch (kind)
+    {
+    case NVCV_DATA_KIND_UNSPECIFIED:
+        return "NVCV_DATA_KIND_UNSPECIFIED";
+    case NVCV_DATA_KIND_UNSIGNED:
+        return "NVCV_DATA_KIND_UNSIGNED";
+    case NVCV_DATA_KIND_SIGNED:
+        return "NVCV_DATA_KIND_SIGNED";
+    case NVCV_DATA_KIND_FLOAT:
+        return "NVCV_DATA_KIND_FLOAT";
+    case NVCV_DATA_KIND_COMPLEX:
+        return "NVCV_DATA_KIND_COMPLEX";
+    }
+    return "Unexpected error retrieving NVCVDataKind string representation";
+}
+
+const char *nvcvMemLayoutGetName(NVCVMemLayout memlayout)
+{
+    return memlayout == NVCV_MEM_LAYOUT_PITCH_LINEAR ? "NVCV_MEM_LAYOUT_PITCH_LINEAR"
+                                                     : ThreadName("NVCV_MEM_LAYOUT_BLOCK%d_LINEAR",
+                                                                  1 << ((int)memlayout - 1));
+}
+
+const char *nvcvSwizzleGetName(NVCVSwizzle swizzle)
+{
+    if ((int)swizzle >= 0 && (int)swizzle < kNumSwizzles)
+    {
+        return ThreadName("NVCV_SWIZZLE_%s", kSwizzles[(int)swizzle]);
+    }
+    return "NVCV_SWIZZLE_UNSUPPORTED";
+}
+
+// ---- colour spec -------------------------------------------------------------------------------
+NVCVStatus nvcvChromaSubsamplingGetNumSamples(NVCVChromaSubsampling css, int32_t *outSamplesHoriz,
+                                              int32_t *outSamplesVert)
+{
+    return Protect(
+        [&]
+        {
+            if ((int)css < 0 || (int)css > 7)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid chroma subsampling: %d", (int)css);
+            }
+            // Evaluate the plane-size rule on a 4x4 luma block of a synthetic YCbCr format.
+            uint64_t fmt = MakeFormatWord(NVCV_COLOR_MODEL_YCbCr, NVCV_COLOR_SPEC_BT601, css, NVCV_MEM_LAYOUT_PL,
+                                          NVCV_DATA_KIND_UNSIGNED, NVCV_SWIZZLE_XYZ0, NVCV_ALPHA_ASSOCIATED,
+                                          NVCV_PACKING_X8, NVCV_PACKING_X8_Y8, NVCV_PACKING_0, NVCV_PACKING_0);
+            int32_t  w, h;
+            FormatPlaneSize(fmt, 1, 4, 4, &w, &h);
+            if (outSamplesHoriz)
+            {
+                *outSamplesHoriz = w;
+            }
+            if (outSamplesVert)
+            {
+                *outSamplesVert = h;
+            }
+        });
+}
+
+const char *nvcvColorModelGetName(NVCVColorModel cmodel)
+{
+    switch (cmodel)
+    {
+    case NVCV_COLOR_MODEL_UNDEFINED:
+        return "NVCV_COLOR_MODEL_UNDEFINED";
+    case NVCV_COLOR_MODEL_YCbCr:
+        return "NVCV_COLOR_MODEL_YCbCr";
+    case NVCV_COLOR_MODEL_RGB:
+        return "NVCV_COLOR_MODEL_RGB";
+    case NVCV_COLOR_MODEL_RAW:
+        return "NVCV_COLOR_MODEL_RAW";
+    case NVCV_COLOR_MODEL_XYZ:
+        return "NVCV_COLOR_MODEL_XYZ";
+    case NVCV_COLOR_MODEL_HSV:
+        return "NVCV_COLOR_MODEL_HSV";
+    case NVCV_COLOR_MODEL_CMYK:
+        return "NVCV_COLOR_MODEL_CMYK";
+    case NVCV_COLOR_MODEL_YCCK:
+        return "NVCV_COLOR_MODEL_YCCK";
+    }
+    return ThreadName("NVCVColorModel(%d)", (int)cmodel);
+}
+
+const char *nvcvChromaSubsamplingGetName(NVCVChromaSubsampling css)
+{
+    static const char *const names[] = {"NVCV_CSS_444", "NVCV_CSS_422",  "NVCV_CSS_422R", "NVCV_CSS_411",
+                                        "NVCV_CSS_411R", "NVCV_CSS_420", "NVCV_CSS_410",  "NVCV_CSS_410R"};
+    return ((int)css >= 0 && (int)css < 8) ? names[(int)css] : ThreadName("NVCVChromaSubsampling(%d)", (int)css);
+}
+
+// ---- data type ---------------------------------------------------------------------------------
+NVCVStatus nvcvMakeDataType(NVCVDataType *outDataType, NVCVDataKind dataKind, NVCVPacking packing)
+{
+    return Protect([&]
+                   { *NotNull(outDataType, "Pointer to output data type") = NVCV_DETAIL_MAKE_DATA_TYPE(dataKind, (uint64_t)packing); });
+}
+
+NVCVStatus nvcvDataTypeGetPacking(NVCVDataType type, NVCVPacking *outPacking)
+{
+    return Protect([&] { *NotNull(outPacking, "Pointer to output packing") = DataTypePacking(type); });
+}
+
+NVCVStatus nvcvDataTypeGetBitsPerPixel(NVCVDataType type, int32_t *outBPP)
+{
+    return Protect([&] { *NotNull(outBPP, "Pointer to output") = DecodePacking(DataTypePacking(type)).bitsPerPixel; });
+}
+
+NVCVStatus nvcvDataTypeGetBitsPerChannel(NVCVDataType type, int32_t *outBits)
+{
+    return nvcvPackingGetBitsPerComponent(DataTypePacking(type), outBits);
+}
+
+NVCVStatus nvcvDataTypeGetAlignment(NVCVDataType type, int32_t *outAlignment)
+{
+    return Protect([&] { *NotNull(outAlignment, "Pointer to output") = DataTypeAlignment(type); });
+}
+
+NVCVStatus nvcvDataTypeGetDataKind(NVCVDataType type, NVCVDataKind *outDataKind)
+{
+    return Protect([&] { *NotNull(outDataKind, "Pointer to output") = FormatDataKind(type); });
+}
+
+NVCVStatus nvcvDataTypeGetNumChannels(NVCVDataType type, int32_t *outNumChannels)
+{
+    return Protect([&]
+                   { *NotNull(outNumChannels, "Pointer to output") = DecodePacking(DataTypePacking(type)).numChannels; });
+}
+
+NVCVStatus nvcvDataTypeGetChannelType(NVCVDataType type, int32_t channel, NVCVDataType *outChannelType)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outChannelType, "Pointer to output");
+            PackingInfo pi = DecodePacking(DataTypePacking(type));
+            if (channel < 0 || channel >= pi.numChannels || !pi.known)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Channel %d does not exist in this data type", channel);
+            }
+            NVCVPacking one;
+            switch (pi.bits[channel])
+            {
+            case 8:
+                one = NVCV_PACKING_X8;
+                break;
+            case 16:
+                one = NVCV_PACKING_X16;
+                break;
+            case 32:
+                one = NVCV_PACKING_X32;
+                break;
+            case 64:
+                one = NVCV_PACKING_X64;
+                break;
+            case 128:
+                one = NVCV_PACKING_X128;
+                break;
+            default:
+                throw Error(NVCV_ERROR_NOT_IMPLEMENTED, "Channels of %d bits are not supported", pi.bits[channel]);
+            }
+            *outChannelType = NVCV_DETAIL_MAKE_DATA_TYPE(FormatDataKind(type), (uint64_t)one);
+        });
+}
+
+NVCVStatus nvcvDataTypeGetStrideBytes(NVCVDataType type, int32_t *outStrideBytes)
+{
+    return Protect([&] { *NotNull(outStrideBytes, "Pointer to output") = DataTypeStrideBytes(type); });
+}
+
+const char *nvcvDataTypeGetName(NVCVDataType type)
+{
+    if (type == NVCV_DATA_TYPE_NONE)
+    {
+        return "NVCV_DATA_TYPE_NONE";
+    }
+    PackingInfo pi = DecodePacking(DataTypePacking(type));
+    if (pi.known && pi.numChannels > 0 && pi.bits[0] * pi.numChannels == pi.bitsPerPixel)
+    {
+        return pi.numChannels == 1
+                 ? ThreadName("NVCV_DATA_TYPE_%s%d", KindLetter(FormatDataKind(type)), pi.bits[0])
+                 : ThreadName("NVCV_DATA_TYPE_%d%s%d", pi.numChannels, KindLetter(FormatDataKind(type)), pi.bits[0]);
+    }
+    return ThreadName("NVCVDataType(%s,packing=%d)", nvcvDataKindGetName(FormatDataKind(type)),
+                      (int)DataTypePacking(type));
+}
+
+// ---- image format ------------------------------------------------------------------------------
+NVCVStatus nvcvMakeYCbCrImageFormat(NVCVImageFormat *outFormat, NVCVColorSpec colorSpec,
+                                    NVCVChromaSubsampling chromaSub, NVCVMemLayout memLayout, NVCVDataKind dataKind,
+                                    NVCVSwizzle swizzle, NVCVPacking packing0, NVCVPacking packing1,
+                                    NVCVPacking packing2, NVCVPacking packing3, NVCVAlphaType alphaType,
+                                    const NVCVExtraChannelInfo *exChannelInfo)
+{
+    return MakeFormat(outFormat, NVCV_COLOR_MODEL_YCbCr, colorSpec, chromaSub, memLayout, dataKind, swizzle, packing0,
+                      packing1, packing2, packing3, alphaType, exChannelInfo);
+}
+
+NVCVStatus nvcvMakeColorImageFormat(NVCVImageFormat *outFormat, NVCVColorModel colorModel, NVCVColorSpec colorSpec,
+                                    NVCVMemLayout memLayout, NVCVDataKind dataKind, NVCVSwizzle swizzle,
+                                    NVCVPacking packing0, NVCVPacking packing1, NVCVPacking packing2,
+                                    NVCVPacking packing3, NVCVAlphaType alphaType,
+                                    const NVCVExtraChannelInfo *exChannelInfo)
+{
+    if (colorModel == NVCV_COLOR_MODEL_YCbCr || colorModel == NVCV_COLOR_MODEL_UNDEFINED
+        || colorModel == NVCV_COLOR_MODEL_RAW)
+    {
+        return Protect(
+            [&] {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT,
+                            "Use the YCbCr / non-colour / raw constructors for colour model %s",
+                            nvcvColorModelGetName(colorModel));
+            });
+    }
+    return MakeFormat(outFormat, colorModel, colorSpec, NVCV_CSS_NONE, memLayout, dataKind, swizzle, packing0,
+                      packing1, packing2, packing3, alphaType, exChannelInfo);
+}
+
+NVCVStatus nvcvMakeNonColorImageFormat(NVCVImageFormat *outFormat, NVCVMemLayout memLayout, NVCVDataKind dataKind,
+                                       NVCVSwizzle swizzle, NVCVPacking packing0, NVCVPacking packing1,
+                                       NVCVPacking packing2, NVCVPacking packing3, NVCVAlphaType alphaType,
+                                       const NVCVExtraChannelInfo *exChannelInfo)
+{
+    return MakeFormat(outFormat, NVCV_COLOR_MODEL_UNDEFINED, 0, NVCV_CSS_NONE, memLayout, dataKind, swizzle, packing0,
+                      packing1, packing2, packing3, alphaType, exChannelInfo);
+}
+
+NVCVStatus nvcvImageFormatGetNumPlanes(NVCVImageFormat fmt, int32_t *outNumPlanes)
+{
+    return Protect([&] { *NotNull(outNumPlanes, "Pointer to output") = FormatNumPlanes(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetNumChannels(NVCVImageFormat fmt, int32_t *outNumChannels)
+{
+    return Protect([&] { *NotNull(outNumChannels, "Pointer to output") = FormatNumChannels(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetBitsPerChannel(NVCVImageFormat fmt, int32_t *bits)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(bits, "Pointer to output");
+            int n = 0;
+            for (int p = 0; p < 4; ++p)
+            {
+                NVCVPacking pk = FormatPlanePacking(fmt, p);
+                PackingInfo pi = DecodePacking(pk);
+                if (!pi.known)
+                {
+                    throw Error(NVCV_ERROR_INVALID_IMAGE_FORMAT, "Plane %d has an unknown packing", p);
+                }
+                if (pk == NVCV_PACKING_X8_Y8__X8_Z8 || pk == NVCV_PACKING_Y8_X8__Z8_X8)
+                {
+                    pi.bits[3] = 0; // the luma sample stored twice counts once
+                }
+                for (int c = 0; c < 4 && pi.bits[c] != 0; ++c)
+                {
+                    if (n >= 4)
+                    {
+                        throw Error(NVCV_ERROR_INVALID_IMAGE_FORMAT, "Planes hold more than 4 channels in total");
+                    }
+                    bits[n++] = pi.bits[c];
+                }
+            }
+            for (; n < 4; ++n)
+            {
+                bits[n] = 0;
+            }
+        });
+}
+
+NVCVStatus nvcvImageFormatGetPlanePacking(NVCVImageFormat fmt, int32_t plane, NVCVPacking *outPacking)
+{
+    return Protect(
+        [&]
+        {
+            CheckPlane(plane);
+            *NotNull(outPacking, "Pointer to output") = FormatPlanePacking(fmt, plane);
+        });
+}
+
+NVCVStatus nvcvImageFormatGetPlaneNumChannels(NVCVImageFormat fmt, int32_t plane, int32_t *outPlaneNumChannels)
+{
+    return Protect(
+        [&]
+        {
+            CheckPlane(plane);
+            *NotNull(outPlaneNumChannels, "Pointer to output") = DecodePacking(FormatPlanePacking(fmt, plane)).numChannels;
+        });
+}
+
+NVCVStatus nvcvImageFormatGetPlaneBitsPerPixel(NVCVImageFormat fmt, int32_t plane, int32_t *outBPP)
+{
+    return Protect(
+        [&]
+        {
+            CheckPlane(plane);
+            *NotNull(outBPP, "Pointer to output") = DecodePacking(FormatPlanePacking(fmt, plane)).bitsPerPixel;
+        });
+}
+
+NVCVStatus nvcvImageFormatGetPlanePixelStrideBytes(NVCVImageFormat fmt, int32_t plane, int32_t *outStrideBytes)
+{
+    return Protect(
+        [&]
+        {
+            CheckPlane(plane);
+            *NotNull(outStrideBytes, "Pointer to output") = FormatPlanePixelStrideBytes(fmt, plane);
+        });
+}
+
+NVCVStatus nvcvImageFormatGetPlaneDataType(NVCVImageFormat fmt, int32_t plane, NVCVDataType *outDataType)
+{
+    return Protect(
+        [&]
+        {
+            CheckPlane(plane);
+            *NotNull(outDataType, "Pointer to output") = FormatPlaneDataType(fmt, plane);
+        });
+}
+
+NVCVStatus nvcvImageFormatGetPlaneSize(NVCVImageFormat fmt, int32_t plane, int32_t imgWidth, int32_t imgHeight,
+                                       int32_t *outPlaneWidth, int32_t *outPlaneHeight)
+{
+    return Protect(
+        [&]
+        {
+            CheckPlane(plane);
+            int32_t w, h;
+            FormatPlaneSize(fmt, plane, imgWidth, imgHeight, &w, &h);
+            if (outPlaneWidth)
+            {
+                *outPlaneWidth = w;
+            }
+            if (outPlaneHeight)
+            {
+                *outPlaneHeight = h;
+            }
+        });
+}
+
+NVCVStatus nvcvImageFormatGetDataKind(NVCVImageFormat fmt, NVCVDataKind *outDataKind)
+{
+    return Protect([&] { *NotNull(outDataKind, "Pointer to output") = FormatDataKind(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetSwizzle(NVCVImageFormat fmt, NVCVSwizzle *outSwizzle)
+{
+    return Protect([&] { *NotNull(outSwizzle, "Pointer to output") = FormatSwizzle(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetMemLayout(NVCVImageFormat fmt, NVCVMemLayout *outMemLayout)
+{
+    return Protect([&] { *NotNull(outMemLayout, "Pointer to output") = FormatMemLayout(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetColorSpec(NVCVImageFormat fmt, NVCVColorSpec *outColorSpec)
+{
+    return Protect([&] { *NotNull(outColorSpec, "Pointer to output") = FormatColorSpec(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetColorModel(NVCVImageFormat fmt, NVCVColorModel *outColorModel)
+{
+    return Protect([&] { *NotNull(outColorModel, "Pointer to output") = FormatColorModel(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetChromaSubsampling(NVCVImageFormat fmt, NVCVChromaSubsampling *outCSS)
+{
+    return Protect([&] { *NotNull(outCSS, "Pointer to output") = FormatCSS(fmt); });
+}
+
+NVCVStatus nvcvImageFormatGetAlphaType(NVCVImageFormat fmt, NVCVAlphaType *outAlphaType)
+{
+    return Protect([&] { *NotNull(outAlphaType, "Pointer to output") = (NVCVAlphaType)NVCV_DETAIL_BITS_GET(fmt, 6, 1); });
+}
+
+NVCVStatus nvcvImageFormatHasSameDataLayout(NVCVImageFormat a, NVCVImageFormat b, int8_t *outBool)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outBool, "Pointer to output");
+            bool same = FormatNumPlanes(a) == FormatNumPlanes(b) && FormatCSS(a) == FormatCSS(b)
+                     && FormatMemLayout(a) == FormatMemLayout(b) && FormatDataKind(a) == FormatDataKind(b);
+            for (int p = 0; same && p < 4; ++p)
+            {
+                same = FormatPlanePacking(a, p) == FormatPlanePacking(b, p);
+            }
+            *outBool = same ? 1 : 0;
+        });
+}
+
+const char *nvcvImageFormatGetName(NVCVImageFormat fmt)
+{
+    if (fmt == NVCV_IMAGE_FORMAT_NONE)
+    {
+        return "NVCV_IMAGE_FORMAT_NONE";
+    }
+    static const struct
+    {
+        NVCVImageFormat fmt;
+        const char     *name;
+    } known[] = {
+#define F(x) {NVCV_IMAGE_FORMAT_##x, "NVCV_IMAGE_FORMAT_" #x}
+        F(U8),     F(S8),     F(U16),     F(S16),     F(U32),     F(S32),    F(F16),    F(F32),     F(F64),
+        F(2S16),   F(2F32),   F(Y8),      F(Y8_ER),   F(NV12),    F(NV12_ER), F(UYVY),  F(YUYV),    F(YUV8),
+        F(YUV8p),  F(RGB8),   F(BGR8),    F(RGBA8),   F(BGRA8),   F(RGBf32), F(BGRf32), F(RGBAf32), F(BGRAf32),
+        F(RGBf16), F(BGRf16), F(RGBAf16), F(BGRAf16), F(HSV8),    F(RGB8p),  F(BGR8p),  F(RGBA8p),  F(BGRA8p),
+        F(RGBf32p), F(BGRf32p), F(RGBAf32p), F(BGRAf32p), F(RGBf16p), F(BGRf16p),
+#undef F
+    };
+    for (const auto &k : known)
+    {
+        if (k.fmt == fmt)
+        {
+            return k.name;
+        }
+    }
+    return ThreadName("NVCVImageFormat(%s,%s,%s,%s,planes=%d)", nvcvColorModelGetName(FormatColorModel(fmt)),
+                      nvcvChromaSubsamplingGetName(FormatCSS(fmt)), nvcvDataKindGetName(FormatDataKind(fmt)),
+                      nvcvSwizzleGetName(FormatSwizzle(fmt)), FormatNumPlanes(fmt));
+}
+}

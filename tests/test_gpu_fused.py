@@ -1,0 +1,170 @@
+"""GPU parity of cvcudaResizeCropConvertReformat[VarShape]Submit against the CPU oracle.
+
+Rows follow the reference's own table (tests/cvcuda/system/TestOpResizeCropConvertReformat.cpp:232-329:
+sizes, resize targets, crops, interpolation, scale/offset, srcCast, layouts) with its deterministic
+input recipe (x+y+c)&255 (:198-221), plus seeded random inputs and the benchmark configuration.
+Tolerances: nearest bit-exact; u8 output <= 1 LSB; f32 output |d| <= 1e-5*max(1,|ref|).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+NEAREST, LINEAR = 0, 1
+
+
+def ramp(n, h, w):
+    y, x, c = np.meshgrid(np.arange(h), np.arange(w), np.arange(3), indexing="ij")
+    img = ((x + y + c) & 255).astype(np.uint8)
+    return np.stack([np.roll(img, i, axis=1) for i in range(n)])
+
+
+def run_tensor(cv, src, out_hw, resize_dim, crop, interp, out_dtype, planar, manip, scale, offset, src_cast,
+               batch_dim=True):
+    n = src.shape[0]
+    tin = cv.Tensor.from_numpy(src if batch_dim else src[0], "NHWC" if batch_dim else "HWC")
+    h, w = out_hw
+    if planar:
+        shape, layout = ([n, 3, h, w], "NCHW") if batch_dim else ([3, h, w], "CHW")
+    else:
+        shape, layout = ([n, h, w, 3], "NHWC") if batch_dim else ([h, w, 3], "HWC")
+    tout = cv.Tensor.alloc(shape, out_dtype, layout)
+    tout.torch_view().zero_()
+    op = cv.ResizeCropConvertReformat()
+    op(None, tin, tout, resize_dim, interp, crop, manip, scale, offset, src_cast)
+    torch.cuda.synchronize()
+    res = tout.numpy()
+    return res if batch_dim else res[None]
+
+
+def compare(res, ref, interp, out_dtype):
+    assert res.shape == ref.shape
+    if out_dtype == np.uint8:
+        d = np.abs(res.astype(np.int32) - ref.astype(np.int32))
+        assert d.max() <= (0 if interp == NEAREST else 1), "max diff %d" % d.max()
+    else:
+        if interp == NEAREST:
+            np.testing.assert_array_equal(res, ref)
+        else:
+            tol = 1e-5 * np.maximum(1.0, np.abs(ref))
+            bad = np.abs(res - ref) > tol
+            assert not bad.any(), "max err %g at %d elements" % (np.abs(res - ref).max(), bad.sum())
+
+
+# srcW, srcH, newW, newH, cropX, cropY, outW, outH, N, interp, out dtype, planar, manip, scale, offset, srcCast
+ROWS = [
+    (8, 8, 8, 8, 0, 0, 8, 8, 1, NEAREST, np.uint8, False, 0, 1.0, 0.0, True),
+    (8, 8, 8, 8, 0, 0, 8, 8, 1, LINEAR, np.uint8, False, 0, 1.0, 0.0, True),
+    (8, 8, 16, 16, 0, 0, 16, 16, 2, LINEAR, np.uint8, False, 0, 1.0, 0.0, True),
+    (42, 48, 23, 24, 0, 0, 23, 24, 2, NEAREST, np.uint8, False, 0, 1.0, 0.0, True),
+    (42, 40, 21, 20, 0, 0, 21, 20, 2, LINEAR, np.uint8, True, 1, 1.0, 0.0, True),
+    (17, 151, 23, 191, 1, 2, 21, 185, 3, LINEAR, np.float32, True, 0, 1.0, 0.0, False),
+    (353, 450, 256, 326, 16, 51, 224, 224, 3, LINEAR, np.float32, True, 1, 1 / 127.5, -1.0, False),
+    (353, 450, 256, 326, 16, 51, 224, 224, 2, LINEAR, np.float32, False, 0, 1 / 255.0, 0.0, True),
+    (353, 450, 256, 326, 16, 51, 224, 224, 2, NEAREST, np.float32, True, 1, 1 / 127.5, -1.0, False),
+    (1080, 1920, 400, 711, 88, 243, 224, 224, 2, LINEAR, np.uint8, True, 0, 1.0, 0.0, True),
+    (1920, 1080, 455, 256, 115, 16, 224, 224, 2, LINEAR, np.float32, True, 0, 1 / (255 * 0.226), -0.449 / 0.226, False),
+    (1920, 1080, 455, 256, 115, 16, 224, 224, 2, NEAREST, np.uint8, False, 1, 1.0, 0.0, False),
+    (640, 480, 1280, 960, 100, 50, 1000, 800, 1, LINEAR, np.float32, True, 0, 2.0, -3.0, False),
+    (31, 29, 97, 93, 0, 0, 97, 93, 1, NEAREST, np.float32, False, 0, 0.5, 0.25, False),
+]
+
+
+@pytest.mark.parametrize("row", ROWS, ids=lambda r: "%dx%d-%dx%d-%s-%s%s" % (
+    r[0], r[1], r[6], r[7], "nn" if r[9] == 0 else "lin", np.dtype(r[10]).name, "p" if r[11] else "i"))
+@pytest.mark.parametrize("data", ["ramp", "random"])
+def test_tensor_rows(cv, orc, gpu, row, data):
+    sw, sh, nw, nh, cx, cy, ow, oh, n, interp, odt, planar, manip, scale, offset, cast = row
+    src = ramp(n, sh, sw) if data == "ramp" else orc.fill_u8((n, sh, sw, 3), 0xC0FFEE00 + sw * 7 + sh)
+    ref = orc.fused_rccr(src, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast, order=0)
+    res = run_tensor(cv, src, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast)
+    compare(res, ref, interp, odt)
+    # the device-order restatement must agree with the golden-order one within the same bar
+    ref1 = orc.fused_rccr(src, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast, order=1)
+    compare(ref1, ref, interp, odt)
+
+
+def test_single_image_layouts(cv, orc, gpu):
+    src = orc.fill_u8((1, 37, 53, 3), 11)
+    for planar in (True, False):
+        ref = orc.fused_rccr(src, (20, 30), (40, 24), (3, 2), LINEAR, np.float32, planar, 0, 0.25, 1.0, False)
+        res = run_tensor(cv, src, (20, 30), (40, 24), (3, 2), LINEAR, np.float32, planar, 0, 0.25, 1.0, False,
+                         batch_dim=False)
+        compare(res, ref, LINEAR, np.float32)
+
+
+def test_identity_and_constant_closed_forms(cv, gpu):
+    # resize to the source size with no crop is an exact cast; a constant image maps to scale*k+offset
+    rng = np.random.default_rng(5)
+    src = rng.integers(0, 256, (2, 19, 23, 3), dtype=np.uint8)
+    res = run_tensor(cv, src, (19, 23), (23, 19), (0, 0), LINEAR, np.float32, False, 0, 1.0, 0.0, False)
+    np.testing.assert_array_equal(res, src.astype(np.float32))
+    const = np.full((1, 64, 48, 3), 77, np.uint8)
+    res = run_tensor(cv, const, (20, 20), (30, 33), (5, 6), LINEAR, np.float32, True, 0, 0.5, 3.0, False)
+    np.testing.assert_array_equal(res, np.full((1, 3, 20, 20), np.float32(0.5) * 77 + np.float32(3.0), np.float32))
+
+
+def test_pitched_unaligned_source_view(cv, orc, gpu):
+    # source tensor that is a window into a larger buffer: odd base address, pitch not a multiple of 4,
+    # last row ends exactly at the end of the allocation (exercises the tail path of the 8-byte loads)
+    H, W = 45, 71
+    pitch = W * 3 + 5
+    host = orc.fill_u8((2 * H * pitch + 1,), 99)
+    buf = torch.from_numpy(host).cuda()
+    base = 1
+    nbytes = (2 * H - 1) * pitch + W * 3
+    assert base + nbytes <= buf.numel()
+    view = buf[base:base + nbytes]
+    tin = cv.Tensor.wrap(view.data_ptr(), [2, H, W, 3], [H * pitch, pitch, 3, 1], np.uint8, "NHWC", keep=buf)
+    src = np.stack([host[base + n * H * pitch: base + n * H * pitch + H * pitch - 5 + 5][: H * pitch]
+                    .reshape(-1)[: (H - 1) * pitch + W * 3 if n == 1 else H * pitch] for n in range(2)], axis=0) \
+        if False else None
+    dense = np.zeros((2, H, W, 3), np.uint8)
+    for n in range(2):
+        for y in range(H):
+            o = base + n * H * pitch + y * pitch
+            dense[n, y] = host[o:o + W * 3].reshape(W, 3)
+    tout = cv.Tensor.alloc([2, 3, 30, 40], np.float32, "NCHW")
+    op = cv.ResizeCropConvertReformat()
+    op(None, tin, tout, (50, 33), LINEAR, (4, 2), 0, 1.0, 0.0, False)
+    torch.cuda.synchronize()
+    ref = orc.fused_rccr(dense, (30, 40), (50, 33), (4, 2), LINEAR, np.float32, True)
+    compare(tout.numpy(), ref, LINEAR, np.float32)
+    del src
+
+
+def test_varshape(cv, K, orc, gpu):
+    rng = np.random.default_rng(3)
+    sizes = [(int(rng.integers(60, 140)), int(rng.integers(50, 120))) for _ in range(5)]
+    for interp, odt, planar in ((LINEAR, np.float32, True), (NEAREST, np.uint8, False), (LINEAR, np.uint8, True)):
+        batch = cv.ImageBatchVarShape(8)
+        hosts = []
+        for i, (w, h) in enumerate(sizes):
+            a = orc.fill_u8((h, w, 3), 1000 + i)
+            hosts.append(a)
+            batch.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_RGB8))
+        shape, layout = ([5, 3, 32, 40], "NCHW") if planar else ([5, 32, 40, 3], "NHWC")
+        tout = cv.Tensor.alloc(shape, odt, layout)
+        op = cv.ResizeCropConvertReformat()
+        op(None, batch, tout, (48, 40), interp, (4, 3), 1, 0.5, 1.0, False)
+        torch.cuda.synchronize()
+        res = tout.numpy()
+        for i, a in enumerate(hosts):
+            ref = orc.fused_rccr(a[None], (32, 40), (48, 40), (4, 3), interp, odt, planar, 1, 0.5, 1.0, False)
+            compare(res[i:i + 1], ref, interp, odt)
+
+
+def test_benchmark_config_full_size(cv, orc, gpu):
+    # BASELINE config 2 at full size: batch 64 of 1080p; oracle on 4 threads over a subset of images,
+    # plus a size-independent property on the whole batch: identical images give identical outputs.
+    N = 64
+    one = orc.fill_u8((4, 1080, 1920, 3), 0xC0FFEE02)
+    src = np.concatenate([one] * (N // 4))
+    res = run_tensor(cv, src, (224, 224), (455, 256), (115, 16), LINEAR, np.float32, True, 0,
+                     1 / (255 * 0.226), -0.449 / 0.226, False)
+    ref = orc.fused_rccr(one, (224, 224), (455, 256), (115, 16), LINEAR, np.float32, True, 0,
+                         1 / (255 * 0.226), -0.449 / 0.226, False, threads=4)
+    compare(res[:4], ref, LINEAR, np.float32)
+    for k in range(1, N // 4):
+        np.testing.assert_array_equal(res[4 * k:4 * k + 4], res[:4])
