@@ -1,0 +1,441 @@
+// Resize with nearest / bilinear / bicubic sampling, tensors and var-shape batches.
+//
+// Index maps and weights follow the reference kernels expression for expression in float32
+// (src/cvcuda/priv/OpResize.cu:142-164 nearest, 177-330 bilinear, 334-388 bicubic;
+// src/cvcuda/priv/legacy/resize_var_shape.cu:92-231 for the var-shape association of the sums).
+// The nearest-neighbour source index uses the single-multiply form floor((d+.5f)*scale) of the
+// reference's CPU golden (tests/cvcuda/system/ResizeUtils.cpp:206-221) for every pixel, so results
+// are bit-exact against it also where the coordinate lands on an integer.
+//
+// Kernel shape: one lane per output pixel, a 256-thread block covers 64 columns x 4 rows; pixels
+// are moved as whole C-channel vectors (one load/store instruction each where the element size
+// allows), outputs use streaming stores. Var-shape batches run on a packed tile grid.
+#include "DeviceUtils.hpp"
+#include "OpCommon.hpp"
+#include "VarShapeTiles.hpp"
+
+#include <cvcuda/OpResize.h>
+
+#include <algorithm>
+
+namespace cvamd {
+
+namespace {
+
+constexpr int kTileW = 64;
+constexpr int kTileH = 4;
+
+// C interleaved elements of type T, naturally aligned to one element: the compiler may merge the
+// accesses into wider instructions (unaligned vector access is legal on gfx950).
+template<class T, int C>
+struct __attribute__((packed, aligned(sizeof(T)))) Pixel
+{
+    T v[C];
+};
+
+struct ResizeArgs
+{
+    // tensors
+    const uint8_t *srcBase;
+    uint8_t       *dstBase;
+    int64_t        srcSampleStride, dstSampleStride;
+    int32_t        srcRowStride, dstRowStride;
+    int32_t        srcW, srcH, dstW, dstH;
+    // var-shape
+    const NVCVImageBufferStrided *srcList;
+    const NVCVImageBufferStrided *dstList;
+};
+
+struct Plane
+{
+    const uint8_t *src;
+    uint8_t       *dst;
+    int32_t        srcRow, dstRow, srcW, srcH, dstW, dstH;
+};
+
+template<bool VARSHAPE>
+__device__ __forceinline__ Plane GetPlanes(const ResizeArgs &a, int n)
+{
+    Plane p;
+    if constexpr (VARSHAPE)
+    {
+        const NVCVImagePlaneStrided &s = a.srcList[n].planes[0];
+        const NVCVImagePlaneStrided &d = a.dstList[n].planes[0];
+        p = {s.basePtr, d.basePtr, s.rowStride, d.rowStride, s.width, s.height, d.width, d.height};
+    }
+    else
+    {
+        p = {a.srcBase + n * a.srcSampleStride,
+             a.dstBase + n * a.dstSampleStride,
+             a.srcRowStride,
+             a.dstRowStride,
+             a.srcW,
+             a.srcH,
+             a.dstW,
+             a.dstH};
+    }
+    return p;
+}
+
+template<class T, int C>
+__device__ __forceinline__ Pixel<T, C> LoadPx(const uint8_t *row, int x)
+{
+    return reinterpret_cast<const Pixel<T, C> *>(row)[x];
+}
+
+template<class T, int C>
+__device__ __forceinline__ void StorePx(uint8_t *row, int x, const Pixel<T, C> &px)
+{
+    Pixel<T, C> *p = reinterpret_cast<Pixel<T, C> *>(row) + x;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        __builtin_nontemporal_store(px.v[c], &p->v[c]);
+    }
+}
+
+__device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
+{
+    constexpr float A = -0.75f;
+    w[0]              = ((A * (d + 1) - 5 * A) * (d + 1) + 8 * A) * (d + 1) - 4 * A;
+    w[1]              = ((A + 2) * d - (A + 3)) * d * d + 1;
+    w[2]              = ((A + 2) * (1 - d) - (A + 3)) * (1 - d) * (1 - d) + 1;
+    w[3]              = 1.f - w[0] - w[1] - w[2];
+}
+
+template<class T, int C, int INTERP, bool VARSHAPE>
+__device__ __forceinline__ void ResizePixel(const Plane &p, int dx, int dy)
+{
+    const float scaleX = static_cast<float>(p.srcW) / p.dstW;
+    const float scaleY = static_cast<float>(p.srcH) / p.dstH;
+    uint8_t    *dstRow = p.dst + (int64_t)dy * p.dstRow;
+    Pixel<T, C> out;
+
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        const int sx = min((int)floorf(scaleX * (dx + 0.5f)), p.srcW - 1);
+        const int sy = min((int)floorf(scaleY * (dy + 0.5f)), p.srcH - 1);
+        out          = LoadPx<T, C>(p.src + (int64_t)sy * p.srcRow, sx);
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const float fx = (dx + .5f) * scaleX - .5f;
+        const float fy = (dy + .5f) * scaleY - .5f;
+        int         sx = (int)floorf(fx);
+        int         sy = (int)floorf(fy);
+        const float wx = (sx < 0) ? 0.f : ((sx > p.srcW - 2) ? 1.f : fx - sx);
+        const float wy = (sy < 0) ? 0.f : ((sy > p.srcH - 2) ? 1.f : fy - sy);
+        sx             = max(0, min(sx, p.srcW - 2));
+        sy             = max(0, min(sy, p.srcH - 2));
+        // a 1-pixel-wide (or -high) source has no second tap: reuse the first (its weight is then 0 or
+        // multiplies an equal value)
+        const int sx1 = min(sx + 1, p.srcW - 1);
+        sx            = max(sx, 0);
+        const uint8_t *r0 = p.src + (int64_t)max(sy, 0) * p.srcRow;
+        const uint8_t *r1 = p.src + (int64_t)min(sy + 1, p.srcH - 1) * p.srcRow;
+        const Pixel<T, C> p00 = LoadPx<T, C>(r0, sx), p01 = LoadPx<T, C>(r0, sx1);
+        const Pixel<T, C> p10 = LoadPx<T, C>(r1, sx), p11 = LoadPx<T, C>(r1, sx1);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            float v;
+            if constexpr (VARSHAPE)
+            {
+                v = (1.0f - wx) * ((float)p00.v[c] * (1.0f - wy) + (float)p10.v[c] * wy)
+                  + wx * ((float)p01.v[c] * (1.0f - wy) + (float)p11.v[c] * wy);
+            }
+            else
+            {
+                v = (float)p00.v[c] * ((1.f - wx) * (1.f - wy)) + (float)p01.v[c] * (wx * (1.f - wy))
+                  + (float)p10.v[c] * ((1.f - wx) * wy) + (float)p11.v[c] * (wx * wy);
+            }
+            out.v[c] = SaturateCast<T>(v);
+        }
+    }
+    else // cubic
+    {
+        const float cx = (dx + .5f) * scaleX - .5f;
+        const float cy = (dy + .5f) * scaleY - .5f;
+        int         sx = (int)floorf(cx);
+        int         sy = (int)floorf(cy);
+        float       fx = cx - sx;
+        const float fy = cy - sy;
+        fx             = (sx < 1 || sx >= p.srcW - 3) ? 0.f : fx;
+        sy             = max(1, min(sy, p.srcH - 3));
+        sx             = max(1, min(sx, p.srcW - 3));
+        float wx[4], wy[4];
+        CubicCoeffs(fx, wx);
+        CubicCoeffs(fy, wy);
+        float sum[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            sum[c] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            // sources narrower/lower than 4 pixels: clamp the taps into the image
+            const int      yy  = max(0, min(sy - 1 + j, p.srcH - 1));
+            const uint8_t *row = p.src + (int64_t)yy * p.srcRow;
+            Pixel<T, C>    t[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                t[i] = LoadPx<T, C>(row, max(0, min(sx - 1 + i, p.srcW - 1)));
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                if constexpr (VARSHAPE)
+                {
+                    sum[c] += wy[j]
+                            * (wx[0] * (float)t[0].v[c] + wx[1] * (float)t[1].v[c] + wx[2] * (float)t[2].v[c]
+                               + wx[3] * (float)t[3].v[c]);
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        sum[c] += (float)t[i].v[c] * (wx[i] * wy[j]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out.v[c] = SaturateCast<T>(fabsf(sum[c]));
+        }
+    }
+    StorePx<T, C>(dstRow, dx, out);
+}
+
+template<class T, int C, int INTERP>
+__global__ __launch_bounds__(256) void ResizeTensorKernel(const ResizeArgs a)
+{
+    const int dx = blockIdx.x * kTileW + (threadIdx.x & 63);
+    const int dy = blockIdx.y * kTileH + (threadIdx.x >> 6);
+    if (dx >= a.dstW || dy >= a.dstH)
+    {
+        return;
+    }
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizePixel<T, C, INTERP, false>(p, dx, dy);
+}
+
+template<class T, int C, int INTERP>
+__global__ __launch_bounds__(256) void ResizeVarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc = LocateTile(tiles, blockIdx.x);
+    const Plane     p  = GetPlanes<true>(a, tc.image);
+    const int       dx = tc.tx * kTileW + (threadIdx.x & 63);
+    const int       dy = tc.ty * kTileH + (threadIdx.x >> 6);
+    if (dx >= p.dstW || dy >= p.dstH)
+    {
+        return;
+    }
+    ResizePixel<T, C, INTERP, true>(p, dx, dy);
+}
+
+template<class T, int C, int INTERP>
+void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
+{
+    dim3 grid(DivUp(a.dstW, kTileW), DivUp(a.dstH, kTileH), N);
+    hipLaunchKernelGGL((ResizeTensorKernel<T, C, INTERP>), grid, dim3(256), 0, stream, a);
+    CheckLaunch("ResizeTensorKernel");
+}
+
+template<class T, int C, int INTERP>
+void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, int N, hipStream_t stream)
+{
+    for (int first = 0; first < N; first += kMaxTileImages)
+    {
+        VarTiles tiles;
+        int      total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kTileW, kTileH);
+        if (total > 0)
+        {
+            hipLaunchKernelGGL((ResizeVarShapeKernel<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a, tiles);
+            CheckLaunch("ResizeVarShapeKernel");
+        }
+    }
+}
+
+template<class T, int C>
+void DispatchInterp(bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, int N, int interp,
+                    hipStream_t stream)
+{
+    switch (interp)
+    {
+    case NVCV_INTERP_NEAREST:
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_NEAREST>(a, dstHost, N, stream)
+                 : LaunchTensor<T, C, NVCV_INTERP_NEAREST>(a, N, stream);
+        break;
+    case NVCV_INTERP_LINEAR:
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_LINEAR>(a, dstHost, N, stream)
+                 : LaunchTensor<T, C, NVCV_INTERP_LINEAR>(a, N, stream);
+        break;
+    case NVCV_INTERP_CUBIC:
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_CUBIC>(a, dstHost, N, stream)
+                 : LaunchTensor<T, C, NVCV_INTERP_CUBIC>(a, N, stream);
+        break;
+    default:
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid interpolation (supported: NEAREST, LINEAR, CUBIC)");
+    }
+}
+
+template<class T>
+void DispatchChannels(int channels, bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, int N,
+                      int interp, hipStream_t stream)
+{
+    switch (channels)
+    {
+    case 1:
+        DispatchInterp<T, 1>(varshape, a, dstHost, N, interp, stream);
+        break;
+    case 3:
+        DispatchInterp<T, 3>(varshape, a, dstHost, N, interp, stream);
+        break;
+    case 4:
+        DispatchInterp<T, 4>(varshape, a, dstHost, N, interp, stream);
+        break;
+    default:
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input data type");
+    }
+}
+
+void DispatchType(ElemType elem, int channels, bool varshape, const ResizeArgs &a,
+                  const NVCVImageBufferStrided *dstHost, int N, int interp, hipStream_t stream)
+{
+    if (N == 0)
+    {
+        return;
+    }
+    switch (elem)
+    {
+    case kU8:
+        DispatchChannels<uint8_t>(channels, varshape, a, dstHost, N, interp, stream);
+        break;
+    case kU16:
+        DispatchChannels<uint16_t>(channels, varshape, a, dstHost, N, interp, stream);
+        break;
+    case kS16:
+        DispatchChannels<int16_t>(channels, varshape, a, dstHost, N, interp, stream);
+        break;
+    case kF32:
+        DispatchChannels<float>(channels, varshape, a, dstHost, N, interp, stream);
+        break;
+    default:
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input data type");
+    }
+}
+
+class Resize final : public IOperator
+{
+public:
+    void submit(hipStream_t stream, NVCVTensorHandle hin, NVCVTensorHandle hout, NVCVInterpolationType interp) const
+    {
+        NVCVTensorData din, dout;
+        ExportTensor(hin, din, "Input");
+        ExportTensor(hout, dout, "Output");
+        if (din.dtype != dout.dtype)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input and output data type are different");
+        }
+        if (nvcvTensorLayoutCompare(din.layout, dout.layout) != 0)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input and output data layout are different");
+        }
+        if (nvcvTensorLayoutCompare(din.layout, NVCV_TENSOR_HWC) != 0
+            && nvcvTensorLayoutCompare(din.layout, NVCV_TENSOR_NHWC) != 0)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input must have (N)HWC layout");
+        }
+        ImageBatchView in  = RequireImageBatchView(din, "Input", NVCV_ERROR_INVALID_ARGUMENT);
+        ImageBatchView out = RequireImageBatchView(dout, "Output", NVCV_ERROR_INVALID_ARGUMENT);
+        if (in.N != out.N)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input and output samples are different");
+        }
+        if (in.C != out.C)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input and output channels are different");
+        }
+        if (in.C > 4 || in.C < 1)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid number of channels");
+        }
+        if (std::max(in.bytesSpanned(), out.bytesSpanned()) > INT32_MAX)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input or output tensors are too large");
+        }
+        ResizeArgs a      = {};
+        a.srcBase         = in.base;
+        a.dstBase         = out.base;
+        a.srcSampleStride = in.strideN;
+        a.dstSampleStride = out.strideN;
+        a.srcRowStride    = (int32_t)in.strideH;
+        a.dstRowStride    = (int32_t)out.strideH;
+        a.srcW            = in.W;
+        a.srcH            = in.H;
+        a.dstW            = out.W;
+        a.dstH            = out.H;
+        if (out.W == 0 || out.H == 0)
+        {
+            return;
+        }
+        DispatchType(in.elem, in.C, false, a, nullptr, in.N, interp, stream);
+    }
+
+    void submit(hipStream_t stream, NVCVImageBatchHandle hin, NVCVImageBatchHandle hout,
+                NVCVInterpolationType interp) const
+    {
+        VarShapeView in  = ExportVarShape(hin, stream, "Input");
+        VarShapeView out = ExportVarShape(hout, stream, "Output");
+        if (in.N != out.N)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input and output batch sizes: %d != %d", in.N, out.N);
+        }
+        if (in.uniqueFormat == NVCV_IMAGE_FORMAT_NONE || in.uniqueFormat != out.uniqueFormat)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "All images in the input and output batches must share one format");
+        }
+        FormatInfo fi = DecodeFormat(in.uniqueFormat);
+        if (fi.planes != 1)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Images must have a single interleaved plane");
+        }
+        ResizeArgs a = {};
+        a.srcList    = in.data.buffer.varShapeStrided.imageList;
+        a.dstList    = out.data.buffer.varShapeStrided.imageList;
+        DispatchType(fi.elem, fi.channels, true, a, out.hostList, in.N, interp, stream);
+    }
+};
+
+} // namespace
+} // namespace cvamd
+
+using namespace cvamd;
+
+extern "C"
+{
+CVCUDA_PUBLIC NVCVStatus cvcudaResizeCreate(NVCVOperatorHandle *handle)
+{
+    return CreateOperator<Resize>(handle);
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaResizeSubmit(NVCVOperatorHandle handle, hipStream_t stream, NVCVTensorHandle in,
+                                            NVCVTensorHandle out, const NVCVInterpolationType interpolation)
+{
+    return Protect([&] { ToOperator<Resize>(handle).submit(stream, in, out, interpolation); });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaResizeVarShapeSubmit(NVCVOperatorHandle handle, hipStream_t stream,
+                                                    NVCVImageBatchHandle in, NVCVImageBatchHandle out,
+                                                    const NVCVInterpolationType interpolation)
+{
+    return Protect([&] { ToOperator<Resize>(handle).submit(stream, in, out, interpolation); });
+}
+}

@@ -307,6 +307,8 @@ public:
     Allocator(const NVCVResourceAllocator *custom, int32_t n)
         : Allocator()
     {
+        // Validate everything before taking ownership of any entry: if construction fails the
+        // caller keeps its contexts and no cleanup callback must run.
         bool seen[NVCV_NUM_RESOURCE_TYPES] = {};
         for (int i = 0; i < n; ++i)
         {
@@ -324,8 +326,11 @@ public:
             {
                 throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Custom allocation and deallocation functions must not be NULL");
             }
-            seen[c.resType]  = true;
-            m_res[c.resType] = c;
+            seen[c.resType] = true;
+        }
+        for (int i = 0; i < n; ++i)
+        {
+            m_res[custom[i].resType] = custom[i];
         }
     }
 

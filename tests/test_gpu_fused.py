@@ -68,6 +68,9 @@ ROWS = [
     (1920, 1080, 455, 256, 115, 16, 224, 224, 2, NEAREST, np.uint8, False, 1, 1.0, 0.0, False),
     (640, 480, 1280, 960, 100, 50, 1000, 800, 1, LINEAR, np.float32, True, 0, 2.0, -3.0, False),
     (31, 29, 97, 93, 0, 0, 97, 93, 1, NEAREST, np.float32, False, 0, 0.5, 0.25, False),
+    (1, 1, 2, 2, 0, 0, 2, 2, 2, LINEAR, np.float32, True, 0, 1.0, 0.0, False),   # images smaller than one 8-byte load
+    (2, 1, 5, 3, 1, 0, 3, 3, 1, LINEAR, np.uint8, False, 1, 1.0, 0.0, True),
+    (3, 1, 7, 2, 0, 0, 7, 2, 1, LINEAR, np.float32, False, 0, 1.0, 0.0, False),  # exactly 9 bytes: shifted tail load
 ]
 
 
@@ -102,7 +105,7 @@ def test_identity_and_constant_closed_forms(cv, gpu):
     np.testing.assert_array_equal(res, src.astype(np.float32))
     const = np.full((1, 64, 48, 3), 77, np.uint8)
     res = run_tensor(cv, const, (20, 20), (30, 33), (5, 6), LINEAR, np.float32, True, 0, 0.5, 3.0, False)
-    np.testing.assert_array_equal(res, np.full((1, 3, 20, 20), np.float32(0.5) * 77 + np.float32(3.0), np.float32))
+    assert np.abs(res - (0.5 * 77 + 3.0)).max() <= 0.5 * 4 * 77 * np.finfo(np.float32).eps
 
 
 def test_pitched_unaligned_source_view(cv, orc, gpu):
@@ -117,9 +120,6 @@ def test_pitched_unaligned_source_view(cv, orc, gpu):
     assert base + nbytes <= buf.numel()
     view = buf[base:base + nbytes]
     tin = cv.Tensor.wrap(view.data_ptr(), [2, H, W, 3], [H * pitch, pitch, 3, 1], np.uint8, "NHWC", keep=buf)
-    src = np.stack([host[base + n * H * pitch: base + n * H * pitch + H * pitch - 5 + 5][: H * pitch]
-                    .reshape(-1)[: (H - 1) * pitch + W * 3 if n == 1 else H * pitch] for n in range(2)], axis=0) \
-        if False else None
     dense = np.zeros((2, H, W, 3), np.uint8)
     for n in range(2):
         for y in range(H):
@@ -131,7 +131,6 @@ def test_pitched_unaligned_source_view(cv, orc, gpu):
     torch.cuda.synchronize()
     ref = orc.fused_rccr(dense, (30, 40), (50, 33), (4, 2), LINEAR, np.float32, True)
     compare(tout.numpy(), ref, LINEAR, np.float32)
-    del src
 
 
 def test_varshape(cv, K, orc, gpu):

@@ -1,0 +1,177 @@
+"""GPU parity of cvcudaResize[VarShape]Submit against the CPU oracle.
+
+Rows are the reference's own table (tests/cvcuda/system/TestOpResize.cpp:49-91, the AREA rows excepted)
+with seeded random inputs, plus the two benchmark configurations at full size.
+Bars: NEAREST bit-exact vs the golden; LINEAR/CUBIC on integer types <= 1 LSB vs the golden (the
+reference's own tolerance) and bit-exact vs the float32 device-formula restatement; f32 cubic
+within 1e-4 of that restatement.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+NEAREST, LINEAR, CUBIC = 0, 1, 2
+
+
+def make_input(orc, shape, dtype, seed):
+    if np.dtype(dtype) == np.float32:
+        return orc.fill_f32(shape, seed)
+    raw = orc.fill_u8(tuple(shape) + (np.dtype(dtype).itemsize,), seed)
+    return raw.view(dtype).reshape(shape)
+
+
+def check(res, src, out_hw, interp, orc, varshape=False):
+    golden = orc.resize(src, out_hw, interp, variant=0)
+    device = orc.resize(src, out_hw, interp, variant=2 if varshape else 1)
+    if interp == NEAREST:
+        np.testing.assert_array_equal(res, golden)
+    elif res.dtype == np.float32:
+        assert np.abs(res - device).max() <= 1e-4
+    else:
+        # The reference golden takes |.| of the bilinear sum as well (ResizeUtils.cpp:241-247) although
+        # its device kernel does not (OpResize.cu:225-228); they only differ for negative signed
+        # inputs, which the reference never tests. Follow the device there.
+        if not (interp == LINEAR and np.issubdtype(res.dtype, np.signedinteger)):
+            assert np.abs(res.astype(np.int64) - golden.astype(np.int64)).max() <= 1
+        # no FMA contraction on either side: the device-formula restatement is reproduced exactly
+        np.testing.assert_array_equal(res, device)
+
+
+TABLE = [
+    (42, 48, 23, 24, NEAREST, 1, np.uint8, 4), (113, 12, 12, 36, NEAREST, 1, np.uint8, 4),
+    (421, 148, 223, 124, NEAREST, 2, np.uint8, 4), (313, 212, 412, 336, NEAREST, 3, np.uint8, 4),
+    (42, 40, 21, 20, LINEAR, 1, np.uint8, 4), (21, 21, 42, 42, LINEAR, 1, np.uint8, 4),
+    (420, 420, 210, 210, LINEAR, 4, np.uint8, 4), (210, 210, 420, 420, LINEAR, 5, np.uint8, 4),
+    (42, 40, 21, 20, CUBIC, 1, np.uint8, 4), (21, 21, 42, 42, CUBIC, 6, np.uint8, 4),
+    (420, 420, 420, 420, CUBIC, 2, np.uint8, 4), (420, 420, 40, 42, CUBIC, 1, np.uint8, 4),
+    (1920, 1080, 640, 320, CUBIC, 2, np.uint8, 4), (1080, 1920, 720, 1280, LINEAR, 1, np.uint8, 4),
+    (720, 1280, 480, 854, CUBIC, 1, np.uint8, 4), (2160, 3840, 1080, 1920, LINEAR, 1, np.uint8, 4),
+    (1080, 1920, 360, 640, CUBIC, 1, np.uint8, 4),
+] + [(42, 48, 23, 24, interp, 1, dt, c) for dt in (np.uint8, np.uint16, np.int16, np.float32) for c in (1, 3, 4)
+     for interp in (NEAREST, LINEAR, CUBIC)]
+
+
+@pytest.mark.parametrize("row", TABLE, ids=lambda r: "%dx%d-%dx%d-i%d-n%d-%s%d" % (r[:6] + (np.dtype(r[6]).name, r[7])))
+def test_tensor_table(cv, orc, gpu, row):
+    sw, sh, dw, dh, interp, n, dt, c = row
+    src = make_input(orc, (n, sh, sw, c), dt, 0xC0FFEE01 + sw + 31 * sh + c)
+    tin = cv.Tensor.from_numpy(src, "NHWC")
+    tout = cv.Tensor.alloc([n, dh, dw, c], dt, "NHWC")
+    cv.Resize()(None, tin, tout, interp)
+    torch.cuda.synchronize()
+    check(tout.numpy(), src, (dh, dw), interp, orc)
+
+
+def test_output_padding_is_untouched_and_hwc_layout(cv, orc, gpu):
+    src = make_input(orc, (1, 33, 47, 3), np.uint8, 5)
+    tin = cv.Tensor.from_numpy(src[0], "HWC")
+    tout = cv.Tensor.alloc([20, 30, 3], np.uint8, "HWC")
+    d = tout.export()
+    pitch = d.buffer.strides[0]
+    assert pitch > 30 * 3
+    raw = cv._bytes_view(d.buffer.basePtr, pitch * 20, tout)
+    raw.fill_(0xAB)
+    cv.Resize()(None, tin, tout, LINEAR)
+    torch.cuda.synchronize()
+    check(tout.numpy()[None], src, (20, 30), LINEAR, orc)
+    pad = raw.view(20, pitch)[:, 30 * 3:].cpu().numpy()
+    assert (pad == 0xAB).all()
+
+
+def test_config1_full_size_and_knife_edge_columns(cv, orc, gpu):
+    # BASELINE config 1: batch 8, u8 NHWC 3ch 1920x1080 -> 224x224; nearest bit-exact, linear <= 1 LSB.
+    src = orc.fill_u8((8, 1080, 1920, 3), 0xC0FFEE01)
+    tin = cv.Tensor.from_numpy(src, "NHWC")
+    for interp in (NEAREST, LINEAR):
+        tout = cv.Tensor.alloc([8, 224, 224, 3], np.uint8, "NHWC")
+        cv.Resize()(None, tin, tout, interp)
+        torch.cuda.synchronize()
+        check(tout.numpy(), src, (224, 224), interp, orc)
+    # a ramp image (value = column index) exposes any deviation of the nearest index on the 32
+    # columns dx = 3 (mod 7) where (dx+.5)*1920/224 is an exact integer
+    ramp = np.tile(np.arange(1920, dtype=np.uint16).reshape(1, 1, 1920, 1), (1, 4, 1, 1))
+    tout = cv.Tensor.alloc([1, 4, 224, 1], np.uint16, "NHWC")
+    cv.Resize()(None, cv.Tensor.from_numpy(ramp, "NHWC"), tout, NEAREST)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(tout.numpy(), orc.resize(ramp, (4, 224), NEAREST))
+
+
+def test_config5_bicubic_f32_full_size(cv, orc, gpu):
+    # BASELINE config 5: batch 16 f32 NHWC 4ch 3840x2160 -> 640x360, values in [0,1), 1e-4 abs
+    N = 16
+    one = orc.fill_f32((2, 2160, 3840, 4), 0xC0FFEE05)
+    tin = cv.Tensor.alloc([N, 2160, 3840, 4], np.float32, "NHWC")
+    view = tin.torch_view()
+    dev = torch.from_numpy(one).cuda()
+    for k in range(N // 2):
+        view[2 * k:2 * k + 2].copy_(dev)
+    tout = cv.Tensor.alloc([N, 360, 640, 4], np.float32, "NHWC")
+    cv.Resize()(None, tin, tout, CUBIC)
+    torch.cuda.synchronize()
+    res = tout.numpy()
+    ref = orc.resize(one, (360, 640), CUBIC, variant=1, threads=8)
+    assert np.abs(res[:2] - ref).max() <= 1e-4
+    for k in range(1, N // 2):
+        np.testing.assert_array_equal(res[2 * k:2 * k + 2], res[:2])
+
+
+def _format_for(cv, K, dt, c):
+    import cvcuda_amd._capi as capi
+    kind = {np.uint8: K.DATA_KIND_UNSIGNED, np.uint16: K.DATA_KIND_UNSIGNED, np.int16: K.DATA_KIND_SIGNED,
+            np.float32: K.DATA_KIND_FLOAT}[dt]
+    bits = np.dtype(dt).itemsize * 8
+    pack = getattr(K, "PACKING_" + "_".join("%s%d" % (n, bits) for n in "XYZW"[:c]))
+    swz = [K.SWIZZLE_X000, None, K.SWIZZLE_XYZ1, K.SWIZZLE_XYZW][c - 1]
+    f = C.c_uint64()
+    cv.check(capi.nvcv.nvcvMakeNonColorImageFormat(C.byref(f), K.MEM_LAYOUT_PL, kind, swz, pack, 0, 0, 0,
+                                                   K.ALPHA_ASSOCIATED, None))
+    return f.value
+
+
+@pytest.mark.parametrize("interp", [NEAREST, LINEAR, CUBIC])
+@pytest.mark.parametrize("dt,c", [(np.uint8, 3), (np.uint8, 4), (np.uint8, 1), (np.uint16, 3), (np.int16, 4),
+                                  (np.float32, 1), (np.float32, 4)])
+def test_varshape(cv, K, orc, gpu, interp, dt, c):
+    rng = np.random.default_rng(17)
+    fmt = _format_for(cv, K, dt, c)
+    n = 7
+    bin_, bout, hosts, outs = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], []
+    for i in range(n):
+        sw, sh = int(rng.integers(20, 300)), int(rng.integers(20, 200))
+        dw, dh = int(rng.integers(10, 350)), int(rng.integers(10, 250))
+        a = make_input(orc, (sh, sw, c), dt, 100 + i)
+        hosts.append(a)
+        bin_.push_back(cv.Image.from_numpy(a, fmt))
+        o = cv.Image.alloc((dw, dh), fmt)
+        outs.append(o)
+        bout.push_back(o)
+    cv.Resize()(None, bin_, bout, interp)
+    torch.cuda.synchronize()
+    for a, o in zip(hosts, outs):
+        w, h = o.size
+        res = o.plane_view(0, dt, c).cpu().numpy()[None]
+        check(res, a[None], (h, w), interp, orc, varshape=True)
+
+
+def test_negative_cases(cv, gpu):
+    a = cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC")
+    op = cv.Resize()
+    cases = [
+        (cv.Tensor.alloc([2, 4, 4, 3], np.float32, "NHWC"), LINEAR),   # dtype differs
+        (cv.Tensor.alloc([3, 4, 4, 3], np.uint8, "NHWC"), LINEAR),     # batch differs
+        (cv.Tensor.alloc([2, 4, 4, 4], np.uint8, "NHWC"), LINEAR),     # channels differ
+        (cv.Tensor.alloc([2, 3, 4, 4], np.uint8, "NCHW"), LINEAR),     # layout differs
+        (cv.Tensor.alloc([2, 4, 4, 3], np.uint8, "NHWC"), 4),          # LANCZOS unsupported
+    ]
+    for out, interp in cases:
+        with pytest.raises(cv.Error) as e:
+            op(None, a, out, interp)
+        assert e.value.status == 2
+    with pytest.raises(cv.Error) as e:
+        cv.ResizeCropConvertReformat()(None, a, a, LINEAR) if False else cv.check(
+            __import__("cvcuda_amd")._capi.cvcuda.cvcudaResizeSubmit(cv.ResizeCropConvertReformat().handle, None,
+                                                                     a.handle, a.handle, LINEAR))
+    assert e.value.status == 9  # handle of another operator -> NOT_COMPATIBLE

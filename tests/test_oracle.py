@@ -1,0 +1,326 @@
+"""Pins the CPU oracle (oracle/cv_oracle.cpp) WITHOUT running the reference: closed forms, textbook
+values, brute force and independent library routines (torch interpolate, numpy pad), chosen so that a
+dropped term, a wrong sign/index or a swapped operand fails at least one check.
+
+Known answers taken from the reference's texts are cited where used.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+NEAREST, LINEAR, CUBIC = 0, 1, 2
+
+
+# ------------------------------------------------------------------------------------------ saturate
+def test_saturate_cast_known_answers(orc):
+    # round-half-to-even then clamp (reference: cuda_tools/detail/SaturateCastImpl.hpp:41-50, 125;
+    # known-answer style of tests/nvcv_types/cudatools_system/TestSaturateCast.cpp)
+    ka = [(0.5, 0), (1.5, 2), (2.5, 2), (3.5, 4), (-0.5, 0), (-1.0, 0), (254.5, 254), (255.5, 255), (300.0, 255),
+          (1e9, 255), (-1e9, 0), (127.49, 127), (float("nan"), 0)]
+    for v, want in ka:
+        assert orc.saturate_f32(v, np.uint8) == want, v
+    for v, want in [(32767.5, 32767), (-32768.5, -32768), (-40000.0, -32768), (1.5, 2), (-1.5, -2), (-2.5, -2)]:
+        assert orc.saturate_f32(v, np.int16) == want, v
+    for v, want in [(65535.5, 65535), (70000.0, 65535), (-1.0, 0), (1234.5, 1234)]:
+        assert orc.saturate_f32(v, np.uint16) == want, v
+    xs = np.linspace(-3, 258, 4177).astype(np.float32)
+    want = np.clip(np.rint(xs), 0, 255).astype(np.int64)  # np.rint is half-to-even
+    got = np.array([orc.saturate_f32(float(x), np.uint8) for x in xs])
+    np.testing.assert_array_equal(got, want)
+
+
+# ------------------------------------------------------------------------------------------ borders
+def test_border_index_maps_against_numpy_pad(orc):
+    modes = {1: "edge", 2: "symmetric", 3: "wrap", 4: "reflect"}  # replicate, reflect, wrap, reflect101
+    for s in range(1, 9):
+        for mode, npmode in modes.items():
+            if npmode == "reflect" and s == 1:
+                assert all(orc.border_index(mode, c, 1) == 0 for c in range(-5, 6))
+                continue
+            pad = 24
+            padded = np.pad(np.arange(s), pad, mode=npmode)
+            for c in range(-20, 21):
+                assert orc.border_index(mode, c, s) == padded[c + pad], (mode, s, c)
+    # the device's closed form for REFLECT (BorderWrap.hpp:100-108) equals the golden's branchy form
+    for s in range(1, 9):
+        for c in range(-40, 41):
+            assert orc.border_index_reflect_device(c, s) == orc.border_index(2, c, s)
+
+
+# ------------------------------------------------------------------------------------------ fused op
+def test_fused_identity_constant_and_crop_consistency(orc):
+    rng = np.random.default_rng(1)
+    src = rng.integers(0, 256, (2, 13, 17, 3), dtype=np.uint8)
+    for order in (0, 1):
+        out = orc.fused_rccr(src, (13, 17), (17, 13), (0, 0), LINEAR, np.float32, False, order=order)
+        np.testing.assert_array_equal(out, src.astype(np.float32))  # same size, no crop: exact cast
+    const = np.full((1, 40, 50, 3), 200, np.uint8)
+    out = orc.fused_rccr(const, (9, 11), (23, 19), (3, 4), LINEAR, np.float32, True, scale=0.25, offset=-7.0)
+    # a constant image stays constant up to a few float32 roundings of the lerp
+    assert np.abs(out - (0.25 * 200 - 7.0)).max() <= 0.25 * 4 * 200 * np.finfo(np.float32).eps
+    # cropping the uncropped result == asking for the crop (same per-pixel coordinates)
+    full = orc.fused_rccr(src, (11, 9), (9, 11), (0, 0), LINEAR, np.float32, False)
+    part = orc.fused_rccr(src, (5, 4), (9, 11), (3, 2), LINEAR, np.float32, False)
+    np.testing.assert_array_equal(part, full[:, 2:7, 3:7])
+    # channel reversal and planar layout are pure index permutations
+    a = orc.fused_rccr(src, (7, 8), (12, 9), (1, 1), LINEAR, np.float32, False, manip=0)
+    b = orc.fused_rccr(src, (7, 8), (12, 9), (1, 1), LINEAR, np.float32, True, manip=1)
+    np.testing.assert_array_equal(b, a[..., ::-1].transpose(0, 3, 1, 2))
+
+
+def test_fused_bilinear_matches_torch_interpolate(orc):
+    # half-pixel-centre bilinear without antialias is exactly torch's align_corners=False mode
+    # (edge handling by tap clamping is equivalent); differences are float rounding only.
+    rng = np.random.default_rng(2)
+    for (h, w, nh, nw) in [(40, 56, 17, 23), (23, 31, 50, 64), (1080 // 8, 1920 // 8, 32, 57)]:
+        src = rng.integers(0, 256, (2, h, w, 3), dtype=np.uint8)
+        ref = F.interpolate(torch.from_numpy(src).permute(0, 3, 1, 2).double(), size=(nh, nw), mode="bilinear",
+                            align_corners=False, antialias=False).numpy()
+        for order in (0, 1):
+            out = orc.fused_rccr(src, (nh, nw), (nw, nh), (0, 0), LINEAR, np.float32, True, order=order)
+            assert np.abs(out - ref).max() < 1e-2  # float32 coordinate rounding (|coord|*eps) times a slope of up to 255
+        # the two summation orders agree far inside the parity bar
+        o0 = orc.fused_rccr(src, (nh, nw), (nw, nh), (0, 0), LINEAR, np.float32, True, order=0)
+        o1 = orc.fused_rccr(src, (nh, nw), (nw, nh), (0, 0), LINEAR, np.float32, True, order=1)
+        assert np.abs(o0 - o1).max() <= 4 * 255 * np.finfo(np.float32).eps
+
+
+def test_fused_nearest_matches_torch_nearest_exact_and_srccast(orc):
+    rng = np.random.default_rng(3)
+    src = rng.integers(0, 256, (1, 33, 47, 3), dtype=np.uint8)
+    # sizes with no coordinate landing within float rounding of an integer
+    out = orc.fused_rccr(src, (13, 19), (19, 13), (0, 0), NEAREST, np.uint8, False)
+    ref = F.interpolate(torch.from_numpy(src).permute(0, 3, 1, 2).float(), size=(13, 19), mode="nearest-exact")
+    np.testing.assert_array_equal(out, ref.permute(0, 2, 3, 1).numpy().astype(np.uint8))
+    # srcCast rounds the interpolated value to u8 (half-to-even) before scaling
+    lin = orc.fused_rccr(src, (13, 19), (19, 13), (0, 0), LINEAR, np.float32, False, scale=1.0, src_cast=False)
+    cast = orc.fused_rccr(src, (13, 19), (19, 13), (0, 0), LINEAR, np.float32, False, scale=1.0, src_cast=True)
+    np.testing.assert_array_equal(cast, np.clip(np.rint(lin), 0, 255))
+    u8 = orc.fused_rccr(src, (13, 19), (19, 13), (0, 0), LINEAR, np.uint8, False, scale=2.0, offset=-100.0)
+    np.testing.assert_array_equal(u8, np.clip(np.rint(np.float32(2.0) * lin + np.float32(-100.0)), 0, 255))
+
+
+# ------------------------------------------------------------------------------------------ resize
+def test_resize_nearest_knife_edge_columns(orc):
+    # 1920 -> 224: (dx+.5)*60/7 is an exact integer for dx = 3 (mod 7). The golden's float32 expression
+    # floor(scaleW*(dx+0.5f)) and the reference device's pack expression floor((dx0+.5f)*s + k*s)
+    # disagree on exactly these 13 columns (documented analysis of tests/cvcuda/system/ResizeUtils.cpp:195-215
+    # vs src/cvcuda/priv/OpResize.cu:79-83,152-162); the oracle must follow the golden.
+    w_src, w_dst = 1920, 224
+    src = np.arange(w_src, dtype=np.uint16).reshape(1, 1, w_src, 1).repeat(2, axis=1)
+    out = orc.resize(src, (2, w_dst), NEAREST)[0, 0, :, 0].astype(np.int64)
+    s = np.float32(w_src) / np.float32(w_dst)
+    dx = np.arange(w_dst)
+    golden = np.minimum(np.floor(s * (dx.astype(np.float32) + np.float32(0.5))), w_src - 1).astype(np.int64)
+    np.testing.assert_array_equal(out, golden)
+    dx0 = (dx // 4) * 4
+    k = (dx % 4).astype(np.float32)
+    pack = np.floor((dx0.astype(np.float32) + np.float32(0.5)) * s + k * s).astype(np.int64)
+    assert list(np.nonzero(pack != golden)[0]) == [59, 73, 101, 115, 122, 143, 150, 171, 178, 185, 199, 206, 213]
+    # away from the knife edges the result is the exact rational floor
+    exact = ((2 * dx + 1) * w_src) // (2 * w_dst)
+    safe = (dx % 7) != 3
+    np.testing.assert_array_equal(out[safe], exact[safe])
+
+
+def test_resize_identity_and_constant(orc):
+    rng = np.random.default_rng(4)
+    for dt in (np.uint8, np.uint16, np.int16, np.float32):
+        a = (rng.random((2, 9, 11, 4)) * 200).astype(dt)
+        for interp in (NEAREST, LINEAR):
+            for variant in (0, 1, 2):
+                if dt == np.float32 and variant == 0 and interp == LINEAR:
+                    continue  # the golden rounds floats to integers (known quirk of the reference's golden)
+                np.testing.assert_array_equal(orc.resize(a, (9, 11), interp, variant), a)
+        c = np.full((1, 20, 30, 3), 37, dt)
+        for interp in (NEAREST, LINEAR, CUBIC):
+            for variant in (0, 1, 2):
+                out = orc.resize(c, (7, 13), interp, variant)
+                assert np.abs(out.astype(np.float64) - 37).max() <= (1e-4 if dt == np.float32 else 0)
+
+
+def test_resize_linear_and_cubic_match_torch(orc):
+    rng = np.random.default_rng(5)
+    a = rng.random((1, 64, 80, 4)).astype(np.float32)
+    t = torch.from_numpy(a).permute(0, 3, 1, 2).double()
+    for (h, w) in [(16, 20), (31, 37), (100, 90)]:
+        ref = F.interpolate(t, size=(h, w), mode="bilinear", align_corners=False).permute(0, 2, 3, 1).numpy()
+        for variant in (1, 2):
+            assert np.abs(orc.resize(a, (h, w), LINEAR, variant) - ref).max() < 1e-4
+        # cubic: torch uses the same Keys kernel (A = -0.75); borders differ, compare the interior only
+        ref = F.interpolate(t, size=(h, w), mode="bicubic", align_corners=False).permute(0, 2, 3, 1).numpy()
+        sy, sx = 64 / h, 80 / w
+        m_y, m_x = int(np.ceil(3 / sy)) + 1, int(np.ceil(3 / sx)) + 1
+        for variant in (1, 2):
+            out = orc.resize(a, (h, w), CUBIC, variant)
+            inner = (slice(None), slice(m_y, h - m_y), slice(m_x, w - m_x))
+            # |.| of the device formula only matters for negative overshoot; inputs are in [0,1)
+            assert np.abs(out[inner] - np.abs(ref[inner])).max() < 1e-4
+    # u8: golden (double, rint) vs device (float32) within 1 LSB, the reference's own tolerance
+    b = rng.integers(0, 256, (1, 50, 70, 3), dtype=np.uint8)
+    for interp in (LINEAR, CUBIC):
+        g = orc.resize(b, (21, 33), interp, 0).astype(np.int32)
+        for variant in (1, 2):
+            d = orc.resize(b, (21, 33), interp, variant).astype(np.int32)
+            assert np.abs(g - d).max() <= 1
+
+
+def test_resize_cubic_edge_quirk(orc):
+    # the x weight is forced to zero-offset when the centre column is within the border band, the y
+    # weight is not (src/cvcuda/priv/OpResize.cu:357-366): with a horizontal ramp the first output
+    # columns reproduce source column 1 exactly (taps (0,1,0,0) on clamped centre 1).
+    w = 40
+    img = np.tile(np.arange(w, dtype=np.float32), (12, 1)).reshape(1, 12, w, 1)
+    out = orc.resize(img, (12, 20), CUBIC, 1)[0, :, :, 0]
+    assert np.all(out[:, 0] == 1.0)
+
+
+# ------------------------------------------------------------------------------------------ NV12
+def _all_triples_nv12():
+    W = H = 4096
+    by, bx = np.meshgrid(np.arange(H // 2), np.arange(W // 2), indexing="ij")
+    blk = by * (W // 2) + bx
+    U = (blk % 256).astype(np.uint8)
+    V = ((blk // 256) % 256).astype(np.uint8)
+    yb = (blk // 65536) * 4
+    Y = np.zeros((H, W), np.uint8)
+    Y[0::2, 0::2] = yb
+    Y[0::2, 1::2] = yb + 1
+    Y[1::2, 0::2] = yb + 2
+    Y[1::2, 1::2] = yb + 3
+    uv = np.zeros((H // 2, W), np.uint8)
+    uv[:, 0::2] = U
+    uv[:, 1::2] = V
+    return np.concatenate([Y, uv])[None], Y, np.repeat(np.repeat(U, 2, 0), 2, 1), np.repeat(np.repeat(V, 2, 0), 2, 1)
+
+
+def test_nv12_textbook_colours_and_exhaustive_cross_check(orc):
+    # BT.601 limited-range primaries (textbook YCbCr values of pure colours)
+    for (y, u, v), rgb in {(16, 128, 128): (0, 0, 0), (235, 128, 128): (255, 255, 255), (81, 90, 240): (255, 0, 0),
+                           (145, 54, 34): (0, 255, 0), (41, 240, 110): (0, 0, 255)}.items():
+        got = orc.yuv_to_rgb_int(y, u, v)
+        assert max(abs(int(g) - w) for g, w in zip(got, rgb)) <= 1, ((y, u, v), got)
+    # every (Y,U,V) in 256^3: the integer device formula stays within 2 of the reference's
+    # double-precision golden (its own test tolerance, tests/cvcuda/system/TestOpCvtColor.cpp:626-646)
+    nv12, Y, U, V = _all_triples_nv12()
+    seen = np.zeros(1 << 24, bool)
+    seen[(Y.astype(np.int64) << 16 | U.astype(np.int64) << 8 | V).ravel()] = True
+    assert seen.all()
+    a = orc.yuv420_to_rgb(nv12, variant=0, threads=8).astype(np.int16)
+    b = orc.yuv420_to_rgb(nv12, variant=1, threads=8).astype(np.int16)
+    assert np.abs(a - b).max() <= 2
+    # channel order / alpha / NV21 are index permutations of the same values
+    small = nv12[:, :, :64][:, list(range(32)) + list(range(4096, 4096 + 16))]
+    rgb = orc.yuv420_to_rgb(small)
+    np.testing.assert_array_equal(orc.yuv420_to_rgb(small, bgr=True), rgb[..., ::-1])
+    rgba = orc.yuv420_to_rgb(small, dcn=4)
+    np.testing.assert_array_equal(rgba[..., :3], rgb)
+    assert (rgba[..., 3] == 255).all()
+    swapped = small.copy()
+    swapped[:, 32:, 0::2], swapped[:, 32:, 1::2] = small[:, 32:, 1::2], small[:, 32:, 0::2]
+    np.testing.assert_array_equal(orc.yuv420_to_rgb(swapped, uidx=1), rgb)
+
+
+def test_i420_equals_nv12_after_deinterleave(orc):
+    rng = np.random.default_rng(6)
+    H, W = 8, 12
+    Y = rng.integers(0, 256, (H, W), dtype=np.uint8)
+    U = rng.integers(0, 256, (H // 2, W // 2), dtype=np.uint8)
+    V = rng.integers(0, 256, (H // 2, W // 2), dtype=np.uint8)
+    uv = np.zeros((H // 2, W), np.uint8)
+    uv[:, 0::2], uv[:, 1::2] = U, V
+    nv12 = np.concatenate([Y, uv])[None]
+    i420 = np.concatenate([Y, U.reshape(H // 4, W), V.reshape(H // 4, W)])[None]
+    np.testing.assert_array_equal(orc.yuv420_to_rgb(i420, semi_planar=False), orc.yuv420_to_rgb(nv12))
+
+
+# ------------------------------------------------------------------------------------------ normalize
+def test_normalize_identity_broadcast_and_stddev(orc):
+    rng = np.random.default_rng(7)
+    for dt in (np.uint8, np.int16, np.float32):
+        a = (rng.random((3, 5, 7, 3)) * 100).astype(dt)
+        one = np.ones((1, 1, 1, 1), np.float32)
+        np.testing.assert_array_equal(orc.normalize(a, 0 * one, one), a)
+    a = rng.random((2, 4, 6, 3)).astype(np.float32)
+    base = rng.random((1, 1, 1, 3)).astype(np.float32)
+    scale = (rng.random((2, 4, 1, 1)) + 0.5).astype(np.float32)
+    out = orc.normalize(a, base, scale, 1.5, 0.25)
+    want = (a - base) * scale * np.float32(1.5) + np.float32(0.25)  # float32, left to right
+    np.testing.assert_array_equal(out, want.astype(np.float32))
+    out = orc.normalize(a, base, scale, 2.0, 1.0, epsilon=0.5, stddev=True)
+    mul = np.float32(1.0) / np.sqrt(scale * scale + np.float32(0.5))
+    np.testing.assert_array_equal(out, ((a - base) * mul * np.float32(2.0) + np.float32(1.0)).astype(np.float32))
+    # u8 saturates and rounds half to even
+    b = np.array([[[[10, 250, 3]]]], np.uint8)
+    out = orc.normalize(b, np.zeros((1, 1, 1, 1), np.float32), np.full((1, 1, 1, 1), 1.5, np.float32), 1.0, 0.0)
+    np.testing.assert_array_equal(out, np.array([[[[15, 255, 4]]]], np.uint8))  # 4.5 -> 4
+
+
+# ------------------------------------------------------------------------------------------ warp
+def test_invert_affine(orc):
+    m = np.array([1.2, 0.3, 5.0, -0.4, 0.9, -7.0], np.float32)
+    inv = orc.invert_affine(m).astype(np.float64)
+    A = np.vstack([m.reshape(2, 3).astype(np.float64), [0, 0, 1]])
+    B = np.vstack([inv.reshape(2, 3), [0, 0, 1]])
+    assert np.abs(A @ B - np.eye(3)).max() < 1e-5
+    np.testing.assert_array_equal(orc.invert_affine([1, 2, 3, 2, 4, 5]), np.zeros(6, np.float32))  # singular
+
+
+def test_warp_identity_translation_borders_rotation(orc):
+    rng = np.random.default_rng(8)
+    src = rng.integers(0, 256, (1, 7, 9, 3), dtype=np.uint8)
+    ident = [1, 0, 0, 0, 1, 0]
+    for interp in (NEAREST, LINEAR, CUBIC):
+        for variant in (0, 1):
+            np.testing.assert_array_equal(orc.warp(src, (7, 9), ident, interp, variant=variant), src)
+    # integer translation: dst(x,y) = src(x+3, y-2); outside -> border policy == numpy pad
+    pads = {0: ("constant", {"constant_values": 0}), 1: ("edge", {}), 2: ("symmetric", {}), 3: ("wrap", {}),
+            4: ("reflect", {})}
+    for border, (mode, kw) in pads.items():
+        padded = np.pad(src[0], ((12, 12), (12, 12), (0, 0)), mode=mode, **kw)
+        want = padded[12 - 2:12 - 2 + 7, 12 + 3:12 + 3 + 9]
+        for interp in (NEAREST, LINEAR):
+            for variant in (0, 1):
+                got = orc.warp(src, (7, 9), [1, 0, 3, 0, 1, -2], interp, border=border, variant=variant)[0]
+                np.testing.assert_array_equal(got, want)
+    # constant border takes the per-channel value
+    got = orc.warp(src, (7, 9), [1, 0, 100, 0, 1, 0], NEAREST, border=0, border_value=(7, 8, 9, 0))[0]
+    assert (got == np.array([7, 8, 9], np.uint8)).all()
+    # 90-degree rotation with an integer matrix is an exact index permutation
+    sq = rng.integers(0, 256, (1, 6, 6, 1), dtype=np.uint8)
+    got = orc.warp(sq, (6, 6), [0, 1, 0, -1, 0, 5], LINEAR)[0, :, :, 0]  # src = (y, 5 - x)
+    np.testing.assert_array_equal(got, np.rot90(sq[0, :, :, 0], 1).T[::-1].T if False else
+                                  np.array([[sq[0, 5 - x, y, 0] for x in range(6)] for y in range(6)]))
+    # half-pixel shift in x: bilinear is the mean of horizontal neighbours
+    f = rng.random((1, 5, 8, 1)).astype(np.float32)
+    got = orc.warp(f, (5, 7), [1, 0, 0.5, 0, 1, 0], LINEAR, variant=1)[0, :, :, 0]
+    np.testing.assert_allclose(got, 0.5 * (f[0, :, :-1, 0] + f[0, :, 1:, 0]), rtol=0, atol=1e-6)
+
+
+def test_warp_cubic_golden_vs_device_and_perspective(orc):
+    rng = np.random.default_rng(9)
+    src = rng.integers(0, 256, (2, 20, 24, 3), dtype=np.uint8)
+    m = orc.invert_affine([0.9, 0.2, 1.5, -0.15, 1.1, -2.0])
+    g = orc.warp(src, (20, 24), m, CUBIC, border=1, variant=0).astype(np.int32)
+    d = orc.warp(src, (20, 24), m, CUBIC, border=1, variant=1).astype(np.int32)
+    assert np.abs(g - d).max() <= 1  # Catmull-Rom taps; golden normalises by the weight sum (== 1)
+    # a perspective matrix with last row (0,0,1) is the affine map
+    a = orc.warp(src, (20, 24), m, LINEAR, border=4, variant=1)
+    p = orc.warp(src, (20, 24), list(m) + [0, 0, 1], LINEAR, border=4, perspective=True, variant=1)
+    np.testing.assert_array_equal(a, p)
+
+
+# ------------------------------------------------------------------------------------------ generator
+def test_seeded_generators(orc):
+    a = orc.fill_u8((1000,), 42)
+    b = orc.fill_u8((1000,), 42)
+    np.testing.assert_array_equal(a, b)
+    assert a.min() < 5 and a.max() > 250
+    c = orc.fill_u8((4096,), 7, 16, 235)
+    assert c.min() == 16 and c.max() == 235
+    f = orc.fill_f32((4096,), 3)
+    assert 0.0 <= f.min() and f.max() < 1.0 and abs(f.mean() - 0.5) < 0.03
+    # splitmix64 reference value: first output for seed 0 is 0xE220A8397B1DCDAF (published test vector)
+    first8 = orc.fill_u8((8,), 0)
+    assert int.from_bytes(bytes(first8), "little") == 0xE220A8397B1DCDAF
