@@ -195,7 +195,7 @@ class Tensor(_Handle):
         strides = [d.buffer.strides[i] for i in range(d.rank)]
         nbytes = max(1, sum((s - 1) * st for s, st in zip(shape, strides)) + es)
         raw = _bytes_view(d.buffer.basePtr, nbytes, self)
-        if es > 1:
+        if npdt != np.dtype(np.uint8):
             assert all(st % es == 0 for st in strides), "strides must be multiples of the element size"
             raw = raw[: (nbytes // es) * es].view(_NP2TORCH[npdt])
         return torch.as_strided(raw, shape, [st // es for st in strides])
@@ -276,7 +276,7 @@ class Image(_Handle):
         es = npdt.itemsize
         nbytes = (pl.height - 1) * pl.rowStride + pl.width * channels * es
         raw = _bytes_view(pl.basePtr, nbytes, self)
-        if es > 1:
+        if npdt != np.dtype(np.uint8):
             raw = raw[: (nbytes // es) * es].view(_NP2TORCH[npdt])
         return torch.as_strided(raw, (pl.height, pl.width, channels), (pl.rowStride // es, channels, 1))
 

@@ -1,0 +1,703 @@
+// WarpAffine and WarpPerspective, tensors and var-shape batches.
+//
+// Coordinates, sampling and border handling follow the reference in float32 without FMA
+// contraction: destination->source map src/cvcuda/priv/legacy/CvCudaLegacy.h:143-183, matrix
+// inversion warp.cu:139-150 (affine) and cuda_tools/math/LinAlg.hpp:1446-1450, 1640-1654 (3x3),
+// samplers cuda_tools/InterpolationWrap.hpp:83-104, 332-339, 429-447, 535-565, border index maps
+// cuda_tools/BorderWrap.hpp:62-121. Validation follows warp.cu:152-232 and warp_var_shape.cu:194-299.
+//
+// Differences by design: the var-shape kernels read each image's matrix straight from the caller's
+// [N,6] / [N,9] tensor and invert it in the block prologue (a few scalar operations), so the operator
+// owns no device buffer and launches no separate inversion kernel; several var-shape submissions of
+// one operator handle may therefore be in flight at once. Var-shape batches run on a packed tile grid.
+//
+// Kernel shape: one lane per destination pixel, 32 x 8 pixels per block (a squarish tile keeps the
+// rotated source footprint of a block compact); all channels of a tap move as one vector access.
+#include "DeviceUtils.hpp"
+#include "OpCommon.hpp"
+#include "VarShapeTiles.hpp"
+
+#include <cvcuda/OpWarpAffine.h>
+#include <cvcuda/OpWarpPerspective.h>
+
+#include <algorithm>
+#include <cmath>
+
+namespace cvamd {
+
+namespace {
+
+constexpr int kTileW = 32;
+constexpr int kTileH = 8;
+
+struct WarpArgs
+{
+    const uint8_t *src;
+    uint8_t       *dst;
+    int64_t        srcN, dstN;
+    int32_t        srcRow, dstRow;
+    int32_t        srcW, srcH, dstW, dstH;
+    const NVCVImageBufferStrided *srcList;
+    const NVCVImageBufferStrided *dstList;
+    // matrix: tensor path -> m[] already maps dst->src; var-shape -> rows of `xforms`
+    float          m[9];
+    const uint8_t *xforms;
+    int64_t        xformStride; // bytes between matrices
+    int32_t        inverseGiven; // var-shape: 1 = matrices already map dst->src
+    int32_t        perspective;
+    int32_t        border;
+    float          bval[4];
+};
+
+template<class T, int C>
+struct __attribute__((packed, aligned(sizeof(T)))) Vec
+{
+    T v[C];
+};
+
+struct Img
+{
+    const uint8_t *base;
+    int32_t        row, w, h;
+};
+
+__device__ __forceinline__ int BorderIndex(int border, int c, int s)
+{
+    switch (border)
+    {
+    case NVCV_BORDER_REPLICATE:
+        return c < 0 ? 0 : (c >= s ? s - 1 : c);
+    case NVCV_BORDER_WRAP:
+        c = c % s;
+        return c < 0 ? c + s : c;
+    case NVCV_BORDER_REFLECT:
+    {
+        const int s2 = s * 2;
+        c            = c % s2;
+        if (c < 0)
+        {
+            c += s2;
+        }
+        return s - 1 - (abs(2 * c + 1 - s2) >> 1);
+    }
+    default: // REFLECT101
+        if (s == 1)
+        {
+            return 0;
+        }
+        c = c % (2 * s - 2);
+        if (c < 0)
+        {
+            c += 2 * s - 2;
+        }
+        return s - 1 - abs(s - 1 - c);
+    }
+}
+
+template<class T>
+__device__ __forceinline__ T BorderCast(float v)
+{
+    if constexpr (std::is_same_v<T, float>)
+    {
+        return v;
+    }
+    else
+    {
+        // truncation toward zero, saturated to the range of T
+        const float lo = (float)std::numeric_limits<T>::min(), hi = (float)std::numeric_limits<T>::max();
+        return (T)(int)fminf(fmaxf(truncf(v), lo), hi);
+    }
+}
+
+template<class T, int C>
+__device__ __forceinline__ void Fetch(const Img &im, const WarpArgs &a, int x, int y, float (&out)[C])
+{
+    if (a.border == NVCV_BORDER_CONSTANT)
+    {
+        if (x < 0 || x >= im.w || y < 0 || y >= im.h)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                out[c] = (float)BorderCast<T>(a.bval[c]);
+            }
+            return;
+        }
+    }
+    else
+    {
+        x = BorderIndex(a.border, x, im.w);
+        y = BorderIndex(a.border, y, im.h);
+    }
+    const Vec<T, C> px = reinterpret_cast<const Vec<T, C> *>(im.base + (int64_t)y * im.row)[x];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        out[c] = (float)px.v[c];
+    }
+}
+
+__device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
+{
+    w[0] = -.5f;
+    w[0] = w[0] * d + 1.f;
+    w[0] = w[0] * d - .5f;
+    w[0] = w[0] * d;
+    w[1] = 1.5f;
+    w[1] = w[1] * d - 2.5f;
+    w[1] = w[1] * d;
+    w[1] = w[1] * d + 1.f;
+    w[2] = -1.5f;
+    w[2] = w[2] * d + 2.f;
+    w[2] = w[2] * d + .5f;
+    w[2] = w[2] * d;
+    w[3] = 1 - w[0] - w[1] - w[2];
+}
+
+// float -> int index like the reference's round-down conversion; huge / non-finite coordinates
+// saturate instead of invoking undefined behaviour
+__device__ __forceinline__ int FloorToInt(float v)
+{
+    return (int)fminf(fmaxf(floorf(v), -1073741824.f), 1073741824.f);
+}
+
+template<class T, int C, int INTERP>
+__device__ __forceinline__ void WarpPixel(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dstRow, int dx,
+                                          int dy)
+{
+    float sx, sy;
+    if (a.perspective)
+    {
+        const float coeff = 1.0f / (m[6] * dx + m[7] * dy + m[8]);
+        sx                = coeff * (m[0] * dx + m[1] * dy + m[2]);
+        sy                = coeff * (m[3] * dx + m[4] * dy + m[5]);
+    }
+    else
+    {
+        sx = m[0] * dx + m[1] * dy + m[2];
+        sy = m[3] * dx + m[4] * dy + m[5];
+    }
+    float acc[C];
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        Fetch<T, C>(im, a, FloorToInt(sx + .5f), FloorToInt(sy + .5f), acc);
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const int x1 = FloorToInt(sx), y1 = FloorToInt(sy);
+        const int x2 = x1 + 1, y2 = y1 + 1;
+        float     t[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] = 0.f;
+        }
+        Fetch<T, C>(im, a, x1, y1, t);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] += t[c] * (x2 - sx) * (y2 - sy);
+        }
+        Fetch<T, C>(im, a, x2, y1, t);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] += t[c] * (sx - x1) * (y2 - sy);
+        }
+        Fetch<T, C>(im, a, x1, y2, t);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] += t[c] * (x2 - sx) * (sy - y1);
+        }
+        Fetch<T, C>(im, a, x2, y2, t);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] += t[c] * (sx - x1) * (sy - y1);
+        }
+    }
+    else
+    {
+        const int ix = FloorToInt(sx), iy = FloorToInt(sy);
+        float     wx[4], wy[4];
+        CubicCoeffs(sx - ix, wx);
+        CubicCoeffs(sy - iy, wy);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] = 0.f;
+        }
+#pragma unroll
+        for (int cy = -1; cy <= 2; ++cy)
+        {
+#pragma unroll
+            for (int cx = -1; cx <= 2; ++cx)
+            {
+                float t[C];
+                Fetch<T, C>(im, a, ix + cx, iy + cy, t);
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    acc[c] += t[c] * (wx[cx + 1] * wy[cy + 1]);
+                }
+            }
+        }
+    }
+    Vec<T, C> *o = reinterpret_cast<Vec<T, C> *>(dstRow) + dx;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        T v;
+        if constexpr (INTERP == NVCV_INTERP_NEAREST)
+        {
+            v = (T)acc[c]; // the tap itself (exactly representable), no rounding involved
+        }
+        else
+        {
+            v = SaturateCast<T>(acc[c]);
+        }
+        __builtin_nontemporal_store(v, &o->v[c]);
+    }
+}
+
+// Inverts one caller-supplied forward matrix (uniform per block).
+__device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (&m)[9])
+{
+    const float *p = reinterpret_cast<const float *>(a.xforms + image * a.xformStride);
+    const int    n = a.perspective ? 9 : 6;
+    float        f[9];
+    for (int i = 0; i < 9; ++i)
+    {
+        f[i] = i < n ? p[i] : 0.f;
+    }
+    if (a.inverseGiven)
+    {
+        for (int i = 0; i < 9; ++i)
+        {
+            m[i] = f[i];
+        }
+        return;
+    }
+    if (!a.perspective)
+    {
+        float den = f[0] * f[4] - f[1] * f[3];
+        den       = fabsf(den) > 1e-5 ? (float)(1. / (double)den) : 0.f;
+        m[0]      = f[4] * den;
+        m[1]      = -f[1] * den;
+        m[2]      = (f[1] * f[5] - f[4] * f[2]) * den;
+        m[3]      = -f[3] * den;
+        m[4]      = f[0] * den;
+        m[5]      = (f[3] * f[2] - f[0] * f[5]) * den;
+        m[6] = m[7] = m[8] = 0.f;
+    }
+    else
+    {
+        const float d = f[0] * (f[4] * f[8] - f[5] * f[7]) + f[1] * (f[5] * f[6] - f[3] * f[8])
+                      + f[2] * (f[3] * f[7] - f[4] * f[6]);
+        if (d == 0)
+        {
+            for (int i = 0; i < 9; ++i)
+            {
+                m[i] = f[i]; // singular: left as given, like the reference's failed in-place inverse
+            }
+            return;
+        }
+        m[0] = (f[4] * f[8] - f[5] * f[7]) / d;
+        m[1] = -(f[1] * f[8] - f[2] * f[7]) / d;
+        m[2] = (f[1] * f[5] - f[2] * f[4]) / d;
+        m[3] = -(f[3] * f[8] - f[5] * f[6]) / d;
+        m[4] = (f[0] * f[8] - f[2] * f[6]) / d;
+        m[5] = -(f[0] * f[5] - f[2] * f[3]) / d;
+        m[6] = (f[3] * f[7] - f[4] * f[6]) / d;
+        m[7] = -(f[0] * f[7] - f[1] * f[6]) / d;
+        m[8] = (f[0] * f[4] - f[1] * f[3]) / d;
+    }
+}
+
+template<class T, int C, int INTERP>
+__global__ __launch_bounds__(256) void WarpTensor(const WarpArgs a)
+{
+    const int dx = blockIdx.x * kTileW + (threadIdx.x & (kTileW - 1));
+    const int dy = blockIdx.y * kTileH + (threadIdx.x / kTileW);
+    if (dx >= a.dstW || dy >= a.dstH)
+    {
+        return;
+    }
+    const int n  = blockIdx.z;
+    const Img im = {a.src + n * a.srcN, a.srcRow, a.srcW, a.srcH};
+    float     m[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i)
+    {
+        m[i] = a.m[i];
+    }
+    WarpPixel<T, C, INTERP>(im, a, m, a.dst + n * a.dstN + (int64_t)dy * a.dstRow, dx, dy);
+}
+
+template<class T, int C, int INTERP>
+__global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarTiles tiles)
+{
+    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
+    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
+    float                        m[9];
+    LoadMatrix(a, tc.image, m);
+    const int dx = tc.tx * kTileW + (threadIdx.x & (kTileW - 1));
+    const int dy = tc.ty * kTileH + (threadIdx.x / kTileW);
+    if (dx >= d.width || dy >= d.height)
+    {
+        return;
+    }
+    const Img im = {s.basePtr, s.rowStride, s.width, s.height};
+    WarpPixel<T, C, INTERP>(im, a, m, d.basePtr + (int64_t)dy * d.rowStride, dx, dy);
+}
+
+template<class T, int C, int INTERP>
+void Launch(const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
+{
+    if (dstHost == nullptr)
+    {
+        dim3 grid(DivUp(a.dstW, kTileW), DivUp(a.dstH, kTileH), N);
+        hipLaunchKernelGGL((WarpTensor<T, C, INTERP>), grid, dim3(256), 0, stream, a);
+        CheckLaunch("WarpTensor");
+        return;
+    }
+    for (int first = 0; first < N; first += kMaxTileImages)
+    {
+        VarTiles tiles;
+        int      total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kTileW, kTileH);
+        if (total > 0)
+        {
+            hipLaunchKernelGGL((WarpVarShape<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a, tiles);
+            CheckLaunch("WarpVarShape");
+        }
+    }
+}
+
+template<class T, int C>
+void DispatchInterp(int interp, const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
+{
+    switch (interp)
+    {
+    case NVCV_INTERP_NEAREST:
+        Launch<T, C, NVCV_INTERP_NEAREST>(a, N, dstHost, stream);
+        break;
+    case NVCV_INTERP_LINEAR:
+        Launch<T, C, NVCV_INTERP_LINEAR>(a, N, dstHost, stream);
+        break;
+    case NVCV_INTERP_CUBIC:
+        Launch<T, C, NVCV_INTERP_CUBIC>(a, N, dstHost, stream);
+        break;
+    default:
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid interpolation (supported: NEAREST, LINEAR, CUBIC)");
+    }
+}
+
+template<class T>
+void DispatchC(int C, int interp, const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
+{
+    switch (C)
+    {
+    case 1:
+        DispatchInterp<T, 1>(interp, a, N, dstHost, stream);
+        break;
+    case 3:
+        DispatchInterp<T, 3>(interp, a, N, dstHost, stream);
+        break;
+    case 4:
+        DispatchInterp<T, 4>(interp, a, N, dstHost, stream);
+        break;
+    default:
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid channel number %d", C);
+    }
+}
+
+void DispatchType(ElemType e, int C, int interp, const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost,
+                  hipStream_t stream)
+{
+    if (N == 0)
+    {
+        return;
+    }
+    switch (e)
+    {
+    case kU8:
+        DispatchC<uint8_t>(C, interp, a, N, dstHost, stream);
+        break;
+    case kU16:
+        DispatchC<uint16_t>(C, interp, a, N, dstHost, stream);
+        break;
+    case kS16:
+        DispatchC<int16_t>(C, interp, a, N, dstHost, stream);
+        break;
+    case kF32:
+        DispatchC<float>(C, interp, a, N, dstHost, stream);
+        break;
+    default:
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid DataType");
+    }
+}
+
+void CheckBorder(NVCVBorderType b)
+{
+    if ((int)b < NVCV_BORDER_CONSTANT || (int)b > NVCV_BORDER_REFLECT101)
+    {
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid border mode %d", (int)b);
+    }
+}
+
+void InvertAffineHost(const float *M, float *out)
+{
+    float den = M[0] * M[4] - M[1] * M[3];
+    den       = std::abs(den) > 1e-5 ? 1. / den : .0;
+    out[0]    = (float)M[4] * den;
+    out[1]    = (float)-M[1] * den;
+    out[2]    = (float)(M[1] * M[5] - M[4] * M[2]) * den;
+    out[3]    = (float)-M[3] * den;
+    out[4]    = (float)M[0] * den;
+    out[5]    = (float)(M[3] * M[2] - M[0] * M[5]) * den;
+    out[6] = out[7] = out[8] = 0.f;
+}
+
+void InvertPerspectiveHost(const float *f, float *m)
+{
+    const float d
+        = f[0] * (f[4] * f[8] - f[5] * f[7]) + f[1] * (f[5] * f[6] - f[3] * f[8]) + f[2] * (f[3] * f[7] - f[4] * f[6]);
+    if (d == 0)
+    {
+        std::copy_n(f, 9, m);
+        return;
+    }
+    m[0] = (f[4] * f[8] - f[5] * f[7]) / d;
+    m[1] = -(f[1] * f[8] - f[2] * f[7]) / d;
+    m[2] = (f[1] * f[5] - f[2] * f[4]) / d;
+    m[3] = -(f[3] * f[8] - f[5] * f[6]) / d;
+    m[4] = (f[0] * f[8] - f[2] * f[6]) / d;
+    m[5] = -(f[0] * f[5] - f[2] * f[3]) / d;
+    m[6] = (f[3] * f[7] - f[4] * f[6]) / d;
+    m[7] = -(f[0] * f[7] - f[1] * f[6]) / d;
+    m[8] = (f[0] * f[4] - f[1] * f[3]) / d;
+}
+
+class Warp : public IOperator
+{
+public:
+    Warp(bool perspective, int32_t maxVarShapeBatchSize)
+        : m_perspective(perspective)
+        , m_maxBatch(maxVarShapeBatchSize)
+    {
+        if (maxVarShapeBatchSize < 0)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "maxVarShapeBatchSize must be >= 0");
+        }
+    }
+
+    void submit(hipStream_t stream, NVCVTensorHandle hin, NVCVTensorHandle hout, const float *xform, int32_t flags,
+                NVCVBorderType border, float4 bval) const
+    {
+        if (xform == nullptr)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Transformation matrix must not be NULL");
+        }
+        NVCVTensorData din, dout;
+        ExportTensor(hin, din, "Input");
+        ExportTensor(hout, dout, "Output");
+        ImageBatchView in  = RequireImageBatchView(din, "Input", NVCV_ERROR_INVALID_ARGUMENT);
+        ImageBatchView out = RequireImageBatchView(dout, "Output", NVCV_ERROR_INVALID_ARGUMENT);
+        if (in.layout != kLayoutNHWC || out.layout != kLayoutNHWC || in.hasBatchDim != out.hasBatchDim)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Invalid DataFormat between input (%s) and output (%s): both must be \"NHWC\" or \"HWC\"",
+                          in.layoutName, out.layoutName);
+        }
+        if (in.C > 4)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid channel number %d", in.C);
+        }
+        if (in.elem != out.elem || in.C != out.C || in.N != out.N)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Input and output must have the same data type, channel count and batch size");
+        }
+        if (std::max(in.bytesSpanned(), out.bytesSpanned()) > INT32_MAX)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Input or output size exceeds %d. Tensor is too large.",
+                          INT32_MAX);
+        }
+        CheckBorder(border);
+        WarpArgs a = makeArgs(border, bval);
+        if (flags & NVCV_WARP_INVERSE_MAP)
+        {
+            for (int i = 0; i < 9; ++i)
+            {
+                a.m[i] = i < (m_perspective ? 9 : 6) ? xform[i] : 0.f;
+            }
+        }
+        else if (m_perspective)
+        {
+            InvertPerspectiveHost(xform, a.m);
+        }
+        else
+        {
+            InvertAffineHost(xform, a.m);
+        }
+        a.src    = in.base;
+        a.dst    = out.base;
+        a.srcN   = in.strideN;
+        a.dstN   = out.strideN;
+        a.srcRow = (int32_t)in.strideH;
+        a.dstRow = (int32_t)out.strideH;
+        a.srcW   = in.W;
+        a.srcH   = in.H;
+        a.dstW   = out.W;
+        a.dstH   = out.H;
+        if (out.W == 0 || out.H == 0 || in.W == 0 || in.H == 0)
+        {
+            return;
+        }
+        DispatchType(in.elem, in.C, flags & NVCV_INTERP_MAX, a, in.N, nullptr, stream);
+    }
+
+    void submit(hipStream_t stream, NVCVImageBatchHandle hin, NVCVImageBatchHandle hout, NVCVTensorHandle hxform,
+                int32_t flags, NVCVBorderType border, float4 bval) const
+    {
+        if (m_maxBatch <= 0)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Operator was not created for var-shape use, maxVarShapeBatchSize: %d", m_maxBatch);
+        }
+        VarShapeView in  = ExportVarShape(hin, stream, "Input");
+        VarShapeView out = ExportVarShape(hout, stream, "Output");
+        if (in.N > m_maxBatch)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid number of images, it should not exceed %d", m_maxBatch);
+        }
+        if (in.N != out.N)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input and output batch sizes: %d != %d", in.N, out.N);
+        }
+        if (in.uniqueFormat == NVCV_IMAGE_FORMAT_NONE || in.uniqueFormat != out.uniqueFormat)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Images in the input and output varshape must all have the same format");
+        }
+        FormatInfo fi = DecodeFormat(in.uniqueFormat);
+        if (fi.planes != 1)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Images must have a single interleaved plane");
+        }
+        if (fi.channels > 4)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid channel number %d", fi.channels);
+        }
+        CheckBorder(border);
+        NVCVTensorData dx;
+        ExportTensor(hxform, dx, "Transformation matrix");
+        const int  cols = m_perspective ? 9 : 6;
+        DTypeInfo  dt   = DecodeDataType(dx.dtype);
+        const bool ok   = dt.elem == kF32 && dt.channels == 1 && dx.rank == 2 && dx.shape[0] >= in.N
+                     && dx.shape[1] == cols && dx.buffer.strided.strides[1] == 4;
+        if (!ok)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Transformation matrix tensor must be float32 of shape [N,%d] with packed rows, N >= %d", cols,
+                          in.N);
+        }
+        WarpArgs a     = makeArgs(border, bval);
+        a.srcList      = in.data.buffer.varShapeStrided.imageList;
+        a.dstList      = out.data.buffer.varShapeStrided.imageList;
+        a.xforms       = dx.buffer.strided.basePtr;
+        a.xformStride  = dx.buffer.strided.strides[0];
+        a.inverseGiven = (flags & NVCV_WARP_INVERSE_MAP) ? 1 : 0;
+        DispatchType(fi.elem, fi.channels, flags & NVCV_INTERP_MAX, a, in.N, out.hostList, stream);
+    }
+
+private:
+    WarpArgs makeArgs(NVCVBorderType border, float4 bval) const
+    {
+        WarpArgs a    = {};
+        a.perspective = m_perspective ? 1 : 0;
+        a.border      = (int32_t)border;
+        a.bval[0]     = bval.x;
+        a.bval[1]     = bval.y;
+        a.bval[2]     = bval.z;
+        a.bval[3]     = bval.w;
+        return a;
+    }
+
+    bool    m_perspective;
+    int32_t m_maxBatch;
+};
+
+class WarpAffine final : public Warp
+{
+public:
+    explicit WarpAffine(int32_t maxBatch)
+        : Warp(false, maxBatch)
+    {
+    }
+};
+
+class WarpPerspective final : public Warp
+{
+public:
+    explicit WarpPerspective(int32_t maxBatch)
+        : Warp(true, maxBatch)
+    {
+    }
+};
+
+} // namespace
+} // namespace cvamd
+
+using namespace cvamd;
+
+extern "C"
+{
+CVCUDA_PUBLIC NVCVStatus cvcudaWarpAffineCreate(NVCVOperatorHandle *handle, const int32_t maxVarShapeBatchSize)
+{
+    return CreateOperator<WarpAffine>(handle, maxVarShapeBatchSize);
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaWarpAffineSubmit(NVCVOperatorHandle handle, hipStream_t stream, NVCVTensorHandle in,
+                                                NVCVTensorHandle out, const NVCVAffineTransform xform,
+                                                const int32_t flags, const NVCVBorderType borderMode,
+                                                const float4 borderValue)
+{
+    return Protect([&] { ToOperator<WarpAffine>(handle).submit(stream, in, out, xform, flags, borderMode, borderValue); });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaWarpAffineVarShapeSubmit(NVCVOperatorHandle handle, hipStream_t stream,
+                                                        NVCVImageBatchHandle in, NVCVImageBatchHandle out,
+                                                        NVCVTensorHandle transMatrix, const int32_t flags,
+                                                        const NVCVBorderType borderMode, const float4 borderValue)
+{
+    return Protect(
+        [&] { ToOperator<WarpAffine>(handle).submit(stream, in, out, transMatrix, flags, borderMode, borderValue); });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaWarpPerspectiveCreate(NVCVOperatorHandle *handle, const int32_t maxVarShapeBatchSize)
+{
+    return CreateOperator<WarpPerspective>(handle, maxVarShapeBatchSize);
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaWarpPerspectiveSubmit(NVCVOperatorHandle handle, hipStream_t stream, NVCVTensorHandle in,
+                                                     NVCVTensorHandle out, const NVCVPerspectiveTransform transMatrix,
+                                                     const int32_t flags, const NVCVBorderType borderMode,
+                                                     const float4 borderValue)
+{
+    return Protect(
+        [&] { ToOperator<WarpPerspective>(handle).submit(stream, in, out, transMatrix, flags, borderMode, borderValue); });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaWarpPerspectiveVarShapeSubmit(NVCVOperatorHandle handle, hipStream_t stream,
+                                                             NVCVImageBatchHandle in, NVCVImageBatchHandle out,
+                                                             NVCVTensorHandle transMatrix, const int32_t flags,
+                                                             const NVCVBorderType borderMode, const float4 borderValue)
+{
+    return Protect(
+        [&]
+        { ToOperator<WarpPerspective>(handle).submit(stream, in, out, transMatrix, flags, borderMode, borderValue); });
+}
+}

@@ -1,0 +1,202 @@
+"""GPU parity of cvcudaWarpAffine / cvcudaWarpPerspective [VarShape] Submit.
+
+Exact-equality rows: the reference's table on tiny RGBA8 images with small integer matrices, all
+five borders, three interpolations, forward and inverse maps
+(tests/cvcuda/system/TestOpWarpAffine.cpp:232-319). Random rotations/scales: <= 1 LSB against the
+reference's golden (oracle variant 0) and bit-exact against the device-formula restatement
+(variant 1). BASELINE configuration 4 at full size."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+NEAREST, LINEAR, CUBIC = 0, 1, 2
+INVERSE_MAP = 16
+
+SIZES = [(5, 4, 5, 4), (5, 4, 6, 8), (7, 8, 4, 5)]
+MATS = [(1, 0, 0, 0, 1, 0), (1, 0, 1, 0, 1, 2), (1, 2, 1, 2, 1, 2), (2, 2, 1, 3, 1, 2), (1, 2, 0, 1, 1, 0),
+        (2, 2, 0, 3, 1, 1), (1, 0, 0, 0, 1, 1), (1, 2, 0, 2, 1, 1), (2, 2, 0, 3, 1, 0), (0.5, 2, 1, 0.75, 1, 2)]
+
+
+def to_inverse(orc, m, inverse_given):
+    return np.asarray(m, np.float32) if inverse_given else orc.invert_affine(m)
+
+
+@pytest.mark.parametrize("interp", [NEAREST, LINEAR, CUBIC])
+@pytest.mark.parametrize("border", [0, 1, 2, 3, 4])
+def test_reference_table_exact(cv, orc, gpu, interp, border):
+    op = cv.WarpAffine(0)
+    for (sw, sh, dw, dh), m, inv in itertools.product(SIZES, MATS, (True, False)):
+        src = orc.fill_u8((4, sh, sw, 4), sw * 100 + dh + int(m[1]))
+        tin = cv.Tensor.from_numpy(src, "NHWC")
+        tout = cv.Tensor.alloc([4, dh, dw, 4], np.uint8, "NHWC")
+        op(None, tin, tout, m, interp | (INVERSE_MAP if inv else 0), border, (1, 2, 3, 4))
+        torch.cuda.synchronize()
+        res = tout.numpy()
+        minv = to_inverse(orc, m, inv)
+        dev = orc.warp(src, (dh, dw), minv, interp, border, (1, 2, 3, 4), variant=1)
+        np.testing.assert_array_equal(res, dev, err_msg=str((sw, sh, dw, dh, m, inv)))
+        gold = orc.warp(src, (dh, dw), minv, interp, border, (1, 2, 3, 4), variant=0)
+        exact = interp != CUBIC and all(float(v).is_integer() for v in minv)
+        tol = 0 if exact else 1
+        assert np.abs(res.astype(np.int16) - gold.astype(np.int16)).max() <= tol, (sw, sh, dw, dh, m, inv)
+
+
+def rotation(w, h, deg, s):
+    t = np.deg2rad(deg)
+    c, sn = s * np.cos(t), s * np.sin(t)
+    cx, cy = (w - 1) / 2.0, (h - 1) / 2.0
+    return [c, -sn, cx - c * cx + sn * cy, sn, c, cy - sn * cx - c * cy]
+
+
+@pytest.mark.parametrize("dt,c", [(np.uint8, 3), (np.uint8, 1), (np.uint8, 4), (np.uint16, 3), (np.int16, 4),
+                                  (np.float32, 1), (np.float32, 3)])
+@pytest.mark.parametrize("interp", [NEAREST, LINEAR, CUBIC])
+def test_random_rotations_tensor(cv, orc, gpu, dt, c, interp):
+    n, h, w = 2, 97, 131
+    if dt == np.float32:
+        src = orc.fill_f32((n, h, w, c), 7) * 255
+    else:
+        src = orc.fill_u8((n, h, w, c, np.dtype(dt).itemsize), 7).view(dt).reshape(n, h, w, c)
+    op = cv.WarpAffine(0)
+    for deg, s, border in [(17.0, 1.1, 0), (-29.0, 0.85, 1), (5.5, 1.0, 4), (30.0, 1.2, 3), (-11.0, 0.9, 2)]:
+        m = rotation(w, h, deg, s)
+        tout = cv.Tensor.alloc([n, 80, 150, c], dt, "NHWC")
+        op(None, cv.Tensor.from_numpy(src, "NHWC"), tout, m, interp, border, (9, 8, 7, 6))
+        torch.cuda.synchronize()
+        res = tout.numpy()
+        minv = orc.invert_affine(m)
+        dev = orc.warp(src, (80, 150), minv, interp, border, (9, 8, 7, 6), variant=1)
+        if dt == np.float32:
+            assert np.abs(res - dev).max() <= 1e-3
+        else:
+            np.testing.assert_array_equal(res, dev)
+            if dt == np.uint8 and interp != NEAREST:
+                gold = orc.warp(src, (80, 150), minv, interp, border, (9, 8, 7, 6), variant=0)
+                assert np.abs(res.astype(np.int16) - gold.astype(np.int16)).max() <= 1
+
+
+def make_c4_batch(cv, K, orc, n, seed):
+    rng = np.random.default_rng(seed)
+    bi, bo, hosts, outs, mats = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], [], []
+    for i in range(n):
+        w, h = int(rng.integers(640, 1921)), int(rng.integers(480, 1081))
+        a = orc.fill_u8((h, w, 3), 0xC0FFEE04 + i)
+        hosts.append(a)
+        bi.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_RGB8))
+        o = cv.Image.alloc((w, h), K.IMAGE_FORMAT_RGB8)
+        outs.append(o)
+        bo.push_back(o)
+        mats.append(rotation(w, h, float(rng.uniform(-30, 30)), float(rng.uniform(0.8, 1.2))))
+    return bi, bo, hosts, outs, np.asarray(mats, np.float32)
+
+
+def test_config4_varshape_full_size(cv, K, orc, gpu):
+    # BASELINE config 4: 32 u8 RGB images, sizes in [640,1920]x[480,1080], rotation +-30deg / scale
+    # 0.8-1.2 about the centre as forward maps, bilinear, constant border 0; <= 1 LSB vs golden
+    n = 32
+    bi, bo, hosts, outs, mats = make_c4_batch(cv, K, orc, n, 4)
+    txf = cv.Tensor.from_numpy(mats, "NW")
+    cv.WarpAffine(n)(None, bi, bo, txf, LINEAR, 0, (0, 0, 0, 0))
+    torch.cuda.synchronize()
+    for i in range(n):
+        a, o = hosts[i], outs[i]
+        res = o.plane_view(0, np.uint8, 3).cpu().numpy()
+        minv = orc.invert_affine(mats[i])
+        gold = orc.warp(a[None], a.shape[:2], minv, LINEAR, 0, (0, 0, 0, 0), variant=0, threads=1)[0]
+        assert np.abs(res.astype(np.int16) - gold.astype(np.int16)).max() <= 1
+        if i < 4:
+            dev = orc.warp(a[None], a.shape[:2], minv, LINEAR, 0, (0, 0, 0, 0), variant=1)[0]
+            np.testing.assert_array_equal(res, dev)
+
+
+def test_varshape_small_all_modes_and_inverse_flag(cv, K, orc, gpu):
+    rng = np.random.default_rng(11)
+    n = 5
+    bi, bo, hosts, outs, mats = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], [], []
+    for i in range(n):
+        w, h = int(rng.integers(20, 120)), int(rng.integers(20, 90))
+        dw, dh = int(rng.integers(20, 140)), int(rng.integers(20, 100))
+        a = orc.fill_u8((h, w, 4), 200 + i)
+        hosts.append(a)
+        bi.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_RGBA8))
+        o = cv.Image.alloc((dw, dh), K.IMAGE_FORMAT_RGBA8)
+        outs.append(o)
+        bo.push_back(o)
+        mats.append(rotation(w, h, float(rng.uniform(-40, 40)), float(rng.uniform(0.7, 1.4))))
+    mats = np.asarray(mats, np.float32)
+    op = cv.WarpAffine(8)
+    for interp, border, inv in itertools.product((NEAREST, LINEAR, CUBIC), range(5), (False, True)):
+        op(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), interp | (INVERSE_MAP if inv else 0), border,
+           (10, 20, 30, 40))
+        torch.cuda.synchronize()
+        for i in range(n):
+            w, h = outs[i].size
+            res = outs[i].plane_view(0, np.uint8, 4).cpu().numpy()
+            minv = mats[i] if inv else orc.invert_affine(mats[i])
+            dev = orc.warp(hosts[i][None], (h, w), minv, interp, border, (10, 20, 30, 40), variant=1)[0]
+            np.testing.assert_array_equal(res, dev, err_msg=str((interp, border, inv, i)))
+    with pytest.raises(cv.Error) as e:
+        cv.WarpAffine(4)(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), LINEAR)  # batch 5 > max 4
+    assert e.value.status == 2
+    with pytest.raises(cv.Error) as e:
+        cv.WarpAffine(0)(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), LINEAR)
+    assert e.value.status == 2
+
+
+def homography_inverse(m):
+    f = np.asarray(m, np.float32)
+    d = f[0] * (f[4] * f[8] - f[5] * f[7]) + f[1] * (f[5] * f[6] - f[3] * f[8]) + f[2] * (f[3] * f[7] - f[4] * f[6])
+    return np.array([(f[4] * f[8] - f[5] * f[7]) / d, -(f[1] * f[8] - f[2] * f[7]) / d, (f[1] * f[5] - f[2] * f[4]) / d,
+                     -(f[3] * f[8] - f[5] * f[6]) / d, (f[0] * f[8] - f[2] * f[6]) / d, -(f[0] * f[5] - f[2] * f[3]) / d,
+                     (f[3] * f[7] - f[4] * f[6]) / d, -(f[0] * f[7] - f[1] * f[6]) / d, (f[0] * f[4] - f[1] * f[3]) / d],
+                    np.float32)
+
+
+def test_warp_perspective(cv, K, orc, gpu):
+    src = orc.fill_u8((2, 60, 80, 3), 21)
+    H = [1.05, 0.08, -3.0, -0.04, 0.97, 2.0, 2e-4, -1e-4, 1.0]
+    op = cv.WarpPerspective(4)
+    for interp, border in itertools.product((NEAREST, LINEAR, CUBIC), (0, 1, 4)):
+        for inv in (True, False):
+            tout = cv.Tensor.alloc([2, 50, 90, 3], np.uint8, "NHWC")
+            op(None, cv.Tensor.from_numpy(src, "NHWC"), tout, H, interp | (INVERSE_MAP if inv else 0), border,
+               (5, 6, 7, 0))
+            torch.cuda.synchronize()
+            minv = np.asarray(H, np.float32) if inv else homography_inverse(H)
+            ref = orc.warp(src, (50, 90), minv, interp, border, (5, 6, 7, 0), perspective=True, variant=1)
+            d = np.abs(tout.numpy().astype(np.int16) - ref.astype(np.int16))
+            # 1/x on the device is correctly rounded like the host's; allow 1 LSB for the inverse path whose
+            # matrix entries come from float divisions evaluated on host in this test
+            assert d.max() <= (0 if inv else 1)
+    # var-shape: two images, matrices in a [N,9] tensor
+    bi, bo = cv.ImageBatchVarShape(2), cv.ImageBatchVarShape(2)
+    outs = []
+    for i in range(2):
+        bi.push_back(cv.Image.from_numpy(src[i], K.IMAGE_FORMAT_RGB8))
+        o = cv.Image.alloc((90, 50), K.IMAGE_FORMAT_RGB8)
+        outs.append(o)
+        bo.push_back(o)
+    mats = np.asarray([H, H], np.float32)
+    op(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), LINEAR | INVERSE_MAP, 1, (0, 0, 0, 0))
+    torch.cuda.synchronize()
+    ref = orc.warp(src, (50, 90), H, LINEAR, 1, perspective=True, variant=1)
+    for i in range(2):
+        np.testing.assert_array_equal(outs[i].plane_view(0, np.uint8, 3).cpu().numpy(), ref[i])
+
+
+def test_tensor_negative(cv, gpu):
+    op = cv.WarpAffine(0)
+    a = cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC")
+    ident = [1, 0, 0, 0, 1, 0]
+    for out, flags, border in [(cv.Tensor.alloc([2, 8, 8, 3], np.float32, "NHWC"), LINEAR, 0),
+                               (cv.Tensor.alloc([3, 8, 8, 3], np.uint8, "NHWC"), LINEAR, 0),
+                               (cv.Tensor.alloc([2, 8, 8, 4], np.uint8, "NHWC"), LINEAR, 0),
+                               (cv.Tensor.alloc([2, 3, 8, 8], np.uint8, "NCHW"), LINEAR, 0),
+                               (cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC"), 3, 0),     # AREA
+                               (cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC"), LINEAR, 9)]:
+        with pytest.raises(cv.Error) as e:
+            op(None, a, out, ident, flags, border)
+        assert e.value.status == 2
