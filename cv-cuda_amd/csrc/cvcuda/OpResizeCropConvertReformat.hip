@@ -44,7 +44,35 @@ struct FusedArgs
     float   scaleX, scaleY; // tensor path: srcW/newW, srcH/newH
     float   scale, offset;
     int32_t srcCast;
+    // launch shape: column tiles and row tiles per image; the grid is 1-D
+    uint32_t tilesX, tilesY;
+    uint32_t rowTiles; // tilesY * N
 };
+
+struct TilePos
+{
+    int n, tx, ty;
+};
+
+// Hardware workgroup id -> (image, row tile, column tile).
+// The column tiles of one row tile read overlapping cache lines (a 128-byte line straddles each
+// tile boundary). MI355X deals workgroups to its 8 XCDs round-robin and each XCD has its own L2, so
+// with the natural order both neighbours would fetch the shared line from memory. Here the column
+// tiles of a row tile go to ONE XCD on consecutive turns (the second hits in L2), while consecutive
+// row tiles still go to consecutive XCDs, so that all XCDs stream through the same region of the
+// batch at the same time. The launch is padded to a multiple of 8 row tiles; padding workgroups
+// get an out-of-range column and leave at once.
+__device__ __forceinline__ TilePos LocateFusedTile(const FusedArgs &a)
+{
+    const uint32_t xcd = blockIdx.x % kXcdCount, turn = blockIdx.x / kXcdCount;
+    const uint32_t inRow   = turn % a.tilesX;
+    const uint32_t rowTile = (turn / a.tilesX) * kXcdCount + xcd; // over all images
+    TilePos        p;
+    p.n  = (int)(rowTile / a.tilesY);
+    p.ty = (int)(rowTile - (uint32_t)p.n * a.tilesY);
+    p.tx = rowTile < a.rowTiles ? (int)inRow : (1 << 24);
+    return p;
+}
 
 struct SrcImage
 {
@@ -93,10 +121,11 @@ __device__ __forceinline__ void StorePixel(const FusedArgs &a, DstT *out, float 
 template<class DstT, bool VARSHAPE>
 __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
 {
-    const int n    = blockIdx.z;
-    const int dx   = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int wave = threadIdx.x >> 6;
-    const int dy0  = blockIdx.y * kRowsPerBlock + wave * kRowsPerWave;
+    const TilePos tp   = LocateFusedTile(a);
+    const int     n    = tp.n;
+    const int     dx   = tp.tx * 64 + (threadIdx.x & 63);
+    const int     wave = threadIdx.x >> 6;
+    const int     dy0  = tp.ty * kRowsPerBlock + wave * kRowsPerWave;
     if (dx >= a.dstW)
     {
         return;
@@ -129,10 +158,11 @@ __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
 template<class DstT, bool VARSHAPE, bool BYTEWISE>
 __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
 {
-    const int n    = blockIdx.z;
-    const int dx   = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int wave = threadIdx.x >> 6;
-    const int dy0  = blockIdx.y * kRowsPerBlock + wave * kRowsPerWave;
+    const TilePos tp   = LocateFusedTile(a);
+    const int     n    = tp.n;
+    const int     dx   = tp.tx * 64 + (threadIdx.x & 63);
+    const int     wave = threadIdx.x >> 6;
+    const int     dy0  = tp.ty * kRowsPerBlock + wave * kRowsPerWave;
     if (dx >= a.dstW)
     {
         return;
@@ -211,14 +241,23 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
 }
 
 template<class DstT, bool VARSHAPE>
-void Launch(const FusedArgs &a, int N, NVCVInterpolationType interp, bool tinyImages, hipStream_t stream)
+void Launch(FusedArgs a, int N, NVCVInterpolationType interp, bool tinyImages, hipStream_t stream)
 {
-    dim3 block(256);
-    dim3 grid(DivUp(a.dstW, 64), DivUp(a.dstH, kRowsPerBlock), N);
     if (N == 0 || a.dstW == 0 || a.dstH == 0)
     {
         return;
     }
+    a.tilesX            = DivUp(a.dstW, 64);
+    a.tilesY            = DivUp(a.dstH, kRowsPerBlock);
+    a.rowTiles          = a.tilesY * N;
+    const int64_t total = (int64_t)a.tilesX * DivUp(a.rowTiles, kXcdCount) * kXcdCount;
+    if (total > INT32_MAX)
+    {
+        throw OpError(NVCV_ERROR_OVERFLOW, "Output of %d images of %d x %d needs too many tiles for one launch", N,
+                      a.dstW, a.dstH);
+    }
+    dim3 block(256);
+    dim3 grid((uint32_t)total);
     if (interp == NVCV_INTERP_NEAREST)
     {
         hipLaunchKernelGGL((FusedNearest<DstT, VARSHAPE>), grid, block, 0, stream, a);
