@@ -1,58 +1,311 @@
 #!/usr/bin/env python3
-"""Benchmark of the fused ResizeCropConvertReformat hot path on one MI355X.
+"""Benchmark of the image pre-processing hot path on one MI355X.
 
-A step = one cvcudaResizeCropConvertReformatSubmit over a batch of 64 1080p u8 RGB images
-(bilinear resize to 455x256, centre crop 224x224, scale/offset, f32 NCHW output). Inputs are
-generated on the host from a fixed seed and uploaded before the timed region. To keep the reads
-coming from HBM rather than from the 256 MB on-die cache, consecutive steps cycle through
-`--rotate` distinct input/output buffer sets (default 4; 1 = same buffers every step).
+Default workload (the headline one): a step = one cvcudaResizeCropConvertReformatSubmit over a batch
+of 64 1080p u8 RGB images (bilinear resize to 455x256, centre crop 224x224, scale/offset, f32 NCHW
+output). `--workload` selects the other configurations (plain resize, NV12->RGB, var-shape affine warp,
+4K cubic resize); each is one Submit per step.
 
-Prints ONE JSON line: throughput (images/s), the HBM roofline fraction of the kernel
-(algorithmic bytes / mean kernel time / 8 TB/s) and the CPU oracle's throughput on the same workload.
+Inputs are generated on the host from a fixed seed and uploaded before the timed region. To keep
+the reads coming from HBM rather than from the 256 MB on-die cache, consecutive steps cycle through
+`--rotate` distinct input/output buffer sets (default: enough sets to touch >= 450 MB; 1 = same
+buffers every step).
+
+Prints ONE JSON line: throughput (images/s), the HBM roofline fraction of the kernel (algorithmic
+bytes / mean kernel time / 8 TB/s) and the CPU oracle's throughput on a bounded sample of the same
+workload.
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
 
 HBM_PEAK_GBS = 8000.0
+SEED_BASE = 0xC0FFEE00
+NEAREST, LINEAR, CUBIC = 0, 1, 2
 
-# workload: BASELINE configuration 2
-N, SRC_H, SRC_W = 64, 1080, 1920
-NEW_W, NEW_H = 455, 256
-CROP_X, CROP_Y = 115, 16
-OUT_H, OUT_W = 224, 224
-SCALE, OFFSET = 1.0 / (255.0 * 0.226), -0.449 / 0.226
-SEED = 0xC0FFEE02
-
-# HBM bytes one launch of the kernel moves, from hardware counters (rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE in separate runs, each scaled by what the same counter reads for a 128 MiB device
-# copy: x1.99965 and x1.00000). It is a property of the kernel and this workload, not of a run, so it
-# is recorded here rather than re-measured: 84,436,703 read + 38,535,168 written.
-MEASURED_TRAFFIC_BYTES = 122971871
+# HBM bytes one launch of the headline kernel moves, from hardware counters (rocprofv3 --pmc
+# FETCH_SIZE and --pmc WRITE_SIZE in separate runs, each scaled by what the same counter reads for a
+# 128 MiB device copy: x1.99965 and x1.00000). It is a property of the kernel and the workload, not
+# of a run, so it is recorded here rather than re-measured: 84,436,703 read + 38,535,168 written.
+MEASURED_TRAFFIC_BYTES = {"fused": 122971871}
 
 
-def algorithmic_bytes_per_image():
-    """Row-span compulsory traffic: distinct source rows referenced x byte span between the first and
-    last referenced pixel of a row, plus the output bytes. Computed from the op's own index map."""
+def span_bytes(n_out, crop, src, new, interp, pixel_bytes):
+    """Distinct source indices referenced along one axis and the byte span first..last (times
+    pixel_bytes), from the operators' own float32 index maps."""
     import numpy as np
     f32 = np.float32
+    s = f32(src) / f32(new)
+    d = np.arange(n_out, dtype=np.float32) + f32(crop)
+    if interp == NEAREST:
+        idx = np.minimum(np.floor((d + f32(0.5)) * s).astype(np.int64), src - 1)
+    elif interp == LINEAR:
+        i0 = np.floor((d + f32(0.5)) * s - f32(0.5)).astype(np.int64)
+        idx = np.concatenate([np.clip(i0, 0, src - 1), np.clip(i0 + 1, 0, src - 1)])
+    else:
+        i0 = np.clip(np.floor((d + f32(0.5)) * s - f32(0.5)).astype(np.int64), 1, src - 3)
+        idx = np.concatenate([i0 - 1, i0, i0 + 1, i0 + 2])
+    return len(np.unique(idx)), (int(idx.max()) - int(idx.min()) + 1) * pixel_bytes
 
-    def taps(n_out, crop, src, new):
-        s = f32(src) / f32(new)
-        f = (np.arange(n_out, dtype=np.float32) + f32(crop) + f32(0.5)) * s - f32(0.5)
-        i0 = np.floor(f).astype(np.int64)
-        i1 = np.minimum(i0 + 1, src - 1)
-        return np.maximum(i0, 0), i1
 
-    y0, y1 = taps(OUT_H, CROP_Y, SRC_H, NEW_H)
-    x0, x1 = taps(OUT_W, CROP_X, SRC_W, NEW_W)
-    rows = len(np.unique(np.concatenate([y0, y1])))
-    span = (int(x1.max()) - int(x0.min()) + 1) * 3
-    read = rows * span
-    write = 3 * OUT_H * OUT_W * 4
-    return read, write
+def polygon_clip_area(poly, w, h):
+    """Area of a convex polygon clipped to [0,w]x[0,h] (Sutherland-Hodgman + shoelace)."""
+    def clip(pts, inside, inter):
+        out = []
+        for i in range(len(pts)):
+            a, b = pts[i - 1], pts[i]
+            ia, ib = inside(a), inside(b)
+            if ia != ib:
+                out.append(inter(a, b))
+            if ib:
+                out.append(b)
+        return out
+
+    def ix(x0):
+        return lambda a, b: (x0, a[1] + (b[1] - a[1]) * (x0 - a[0]) / (b[0] - a[0]))
+
+    def iy(y0):
+        return lambda a, b: (a[0] + (b[0] - a[0]) * (y0 - a[1]) / (b[1] - a[1]), y0)
+
+    pts = list(poly)
+    for inside, inter in ((lambda p: p[0] >= 0, ix(0.0)), (lambda p: p[0] <= w, ix(float(w))),
+                          (lambda p: p[1] >= 0, iy(0.0)), (lambda p: p[1] <= h, iy(float(h)))):
+        if not pts:
+            return 0.0
+        pts = clip(pts, inside, inter)
+    area = 0.0
+    for i in range(len(pts)):
+        area += pts[i - 1][0] * pts[i][1] - pts[i][0] * pts[i - 1][1]
+    return abs(area) / 2
+
+
+# ------------------------------------------------------------------------------------------------
+# Workloads. Each class offers: key, kernel, workload (text), dtype, images (per step), alg_bytes
+# (per step), make_set() -> buffer set, submit(stream, set), check(set) (oracle spot check of what
+# the GPU produced), cpu(threads) -> images the oracle processed.
+class Fused:
+    key, config_id = "fused", 2
+    N, SRC_H, SRC_W = 64, 1080, 1920
+    NEW_W, NEW_H, CROP_X, CROP_Y, OUT_H, OUT_W = 455, 256, 115, 16, 224, 224
+    SCALE, OFFSET = 1.0 / (255.0 * 0.226), -0.449 / 0.226
+    kernel = "FusedBilinear<float,false,false>"
+    dtype = "f32"
+    workload = ("fused ResizeCropConvertReformat: batch 64 u8 NHWC 1920x1080 -> bilinear 455x256 -> "
+                "crop 224x224 @(115,16) -> f32 NCHW, scale/offset")
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        rows, _ = span_bytes(self.OUT_H, self.CROP_Y, self.SRC_H, self.NEW_H, LINEAR, 1)
+        _, span = span_bytes(self.OUT_W, self.CROP_X, self.SRC_W, self.NEW_W, LINEAR, 3)
+        self.alg_bytes = (rows * span + 3 * self.OUT_H * self.OUT_W * 4) * self.N
+        self.host = orc.fill_u8((self.N, self.SRC_H, self.SRC_W, 3), SEED_BASE + self.config_id)
+        self.dev = torch.from_numpy(self.host).cuda()
+        self.op = cv.ResizeCropConvertReformat()
+
+    def make_set(self):
+        tin = self.cv.Tensor.alloc([self.N, self.SRC_H, self.SRC_W, 3], self.np.uint8, "NHWC")
+        tin.torch_view().copy_(self.dev)
+        return tin, self.cv.Tensor.alloc([self.N, 3, self.OUT_H, self.OUT_W], self.np.float32, "NCHW")
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], (self.NEW_W, self.NEW_H), LINEAR, (self.CROP_X, self.CROP_Y), 0, self.SCALE,
+                self.OFFSET, False)
+
+    def _oracle(self, src, threads=1):
+        return self.orc.fused_rccr(src, (self.OUT_H, self.OUT_W), (self.NEW_W, self.NEW_H), (self.CROP_X, self.CROP_Y),
+                                   LINEAR, self.np.float32, True, 0, self.SCALE, self.OFFSET, False, threads=threads)
+
+    def check(self, s):
+        np = self.np
+        ref = self._oracle(self.host[:2])
+        got = s[1].torch_view()[:2].cpu().numpy()
+        assert (np.abs(got - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all(), "bench output differs from oracle"
+
+    def cpu(self, threads):
+        self._oracle(self.host[:8], threads)
+        return 8
+
+
+class ResizeC1:
+    config_id = 1
+    N, SRC_H, SRC_W, OUT_H, OUT_W = 8, 1080, 1920, 224, 224
+    dtype = "f32"
+
+    def __init__(self, cv, orc, np, torch, interp):
+        self.cv, self.orc, self.np, self.torch, self.interp = cv, orc, np, torch, interp
+        name = "NEAREST" if interp == NEAREST else "LINEAR"
+        self.key = "resize-" + name.lower()
+        self.kernel = "ResizeTensorKernel<uint8_t,3,%s>" % name
+        self.workload = "Resize %s: batch 8 u8 NHWC 1920x1080 -> 224x224" % name
+        self.images = self.N
+        rows, _ = span_bytes(self.OUT_H, 0, self.SRC_H, self.OUT_H, interp, 1)
+        _, span = span_bytes(self.OUT_W, 0, self.SRC_W, self.OUT_W, interp, 3)
+        self.alg_bytes = (rows * span + self.OUT_H * self.OUT_W * 3) * self.N
+        self.host = orc.fill_u8((self.N, self.SRC_H, self.SRC_W, 3), SEED_BASE + self.config_id)
+        self.dev = torch.from_numpy(self.host).cuda()
+        self.op = cv.Resize()
+
+    def make_set(self):
+        tin = self.cv.Tensor.alloc([self.N, self.SRC_H, self.SRC_W, 3], self.np.uint8, "NHWC")
+        tin.torch_view().copy_(self.dev)
+        return tin, self.cv.Tensor.alloc([self.N, self.OUT_H, self.OUT_W, 3], self.np.uint8, "NHWC")
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], self.interp)
+
+    def check(self, s):
+        ref = self.orc.resize(self.host[:2], (self.OUT_H, self.OUT_W), self.interp, variant=0)
+        got = s[1].torch_view()[:2].cpu().numpy()
+        tol = 0 if self.interp == NEAREST else 1
+        assert self.np.abs(got.astype(self.np.int16) - ref.astype(self.np.int16)).max() <= tol
+
+    def cpu(self, threads):
+        self.orc.resize(self.host, (self.OUT_H, self.OUT_W), self.interp, variant=0, threads=threads)
+        return self.N
+
+
+class CubicC5:
+    key, config_id = "resize-cubic-4k", 5
+    N, SRC_H, SRC_W, OUT_H, OUT_W = 16, 2160, 3840, 360, 640
+    kernel = "ResizeTensorKernel<float,4,CUBIC>"
+    dtype = "f32"
+    workload = "Resize CUBIC: batch 16 f32 NHWC 3840x2160x4 -> 640x360x4"
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        rows, _ = span_bytes(self.OUT_H, 0, self.SRC_H, self.OUT_H, CUBIC, 1)
+        _, span = span_bytes(self.OUT_W, 0, self.SRC_W, self.OUT_W, CUBIC, 16)
+        self.alg_bytes = (rows * span + self.OUT_H * self.OUT_W * 16) * self.N
+        self.host = orc.fill_f32((self.N, self.SRC_H, self.SRC_W, 4), SEED_BASE + self.config_id)
+        self.dev = torch.from_numpy(self.host).cuda()
+        self.op = cv.Resize()
+
+    def make_set(self):
+        tin = self.cv.Tensor.alloc([self.N, self.SRC_H, self.SRC_W, 4], self.np.float32, "NHWC")
+        tin.torch_view().copy_(self.dev)
+        return tin, self.cv.Tensor.alloc([self.N, self.OUT_H, self.OUT_W, 4], self.np.float32, "NHWC")
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], CUBIC)
+
+    def check(self, s):
+        ref = self.orc.resize(self.host[:1], (self.OUT_H, self.OUT_W), CUBIC, variant=1)
+        got = s[1].torch_view()[:1].cpu().numpy()
+        assert self.np.abs(got - ref).max() <= 1e-4
+
+    def cpu(self, threads):
+        self.orc.resize(self.host[:4], (self.OUT_H, self.OUT_W), CUBIC, variant=1, threads=threads)
+        return 4
+
+
+class Nv12C3:
+    key, config_id = "nv12-to-rgb", 3
+    N, H, W = 32, 1080, 1920
+    kernel = "Yuv420ToRgbTensor<3,true>"
+    dtype = "int32"
+    workload = "CvtColor YUV2RGB_NV12: batch 32 u8 [1620,1920,1] -> [1080,1920,3]"
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        self.alg_bytes = self.N * (self.H * 3 // 2 * self.W + self.H * self.W * 3)
+        y = orc.fill_u8((self.N, self.H, self.W, 1), SEED_BASE + self.config_id, 16, 235)
+        uv = orc.fill_u8((self.N, self.H // 2, self.W, 1), SEED_BASE + self.config_id + 100, 16, 240)
+        self.host = np.concatenate([y, uv], axis=1)
+        self.dev = torch.from_numpy(self.host).cuda()
+        self.op = cv.CvtColor()
+
+    def make_set(self):
+        tin = self.cv.Tensor.alloc([self.N, self.H * 3 // 2, self.W, 1], self.np.uint8, "NHWC")
+        tin.torch_view().copy_(self.dev)
+        return tin, self.cv.Tensor.alloc([self.N, self.H, self.W, 3], self.np.uint8, "NHWC")
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], 90)
+
+    def check(self, s):
+        ref = self.orc.yuv420_to_rgb(self.host[:1, :, :, 0], 3, False, 0, True, variant=0)
+        got = s[1].torch_view()[:1].cpu().numpy()
+        assert (got == ref).all()
+
+    def cpu(self, threads):
+        self.orc.yuv420_to_rgb(self.host[:16, :, :, 0], 3, False, 0, True, variant=0, threads=threads)
+        return 16
+
+
+class WarpC4:
+    key, config_id = "warp-affine-varshape", 4
+    N = 32
+    kernel = "WarpVarShape<uint8_t,3,LINEAR>"
+    dtype = "f32"
+    workload = ("WarpAffine var-shape LINEAR: 32 u8 RGB images, W in [640,1920], H in [480,1080], rotation +-30 deg "
+                "x scale 0.8-1.2 about the centre, constant border 0")
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        rng = np.random.default_rng(SEED_BASE + self.config_id)
+        self.sizes, mats, alg = [], [], 0
+        for _ in range(self.N):
+            w, h = int(rng.integers(640, 1921)), int(rng.integers(480, 1081))
+            t, s = math.radians(float(rng.uniform(-30, 30))), float(rng.uniform(0.8, 1.2))
+            c, sn, cx, cy = s * math.cos(t), s * math.sin(t), (w - 1) / 2.0, (h - 1) / 2.0
+            m = [c, -sn, cx - c * cx + sn * cy, sn, c, cy - sn * cx - c * cy]
+            self.sizes.append((w, h))
+            mats.append(m)
+            inv = orc.invert_affine(m).astype(np.float64)
+            corners = [(inv[0] * x + inv[1] * y + inv[2], inv[3] * x + inv[4] * y + inv[5])
+                       for x, y in ((0, 0), (w, 0), (w, h), (0, h))]
+            alg += min(w * h * 3, int(3 * polygon_clip_area(corners, w, h))) + w * h * 3
+        self.alg_bytes = alg
+        self.mats = np.asarray(mats, np.float32)
+        self.hosts = [orc.fill_u8((h, w, 3), SEED_BASE + self.config_id + 1000 + i)
+                      for i, (w, h) in enumerate(self.sizes)]
+        self.op = cv.WarpAffine(self.N)
+        self.K = cv.K
+
+    def make_set(self):
+        cv = self.cv
+        bi, bo, outs = cv.ImageBatchVarShape(self.N), cv.ImageBatchVarShape(self.N), []
+        for a, (w, h) in zip(self.hosts, self.sizes):
+            bi.push_back(cv.Image.from_numpy(a, self.K.IMAGE_FORMAT_RGB8))
+            o = cv.Image.alloc((w, h), self.K.IMAGE_FORMAT_RGB8)
+            outs.append(o)
+            bo.push_back(o)
+        return bi, bo, cv.Tensor.from_numpy(self.mats, "NW"), outs
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], s[2], LINEAR, 0, (0, 0, 0, 0))
+
+    def check(self, s):
+        np = self.np
+        a = self.hosts[0]
+        ref = self.orc.warp(a[None], a.shape[:2], self.orc.invert_affine(self.mats[0]), LINEAR, 0, variant=0)[0]
+        got = s[3][0].plane_view(0, np.uint8, 3).cpu().numpy()
+        assert np.abs(got.astype(np.int16) - ref.astype(np.int16)).max() <= 1
+
+    def cpu(self, threads):
+        # images differ in size: the oracle threads over the rows of one image at a time
+        for i in range(8):
+            a = self.hosts[i]
+            self.orc.warp(a[None], a.shape[:2], self.orc.invert_affine(self.mats[i]), LINEAR, 0, variant=0,
+                          threads=threads)
+        return 8
+
+
+WORKLOADS = {
+    "fused": Fused,
+    "resize-nearest": lambda *a: ResizeC1(*a, NEAREST),
+    "resize-linear": lambda *a: ResizeC1(*a, LINEAR),
+    "nv12-to-rgb": Nv12C3,
+    "warp-affine-varshape": WarpC4,
+    "resize-cubic-4k": CubicC5,
+}
 
 
 def main():
@@ -60,7 +313,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--rotate", type=int, default=4, help="distinct buffer sets cycled through (1 = cache-resident)")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="fused")
+    ap.add_argument("--rotate", type=int, default=0,
+                    help="distinct buffer sets cycled through (0 = enough to touch >= 450 MB, 1 = cache-resident)")
     ap.add_argument("--no-graph", action="store_true", help="time eager Submits instead of a HIP-graph replay")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget of the CPU-oracle leg (0 = skip)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
@@ -84,26 +339,14 @@ def main():
     torch.cuda.set_device(0)
 
     # ---- inputs resident in HBM ----------------------------------------------------------------
-    sets = []
-    host0 = None
-    for r in range(max(1, args.rotate)):
-        host = orc.fill_u8((N, SRC_H, SRC_W, 3), SEED + r)
-        if r == 0:
-            host0 = host[:8].copy()
-        tin = cv.Tensor.alloc([N, SRC_H, SRC_W, 3], np.uint8, "NHWC")
-        tin.torch_view().copy_(torch.from_numpy(host).cuda())
-        tout = cv.Tensor.alloc([N, 3, OUT_H, OUT_W], np.float32, "NCHW")
-        sets.append((tin, tout))
-        del host
-    op = cv.ResizeCropConvertReformat()
+    wl = WORKLOADS[args.workload](cv, orc, np, torch)
+    nsets = args.rotate if args.rotate > 0 else max(2, math.ceil(450e6 / wl.alg_bytes))
+    sets = [wl.make_set() for _ in range(nsets)]
     stream = torch.cuda.current_stream()
-
-    def step(i):
-        tin, tout = sets[i % len(sets)]
-        op(stream, tin, tout, (NEW_W, NEW_H), 1, (CROP_X, CROP_Y), 0, SCALE, OFFSET, False)
+    torch.cuda.synchronize()
 
     for i in range(args.warmup):
-        step(i)
+        wl.submit(stream, sets[i % nsets])
     torch.cuda.synchronize()
 
     # ---- timed region: exactly K steps between two events on the launch stream.
@@ -118,8 +361,7 @@ def main():
             with torch.cuda.graph(graph):
                 cap = torch.cuda.current_stream()
                 for i in range(args.steps):
-                    tin, tout = sets[i % len(sets)]
-                    op(cap, tin, tout, (NEW_W, NEW_H), 1, (CROP_X, CROP_Y), 0, SCALE, OFFSET, False)
+                    wl.submit(cap, sets[i % nsets])
             graph.replay()  # untimed first replay
             torch.cuda.synchronize()
             mode = "hipgraph"
@@ -134,13 +376,13 @@ def main():
         graph.replay()
     else:
         for i in range(args.steps):
-            step(i)
+            wl.submit(stream, sets[i % nsets])
     e1.record(stream)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     wall = t1 - t0
-    # mean launch-to-launch duration of the kernel over the timed region (includes the ~2 us
-    # dispatch gap between dependent launches, so it is an upper bound of the pure kernel time)
+    # mean launch-to-launch duration of the kernel over the timed region (includes the gap between
+    # dependent launches, so it is an upper bound of the pure kernel time)
     mean_kernel_ms = e0.elapsed_time(e1) / args.steps
 
     if args.copy_probe > 0:
@@ -151,35 +393,28 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
-    # ---- correctness spot check of what was just produced (first 2 images of set 0)
-    ref = orc.fused_rccr(host0[:2], (OUT_H, OUT_W), (NEW_W, NEW_H), (CROP_X, CROP_Y), 1, np.float32, True, 0, SCALE,
-                         OFFSET, False)
-    got = sets[0][1].torch_view()[:2].cpu().numpy()
-    assert (np.abs(got - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all(), "bench output differs from the oracle"
+    # ---- correctness spot check of what was just produced (set 0)
+    wl.check(sets[0])
 
-    rd, wr = algorithmic_bytes_per_image()
-    alg_bytes = (rd + wr) * N
-    achieved = alg_bytes / (mean_kernel_ms * 1e-3) / 1e9
+    achieved = wl.alg_bytes / (mean_kernel_ms * 1e-3) / 1e9
 
     # ---- CPU oracle on the same workload (bounded sample)
     cpu = None
     if args.cpu_seconds > 0:
         threads = min(os.cpu_count() or 1, 16)
-        sample = host0
-        reps, tcpu = 0, 0.0
+        reps, done, tcpu = 0, 0, 0.0
         c0 = time.perf_counter()
         while reps < 2 or tcpu < args.cpu_seconds:
-            orc.fused_rccr(sample, (OUT_H, OUT_W), (NEW_W, NEW_H), (CROP_X, CROP_Y), 1, np.float32, True, 0, SCALE,
-                           OFFSET, False, threads=threads)
+            done += wl.cpu(threads)
             reps += 1
             tcpu = time.perf_counter() - c0
-        cpu = {"value": round(reps * sample.shape[0] / tcpu, 1), "unit": "images/s", "cores": threads, "kind": "port",
-               "sample": "%d x (batch of %d 1080p images) through the C++ oracle, %d threads over images"
-                         % (reps, sample.shape[0], threads)}
+        cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": threads, "kind": "port",
+               "sample": "%d images of this workload through the C++ oracle in %.1f s, %d threads"
+                         % (done, tcpu, threads)}
 
     out = {
         "metric": "images/sec and achieved HBM GB/s (% of roofline), 1 MI355X",
-        "value": round(N * args.steps / wall, 1),
+        "value": round(wl.images * args.steps / wall, 1),
         "unit": "images/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -188,15 +423,13 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": wl.dtype,
         "data": "synthetic",
-        "config": {"workload": "fused ResizeCropConvertReformat: batch 64 u8 NHWC 1920x1080 -> bilinear 455x256 -> "
-                               "crop 224x224 @(115,16) -> f32 NCHW, scale/offset",
-                   "rotate_buffer_sets": len(sets), "launch": mode},
+        "config": {"workload": wl.workload, "rotate_buffer_sets": nsets, "launch": mode},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "FusedBilinear<float,false>", "kernel_ms_mean": round(mean_kernel_ms, 5),
-                     "algorithmic_bytes_per_launch": alg_bytes},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.key),
+                     "kernel": wl.kernel, "kernel_ms_mean": round(mean_kernel_ms, 5),
+                     "algorithmic_bytes_per_launch": wl.alg_bytes},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

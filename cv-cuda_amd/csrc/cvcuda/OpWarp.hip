@@ -11,8 +11,11 @@
 // owns no device buffer and launches no separate inversion kernel; several var-shape submissions of
 // one operator handle may therefore be in flight at once. Var-shape batches run on a packed tile grid.
 //
-// Kernel shape: one lane per destination pixel, 32 x 8 pixels per block (a squarish tile keeps the
-// rotated source footprint of a block compact); all channels of a tap move as one vector access.
+// Kernel shape: one lane produces kPxPerLane = 4 consecutive destination pixels of one row and stores
+// them as whole dwords (12 bytes for u8x3); a wave covers 64 x 4 pixels, a 256-thread block 64 x 16.
+// The block prologue (tile lookup, matrix load / inversion) is paid once per 4 pixels. Taps that lie
+// inside the source image - nearly all of them - skip the border logic and fetch the horizontally
+// adjacent taps of a row with one wide load (u8x3: the 6 bytes of two pixels in one 8-byte load).
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
@@ -27,8 +30,9 @@ namespace cvamd {
 
 namespace {
 
-constexpr int kTileW = 32;
-constexpr int kTileH = 8;
+constexpr int kPxPerLane = 4;
+constexpr int kTileW     = 16 * kPxPerLane;
+constexpr int kTileH     = 16;
 
 struct WarpArgs
 {
@@ -59,7 +63,13 @@ struct Img
 {
     const uint8_t *base;
     int32_t        row, w, h;
+    int64_t        lastLoad; // last byte offset at which an 8-byte load still ends inside the image
 };
+
+__device__ __forceinline__ Img MakeImg(const uint8_t *base, int32_t row, int32_t w, int32_t h, int pixelBytes)
+{
+    return Img{base, row, w, h, (int64_t)(h - 1) * row + (int64_t)w * pixelBytes - 8};
+}
 
 __device__ __forceinline__ int BorderIndex(int border, int c, int s)
 {
@@ -161,11 +171,40 @@ __device__ __forceinline__ int FloorToInt(float v)
     return (int)fminf(fmaxf(floorf(v), -1073741824.f), 1073741824.f);
 }
 
-template<class T, int C, int INTERP>
-__device__ __forceinline__ void WarpPixel(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dstRow, int dx,
-                                          int dy)
+// The two horizontally adjacent taps (x, y) and (x + 1, y), both known to be inside the image.
+template<class T, int C>
+__device__ __forceinline__ void FetchPairInside(const Img &im, int x, int y, float (&p0)[C], float (&p1)[C])
 {
-    float sx, sy;
+    if constexpr (std::is_same_v<T, uint8_t> && C == 3)
+    {
+        // 6 bytes through one 8-byte load; at the very end of the image the load is moved back so
+        // that it ends with the image and the value is shifted into place
+        const int64_t  off  = (int64_t)y * im.row + x * 3;
+        const int      back = (int)max((int64_t)0, off - im.lastLoad);
+        const uint64_t q    = LoadU64Unaligned(im.base + off - back) >> (8 * back);
+        const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
+        p0[0] = (float)(lo & 0xFF);
+        p0[1] = (float)((lo >> 8) & 0xFF);
+        p0[2] = (float)((lo >> 16) & 0xFF);
+        p1[0] = (float)(lo >> 24);
+        p1[1] = (float)(hi & 0xFF);
+        p1[2] = (float)((hi >> 8) & 0xFF);
+    }
+    else
+    {
+        const Vec<T, 2 * C> v
+            = *reinterpret_cast<const Vec<T, 2 * C> *>(im.base + (int64_t)y * im.row + (int64_t)x * (C * sizeof(T)));
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            p0[c] = (float)v.v[c];
+            p1[c] = (float)v.v[C + c];
+        }
+    }
+}
+
+__device__ __forceinline__ void MapCoord(const WarpArgs &a, const float (&m)[9], int dx, int dy, float &sx, float &sy)
+{
     if (a.perspective)
     {
         const float coeff = 1.0f / (m[6] * dx + m[7] * dy + m[8]);
@@ -177,44 +216,46 @@ __device__ __forceinline__ void WarpPixel(const Img &im, const WarpArgs &a, cons
         sx = m[0] * dx + m[1] * dy + m[2];
         sy = m[3] * dx + m[4] * dy + m[5];
     }
+}
+
+// One destination pixel sampled at (sx, sy) with every tap going through the border logic. The tap
+// loops are deliberately not unrolled: this path runs only for the few waves that straddle the image
+// border, and one copy of the border code keeps the kernel small.
+template<class T, int C, int INTERP>
+__device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &a, float sx, float sy, T (&out)[C])
+{
     float acc[C];
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
     {
         Fetch<T, C>(im, a, FloorToInt(sx + .5f), FloorToInt(sy + .5f), acc);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[c] = (T)acc[c]; // the tap itself (exactly representable), no rounding involved
+        }
+        return;
     }
     else if constexpr (INTERP == NVCV_INTERP_LINEAR)
     {
         const int x1 = FloorToInt(sx), y1 = FloorToInt(sy);
         const int x2 = x1 + 1, y2 = y1 + 1;
-        float     t[C];
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
             acc[c] = 0.f;
         }
-        Fetch<T, C>(im, a, x1, y1, t);
-#pragma unroll
-        for (int c = 0; c < C; ++c)
+#pragma nounroll
+        for (int i = 0; i < 4; ++i) // taps (x1,y1) (x2,y1) (x1,y2) (x2,y2) in this order
         {
-            acc[c] += t[c] * (x2 - sx) * (y2 - sy);
-        }
-        Fetch<T, C>(im, a, x2, y1, t);
+            float t[C];
+            Fetch<T, C>(im, a, x1 + (i & 1), y1 + (i >> 1), t);
+            const float wx = (i & 1) ? (sx - x1) : (x2 - sx);
+            const float wy = (i >> 1) ? (sy - y1) : (y2 - sy);
 #pragma unroll
-        for (int c = 0; c < C; ++c)
-        {
-            acc[c] += t[c] * (sx - x1) * (y2 - sy);
-        }
-        Fetch<T, C>(im, a, x1, y2, t);
-#pragma unroll
-        for (int c = 0; c < C; ++c)
-        {
-            acc[c] += t[c] * (x2 - sx) * (sy - y1);
-        }
-        Fetch<T, C>(im, a, x2, y2, t);
-#pragma unroll
-        for (int c = 0; c < C; ++c)
-        {
-            acc[c] += t[c] * (sx - x1) * (sy - y1);
+            for (int c = 0; c < C; ++c)
+            {
+                acc[c] += t[c] * wx * wy;
+            }
         }
     }
     else
@@ -229,35 +270,181 @@ __device__ __forceinline__ void WarpPixel(const Img &im, const WarpArgs &a, cons
             acc[c] = 0.f;
         }
 #pragma unroll
-        for (int cy = -1; cy <= 2; ++cy)
+        for (int cy = 0; cy < 4; ++cy)
         {
 #pragma unroll
-            for (int cx = -1; cx <= 2; ++cx)
+            for (int cx = 0; cx < 4; ++cx)
             {
                 float t[C];
-                Fetch<T, C>(im, a, ix + cx, iy + cy, t);
+                Fetch<T, C>(im, a, ix + cx - 1, iy + cy - 1, t);
 #pragma unroll
                 for (int c = 0; c < C; ++c)
                 {
-                    acc[c] += t[c] * (wx[cx + 1] * wy[cy + 1]);
+                    acc[c] += t[c] * (wx[cx] * wy[cy]);
                 }
             }
         }
     }
-    Vec<T, C> *o = reinterpret_cast<Vec<T, C> *>(dstRow) + dx;
 #pragma unroll
     for (int c = 0; c < C; ++c)
     {
-        T v;
-        if constexpr (INTERP == NVCV_INTERP_NEAREST)
+        out[c] = SaturateCast<T>(acc[c]);
+    }
+}
+
+// True when every tap of the sample at (sx, sy) lies inside the image.
+template<int INTERP>
+__device__ __forceinline__ bool TapsInside(const Img &im, float sx, float sy)
+{
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        const int x = FloorToInt(sx + .5f), y = FloorToInt(sy + .5f);
+        return x >= 0 && y >= 0 && x < im.w && y < im.h;
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const int x = FloorToInt(sx), y = FloorToInt(sy);
+        return x >= 0 && y >= 0 && x + 1 < im.w && y + 1 < im.h;
+    }
+    else
+    {
+        const int x = FloorToInt(sx), y = FloorToInt(sy);
+        return x >= 1 && y >= 1 && x + 2 < im.w && y + 2 < im.h;
+    }
+}
+
+// Same arithmetic as SampleWithBorder for a sample whose taps are all inside the image: no border
+// logic, adjacent taps fetched together, no branches (so the loads of several pixels can be in flight
+// at once).
+template<class T, int C, int INTERP>
+__device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, T (&out)[C])
+{
+    float acc[C];
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        const int       x = FloorToInt(sx + .5f), y = FloorToInt(sy + .5f);
+        const Vec<T, C> px = reinterpret_cast<const Vec<T, C> *>(im.base + (int64_t)y * im.row)[x];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
         {
-            v = (T)acc[c]; // the tap itself (exactly representable), no rounding involved
+            out[c] = px.v[c];
         }
-        else
+        return;
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const int x1 = FloorToInt(sx), y1 = FloorToInt(sy);
+        const int x2 = x1 + 1, y2 = y1 + 1;
+        float     t[4][C];
+        FetchPairInside<T, C>(im, x1, y1, t[0], t[1]);
+        FetchPairInside<T, C>(im, x1, y2, t[2], t[3]);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
         {
-            v = SaturateCast<T>(acc[c]);
+            float v = 0.f;
+            v += t[0][c] * (x2 - sx) * (y2 - sy);
+            v += t[1][c] * (sx - x1) * (y2 - sy);
+            v += t[2][c] * (x2 - sx) * (sy - y1);
+            v += t[3][c] * (sx - x1) * (sy - y1);
+            acc[c] = v;
         }
-        __builtin_nontemporal_store(v, &o->v[c]);
+    }
+    else
+    {
+        const int ix = FloorToInt(sx), iy = FloorToInt(sy);
+        float     wx[4], wy[4];
+        CubicCoeffs(sx - ix, wx);
+        CubicCoeffs(sy - iy, wy);
+        float t[4][4][C];
+#pragma unroll
+        for (int cy = 0; cy < 4; ++cy)
+        {
+            FetchPairInside<T, C>(im, ix - 1, iy + cy - 1, t[cy][0], t[cy][1]);
+            FetchPairInside<T, C>(im, ix + 1, iy + cy - 1, t[cy][2], t[cy][3]);
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            acc[c] = 0.f;
+        }
+#pragma unroll
+        for (int cy = 0; cy < 4; ++cy)
+        {
+#pragma unroll
+            for (int cx = 0; cx < 4; ++cx)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    acc[c] += t[cy][cx][c] * (wx[cx] * wy[cy]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        out[c] = SaturateCast<T>(acc[c]);
+    }
+}
+
+struct __attribute__((packed, aligned(1))) UnalignedWord
+{
+    uint32_t w;
+};
+
+// The kPxPerLane pixels of one lane: dx0 .. dx0+3 of row dy. A full group leaves as whole dwords
+// (streaming stores: the output is not read back); a ragged right edge element by element.
+template<class T, int C, int INTERP>
+__device__ __forceinline__ void WarpQuad(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dstRow, int dx0,
+                                         int dy, int dstW)
+{
+    constexpr int kWords = kPxPerLane * C * (int)sizeof(T) / 4;
+    union
+    {
+        T        px[kPxPerLane][C];
+        uint32_t w[kWords];
+    } q;
+    const int count = min(kPxPerLane, dstW - dx0);
+    float     sx[kPxPerLane], sy[kPxPerLane];
+    bool      allInside = count == kPxPerLane;
+#pragma unroll
+    for (int k = 0; k < kPxPerLane; ++k)
+    {
+        MapCoord(a, m, dx0 + k, dy, sx[k], sy[k]);
+        allInside = allInside && TapsInside<INTERP>(im, sx[k], sy[k]);
+    }
+    uint8_t *o = dstRow + (int64_t)dx0 * (C * sizeof(T));
+    if (allInside)
+    {
+#pragma unroll
+        for (int k = 0; k < kPxPerLane; ++k)
+        {
+            SampleInside<T, C, INTERP>(im, sx[k], sy[k], q.px[k]);
+        }
+        UnalignedWord *ow = reinterpret_cast<UnalignedWord *>(o);
+#pragma unroll
+        for (int i = 0; i < kWords; ++i)
+        {
+            __builtin_nontemporal_store(q.w[i], &ow[i].w);
+        }
+    }
+    else
+    {
+        T *ot = reinterpret_cast<T *>(o);
+#pragma nounroll
+        for (int k = 0; k < count; ++k)
+        {
+            T     px[C];
+            float bx, by; // recomputed rather than indexed: a dynamic index would put sx/sy in scratch
+            MapCoord(a, m, dx0 + k, dy, bx, by);
+            SampleWithBorder<T, C, INTERP>(im, a, bx, by, px);
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                ot[k * C + c] = px[c];
+            }
+        }
     }
 }
 
@@ -267,12 +454,14 @@ __device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (
     const float *p = reinterpret_cast<const float *>(a.xforms + image * a.xformStride);
     const int    n = a.perspective ? 9 : 6;
     float        f[9];
+#pragma unroll
     for (int i = 0; i < 9; ++i)
     {
         f[i] = i < n ? p[i] : 0.f;
     }
     if (a.inverseGiven)
     {
+#pragma unroll
         for (int i = 0; i < 9; ++i)
         {
             m[i] = f[i];
@@ -297,6 +486,7 @@ __device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (
                       + f[2] * (f[3] * f[7] - f[4] * f[6]);
         if (d == 0)
         {
+#pragma unroll
             for (int i = 0; i < 9; ++i)
             {
                 m[i] = f[i]; // singular: left as given, like the reference's failed in-place inverse
@@ -318,39 +508,39 @@ __device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (
 template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void WarpTensor(const WarpArgs a)
 {
-    const int dx = blockIdx.x * kTileW + (threadIdx.x & (kTileW - 1));
-    const int dy = blockIdx.y * kTileH + (threadIdx.x / kTileW);
-    if (dx >= a.dstW || dy >= a.dstH)
+    const int dx0 = blockIdx.x * kTileW + (threadIdx.x & 15) * kPxPerLane;
+    const int dy  = blockIdx.y * kTileH + (threadIdx.x >> 4);
+    if (dx0 >= a.dstW || dy >= a.dstH)
     {
         return;
     }
     const int n  = blockIdx.z;
-    const Img im = {a.src + n * a.srcN, a.srcRow, a.srcW, a.srcH};
+    const Img im = MakeImg(a.src + n * a.srcN, a.srcRow, a.srcW, a.srcH, C * sizeof(T));
     float     m[9];
 #pragma unroll
     for (int i = 0; i < 9; ++i)
     {
         m[i] = a.m[i];
     }
-    WarpPixel<T, C, INTERP>(im, a, m, a.dst + n * a.dstN + (int64_t)dy * a.dstRow, dx, dy);
+    WarpQuad<T, C, INTERP>(im, a, m, a.dst + n * a.dstN + (int64_t)dy * a.dstRow, dx0, dy, a.dstW);
 }
 
 template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarTiles tiles)
 {
-    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
-    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
-    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    float                        m[9];
-    LoadMatrix(a, tc.image, m);
-    const int dx = tc.tx * kTileW + (threadIdx.x & (kTileW - 1));
-    const int dy = tc.ty * kTileH + (threadIdx.x / kTileW);
-    if (dx >= d.width || dy >= d.height)
+    const TileCoord              tc  = LocateTile(tiles, blockIdx.x);
+    const NVCVImagePlaneStrided &s   = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided &d   = a.dstList[tc.image].planes[0];
+    const int                    dx0 = tc.tx * kTileW + (threadIdx.x & 15) * kPxPerLane;
+    const int                    dy  = tc.ty * kTileH + (threadIdx.x >> 4);
+    if (dx0 >= d.width || dy >= d.height)
     {
         return;
     }
-    const Img im = {s.basePtr, s.rowStride, s.width, s.height};
-    WarpPixel<T, C, INTERP>(im, a, m, d.basePtr + (int64_t)dy * d.rowStride, dx, dy);
+    float m[9];
+    LoadMatrix(a, tc.image, m);
+    const Img im = MakeImg(s.basePtr, s.rowStride, s.width, s.height, C * sizeof(T));
+    WarpQuad<T, C, INTERP>(im, a, m, d.basePtr + (int64_t)dy * d.rowStride, dx0, dy, d.width);
 }
 
 template<class T, int C, int INTERP>
