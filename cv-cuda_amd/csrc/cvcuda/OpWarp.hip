@@ -11,11 +11,17 @@
 // owns no device buffer and launches no separate inversion kernel; several var-shape submissions of
 // one operator handle may therefore be in flight at once. Var-shape batches run on a packed tile grid.
 //
-// Kernel shape: one lane produces kPxPerLane = 4 consecutive destination pixels of one row and stores
-// them as whole dwords (12 bytes for u8x3); a wave covers 64 x 4 pixels, a 256-thread block 64 x 16.
-// The block prologue (tile lookup, matrix load / inversion) is paid once per 4 pixels. Taps that lie
-// inside the source image - nearly all of them - skip the border logic and fetch the horizontally
-// adjacent taps of a row with one wide load (u8x3: the 6 bytes of two pixels in one 8-byte load).
+// Kernel shape. A 256-thread block produces a 64 x 16 pixel tile of the destination in two phases.
+// Gather: the cost of the gather is set by how many distinct cache lines one wave-wide load touches,
+// and under a rotation every source row a wave's footprint crosses is another line; so a wave samples
+// compact 8 x 8 pixel patches (one lane per pixel, ~10 source rows per load where a 64 x 1 strip would
+// cross ~20), four patches per wave, i.e. kPxPerLane = 4 independent samples per lane whose loads are
+// in flight together. Taps that lie inside the source image - nearly all of them - skip the border
+// logic and fetch the horizontally adjacent taps of a row with one wide load (u8x3: the 6 bytes of two
+// pixels in one 8-byte load). Store: the results cross over through LDS so that each lane writes 4
+// consecutive pixels of one row as whole dwords (16 lanes cover a 64-pixel row segment); single-byte
+// stores scattered over 8 rows are several times slower. The block prologue (tile lookup, matrix
+// load / inversion) is paid once per 4 pixels.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
@@ -30,9 +36,10 @@ namespace cvamd {
 
 namespace {
 
-constexpr int kPxPerLane = 4;
-constexpr int kTileW     = 16 * kPxPerLane;
-constexpr int kTileH     = 16;
+constexpr int kPatch     = 8;  // gather granule: a wave samples kPatch x kPatch pixels per step
+constexpr int kPxPerLane = 4;  // steps per wave
+constexpr int kTileW     = 64; // = 8 patches
+constexpr int kTileH     = 16; // = 2 patches; 16 patches / 4 waves = kPxPerLane
 
 struct WarpArgs
 {
@@ -63,13 +70,7 @@ struct Img
 {
     const uint8_t *base;
     int32_t        row, w, h;
-    int64_t        lastLoad; // last byte offset at which an 8-byte load still ends inside the image
 };
-
-__device__ __forceinline__ Img MakeImg(const uint8_t *base, int32_t row, int32_t w, int32_t h, int pixelBytes)
-{
-    return Img{base, row, w, h, (int64_t)(h - 1) * row + (int64_t)w * pixelBytes - 8};
-}
 
 __device__ __forceinline__ int BorderIndex(int border, int c, int s)
 {
@@ -171,17 +172,41 @@ __device__ __forceinline__ int FloorToInt(float v)
     return (int)fminf(fmaxf(floorf(v), -1073741824.f), 1073741824.f);
 }
 
-// The two horizontally adjacent taps (x, y) and (x + 1, y), both known to be inside the image.
+// u8x3 taps are fetched with loads wider than the taps (4 bytes for one pixel, 8 for two), which
+// read 1-2 bytes past them. Inside the image that is harmless; the one tap after which the image
+// ends (last pixel of the last row) is kept off this path by TapsInside.
 template<class T, int C>
-__device__ __forceinline__ void FetchPairInside(const Img &im, int x, int y, float (&p0)[C], float (&p1)[C])
+constexpr bool kWideTapLoads = std::is_same_v<T, uint8_t> && C == 3;
+
+// One pixel at p, known to be inside the image.
+template<class T, int C>
+__device__ __forceinline__ void LoadPixelInside(const uint8_t *p, T (&out)[C])
 {
-    if constexpr (std::is_same_v<T, uint8_t> && C == 3)
+    if constexpr (kWideTapLoads<T, C>)
     {
-        // 6 bytes through one 8-byte load; at the very end of the image the load is moved back so
-        // that it ends with the image and the value is shifted into place
-        const int64_t  off  = (int64_t)y * im.row + x * 3;
-        const int      back = (int)max((int64_t)0, off - im.lastLoad);
-        const uint64_t q    = LoadU64Unaligned(im.base + off - back) >> (8 * back);
+        const uint32_t q = LoadU32Unaligned(p);
+        out[0]           = (uint8_t)q;
+        out[1]           = (uint8_t)(q >> 8);
+        out[2]           = (uint8_t)(q >> 16);
+    }
+    else
+    {
+        const Vec<T, C> v = *reinterpret_cast<const Vec<T, C> *>(p);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[c] = v.v[c];
+        }
+    }
+}
+
+// Two horizontally adjacent pixels starting at p, both known to be inside the image.
+template<class T, int C>
+__device__ __forceinline__ void LoadPairInside(const uint8_t *p, float (&p0)[C], float (&p1)[C])
+{
+    if constexpr (kWideTapLoads<T, C>)
+    {
+        const uint64_t q  = LoadU64Unaligned(p);
         const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
         p0[0] = (float)(lo & 0xFF);
         p0[1] = (float)((lo >> 8) & 0xFF);
@@ -192,8 +217,7 @@ __device__ __forceinline__ void FetchPairInside(const Img &im, int x, int y, flo
     }
     else
     {
-        const Vec<T, 2 * C> v
-            = *reinterpret_cast<const Vec<T, 2 * C> *>(im.base + (int64_t)y * im.row + (int64_t)x * (C * sizeof(T)));
+        const Vec<T, 2 * C> v = *reinterpret_cast<const Vec<T, 2 * C> *>(p);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -203,9 +227,19 @@ __device__ __forceinline__ void FetchPairInside(const Img &im, int x, int y, flo
     }
 }
 
-__device__ __forceinline__ void MapCoord(const WarpArgs &a, const float (&m)[9], int dx, int dy, float &sx, float &sy)
+// Byte offset of pixel (x, y), both inside the image. Image planes are below 2 GiB. Uses the 24-bit
+// multiply (full rate; the 32-bit one runs at a quarter): images whose row pitch or height does not
+// fit 23 bits never take the path that calls this.
+template<int PIXEL_BYTES>
+__device__ __forceinline__ uint32_t PixelOffset(const Img &im, int x, int y)
 {
-    if (a.perspective)
+    return (uint32_t)__mul24(y, im.row) + (uint32_t)x * PIXEL_BYTES;
+}
+
+template<bool PERSPECTIVE>
+__device__ __forceinline__ void MapCoord(const float (&m)[9], int dx, int dy, float &sx, float &sy)
+{
+    if constexpr (PERSPECTIVE)
     {
         const float coeff = 1.0f / (m[6] * dx + m[7] * dy + m[8]);
         sx                = coeff * (m[0] * dx + m[1] * dy + m[2]);
@@ -292,75 +326,76 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
     }
 }
 
-// True when every tap of the sample at (sx, sy) lies inside the image.
-template<int INTERP>
-__device__ __forceinline__ bool TapsInside(const Img &im, float sx, float sy)
+// True when every tap of the sample at (sx, sy) lies inside the image (and, with WIDE loads, none of
+// them is the very last pixel of the image). Decided on the float coordinates: for an integer k,
+// floor(v) >= k <=> v >= k and floor(v) < k <=> v < k; a NaN coordinate fails every comparison.
+template<int INTERP, bool WIDE>
+__device__ __forceinline__ bool TapsInside(float wf, float hf, float sx, float sy)
 {
+    // taps span [floor(v) - lo, floor(v) + hi] per axis
+    constexpr float lo = INTERP == NVCV_INTERP_CUBIC ? 1.f : 0.f;
+    constexpr float hi = INTERP == NVCV_INTERP_CUBIC ? 2.f : (INTERP == NVCV_INTERP_LINEAR ? 1.f : 0.f);
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
     {
-        const int x = FloorToInt(sx + .5f), y = FloorToInt(sy + .5f);
-        return x >= 0 && y >= 0 && x < im.w && y < im.h;
+        sx += .5f;
+        sy += .5f;
     }
-    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    // bitwise on purpose: no short-circuit branches
+    bool in = (sx >= lo) & (sy >= lo) & (sx < wf - hi) & (sy < hf - hi);
+    if constexpr (WIDE)
     {
-        const int x = FloorToInt(sx), y = FloorToInt(sy);
-        return x >= 0 && y >= 0 && x + 1 < im.w && y + 1 < im.h;
+        in = in & ((sx < wf - hi - 1.f) | (sy < hf - hi - 1.f));
     }
-    else
-    {
-        const int x = FloorToInt(sx), y = FloorToInt(sy);
-        return x >= 1 && y >= 1 && x + 2 < im.w && y + 2 < im.h;
-    }
+    return in;
 }
 
 // Same arithmetic as SampleWithBorder for a sample whose taps are all inside the image: no border
 // logic, adjacent taps fetched together, no branches (so the loads of several pixels can be in flight
-// at once).
+// at once). floorf(v) is used directly where the generic path converts floor(v) to int and back.
 template<class T, int C, int INTERP>
 __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, T (&out)[C])
 {
-    float acc[C];
+    constexpr int PB = C * sizeof(T);
+    float         acc[C];
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
     {
-        const int       x = FloorToInt(sx + .5f), y = FloorToInt(sy + .5f);
-        const Vec<T, C> px = reinterpret_cast<const Vec<T, C> *>(im.base + (int64_t)y * im.row)[x];
-#pragma unroll
-        for (int c = 0; c < C; ++c)
-        {
-            out[c] = px.v[c];
-        }
+        const int x = (int)floorf(sx + .5f), y = (int)floorf(sy + .5f);
+        LoadPixelInside<T, C>(im.base + PixelOffset<PB>(im, x, y), out);
         return;
     }
     else if constexpr (INTERP == NVCV_INTERP_LINEAR)
     {
-        const int x1 = FloorToInt(sx), y1 = FloorToInt(sy);
-        const int x2 = x1 + 1, y2 = y1 + 1;
-        float     t[4][C];
-        FetchPairInside<T, C>(im, x1, y1, t[0], t[1]);
-        FetchPairInside<T, C>(im, x1, y2, t[2], t[3]);
+        const float fx = floorf(sx), fy = floorf(sy);
+        const float wx1 = sx - fx, wx0 = (fx + 1.f) - sx;
+        const float wy1 = sy - fy, wy0 = (fy + 1.f) - sy;
+        const uint8_t *p = im.base + PixelOffset<PB>(im, (int)fx, (int)fy);
+        float          t[4][C];
+        LoadPairInside<T, C>(p, t[0], t[1]);
+        LoadPairInside<T, C>(p + (uint32_t)im.row, t[2], t[3]);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
-            float v = 0.f;
-            v += t[0][c] * (x2 - sx) * (y2 - sy);
-            v += t[1][c] * (sx - x1) * (y2 - sy);
-            v += t[2][c] * (x2 - sx) * (sy - y1);
-            v += t[3][c] * (sx - x1) * (sy - y1);
+            float v = t[0][c] * wx0 * wy0;
+            v += t[1][c] * wx1 * wy0;
+            v += t[2][c] * wx0 * wy1;
+            v += t[3][c] * wx1 * wy1;
             acc[c] = v;
         }
     }
     else
     {
-        const int ix = FloorToInt(sx), iy = FloorToInt(sy);
-        float     wx[4], wy[4];
-        CubicCoeffs(sx - ix, wx);
-        CubicCoeffs(sy - iy, wy);
-        float t[4][4][C];
+        const float fx = floorf(sx), fy = floorf(sy);
+        float       wx[4], wy[4];
+        CubicCoeffs(sx - fx, wx);
+        CubicCoeffs(sy - fy, wy);
+        const uint8_t *p = im.base + PixelOffset<PB>(im, (int)fx - 1, (int)fy - 1);
+        float          t[4][4][C];
 #pragma unroll
         for (int cy = 0; cy < 4; ++cy)
         {
-            FetchPairInside<T, C>(im, ix - 1, iy + cy - 1, t[cy][0], t[cy][1]);
-            FetchPairInside<T, C>(im, ix + 1, iy + cy - 1, t[cy][2], t[cy][3]);
+            LoadPairInside<T, C>(p, t[cy][0], t[cy][1]);
+            LoadPairInside<T, C>(p + 2 * PB, t[cy][2], t[cy][3]);
+            p += (uint32_t)im.row;
         }
 #pragma unroll
         for (int c = 0; c < C; ++c)
@@ -393,57 +428,113 @@ struct __attribute__((packed, aligned(1))) UnalignedWord
     uint32_t w;
 };
 
-// The kPxPerLane pixels of one lane: dx0 .. dx0+3 of row dy. A full group leaves as whole dwords
-// (streaming stores: the output is not read back); a ragged right edge element by element.
+// One 64 x 16 tile of the destination image `dst` (tile coordinates tx, ty), all 256 threads.
 template<class T, int C, int INTERP>
-__device__ __forceinline__ void WarpQuad(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dstRow, int dx0,
-                                         int dy, int dstW)
+__device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dst, int dstRow,
+                                         int dstW, int dstH, int tx, int ty)
 {
-    constexpr int kWords = kPxPerLane * C * (int)sizeof(T) / 4;
-    union
-    {
-        T        px[kPxPerLane][C];
-        uint32_t w[kWords];
-    } q;
-    const int count = min(kPxPerLane, dstW - dx0);
-    float     sx[kPxPerLane], sy[kPxPerLane];
-    bool      allInside = count == kPxPerLane;
+    constexpr int PB       = C * sizeof(T);
+    constexpr int kLdsRow  = kTileW * PB + 4; // + 1 bank: the 8 rows of a patch start in different banks
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kTileH * kLdsRow];
+
+    // ---- gather: lane (lx, ly) of wave w samples its pixel in patches 4w .. 4w+3
+    const int wave = threadIdx.x >> 6, lx = threadIdx.x & (kPatch - 1), ly = (threadIdx.x >> 3) & (kPatch - 1);
+    const float wf = (float)im.w, hf = (float)im.h;
+    float       sx[kPxPerLane], sy[kPxPerLane];
+    int         ldsAt[kPxPerLane];
+    // rows too long or too many for 24-bit offset arithmetic go through the generic path
+    bool allInside = (im.row | im.h) < (1 << 23);
 #pragma unroll
     for (int k = 0; k < kPxPerLane; ++k)
     {
-        MapCoord(a, m, dx0 + k, dy, sx[k], sy[k]);
-        allInside = allInside && TapsInside<INTERP>(im, sx[k], sy[k]);
+        const int patch = wave * kPxPerLane + k;
+        const int px = (patch & 7) * kPatch + lx, py = (patch >> 3) * kPatch + ly;
+        ldsAt[k]     = py * kLdsRow + px * PB;
+        // pixels of the tile beyond the image edge repeat the edge pixel's sample; they are never stored
+        const int dx = min(tx * kTileW + px, dstW - 1), dy = min(ty * kTileH + py, dstH - 1);
+        if (a.perspective)
+        {
+            MapCoord<true>(m, dx, dy, sx[k], sy[k]);
+        }
+        else
+        {
+            MapCoord<false>(m, dx, dy, sx[k], sy[k]);
+        }
+        allInside = allInside & TapsInside<INTERP, kWideTapLoads<T, C>>(wf, hf, sx[k], sy[k]);
     }
-    uint8_t *o = dstRow + (int64_t)dx0 * (C * sizeof(T));
     if (allInside)
     {
+        T v[kPxPerLane][C];
 #pragma unroll
         for (int k = 0; k < kPxPerLane; ++k)
         {
-            SampleInside<T, C, INTERP>(im, sx[k], sy[k], q.px[k]);
+            SampleInside<T, C, INTERP>(im, sx[k], sy[k], v[k]);
         }
-        UnalignedWord *ow = reinterpret_cast<UnalignedWord *>(o);
 #pragma unroll
-        for (int i = 0; i < kWords; ++i)
+        for (int k = 0; k < kPxPerLane; ++k)
         {
-            __builtin_nontemporal_store(q.w[i], &ow[i].w);
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                reinterpret_cast<T *>(lds + ldsAt[k])[c] = v[k][c];
+            }
         }
     }
     else
     {
-        T *ot = reinterpret_cast<T *>(o);
 #pragma nounroll
-        for (int k = 0; k < count; ++k)
+        for (int k = 0; k < kPxPerLane; ++k)
         {
-            T     px[C];
-            float bx, by; // recomputed rather than indexed: a dynamic index would put sx/sy in scratch
-            MapCoord(a, m, dx0 + k, dy, bx, by);
-            SampleWithBorder<T, C, INTERP>(im, a, bx, by, px);
+            // position and coordinates recomputed rather than indexed: a dynamic index would put the
+            // arrays in scratch memory
+            const int patch = wave * kPxPerLane + k;
+            const int px = (patch & 7) * kPatch + lx, py = (patch >> 3) * kPatch + ly;
+            const int dx = min(tx * kTileW + px, dstW - 1), dy = min(ty * kTileH + py, dstH - 1);
+            float     bx, by;
+            if (a.perspective)
+            {
+                MapCoord<true>(m, dx, dy, bx, by);
+            }
+            else
+            {
+                MapCoord<false>(m, dx, dy, bx, by);
+            }
+            T v[C];
+            SampleWithBorder<T, C, INTERP>(im, a, bx, by, v);
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
-                ot[k * C + c] = px[c];
+                reinterpret_cast<T *>(lds + py * kLdsRow + px * PB)[c] = v[c];
             }
+        }
+    }
+    __syncthreads();
+
+    // ---- store: thread t writes pixels 4*(t & 15) .. +3 of tile row t >> 4
+    const int row = threadIdx.x >> 4, x0 = (threadIdx.x & 15) * 4;
+    const int dy = ty * kTileH + row, dx0 = tx * kTileW + x0;
+    if (dy >= dstH || dx0 >= dstW)
+    {
+        return;
+    }
+    const uint8_t *from  = lds + row * kLdsRow + x0 * PB;
+    uint8_t       *to    = dst + (int64_t)dy * dstRow + (int64_t)dx0 * PB;
+    const int      count = min(4, dstW - dx0);
+    if (count == 4)
+    {
+        // streaming stores: the output is not read back by this kernel
+        UnalignedWord *ow = reinterpret_cast<UnalignedWord *>(to);
+#pragma unroll
+        for (int i = 0; i < PB; ++i) // 4 pixels = PB dwords
+        {
+            __builtin_nontemporal_store(reinterpret_cast<const uint32_t *>(from)[i], &ow[i].w);
+        }
+    }
+    else
+    {
+        for (int i = 0; i < count * C; ++i)
+        {
+            reinterpret_cast<T *>(to)[i] = reinterpret_cast<const T *>(from)[i];
         }
     }
 }
@@ -508,39 +599,27 @@ __device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (
 template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void WarpTensor(const WarpArgs a)
 {
-    const int dx0 = blockIdx.x * kTileW + (threadIdx.x & 15) * kPxPerLane;
-    const int dy  = blockIdx.y * kTileH + (threadIdx.x >> 4);
-    if (dx0 >= a.dstW || dy >= a.dstH)
-    {
-        return;
-    }
     const int n  = blockIdx.z;
-    const Img im = MakeImg(a.src + n * a.srcN, a.srcRow, a.srcW, a.srcH, C * sizeof(T));
+    const Img im = {a.src + n * a.srcN, a.srcRow, a.srcW, a.srcH};
     float     m[9];
 #pragma unroll
     for (int i = 0; i < 9; ++i)
     {
         m[i] = a.m[i];
     }
-    WarpQuad<T, C, INTERP>(im, a, m, a.dst + n * a.dstN + (int64_t)dy * a.dstRow, dx0, dy, a.dstW);
+    WarpTile<T, C, INTERP>(im, a, m, a.dst + n * a.dstN, a.dstRow, a.dstW, a.dstH, blockIdx.x, blockIdx.y);
 }
 
 template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarTiles tiles)
 {
-    const TileCoord              tc  = LocateTile(tiles, blockIdx.x);
-    const NVCVImagePlaneStrided &s   = a.srcList[tc.image].planes[0];
-    const NVCVImagePlaneStrided &d   = a.dstList[tc.image].planes[0];
-    const int                    dx0 = tc.tx * kTileW + (threadIdx.x & 15) * kPxPerLane;
-    const int                    dy  = tc.ty * kTileH + (threadIdx.x >> 4);
-    if (dx0 >= d.width || dy >= d.height)
-    {
-        return;
-    }
-    float m[9];
+    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
+    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
+    float                        m[9];
     LoadMatrix(a, tc.image, m);
-    const Img im = MakeImg(s.basePtr, s.rowStride, s.width, s.height, C * sizeof(T));
-    WarpQuad<T, C, INTERP>(im, a, m, d.basePtr + (int64_t)dy * d.rowStride, dx0, dy, d.width);
+    const Img im = {s.basePtr, s.rowStride, s.width, s.height};
+    WarpTile<T, C, INTERP>(im, a, m, d.basePtr, d.rowStride, d.width, d.height, tc.tx, tc.ty);
 }
 
 template<class T, int C, int INTERP>
