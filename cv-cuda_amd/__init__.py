@@ -366,6 +366,16 @@ class ResizeCropConvertReformat(_Operator):
         check(fn(self.handle, stream_ptr(stream), _h(inp), _h(out), capi.Size2D(*resize_dim), interp,
                  capi.Int2(*crop_pos), manip, scale, offset, src_cast))
 
+    def normalized(self, stream, inp, out, resize_dim, interp, crop_pos, base, nscale, manip=K.CHANNEL_NO_OP,
+                   scale=1.0, offset=0.0, src_cast=False, global_scale=1.0, shift=0.0, epsilon=0.0, flags=0):
+        """Extension: the fused operator followed by a per-channel Normalize in the same kernel."""
+        fn = (_cv.cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit if isinstance(inp, ImageBatchVarShape)
+              else _cv.cvcudaxResizeCropConvertReformatNormalizeSubmit)
+        nrm = capi.ChannelNormalize((C.c_float * 3)(*base), (C.c_float * 3)(*nscale), global_scale, shift, epsilon,
+                                    flags)
+        check(fn(self.handle, stream_ptr(stream), _h(inp), _h(out), capi.Size2D(*resize_dim), interp,
+                 capi.Int2(*crop_pos), manip, scale, offset, src_cast, C.byref(nrm)))
+
 
 class Resize(_Operator):
     _create = "cvcudaResizeCreate"

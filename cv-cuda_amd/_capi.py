@@ -273,6 +273,18 @@ _sig(cvcuda, "cvcudaResizeCropConvertReformatVarShapeSubmit", ST, H, C.c_void_p,
      C.c_int, C.c_float, C.c_float, C.c_bool)
 
 
+class ChannelNormalize(C.Structure):
+    """CVCUDAXChannelNormalize (cvcuda/OpResizeCropConvertReformat.h, extension)."""
+    _fields_ = [("base", C.c_float * 3), ("scale", C.c_float * 3), ("globalScale", C.c_float), ("shift", C.c_float),
+                ("epsilon", C.c_float), ("flags", C.c_uint32)]
+
+
+_sig(cvcuda, "cvcudaxResizeCropConvertReformatNormalizeSubmit", ST, H, C.c_void_p, H, H, Size2D, C.c_int, Int2,
+     C.c_int, C.c_float, C.c_float, C.c_bool, P(ChannelNormalize))
+_sig(cvcuda, "cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit", ST, H, C.c_void_p, H, H, Size2D, C.c_int,
+     Int2, C.c_int, C.c_float, C.c_float, C.c_bool, P(ChannelNormalize))
+
+
 def declare_optional(name, res, *args):
     """Declares an operator entry point if the library exports it; returns whether it does."""
     if hasattr(cvcuda, name):

@@ -14,7 +14,10 @@
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
 
+#include <cvcuda/OpNormalize.h>
 #include <cvcuda/OpResizeCropConvertReformat.h>
+
+#include <cmath>
 
 namespace cvamd {
 
@@ -47,6 +50,10 @@ struct FusedArgs
     // launch shape: column tiles and row tiles per image; the grid is 1-D
     uint32_t tilesX, tilesY;
     uint32_t rowTiles; // tilesY * N
+    // per-channel normalisation of the extension entry points, indexed by source channel:
+    // ((scale*v + offset) - normBase) * normMul * normGlobal + normShift
+    float normBase[3], normMul[3];
+    float normGlobal, normShift;
 };
 
 struct TilePos
@@ -107,18 +114,33 @@ __device__ __forceinline__ SrcImage GetSource(const FusedArgs &a, int n)
     return s;
 }
 
-template<class DstT>
+template<class DstT, bool NORM>
+__device__ __forceinline__ DstT Finish(const FusedArgs &a, float v, int c)
+{
+    if constexpr (NORM)
+    {
+        // the value an f32 fused output would hold, then the Normalize operator's expression
+        const float x = a.scale * v + a.offset;
+        return SaturateCast<DstT>((x - a.normBase[c]) * a.normMul[c] * a.normGlobal + a.normShift);
+    }
+    else
+    {
+        return SaturateCast<DstT>(a.scale * v + a.offset);
+    }
+}
+
+template<class DstT, bool NORM>
 __device__ __forceinline__ void StorePixel(const FusedArgs &a, DstT *out, float v0, float v1, float v2)
 {
     // Streaming (non-temporal) stores: the output is written once and not read back by this
     // kernel, so it should not displace source lines in L2 / the memory-side cache. On MI355X
     // this alone shortens the batch-64 1080p -> 224x224 launch by ~15 %.
-    __builtin_nontemporal_store(SaturateCast<DstT>(a.scale * v0 + a.offset), out + a.dstOffC[0]);
-    __builtin_nontemporal_store(SaturateCast<DstT>(a.scale * v1 + a.offset), out + a.dstOffC[1]);
-    __builtin_nontemporal_store(SaturateCast<DstT>(a.scale * v2 + a.offset), out + a.dstOffC[2]);
+    __builtin_nontemporal_store(Finish<DstT, NORM>(a, v0, 0), out + a.dstOffC[0]);
+    __builtin_nontemporal_store(Finish<DstT, NORM>(a, v1, 1), out + a.dstOffC[1]);
+    __builtin_nontemporal_store(Finish<DstT, NORM>(a, v2, 2), out + a.dstOffC[2]);
 }
 
-template<class DstT, bool VARSHAPE>
+template<class DstT, bool VARSHAPE, bool NORM>
 __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
@@ -146,7 +168,7 @@ __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
         int sy = (int)floorf((dy + a.cropY + 0.5f) * s.scaleY);
         sy     = min(sy, s.h - 1);
         const uint8_t *p = s.base + (int64_t)sy * s.rowStride + sx * 3;
-        StorePixel<DstT>(a, dst + (int64_t)dy * a.dstStrideY + dx * a.dstStrideX, (float)p[0], (float)p[1], (float)p[2]);
+        StorePixel<DstT, NORM>(a, dst + (int64_t)dy * a.dstStrideY + dx * a.dstStrideX, (float)p[0], (float)p[1], (float)p[2]);
     }
 }
 
@@ -155,7 +177,7 @@ __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
 // is harmless, at the very end of the image buffer the load is moved back so that it ends with the
 // buffer and the value is shifted into place (no divergent branch). Needs an image of >= 8 bytes.
 // BYTEWISE=true: plain byte loads, used for images smaller than 8 bytes.
-template<class DstT, bool VARSHAPE, bool BYTEWISE>
+template<class DstT, bool VARSHAPE, bool BYTEWISE, bool NORM>
 __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
@@ -236,12 +258,12 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
             }
             v[c] = t;
         }
-        StorePixel<DstT>(a, dst + (int64_t)dy * a.dstStrideY + dx * a.dstStrideX, v[0], v[1], v[2]);
+        StorePixel<DstT, NORM>(a, dst + (int64_t)dy * a.dstStrideY + dx * a.dstStrideX, v[0], v[1], v[2]);
     }
 }
 
-template<class DstT, bool VARSHAPE>
-void Launch(FusedArgs a, int N, NVCVInterpolationType interp, bool tinyImages, hipStream_t stream)
+template<class DstT, bool VARSHAPE, bool NORM>
+void LaunchKernels(FusedArgs a, int N, NVCVInterpolationType interp, bool tinyImages, hipStream_t stream)
 {
     if (N == 0 || a.dstW == 0 || a.dstH == 0)
     {
@@ -260,20 +282,33 @@ void Launch(FusedArgs a, int N, NVCVInterpolationType interp, bool tinyImages, h
     dim3 grid((uint32_t)total);
     if (interp == NVCV_INTERP_NEAREST)
     {
-        hipLaunchKernelGGL((FusedNearest<DstT, VARSHAPE>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((FusedNearest<DstT, VARSHAPE, NORM>), grid, block, 0, stream, a);
         CheckLaunch("FusedNearest");
     }
     else
     {
         if (tinyImages)
         {
-            hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, true>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, true, NORM>), grid, block, 0, stream, a);
         }
         else
         {
-            hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, false>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, false, NORM>), grid, block, 0, stream, a);
         }
         CheckLaunch("FusedBilinear");
+    }
+}
+
+template<class DstT, bool VARSHAPE>
+void Launch(const FusedArgs &a, bool normalize, int N, NVCVInterpolationType interp, bool tinyImages, hipStream_t stream)
+{
+    if (normalize)
+    {
+        LaunchKernels<DstT, VARSHAPE, true>(a, N, interp, tinyImages, stream);
+    }
+    else
+    {
+        LaunchKernels<DstT, VARSHAPE, false>(a, N, interp, tinyImages, stream);
     }
 }
 
@@ -282,7 +317,7 @@ class ResizeCropConvertReformat final : public IOperator
 public:
     void submit(hipStream_t stream, NVCVTensorHandle hin, NVCVTensorHandle hout, NVCVSize2D resizeDim,
                 NVCVInterpolationType interp, int2 cropPos, NVCVChannelManip manip, float scale, float offset,
-                bool srcCast) const
+                bool srcCast, const CVCUDAXChannelNormalize *norm = nullptr) const
     {
         NVCVTensorData din, dout;
         ExportTensor(hin, din, "Input");
@@ -311,7 +346,7 @@ public:
         }
         checkInterp(interp);
 
-        FusedArgs a       = makeArgs(out, resizeDim, cropPos, manip, scale, offset, srcCast);
+        FusedArgs a       = makeArgs(out, resizeDim, cropPos, manip, scale, offset, srcCast, norm);
         a.srcBase         = in.base;
         a.srcSampleStride = in.strideN;
         a.srcRowStride    = (int32_t)in.strideH;
@@ -322,17 +357,17 @@ public:
         const bool tiny = (int64_t)(in.H - 1) * in.strideH + (int64_t)in.W * 3 < 8;
         if (out.elem == kU8)
         {
-            Launch<uint8_t, false>(a, in.N, interp, tiny, stream);
+            Launch<uint8_t, false>(a, norm != nullptr, in.N, interp, tiny, stream);
         }
         else
         {
-            Launch<float, false>(a, in.N, interp, tiny, stream);
+            Launch<float, false>(a, norm != nullptr, in.N, interp, tiny, stream);
         }
     }
 
     void submit(hipStream_t stream, NVCVImageBatchHandle hin, NVCVTensorHandle hout, NVCVSize2D resizeDim,
                 NVCVInterpolationType interp, int2 cropPos, NVCVChannelManip manip, float scale, float offset,
-                bool srcCast) const
+                bool srcCast, const CVCUDAXChannelNormalize *norm = nullptr) const
     {
         VarShapeView   in = ExportVarShape(hin, stream, "Input");
         NVCVTensorData dout;
@@ -351,7 +386,7 @@ public:
         {
             throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid resize dimensions: %d x %d", resizeDim.w, resizeDim.h);
         }
-        FusedArgs a = makeArgs(out, resizeDim, cropPos, manip, scale, offset, srcCast);
+        FusedArgs a = makeArgs(out, resizeDim, cropPos, manip, scale, offset, srcCast, norm);
         a.srcList   = in.data.buffer.varShapeStrided.imageList;
         bool tiny = false;
         for (int i = 0; i < in.N; ++i)
@@ -361,11 +396,11 @@ public:
         }
         if (out.elem == kU8)
         {
-            Launch<uint8_t, true>(a, in.N, interp, tiny, stream);
+            Launch<uint8_t, true>(a, norm != nullptr, in.N, interp, tiny, stream);
         }
         else
         {
-            Launch<float, true>(a, in.N, interp, tiny, stream);
+            Launch<float, true>(a, norm != nullptr, in.N, interp, tiny, stream);
         }
     }
 
@@ -427,7 +462,7 @@ private:
     }
 
     static FusedArgs makeArgs(const ImageBatchView &out, NVCVSize2D resizeDim, int2 cropPos, NVCVChannelManip manip,
-                              float scale, float offset, bool srcCast)
+                              float scale, float offset, bool srcCast, const CVCUDAXChannelNormalize *norm)
     {
         const int es = ElemSize(out.elem);
         if (out.strideN % es || out.strideH % es || out.strideW % es || out.strideC % es)
@@ -453,6 +488,25 @@ private:
         a.scale   = scale;
         a.offset  = offset;
         a.srcCast = srcCast ? 1 : 0;
+        if (norm != nullptr)
+        {
+            if (norm->flags & ~(uint32_t)CVCUDA_NORMALIZE_SCALE_IS_STDDEV)
+            {
+                throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid normalization flags 0x%x", norm->flags);
+            }
+            for (int c = 0; c < 3; ++c)
+            {
+                // base / scale are given per OUTPUT channel; the kernel indexes by source channel
+                const int   to = manip == NVCV_CHANNEL_REVERSE ? 2 - c : c;
+                const float sc = norm->scale[to];
+                a.normBase[c]  = norm->base[to];
+                // same expression, in float32, as the Normalize operator evaluates on the device
+                a.normMul[c] = (norm->flags & CVCUDA_NORMALIZE_SCALE_IS_STDDEV) ? 1.0f / std::sqrt(sc * sc + norm->epsilon)
+                                                                                : sc;
+            }
+            a.normGlobal = norm->globalScale;
+            a.normShift  = norm->shift;
+        }
         return a;
     }
 };
@@ -495,6 +549,42 @@ CVCUDA_PUBLIC NVCVStatus cvcudaResizeCropConvertReformatVarShapeSubmit(
         {
             ToOperator<ResizeCropConvertReformat>(handle).submit(stream, in, out, resizeDim, interpolation, cropPos,
                                                                  manip, scale, offset, srcCast);
+        });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaxResizeCropConvertReformatNormalizeSubmit(
+    NVCVOperatorHandle handle, hipStream_t stream, NVCVTensorHandle in, NVCVTensorHandle out,
+    const NVCVSize2D resizeDim, const NVCVInterpolationType interpolation, const int2 cropPos,
+    const NVCVChannelManip manip, const float scale, const float offset, const bool srcCast,
+    const CVCUDAXChannelNormalize *normalize)
+{
+    return Protect(
+        [&]
+        {
+            if (normalize == nullptr)
+            {
+                throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Pointer to the normalization parameters must not be NULL");
+            }
+            ToOperator<ResizeCropConvertReformat>(handle).submit(stream, in, out, resizeDim, interpolation, cropPos,
+                                                                 manip, scale, offset, srcCast, normalize);
+        });
+}
+
+CVCUDA_PUBLIC NVCVStatus cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit(
+    NVCVOperatorHandle handle, hipStream_t stream, NVCVImageBatchHandle in, NVCVTensorHandle out,
+    const NVCVSize2D resizeDim, const NVCVInterpolationType interpolation, const int2 cropPos,
+    const NVCVChannelManip manip, const float scale, const float offset, const bool srcCast,
+    const CVCUDAXChannelNormalize *normalize)
+{
+    return Protect(
+        [&]
+        {
+            if (normalize == nullptr)
+            {
+                throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Pointer to the normalization parameters must not be NULL");
+            }
+            ToOperator<ResizeCropConvertReformat>(handle).submit(stream, in, out, resizeDim, interpolation, cropPos,
+                                                                 manip, scale, offset, srcCast, normalize);
         });
 }
 }

@@ -39,6 +39,38 @@ CVCUDA_PUBLIC NVCVStatus cvcudaResizeCropConvertReformatVarShapeSubmit(
     const NVCVSize2D resizeDim, const NVCVInterpolationType interpolation, const int2 cropPos,
     const NVCVChannelManip manip, const float scale, const float offset, const bool srcCast);
 
+/* ---- Extension (no counterpart in the reference) -------------------------------------------------
+ * The fused operator followed, in the same kernel, by a per-channel normalisation: the result is
+ * what cvcudaNormalizeSubmit(base[1,1,1,3], scale[1,1,1,3], globalScale, shift, epsilon, flags)
+ * gives when applied to the f32 output of the fused operator with the same scale/offset, i.e.
+ *     x = scale*v + offset;  out = ((x - base[c]) * m[c]) * globalScale + shift,
+ *     m[c] = scale[c], or 1/sqrt(scale[c]^2 + epsilon) with CVCUDA_NORMALIZE_SCALE_IS_STDDEV,
+ * evaluated in float32 in this order, c being the OUTPUT channel (after manip). It serves the
+ * "resize, crop, /255, subtract mean, divide by std, to planar f32" pre-processing in one pass over
+ * the data; the reference needs three operators (fused, Normalize, Reformat) for it.
+ * Status codes as for the plain entry points; INVALID_ARGUMENT for a NULL `normalize` or unknown flags. */
+typedef struct CVCUDAXChannelNormalizeRec
+{
+    float    base[3];
+    float    scale[3];
+    float    globalScale;
+    float    shift;
+    float    epsilon;
+    uint32_t flags; /* 0 or CVCUDA_NORMALIZE_SCALE_IS_STDDEV (cvcuda/OpNormalize.h) */
+} CVCUDAXChannelNormalize;
+
+CVCUDA_PUBLIC NVCVStatus cvcudaxResizeCropConvertReformatNormalizeSubmit(
+    NVCVOperatorHandle handle, hipStream_t stream, NVCVTensorHandle in, NVCVTensorHandle out,
+    const NVCVSize2D resizeDim, const NVCVInterpolationType interpolation, const int2 cropPos,
+    const NVCVChannelManip manip, const float scale, const float offset, const bool srcCast,
+    const CVCUDAXChannelNormalize *normalize);
+
+CVCUDA_PUBLIC NVCVStatus cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit(
+    NVCVOperatorHandle handle, hipStream_t stream, NVCVImageBatchHandle in, NVCVTensorHandle out,
+    const NVCVSize2D resizeDim, const NVCVInterpolationType interpolation, const int2 cropPos,
+    const NVCVChannelManip manip, const float scale, const float offset, const bool srcCast,
+    const CVCUDAXChannelNormalize *normalize);
+
 #ifdef __cplusplus
 }
 #endif

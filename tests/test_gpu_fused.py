@@ -167,3 +167,63 @@ def test_benchmark_config_full_size(cv, orc, gpu):
     compare(res[:4], ref, LINEAR, np.float32)
     for k in range(1, N // 4):
         np.testing.assert_array_equal(res[4 * k:4 * k + 4], res[:4])
+
+
+# ---- extension: fused + per-channel normalisation in one kernel -------------------------------------
+IMAGENET_MEAN, IMAGENET_STD = (0.485, 0.456, 0.406), (0.229, 0.224, 0.225)
+
+
+@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("manip", [0, 1])
+def test_normalize_extension_equals_three_operator_chain(cv, K, orc, gpu, interp, manip):
+    # the reference-faithful way: fused (scale 1/255, f32 NHWC) -> Normalize(STDDEV) -> Reformat(NCHW);
+    # the extension must give the same bits in one pass
+    src = orc.fill_u8((3, 135, 240, 3), 77)
+    tin = cv.Tensor.from_numpy(src, "NHWC")
+    fused, norm, reformat = cv.ResizeCropConvertReformat(), cv.Normalize(), cv.Reformat()
+    t1 = cv.Tensor.alloc([3, 56, 56, 3], np.float32, "NHWC")
+    t2 = cv.Tensor.alloc([3, 56, 56, 3], np.float32, "NHWC")
+    t3 = cv.Tensor.alloc([3, 3, 56, 56], np.float32, "NCHW")
+    fused(None, tin, t1, (114, 64), interp, (29, 4), manip, 1 / 255.0, 0.0, False)
+    mean = np.asarray(IMAGENET_MEAN, np.float32).reshape(1, 1, 1, 3)
+    std = np.asarray(IMAGENET_STD, np.float32).reshape(1, 1, 1, 3)
+    norm(None, t1, cv.Tensor.from_numpy(mean, "NHWC"), cv.Tensor.from_numpy(std, "NHWC"), t2, 1.0, 0.0, 0.0,
+         K.CVCUDA_NORMALIZE_SCALE_IS_STDDEV)
+    reformat(None, t2, t3)
+    one = cv.Tensor.alloc([3, 3, 56, 56], np.float32, "NCHW")
+    fused.normalized(None, tin, one, (114, 64), interp, (29, 4), IMAGENET_MEAN, IMAGENET_STD, manip, 1 / 255.0, 0.0,
+                     False, 1.0, 0.0, 0.0, K.CVCUDA_NORMALIZE_SCALE_IS_STDDEV)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(one.numpy(), t3.numpy())
+    # and against the oracle: golden fused composed with the Normalize formula
+    x = orc.fused_rccr(src, (56, 56), (114, 64), (29, 4), interp, np.float32, False, manip, 1 / 255.0, 0.0, False)
+    ref = orc.normalize(x, mean, std, 1.0, 0.0, 0.0, True).transpose(0, 3, 1, 2)
+    assert (np.abs(one.numpy() - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all()
+
+
+def test_normalize_extension_varshape_plain_scale_and_errors(cv, K, orc, gpu):
+    rng = np.random.default_rng(3)
+    n = 4
+    batch, hosts = cv.ImageBatchVarShape(n), []
+    for i in range(n):
+        a = orc.fill_u8((int(rng.integers(60, 200)), int(rng.integers(80, 300)), 3), 500 + i)
+        hosts.append(a)
+        batch.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_RGB8))
+    out = cv.Tensor.alloc([n, 3, 32, 48], np.float32, "NCHW")
+    op = cv.ResizeCropConvertReformat()
+    base, nscale = (10.0, 20.0, 30.0), (0.5, 0.25, 2.0)
+    op.normalized(None, batch, out, (64, 40), 1, (8, 4), base, nscale, 0, 1.0, 0.0, False, 0.9, 0.1)
+    torch.cuda.synchronize()
+    got = out.numpy()
+    for i, a in enumerate(hosts):
+        x = orc.fused_rccr(a[None], (32, 48), (64, 40), (8, 4), 1, np.float32, False, 0, 1.0, 0.0, False)
+        ref = orc.normalize(x, np.asarray(base, np.float32).reshape(1, 1, 1, 3),
+                            np.asarray(nscale, np.float32).reshape(1, 1, 1, 3), 0.9, 0.1)[0].transpose(2, 0, 1)
+        assert (np.abs(got[i] - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all()
+    with pytest.raises(cv.Error) as e:
+        op.normalized(None, batch, out, (64, 40), 1, (8, 4), base, nscale, flags=4)
+    assert e.value.status == 2
+    st = cv._cv.cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit(
+        op.handle, cv.stream_ptr(None), batch.handle, out.handle, cv.capi.Size2D(64, 40), 1, cv.capi.Int2(8, 4), 0, 1.0,
+        0.0, False, None)
+    assert st == 2
