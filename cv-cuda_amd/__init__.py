@@ -409,6 +409,44 @@ class Reformat(_Operator):
         check(_cv.cvcudaReformatSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out)))
 
 
+class ConvertTo(_Operator):
+    _create = "cvcudaConvertToCreate"
+
+    def __call__(self, stream, inp, out, alpha=1.0, beta=0.0):
+        check(_cv.cvcudaConvertToSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out), alpha, beta))
+
+
+class CustomCrop(_Operator):
+    _create = "cvcudaCustomCropCreate"
+
+    def __call__(self, stream, inp, out, rect):
+        """rect: (x, y, width, height)"""
+        check(_cv.cvcudaCustomCropSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out), capi.RectI(*rect)))
+
+
+class CenterCrop(_Operator):
+    _create = "cvcudaCenterCropCreate"
+
+    def __call__(self, stream, inp, out, crop_size):
+        """crop_size: (width, height)"""
+        check(_cv.cvcudaCenterCropSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out), crop_size[0],
+                                         crop_size[1]))
+
+
+class Flip(_Operator):
+    _create = "cvcudaFlipCreate"
+
+    def __init__(self, max_varshape_batch_size=0):
+        super().__init__(max_varshape_batch_size)
+
+    def __call__(self, stream, inp, out, flip_code):
+        """flip_code: int for tensors, an int32 Tensor with one code per image for var-shape batches."""
+        if isinstance(inp, ImageBatchVarShape):
+            check(_cv.cvcudaFlipVarShapeSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out), _h(flip_code)))
+        else:
+            check(_cv.cvcudaFlipSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out), flip_code))
+
+
 class WarpAffine(_Operator):
     _create = "cvcudaWarpAffineCreate"
 

@@ -122,6 +122,10 @@ class Int2(C.Structure):
     _fields_ = [("x", C.c_int), ("y", C.c_int)]
 
 
+class RectI(C.Structure):
+    _fields_ = [("x", C.c_int32), ("y", C.c_int32), ("width", C.c_int32), ("height", C.c_int32)]
+
+
 class Float4(C.Structure):
     _fields_ = [("x", C.c_float), ("y", C.c_float), ("z", C.c_float), ("w", C.c_float)]
 
@@ -283,6 +287,16 @@ _sig(cvcuda, "cvcudaxResizeCropConvertReformatNormalizeSubmit", ST, H, C.c_void_
      C.c_int, C.c_float, C.c_float, C.c_bool, P(ChannelNormalize))
 _sig(cvcuda, "cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit", ST, H, C.c_void_p, H, H, Size2D, C.c_int,
      Int2, C.c_int, C.c_float, C.c_float, C.c_bool, P(ChannelNormalize))
+
+_sig(cvcuda, "cvcudaConvertToCreate", ST, P(H))
+_sig(cvcuda, "cvcudaConvertToSubmit", ST, H, C.c_void_p, H, H, C.c_double, C.c_double)
+_sig(cvcuda, "cvcudaCustomCropCreate", ST, P(H))
+_sig(cvcuda, "cvcudaCustomCropSubmit", ST, H, C.c_void_p, H, H, RectI)
+_sig(cvcuda, "cvcudaCenterCropCreate", ST, P(H))
+_sig(cvcuda, "cvcudaCenterCropSubmit", ST, H, C.c_void_p, H, H, C.c_int32, C.c_int32)
+_sig(cvcuda, "cvcudaFlipCreate", ST, P(H), C.c_int32)
+_sig(cvcuda, "cvcudaFlipSubmit", ST, H, C.c_void_p, H, H, C.c_int32)
+_sig(cvcuda, "cvcudaFlipVarShapeSubmit", ST, H, C.c_void_p, H, H, H)
 
 
 def declare_optional(name, res, *args):

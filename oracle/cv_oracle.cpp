@@ -889,6 +889,84 @@ ORC_API int orc_warp(const void *src, int64_t srcStep, int64_t srcImgStep, int N
                         });
 }
 
+// ---- ConvertTo ---------------------------------------------------------------------------------------
+// variant 1 (device): src/cvcuda/priv/legacy/convert_to.cu:36-47, 77-83: alpha*src+beta evaluated in
+// float32, or float64 when either element type is float64, alpha/beta first converted to that type.
+// variant 0 (golden): tests/cvcuda/system/TestOpConvertTo.cpp:132 evaluates it in float64 always.
+template<class TS, class TD>
+void ConvertRows(const TS *src, TD *dst, int64_t count, double alpha, double beta, int variant)
+{
+    constexpr bool dbl = std::is_same_v<TS, double> || std::is_same_v<TD, double>;
+    for (int64_t i = 0; i < count; ++i)
+    {
+        if (dbl || variant == 0)
+        {
+            dst[i] = SatD<TD>(alpha * (double)src[i] + beta);
+        }
+        else
+        {
+            const float v = (float)alpha * (float)src[i] + (float)beta;
+            dst[i]        = SatF<TD>(v);
+        }
+    }
+}
+
+template<class TS>
+int ConvertDst(const TS *src, void *dst, int dstType, int64_t count, double alpha, double beta, int variant)
+{
+    switch (dstType)
+    {
+    case U8:
+        ConvertRows(src, (uint8_t *)dst, count, alpha, beta, variant);
+        return 0;
+    case S8:
+        ConvertRows(src, (int8_t *)dst, count, alpha, beta, variant);
+        return 0;
+    case U16:
+        ConvertRows(src, (uint16_t *)dst, count, alpha, beta, variant);
+        return 0;
+    case S16:
+        ConvertRows(src, (int16_t *)dst, count, alpha, beta, variant);
+        return 0;
+    case S32:
+        ConvertRows(src, (int32_t *)dst, count, alpha, beta, variant);
+        return 0;
+    case F32:
+        ConvertRows(src, (float *)dst, count, alpha, beta, variant);
+        return 0;
+    case F64:
+        ConvertRows(src, (double *)dst, count, alpha, beta, variant);
+        return 0;
+    default:
+        return 1;
+    }
+}
+
+// Packed arrays of `count` scalars.
+ORC_API int orc_convert_to(const void *src, int srcType, void *dst, int dstType, int64_t count, double alpha,
+                           double beta, int variant)
+{
+    switch (srcType)
+    {
+    case U8:
+        return ConvertDst((const uint8_t *)src, dst, dstType, count, alpha, beta, variant);
+    case S8:
+        return ConvertDst((const int8_t *)src, dst, dstType, count, alpha, beta, variant);
+    case U16:
+        return ConvertDst((const uint16_t *)src, dst, dstType, count, alpha, beta, variant);
+    case S16:
+        return ConvertDst((const int16_t *)src, dst, dstType, count, alpha, beta, variant);
+    case S32:
+        return ConvertDst((const int32_t *)src, dst, dstType, count, alpha, beta, variant);
+    case F32:
+        return ConvertDst((const float *)src, dst, dstType, count, alpha, beta, variant);
+    case F64:
+        return ConvertDst((const double *)src, dst, dstType, count, alpha, beta, variant);
+    default:
+        return 1;
+    }
+}
+
 // ---- primitives exposed for known-answer tests ----------------------------------------------------
 ORC_API int orc_saturate_f32(float v, int dtype)
 {

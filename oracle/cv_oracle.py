@@ -32,7 +32,7 @@ def lib():
 
 
 DTYPE_CODE = {np.dtype(np.uint8): 0, np.dtype(np.int8): 1, np.dtype(np.uint16): 2, np.dtype(np.int16): 3,
-              np.dtype(np.int32): 4, np.dtype(np.float32): 5}
+              np.dtype(np.int32): 4, np.dtype(np.float32): 5, np.dtype(np.float64): 6}
 
 
 def _p(a):
@@ -111,6 +111,18 @@ def normalize(src, base, scale, global_scale=1.0, shift=0.0, epsilon=0.0, stddev
                              bC, _p(scale), _i64(sW * sC), _i64(sH * sW * sC), sN, sW, sH, sC,
                              C.c_float(global_scale), C.c_float(shift), C.c_float(epsilon), int(bool(stddev)),
                              int(threads))
+    assert rc == 0
+    return dst
+
+
+def convert_to(src, out_dtype, alpha=1.0, beta=0.0, variant=1):
+    """Element-wise saturate_cast<out_dtype>(alpha*src+beta); variant 1 = device arithmetic, 0 = float64 golden."""
+    src = np.ascontiguousarray(src)
+    dst = np.zeros(src.shape, out_dtype)
+    lib().orc_convert_to.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int64, C.c_double, C.c_double,
+                                     C.c_int]
+    rc = lib().orc_convert_to(_p(src), DTYPE_CODE[src.dtype], _p(dst), DTYPE_CODE[dst.dtype], src.size, alpha, beta,
+                              int(variant))
     assert rc == 0
     return dst
 

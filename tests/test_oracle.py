@@ -324,3 +324,28 @@ def test_seeded_generators(orc):
     # splitmix64 reference value: first output for seed 0 is 0xE220A8397B1DCDAF (published test vector)
     first8 = orc.fill_u8((8,), 0)
     assert int.from_bytes(bytes(first8), "little") == 0xE220A8397B1DCDAF
+
+
+def test_convert_to_known_answers_and_numpy_cross_check(orc):
+    # rows of the reference's own test (tests/cvcuda/system/TestOpConvertTo.cpp:119-240): value 0x10
+    v = np.full((7,), 16, np.uint8)
+    for variant in (0, 1):
+        assert (orc.convert_to(v, np.uint8, 1.0, 1.0, variant) == 17).all()
+        assert (orc.convert_to(v, np.uint8, 2.1, 2.0, variant) == 36).all()
+        assert (orc.convert_to(v, np.uint8, 2.1, -1.0, variant) == 33).all()
+        assert (orc.convert_to(v, np.uint16, 2.1, 2.0, variant) == 36).all()
+    assert (orc.convert_to(v, np.float32, 2.1, 2.0, 1) == np.float32(2.1) * np.float32(16) + np.float32(2)).all()
+    assert (orc.convert_to(v.astype(np.float32), np.float64, 2.1, 2.0, 1) == 2.1 * 16 + 2.0).all()
+    # identity, saturation at both ends, ties to even, NaN
+    x = np.arange(-300, 300, dtype=np.int16)
+    np.testing.assert_array_equal(orc.convert_to(x, np.int16), x)
+    np.testing.assert_array_equal(orc.convert_to(x, np.uint8), np.clip(x, 0, 255))
+    np.testing.assert_array_equal(orc.convert_to(x, np.int8), np.clip(x, -128, 127))
+    np.testing.assert_array_equal(orc.convert_to(np.array([1, 3, 5, 7], np.uint8), np.uint8, 0.5, 0.0), [0, 2, 2, 4])
+    assert orc.convert_to(np.array([np.nan, 1e20, -1e20], np.float32), np.int32).tolist() == [0, 2**31 - 1, -2**31]
+    # every integer target against numpy arithmetic in float32
+    f = (orc.fill_f32((4096,), 5) - 0.5) * 1e5
+    for dt in (np.uint8, np.int8, np.uint16, np.int16, np.int32):
+        info = np.iinfo(dt)
+        ref = np.clip(np.rint(np.float32(0.37) * f + np.float32(-11.5)), info.min, info.max).astype(dt)
+        np.testing.assert_array_equal(orc.convert_to(f, dt, 0.37, -11.5), ref)
