@@ -409,6 +409,16 @@ class Reformat(_Operator):
         check(_cv.cvcudaReformatSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out)))
 
 
+class CropFlipNormalizeReformat(_Operator):
+    _create = "cvcudaCropFlipNormalizeReformatCreate"
+
+    def __call__(self, stream, inp, out, crop_rect, border, border_value, flip_code, base, scale, global_scale=1.0,
+                 shift=0.0, epsilon=0.0, flags=0):
+        check(_cv.cvcudaCropFlipNormalizeReformatSubmit(self.handle, stream_ptr(stream), _h(inp), _h(out),
+                                                        _h(crop_rect), border, border_value, _h(flip_code), _h(base),
+                                                        _h(scale), global_scale, shift, epsilon, flags))
+
+
 class ConvertTo(_Operator):
     _create = "cvcudaConvertToCreate"
 

@@ -288,6 +288,9 @@ _sig(cvcuda, "cvcudaxResizeCropConvertReformatNormalizeSubmit", ST, H, C.c_void_
 _sig(cvcuda, "cvcudaxResizeCropConvertReformatNormalizeVarShapeSubmit", ST, H, C.c_void_p, H, H, Size2D, C.c_int,
      Int2, C.c_int, C.c_float, C.c_float, C.c_bool, P(ChannelNormalize))
 
+_sig(cvcuda, "cvcudaCropFlipNormalizeReformatCreate", ST, P(H))
+_sig(cvcuda, "cvcudaCropFlipNormalizeReformatSubmit", ST, H, C.c_void_p, H, H, H, C.c_int, C.c_float, H, H, H,
+     C.c_float, C.c_float, C.c_float, C.c_uint32)
 _sig(cvcuda, "cvcudaConvertToCreate", ST, P(H))
 _sig(cvcuda, "cvcudaConvertToSubmit", ST, H, C.c_void_p, H, H, C.c_double, C.c_double)
 _sig(cvcuda, "cvcudaCustomCropCreate", ST, P(H))

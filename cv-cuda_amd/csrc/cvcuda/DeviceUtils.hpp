@@ -3,6 +3,7 @@
 #define CVCUDA_AMD_DEVICEUTILS_HPP
 
 #include <hip/hip_runtime.h>
+#include <nvcv/BorderType.h>
 
 #include <cstdint>
 #include <type_traits>
@@ -90,6 +91,42 @@ __device__ __forceinline__ uint32_t LoadU32Unaligned(const uint8_t *p)
 __device__ __forceinline__ uint64_t LoadU64Unaligned(const uint8_t *p)
 {
     return reinterpret_cast<const UnalignedU64 *>(p)->v;
+}
+
+// Coordinate c outside [0, s) -> the coordinate inside that the border mode stands for (every mode
+// but NVCV_BORDER_CONSTANT); index maps of the reference's border wrappers
+// (cuda_tools/BorderWrap.hpp:62-121, BorderVarShapeWrap.hpp:290-368).
+__device__ __forceinline__ int BorderIndex(int border, int c, int s)
+{
+    switch (border)
+    {
+    case NVCV_BORDER_REPLICATE:
+        return c < 0 ? 0 : (c >= s ? s - 1 : c);
+    case NVCV_BORDER_WRAP:
+        c = c % s;
+        return c < 0 ? c + s : c;
+    case NVCV_BORDER_REFLECT:
+    {
+        const int s2 = s * 2;
+        c            = c % s2;
+        if (c < 0)
+        {
+            c += s2;
+        }
+        return s - 1 - (abs(2 * c + 1 - s2) >> 1);
+    }
+    default: // REFLECT101
+        if (s == 1)
+        {
+            return 0;
+        }
+        c = c % (2 * s - 2);
+        if (c < 0)
+        {
+            c += 2 * s - 2;
+        }
+        return s - 1 - abs(s - 1 - c);
+    }
 }
 
 // MI355X hands the workgroups of a launch to its 8 XCDs round-robin (hardware id % 8) and every

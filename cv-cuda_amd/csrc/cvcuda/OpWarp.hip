@@ -72,39 +72,6 @@ struct Img
     int32_t        row, w, h;
 };
 
-__device__ __forceinline__ int BorderIndex(int border, int c, int s)
-{
-    switch (border)
-    {
-    case NVCV_BORDER_REPLICATE:
-        return c < 0 ? 0 : (c >= s ? s - 1 : c);
-    case NVCV_BORDER_WRAP:
-        c = c % s;
-        return c < 0 ? c + s : c;
-    case NVCV_BORDER_REFLECT:
-    {
-        const int s2 = s * 2;
-        c            = c % s2;
-        if (c < 0)
-        {
-            c += s2;
-        }
-        return s - 1 - (abs(2 * c + 1 - s2) >> 1);
-    }
-    default: // REFLECT101
-        if (s == 1)
-        {
-            return 0;
-        }
-        c = c % (2 * s - 2);
-        if (c < 0)
-        {
-            c += 2 * s - 2;
-        }
-        return s - 1 - abs(s - 1 - c);
-    }
-}
-
 template<class T>
 __device__ __forceinline__ T BorderCast(float v)
 {

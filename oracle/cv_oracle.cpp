@@ -967,6 +967,98 @@ ORC_API int orc_convert_to(const void *src, int srcType, void *dst, int dstType,
     }
 }
 
+// ---- CropFlipNormalizeReformat ------------------------------------------------------------------------
+// follows the golden tests/cvcuda/system/TestOpCropFlipNormalizeReformat.cpp:44-170 (identical to the
+// device expression src/cvcuda/priv/OpCropFlipNormalizeReformat.cu:73-74, 165-187): one image, source
+// and destination as packed HWC arrays.
+template<class TS, class TD>
+void CropFlipNormOne(const TS *src, int W, int H, int C, TD *dst, int dw, int dh, const int *crop, int flip, int border,
+                     float borderValue, const float *base, const float *scale, float gscale, float shift, float eps,
+                     int stddev)
+{
+    for (int i = 0; i < dh; ++i)
+    {
+        for (int j = 0; j < dw; ++j)
+        {
+            TD *o = dst + ((int64_t)i * dw + j) * C;
+            if (i >= crop[3] || j >= crop[2])
+            {
+                for (int k = 0; k < C; ++k)
+                {
+                    o[k] = 0;
+                }
+                continue;
+            }
+            int x = j + crop[0], y = i + crop[1];
+            if (flip == 1 || flip == -1)
+            {
+                x = crop[2] - 1 - j + crop[0];
+            }
+            if (flip == 0 || flip == -1)
+            {
+                y = crop[3] - 1 - i + crop[1];
+            }
+            const bool outside = x < 0 || x >= W || y < 0 || y >= H;
+            if (outside && border != 0)
+            {
+                x = BorderIndex(border, x, W);
+                y = BorderIndex(border, y, H);
+            }
+            for (int k = 0; k < C; ++k)
+            {
+                float mul = scale[k];
+                if (stddev)
+                {
+                    float t = scale[k] * scale[k] + eps;
+                    mul     = 1.0f / std::sqrt(t);
+                }
+                TS v;
+                if (outside && border == 0)
+                {
+                    if constexpr (std::is_same_v<TS, float>)
+                    {
+                        v = borderValue;
+                    }
+                    else
+                    {
+                        float t = std::trunc(borderValue);
+                        t       = std::min(std::max(t, (float)std::numeric_limits<TS>::min()),
+                                           (float)std::numeric_limits<TS>::max());
+                        v       = (TS)(int64_t)t;
+                    }
+                }
+                else
+                {
+                    v = src[((int64_t)y * W + x) * C + k];
+                }
+                o[k] = SatF<TD>(((float)v - base[k]) * mul * gscale + shift);
+            }
+        }
+    }
+}
+
+ORC_API int orc_crop_flip_normalize(const void *src, int W, int H, int C, int srcType, void *dst, int dw, int dh,
+                                    int dstType, const int *crop, int flip, int border, float borderValue,
+                                    const float *base, const float *scale, float gscale, float shift, float eps,
+                                    int stddev)
+{
+    int rc = 1;
+    DispatchType(srcType,
+                 [&](auto ts)
+                 {
+                     using TS = decltype(ts);
+                     rc       = DispatchType(dstType,
+                                             [&](auto td)
+                                             {
+                                           using TD = decltype(td);
+                                           CropFlipNormOne<TS, TD>((const TS *)src, W, H, C, (TD *)dst, dw, dh, crop, flip,
+                                                                   border, borderValue, base, scale, gscale, shift, eps,
+                                                                   stddev);
+                                       });
+                 });
+    return rc;
+}
+
 // ---- primitives exposed for known-answer tests ----------------------------------------------------
 ORC_API int orc_saturate_f32(float v, int dtype)
 {

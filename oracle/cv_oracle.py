@@ -127,6 +127,24 @@ def convert_to(src, out_dtype, alpha=1.0, beta=0.0, variant=1):
     return dst
 
 
+def crop_flip_normalize(src, out_hw, out_dtype, crop, flip, border, border_value, base, scale, global_scale=1.0,
+                        shift=0.0, epsilon=0.0, stddev=False):
+    """One image src [H,W,C] -> [h,w,C]; crop = (x, y, width, height); base/scale: C floats."""
+    src = np.ascontiguousarray(src)
+    H, W, Cc = src.shape
+    h, w = out_hw
+    dst = np.zeros((h, w, Cc), out_dtype)
+    cr = np.asarray(crop, np.int32)
+    b = np.ascontiguousarray(np.broadcast_to(np.asarray(base, np.float32).reshape(-1), (Cc,)))
+    sc = np.ascontiguousarray(np.broadcast_to(np.asarray(scale, np.float32).reshape(-1), (Cc,)))
+    rc = lib().orc_crop_flip_normalize(_p(src), W, H, Cc, DTYPE_CODE[src.dtype], _p(dst), w, h, DTYPE_CODE[dst.dtype],
+                                       _p(cr), int(flip), int(border), C.c_float(border_value), _p(b), _p(sc),
+                                       C.c_float(global_scale), C.c_float(shift), C.c_float(epsilon),
+                                       int(bool(stddev)))
+    assert rc == 0
+    return dst
+
+
 def invert_affine(m):
     m = np.ascontiguousarray(m, dtype=np.float32).reshape(6)
     out = np.zeros(6, np.float32)

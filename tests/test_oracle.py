@@ -349,3 +349,29 @@ def test_convert_to_known_answers_and_numpy_cross_check(orc):
         info = np.iinfo(dt)
         ref = np.clip(np.rint(np.float32(0.37) * f + np.float32(-11.5)), info.min, info.max).astype(dt)
         np.testing.assert_array_equal(orc.convert_to(f, dt, 0.37, -11.5), ref)
+
+
+def test_crop_flip_normalize_closed_forms(orc):
+    a = orc.fill_u8((20, 30, 3), 8)
+    # identity parameters = numpy crop (+ flips), zeros beyond the rectangle
+    for code, pick in [(7, lambda w: w), (1, lambda w: w[:, ::-1]), (0, lambda w: w[::-1]), (-1, lambda w: w[::-1, ::-1])]:
+        r = orc.crop_flip_normalize(a, (16, 24), np.uint8, (4, 2, 20, 12), code, 0, 0.0, [0], [1])
+        np.testing.assert_array_equal(r[:12, :20], pick(a[2:14, 4:24]))
+        assert (r[12:] == 0).all() and (r[:, 20:] == 0).all()
+    # rectangle leaving the image: numpy.pad supplies the border
+    pads = {0: dict(mode="constant", constant_values=9), 1: dict(mode="edge"), 2: dict(mode="symmetric"),
+            3: dict(mode="wrap"), 4: dict(mode="reflect")}
+    for border, kw in pads.items():
+        padded = np.pad(a, ((5, 5), (5, 5), (0, 0)), **kw)
+        r = orc.crop_flip_normalize(a, (26, 36), np.uint8, (-3, -4, 36, 26), 2, border, 9.0, [0], [1])
+        np.testing.assert_array_equal(r, padded[1:27, 2:38])
+    # normalisation arithmetic against numpy float32, scalar and per-channel, stddev mode
+    base, scale = np.array([10.5, 20.25, 3.0], np.float32), np.array([0.5, 0.25, 2.0], np.float32)
+    x = a[2:14, 4:24].astype(np.float32)
+    r = orc.crop_flip_normalize(a, (12, 20), np.float32, (4, 2, 20, 12), 2, 0, 0.0, base, scale, 1.5, -2.0)
+    np.testing.assert_array_equal(r, (x - base) * scale * np.float32(1.5) + np.float32(-2.0))
+    r = orc.crop_flip_normalize(a, (12, 20), np.float32, (4, 2, 20, 12), 2, 0, 0.0, base, scale, 1.0, 0.0, 0.01, True)
+    mul = np.float32(1) / np.sqrt(scale * scale + np.float32(0.01))
+    np.testing.assert_array_equal(r, (x - base) * mul * np.float32(1.0) + np.float32(0.0))
+    r8 = orc.crop_flip_normalize(a, (12, 20), np.int8, (4, 2, 20, 12), 2, 0, 0.0, [128], [1])
+    np.testing.assert_array_equal(r8, np.clip(a[2:14, 4:24].astype(np.int32) - 128, -128, 127))
