@@ -318,6 +318,9 @@ def main():
                     help="distinct buffer sets cycled through (0 = enough to touch >= 450 MB, 1 = cache-resident)")
     ap.add_argument("--no-graph", action="store_true", help="time eager Submits instead of a HIP-graph replay")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget of the CPU-oracle leg (0 = skip)")
+    ap.add_argument("--streams", type=int, default=1,
+                    help="independent streams the K steps are dealt to inside the captured graph (default 1: every "
+                         "step waits for the one before, as consecutive Submits on one stream do)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="after the timed region, also run a plain device copy of this many MiB three times "
                          "(a kernel of known traffic to scale hardware byte counters against)")
@@ -358,10 +361,15 @@ def main():
     if not args.no_graph:
         try:
             graph = torch.cuda.CUDAGraph()
+            sides = [torch.cuda.Stream() for _ in range(args.streams)] if args.streams > 1 else []
             with torch.cuda.graph(graph):
                 cap = torch.cuda.current_stream()
+                for sd in sides:
+                    sd.wait_stream(cap)
                 for i in range(args.steps):
-                    wl.submit(cap, sets[i % nsets])
+                    wl.submit(sides[i % len(sides)] if sides else cap, sets[i % nsets])
+                for sd in sides:
+                    cap.wait_stream(sd)
             graph.replay()  # untimed first replay
             torch.cuda.synchronize()
             mode = "hipgraph"
@@ -425,7 +433,8 @@ def main():
         "vs_baseline": None,
         "dtype": wl.dtype,
         "data": "synthetic",
-        "config": {"workload": wl.workload, "rotate_buffer_sets": nsets, "launch": mode},
+        "config": {"workload": wl.workload, "rotate_buffer_sets": nsets, "launch": mode,
+                   "streams": args.streams if graph is not None else 1},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.key),
                      "kernel": wl.kernel, "kernel_ms_mean": round(mean_kernel_ms, 5),
