@@ -79,9 +79,13 @@ def build(force=False, jobs=8, verbose=True):
     nvcv_so = os.path.join(LIBDIR, "libnvcv_types.so")
     cvcuda_so = os.path.join(LIBDIR, "libcvcuda.so")
     link = ["hipcc", "-shared", "-fPIC", "--offload-arch=" + ARCH, "-Wl,--no-undefined"]
-    subprocess.run(link + core_objs + ["-o", nvcv_so, "-Wl,-soname,libnvcv_types.so"], check=True)
+    # ELF symbol versions of the reference's ABI (FUNC@@NVCV_x.y / FUNC@@CVCUDA_x.y), see csrc/abi
+    maps = os.path.join(CSRC, "abi")
+    subprocess.run(link + core_objs + ["-o", nvcv_so, "-Wl,-soname,libnvcv_types.so",
+                                       "-Wl,--version-script=" + os.path.join(maps, "nvcv_types.map")], check=True)
     subprocess.run(link + ops_objs + ["-o", cvcuda_so, "-Wl,-soname,libcvcuda.so", "-L" + LIBDIR, "-lnvcv_types",
-                                      "-Wl,-rpath,$ORIGIN"], check=True)
+                                      "-Wl,-rpath,$ORIGIN",
+                                      "-Wl,--version-script=" + os.path.join(maps, "cvcuda.map")], check=True)
     return nvcv_so, cvcuda_so
 
 

@@ -115,3 +115,28 @@ int main(void) {
     assert out[0].startswith("2|Invalid resize dimensions: width x hight = 33 x 1")
     assert out[1].startswith("2|Invalid crop region: crop region(x, y, w, h) = (11, 22, 12, 10)")
     assert out[2] == "2|Interpolation not implemented: NVCV_INTERP_CUBIC"
+
+
+def test_symbol_versions_match_reference_tags(cv):
+    """Exported functions carry the ELF symbol versions the reference gives them (NVCV_PROJ_DEFINE_API,
+    src/nvcv/util/SymbolVersioning.hpp:69-92), so binaries linked against the reference resolve."""
+    import os
+    import re
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for lib, mapfile in (("libcvcuda.so", "cvcuda.map"), ("libnvcv_types.so", "nvcv_types.map")):
+        text = open(os.path.join(root, "cv-cuda_amd", "csrc", "abi", mapfile)).read()
+        want = {}
+        for node, body in re.findall(r"(\w+_\d+\.\d+)\s*\{\s*global:(.*?)\};", text, re.S):
+            for f in re.findall(r"(\w+);", body):
+                want[f] = node
+        out = subprocess.run(["nm", "-D", "--with-symbol-versions", os.path.join(root, "cv-cuda_amd", "lib", lib)],
+                             capture_output=True, text=True, check=True).stdout
+        have = dict(re.findall(r" T (\w+)@@(\w+\.\d+)", out))
+        assert len(want) > 20
+        for f, node in want.items():
+            assert have.get(f) == node, (f, node, have.get(f))
+    # spot values read from the reference's sources
+    assert "cvcudaResizeCropConvertReformatSubmit@@CVCUDA_0.10" in subprocess.run(
+        ["nm", "-D", "--with-symbol-versions", os.path.join(root, "cv-cuda_amd", "lib", "libcvcuda.so")],
+        capture_output=True, text=True).stdout
