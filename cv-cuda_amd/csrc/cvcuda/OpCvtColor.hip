@@ -1,4 +1,5 @@
-// Colour conversion: channel swizzles (BGR<->RGB, add/drop alpha) and YUV 4:2:0 -> RGB family.
+// Colour conversion: channel swizzles (BGR<->RGB, add/drop alpha) and YUV 4:2:0 -> RGB family; every other
+// supported code is forwarded to the per-pixel families of OpCvtColorPixel.hip.
 //
 // Arithmetic follows the reference: integer BT.601 limited-range conversion in 20-bit fixed point
 // (src/cvcuda/priv/legacy/cvt_color.cu:64-69, 618-638) with the 4:2:0 addressing of :514-565; swizzle
@@ -9,6 +10,7 @@
 // chroma load (U0 V0 U1 V1 serves all eight pixels), two 12- or 16-byte streaming stores. Consecutive
 // lanes touch consecutive addresses in all three streams, so every cache line is fetched and written
 // exactly once: 1.5 bytes in, 3 (4) bytes out per pixel.
+#include "CvtColorFamilies.hpp"
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
@@ -573,7 +575,32 @@ public:
             break;
         }
         default:
-            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Unsupported conversion code %d", (int)code);
+        {
+            if (out.N != in.N)
+            {
+                throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Shape mismatch -- input and output batch sizes differ");
+            }
+            ColorIO io = {};
+            io.src     = in.base;
+            io.dst     = out.base;
+            io.srcN    = in.strideN;
+            io.dstN    = out.strideN;
+            io.srcRow  = (int32_t)in.strideH;
+            io.dstRow  = (int32_t)out.strideH;
+            io.N       = in.N;
+            io.srcW    = in.W;
+            io.srcH    = in.H;
+            io.srcC    = in.C;
+            io.dstW    = out.W;
+            io.dstH    = out.H;
+            io.dstC    = out.C;
+            io.srcElem = in.elem;
+            io.dstElem = out.elem;
+            if (!RunPixelColorFamily(code, io, stream))
+            {
+                throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Unsupported conversion code %d", (int)code);
+            }
+        }
         }
     }
 
@@ -643,7 +670,22 @@ public:
             break;
         }
         default:
-            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Unsupported conversion code %d", (int)code);
+        {
+            ColorIO io = {};
+            io.N       = in.N;
+            io.srcC    = fi.channels;
+            io.dstC    = fo.channels;
+            io.srcElem = fi.elem;
+            io.dstElem = fo.elem;
+            io.srcList = in.data.buffer.varShapeStrided.imageList;
+            io.dstList = out.data.buffer.varShapeStrided.imageList;
+            io.srcHost = in.hostList;
+            io.dstHost = out.hostList;
+            if (!RunPixelColorFamily(code, io, stream))
+            {
+                throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Unsupported conversion code %d", (int)code);
+            }
+        }
         }
     }
 };

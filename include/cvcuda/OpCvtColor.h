@@ -2,10 +2,19 @@
  * Replaces: src/cvcuda/include/cvcuda/OpCvtColor.h:52, 70-75 (semantics of
  * src/cvcuda/priv/legacy/cvt_color.cu:181-230, 514-674, 1387-1517, 1768-2006).
  *
- * Codes implemented: channel swizzles BGR<->RGB, BGR(A)<->RGB(A), add/drop alpha (0..5) for
- * u8/u16/s32/f16/f32/f64 [N]HWC tensors; NV12/NV21 -> RGB/BGR/RGBA/BGRA (90..97) for u8, where the
- * input is a 1-channel tensor of height H*3/2 (luma rows followed by interleaved chroma rows) and
- * the arithmetic is BT.601 limited-range in 20-bit fixed point. Any other code -> INVALID_ARGUMENT. */
+ * Codes implemented (the set the reference implements, cvt_color.cu:1791-1995); tensors are [N]HWC:
+ *   0..5     channel swizzles BGR<->RGB, BGR(A)<->RGB(A), add/drop alpha: u8/s8/u16/s16/s32/f16/f32/f64
+ *   6, 7     BGR/RGB -> gray (u8, u16: 15-bit fixed point; f32), 8 gray -> BGR (any element size)
+ *   40, 41, 66, 67 BGR/RGB -> HSV and 54, 55, 70, 71 HSV -> BGR/RGB(A), half (180) or full (256) hue
+ *            range for u8, degrees for f32
+ *   82..85   BGR/RGB <-> YUV 4:4:4 (u8, u16: 14-bit fixed point; f32)
+ *   90..105  NV12 / NV21 / YV12 / I420 -> RGB/BGR(A), 106 -> gray: u8, the input is a 1-channel tensor
+ *            of height H*3/2 (luma rows, then chroma rows); BT.601 limited range, 20-bit fixed point
+ *   107, 108, 111, 112, 115..124 UYVY / YUY2 / YVYU -> RGB/BGR(A) or gray: u8, input 1-channel of width 2*W
+ *   127..134, 140..147 RGB/BGR(A) -> I420 / YV12 / NV12 / NV21: u8, chroma from the top-left pixel of
+ *            each 2x2 block
+ * Image batches (VarShapeSubmit) take every code whose input and output have equal sizes, and the
+ * 4:2:0 -> RGB codes. Any other code or combination -> INVALID_ARGUMENT. */
 #ifndef CVCUDA_CVTCOLOR_H
 #define CVCUDA_CVTCOLOR_H
 
