@@ -152,6 +152,99 @@ __device__ __forceinline__ void ResizePixel(const Plane &p, int dx, int dy)
             out.v[c] = SaturateCast<T>(v);
         }
     }
+    else if constexpr (INTERP == NVCV_INTERP_AREA)
+    {
+        // box filter over the source rectangle the output pixel covers, partial pixels weighted by
+        // their covered fraction; taps outside the image read 0 (reference:
+        // cuda_tools/InterpolationWrap.hpp:668-760, accumulation order kept)
+        const float fsx1 = dx * scaleX, fsy1 = dy * scaleY;
+        const float fsx2 = fsx1 + scaleX, fsy2 = fsy1 + scaleY;
+        const int   xmin = (int)ceilf(fsx1), xmax = (int)floorf(fsx2);
+        const int   ymin = (int)ceilf(fsy1), ymax = (int)floorf(fsy2);
+        float       sum[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            sum[c] = 0.f;
+        }
+        auto add = [&](int x, int y, float w)
+        {
+            if (x >= 0 && x < p.srcW && y >= 0 && y < p.srcH)
+            {
+                const Pixel<T, C> t = LoadPx<T, C>(p.src + (int64_t)y * p.srcRow, x);
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    sum[c] += (float)t.v[c] * w;
+                }
+            }
+        };
+        if (ceilf(scaleX) == scaleX && ceilf(scaleY) == scaleY)
+        {
+            const float scale = 1.f / (scaleX * scaleY);
+            for (int cy = ymin; cy < ymax; ++cy)
+            {
+                for (int cx = xmin; cx < xmax; ++cx)
+                {
+                    add(cx, cy, scale);
+                }
+            }
+        }
+        else
+        {
+            const float scale = 1.f / (fminf(scaleX, p.srcW - fsx1) * fminf(scaleY, p.srcH - fsy1));
+            for (int cy = ymin; cy < ymax; ++cy)
+            {
+                for (int cx = xmin; cx < xmax; ++cx)
+                {
+                    add(cx, cy, scale);
+                }
+                if (xmin > fsx1)
+                {
+                    add(xmin - 1, cy, (xmin - fsx1) * scale);
+                }
+                if (xmax < fsx2)
+                {
+                    add(xmax, cy, (fsx2 - xmax) * scale);
+                }
+            }
+            if (ymin > fsy1)
+            {
+                for (int cx = xmin; cx < xmax; ++cx)
+                {
+                    add(cx, ymin - 1, (ymin - fsy1) * scale);
+                }
+                if (xmin > fsx1)
+                {
+                    add(xmin - 1, ymin - 1, (ymin - fsy1) * (xmin - fsx1) * scale);
+                }
+                if (xmax < fsx2)
+                {
+                    add(xmax, ymin - 1, (ymin - fsy1) * (fsx2 - xmax) * scale);
+                }
+            }
+            if (ymax < fsy2)
+            {
+                for (int cx = xmin; cx < xmax; ++cx)
+                {
+                    add(cx, ymax, (fsy2 - ymax) * scale);
+                }
+                if (xmax < fsx2)
+                {
+                    add(xmax, ymax, (fsy2 - ymax) * (fsx2 - xmax) * scale);
+                }
+                if (xmin > fsx1)
+                {
+                    add(xmin - 1, ymax, (fsy2 - ymax) * (xmin - fsx1) * scale);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out.v[c] = SaturateCast<T>(sum[c]);
+        }
+    }
     else // cubic
     {
         const float cx = (dx + .5f) * scaleX - .5f;
@@ -280,8 +373,15 @@ void DispatchInterp(bool varshape, const ResizeArgs &a, const NVCVImageBufferStr
         varshape ? LaunchVarShape<T, C, NVCV_INTERP_CUBIC>(a, dstHost, N, stream)
                  : LaunchTensor<T, C, NVCV_INTERP_CUBIC>(a, N, stream);
         break;
+    case NVCV_INTERP_AREA:
+        if (varshape)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "AREA interpolation is available for tensors only");
+        }
+        LaunchTensor<T, C, NVCV_INTERP_AREA>(a, N, stream);
+        break;
     default:
-        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid interpolation (supported: NEAREST, LINEAR, CUBIC)");
+        throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid interpolation (supported: NEAREST, LINEAR, CUBIC, AREA)");
     }
 }
 

@@ -270,6 +270,98 @@ void FusedOne(const uint8_t *src, int64_t srcRowStride, int srcW, int srcH, DstT
 //                     weight rules, different association: linear (1-fx)*(a0*(1-fy)+b0*fy) +
 //                     fx*(a1*(1-fy)+b1*fy); cubic accumulates wy[row]*(row dot wx); abs as built
 //                     (the legacy-math switch is on).
+// ---- area resize, one output pixel ---------------------------------------------------------------
+// variant 0: golden tests/cvcuda/system/ResizeUtils.cpp:44-186 (tensor branch) in float64;
+// variant 1: device cuda_tools/InterpolationWrap.hpp:668-760 in float32 (taps outside the image read 0).
+template<class T>
+void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C, int dx, int dy, int dstW, int dstH,
+               int variant)
+{
+    auto at = [&](int x, int y, int c) -> double
+    { return (x < 0 || x >= srcW || y < 0 || y >= srcH) ? 0.0 : (double)src[y * srcStep + (int64_t)x * C + c]; };
+    if (variant == 0)
+    {
+        const double scaleH = static_cast<double>(srcH) / dstH, scaleW = static_cast<double>(srcW) / dstW;
+        const double fsx1 = dx * scaleW, fsx2 = fsx1 + scaleW, fsy1 = dy * scaleH, fsy2 = fsy1 + scaleH;
+        const int    sx1 = (int)std::ceil(fsx1), sx2 = (int)std::floor(fsx2);
+        const int    sy1 = (int)std::ceil(fsy1), sy2 = (int)std::floor(fsy2);
+        const double lo = (double)std::numeric_limits<T>::lowest(), hi = (double)std::numeric_limits<T>::max();
+        for (int c = 0; c < C; ++c)
+        {
+            double o = 0.0;
+            if (std::ceil(scaleW) == scaleW && std::ceil(scaleH) == scaleH)
+            {
+                const double inv = 1.f / (scaleW * scaleH);
+                for (int y = sy1; y < sy2; ++y)
+                    for (int x = sx1; x < sx2; ++x) o = o + at(x, y, c) * inv;
+            }
+            else
+            {
+                const double inv = 1.f / (std::min(scaleW, srcW - fsx1) * std::min(scaleH, srcH - fsy1));
+                for (int y = sy1; y < sy2; ++y)
+                {
+                    for (int x = sx1; x < sx2; ++x) o = o + at(x, y, c) * inv;
+                    if (sx1 > fsx1) o = o + at(sx1 - 1, y, c) * ((sx1 - fsx1) * inv);
+                    if (sx2 < fsx2) o = o + at(sx2, y, c) * ((fsx2 - sx2) * inv);
+                }
+                if (sy1 > fsy1)
+                    for (int x = sx1; x < sx2; ++x) o = o + at(x, sy1 - 1, c) * ((sy1 - fsy1) * inv);
+                if (sy2 < fsy2)
+                    for (int x = sx1; x < sx2; ++x) o = o + at(x, sy2, c) * ((fsy2 - sy2) * inv);
+                if (sy1 > fsy1 && sx1 > fsx1) o = o + at(sx1 - 1, sy1 - 1, c) * ((sy1 - fsy1) * (sx1 - fsx1) * inv);
+                if (sy1 > fsy1 && sx2 < fsx2) o = o + at(sx2, sy1 - 1, c) * ((sy1 - fsy1) * (fsx2 - sx2) * inv);
+                if (sy2 < fsy2 && sx2 < fsx2) o = o + at(sx2, sy2, c) * ((fsy2 - sy2) * (fsx2 - sx2) * inv);
+                if (sy2 < fsy2 && sx1 > fsx1) o = o + at(sx1 - 1, sy2, c) * ((fsy2 - sy2) * (sx1 - fsx1) * inv);
+            }
+            if (std::numeric_limits<T>::is_integer)
+            {
+                o = std::rint(std::numeric_limits<T>::is_signed ? o : std::abs(o));
+            }
+            out[c] = (T)(o < lo ? lo : (o > hi ? hi : o));
+        }
+        return;
+    }
+    const float scaleX = static_cast<float>(srcW) / dstW, scaleY = static_cast<float>(srcH) / dstH;
+    const float fsx1 = dx * scaleX, fsy1 = dy * scaleY, fsx2 = fsx1 + scaleX, fsy2 = fsy1 + scaleY;
+    const int   xmin = (int)std::ceil(fsx1), xmax = (int)std::floor(fsx2);
+    const int   ymin = (int)std::ceil(fsy1), ymax = (int)std::floor(fsy2);
+    const bool  integerArea = std::ceil(scaleX) == scaleX && std::ceil(scaleY) == scaleY;
+    for (int c = 0; c < C; ++c)
+    {
+        auto  v = [&](int x, int y) -> float { return (float)at(x, y, c); };
+        float o = 0.f;
+        if (integerArea)
+        {
+            const float scale = 1.f / (scaleX * scaleY);
+            for (int cy = ymin; cy < ymax; ++cy)
+                for (int cx = xmin; cx < xmax; ++cx) o += v(cx, cy) * scale;
+        }
+        else
+        {
+            const float scale = 1.f / (std::min(scaleX, srcW - fsx1) * std::min(scaleY, srcH - fsy1));
+            for (int cy = ymin; cy < ymax; ++cy)
+            {
+                for (int cx = xmin; cx < xmax; ++cx) o += v(cx, cy) * scale;
+                if (xmin > fsx1) o += v(xmin - 1, cy) * ((xmin - fsx1) * scale);
+                if (xmax < fsx2) o += v(xmax, cy) * ((fsx2 - xmax) * scale);
+            }
+            if (ymin > fsy1)
+            {
+                for (int cx = xmin; cx < xmax; ++cx) o += v(cx, ymin - 1) * ((ymin - fsy1) * scale);
+                if (xmin > fsx1) o += v(xmin - 1, ymin - 1) * ((ymin - fsy1) * (xmin - fsx1) * scale);
+                if (xmax < fsx2) o += v(xmax, ymin - 1) * ((ymin - fsy1) * (fsx2 - xmax) * scale);
+            }
+            if (ymax < fsy2)
+            {
+                for (int cx = xmin; cx < xmax; ++cx) o += v(cx, ymax) * ((fsy2 - ymax) * scale);
+                if (xmax < fsx2) o += v(xmax, ymax) * ((fsy2 - ymax) * (fsx2 - xmax) * scale);
+                if (xmin > fsx1) o += v(xmin - 1, ymax) * ((fsy2 - ymax) * (xmin - fsx1) * scale);
+            }
+        }
+        out[c] = SatF<T>(o);
+    }
+}
+
 template<class T>
 void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_t dstStep, int dstW, int dstH, int C,
                int interp, int variant)
@@ -438,6 +530,10 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                     }
                     out[c] = SatF<T>(std::abs(sum));
                 }
+            }
+            else if (interp == 3)
+            {
+                AreaPixel<T>(src, srcStep, srcW, srcH, out, C, dx, dy, dstW, dstH, variant);
             }
         }
     }
@@ -782,7 +878,7 @@ ORC_API int orc_resize(const void *src, int64_t srcStep, int64_t srcImgStep, int
                        int64_t dstStep, int64_t dstImgStep, int dstW, int dstH, int C, int dtype, int interp,
                        int variant, int threads)
 {
-    if (interp < 0 || interp > 2)
+    if (interp < 0 || interp > 3)
     {
         return -1;
     }

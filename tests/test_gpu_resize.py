@@ -1,6 +1,6 @@
 """GPU parity of cvcudaResize[VarShape]Submit against the CPU oracle.
 
-Rows are the reference's own table (tests/cvcuda/system/TestOpResize.cpp:49-91, the AREA rows excepted)
+Rows are the reference's own table (tests/cvcuda/system/TestOpResize.cpp:49-91)
 with seeded random inputs, plus the two benchmark configurations at full size.
 Bars: NEAREST bit-exact vs the golden; LINEAR/CUBIC on integer types <= 1 LSB vs the golden (the
 reference's own tolerance) and bit-exact vs the float32 device-formula restatement; f32 cubic
@@ -154,6 +154,33 @@ def test_varshape(cv, K, orc, gpu, interp, dt, c):
         w, h = o.size
         res = o.plane_view(0, dt, c).cpu().numpy()[None]
         check(res, a[None], (h, w), interp, orc, varshape=True)
+
+
+AREA = 3
+AREA_ROWS = [(44, 40, 22, 20, 2, np.uint8, 4), (30, 30, 20, 20, 2, np.uint8, 4), (30, 30, 60, 60, 4, np.uint8, 4),
+             (1440, 2560, 1080, 1920, 1, np.uint8, 4), (720, 1280, 360, 640, 1, np.uint8, 4),
+             (1440, 2560, 720, 1280, 1, np.uint8, 4), (1920, 1080, 224, 224, 2, np.uint8, 3),
+             (97, 61, 13, 9, 2, np.uint16, 1), (97, 61, 13, 9, 2, np.int16, 3), (97, 61, 40, 33, 2, np.float32, 4)]
+
+
+@pytest.mark.parametrize("row", AREA_ROWS, ids=lambda r: "%dx%d-%dx%d-n%d-%s%d" % (r[:5] + (np.dtype(r[5]).name, r[6])))
+def test_area_tensor(cv, orc, gpu, row):
+    # box-filter resize, tensors (reference rows TestOpResize.cpp:67-78 plus other types and the
+    # 1080p -> 224 case): <= 1 LSB against the float64 golden, and against the float32 device-order
+    # restatement within float rounding of the long sums
+    sw, sh, dw, dh, n, dt, c = row
+    src = make_input(orc, (n, sh, sw, c), dt, 0xA0EA + sw + dh)
+    tout = cv.Tensor.alloc([n, dh, dw, c], dt, "NHWC")
+    cv.Resize()(None, cv.Tensor.from_numpy(src, "NHWC"), tout, AREA)
+    torch.cuda.synchronize()
+    res = tout.numpy()
+    golden = orc.resize(src, (dh, dw), AREA, variant=0, threads=8)
+    device = orc.resize(src, (dh, dw), AREA, variant=1, threads=8)
+    if dt == np.float32:
+        assert np.abs(res - device).max() <= 1e-5 and np.abs(res - golden).max() <= 1e-4
+    else:
+        assert np.abs(res.astype(np.int64) - golden.astype(np.int64)).max() <= 1
+        np.testing.assert_array_equal(res, device)
 
 
 def test_negative_cases(cv, gpu):

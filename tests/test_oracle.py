@@ -375,3 +375,27 @@ def test_crop_flip_normalize_closed_forms(orc):
     np.testing.assert_array_equal(r, (x - base) * mul * np.float32(1.0) + np.float32(0.0))
     r8 = orc.crop_flip_normalize(a, (12, 20), np.int8, (4, 2, 20, 12), 2, 0, 0.0, [128], [1])
     np.testing.assert_array_equal(r8, np.clip(a[2:14, 4:24].astype(np.int32) - 128, -128, 127))
+
+
+def test_resize_area_closed_forms(orc):
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, (1, 24, 36, 3), dtype=np.uint8)
+    # integer factors: the plain block mean
+    for fy, fx in ((2, 2), (3, 4), (1, 6)):
+        ref = a.reshape(1, 24 // fy, fy, 36 // fx, fx, 3).astype(np.float64).mean(axis=(2, 4))
+        for variant in (0, 1):
+            r = orc.resize(a, (24 // fy, 36 // fx), 3, variant=variant)
+            assert np.abs(r - ref).max() <= 0.5 + 1e-4
+    # same size: identity; constant image: constant (weights sum to the covered area)
+    for variant in (0, 1):
+        np.testing.assert_array_equal(orc.resize(a, (24, 36), 3, variant=variant), a)
+        k = np.full((1, 31, 47, 1), 200, np.uint8)
+        r = orc.resize(k, (13, 10), 3, variant=variant)
+        assert np.abs(r.astype(int) - 200).max() <= 1
+    # fractional factor: exact area-weighted mean computed by brute force on a 60x finer grid
+    f = rng.random((1, 7, 9, 1)).astype(np.float32)
+    fine = np.repeat(np.repeat(f, 60, axis=1), 60, axis=2)  # 420 x 540
+    ref = fine.reshape(1, 5, 84, 6, 90, 1).mean(axis=(2, 4))  # 7 -> 5 rows, 9 -> 6 columns
+    for variant in (0, 1):
+        r = orc.resize(f, (5, 6), 3, variant=variant)
+        assert np.abs(r - ref).max() < 1e-5
