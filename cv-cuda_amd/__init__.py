@@ -155,6 +155,39 @@ class Tensor(_Handle):
         return cls.wrap(t.data_ptr(), list(t.shape), [s * es for s in t.stride()], npdt, layout, keep=t)
 
     @classmethod
+    def from_cuda_array_interface(cls, obj, layout):
+        """Zero-copy view of any object exposing __cuda_array_interface__ (version 2 or 3: CuPy, Numba,
+        PyTorch, decoder surfaces ...). The reference offers the same through its external-buffer
+        wrapper (python/mod_nvcv/ExternalBuffer.cpp); on ROCm the protocol carries HIP device pointers."""
+        iface = obj.__cuda_array_interface__
+        npdt = np.dtype(iface["typestr"])
+        shape = list(iface["shape"])
+        strides = iface.get("strides")
+        if strides is None:
+            strides, acc = [], npdt.itemsize
+            for s_ in reversed(shape):
+                strides.insert(0, acc)
+                acc *= s_
+        return cls.wrap(iface["data"][0], shape, list(strides), npdt, layout, keep=obj)
+
+    @classmethod
+    def from_dlpack(cls, obj, layout):
+        """Zero-copy view of a DLPack capsule / producer living on this GPU (via torch.utils.dlpack)."""
+        return cls.from_torch(torch.utils.dlpack.from_dlpack(obj), layout)
+
+    def to_dlpack(self):
+        """DLPack capsule over the tensor's memory; the consumer must not outlive this tensor."""
+        return torch.utils.dlpack.to_dlpack(self.torch_view())
+
+    @property
+    def __cuda_array_interface__(self):
+        d = self.export()
+        npdt = _DT2NP[d.dtype]
+        return {"shape": tuple(d.shape[i] for i in range(d.rank)), "typestr": npdt.str,
+                "data": (int(d.buffer.basePtr or 0), False),
+                "strides": tuple(d.buffer.strides[i] for i in range(d.rank)), "version": 3}
+
+    @classmethod
     def from_numpy(cls, a, layout, row_align=0):
         """Uploads a dense host array into a freshly allocated (pitched) tensor."""
         a = np.ascontiguousarray(a)

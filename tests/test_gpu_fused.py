@@ -227,3 +227,32 @@ def test_normalize_extension_varshape_plain_scale_and_errors(cv, K, orc, gpu):
         op.handle, cv.stream_ptr(None), batch.handle, out.handle, cv.capi.Size2D(64, 40), 1, cv.capi.Int2(8, 4), 0, 1.0,
         0.0, False, None)
     assert st == 2
+
+
+def test_zero_copy_interop_torch_dlpack_cuda_array_interface(cv, orc, gpu):
+    # the pipeline edge: a PyTorch-ROCm tensor in, an NCHW f32 torch tensor out, no copies on either side
+    src = orc.fill_u8((2, 135, 240, 3), 31)
+    t_in = torch.from_numpy(src).cuda()
+    t_out = torch.empty((2, 3, 56, 56), dtype=torch.float32, device="cuda")
+    op = cv.ResizeCropConvertReformat()
+    ref = orc.fused_rccr(src, (56, 56), (114, 64), (29, 4), 1, np.float32, True, 0, 1 / 255.0, 0.0, False)
+    for wrap_in, wrap_out in [(cv.Tensor.from_torch(t_in, "NHWC"), cv.Tensor.from_torch(t_out, "NCHW")),
+                              (cv.Tensor.from_dlpack(torch.utils.dlpack.to_dlpack(t_in), "NHWC"),
+                               cv.Tensor.from_dlpack(t_out, "NCHW")),
+                              (cv.Tensor.from_cuda_array_interface(t_in, "NHWC"),
+                               cv.Tensor.from_cuda_array_interface(t_out, "NCHW"))]:
+        t_out.zero_()
+        op(None, wrap_in, wrap_out, (114, 64), 1, (29, 4), 0, 1 / 255.0, 0.0, False)
+        torch.cuda.synchronize()
+        got = t_out.cpu().numpy()
+        assert (np.abs(got - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all()
+        assert wrap_out.export().buffer.basePtr == t_out.data_ptr()
+    # and outwards: a library-allocated (pitched) tensor seen by torch through both protocols
+    own = cv.Tensor.alloc([2, 56, 56, 3], np.float32, "NHWC")
+    op(None, cv.Tensor.from_torch(t_in, "NHWC"), own, (114, 64), 1, (29, 4), 0, 1 / 255.0, 0.0, False)
+    torch.cuda.synchronize()
+    via_dlpack = torch.utils.dlpack.from_dlpack(own.to_dlpack())
+    via_cai = torch.as_tensor(own, device="cuda")
+    for view in (via_dlpack, via_cai):
+        assert view.data_ptr() == own.export().buffer.basePtr
+        assert np.abs(view.cpu().numpy().transpose(0, 3, 1, 2) - ref).max() <= 1e-5 * np.abs(ref).max()
