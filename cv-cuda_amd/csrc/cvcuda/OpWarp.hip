@@ -1,7 +1,8 @@
 // WarpAffine and WarpPerspective, tensors and var-shape batches.
 //
 // Coordinates, sampling and border handling follow the reference in float32 without FMA
-// contraction: destination->source map src/cvcuda/priv/legacy/CvCudaLegacy.h:143-183, matrix
+// contraction (the bilinear sum in the association of the reference's golden, tap * (wx * wy),
+// tests/cvcuda/system/TestOpWarpAffine.cpp:159-170, so integer results equal the golden's bit for bit): destination->source map src/cvcuda/priv/legacy/CvCudaLegacy.h:143-183, matrix
 // inversion warp.cu:139-150 (affine) and cuda_tools/math/LinAlg.hpp:1446-1450, 1640-1654 (3x3),
 // samplers cuda_tools/InterpolationWrap.hpp:83-104, 332-339, 429-447, 535-565, border index maps
 // cuda_tools/BorderWrap.hpp:62-121. Validation follows warp.cu:152-232 and warp_var_shape.cu:194-299.
@@ -252,10 +253,11 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
             Fetch<T, C>(im, a, x1 + (i & 1), y1 + (i >> 1), t);
             const float wx = (i & 1) ? (sx - x1) : (x2 - sx);
             const float wy = (i >> 1) ? (sy - y1) : (y2 - sy);
+            const float w  = wx * wy;
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
-                acc[c] += t[c] * wx * wy;
+                acc[c] += t[c] * w;
             }
         }
     }
@@ -339,13 +341,14 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
         float          t[4][C];
         LoadPairInside<T, C>(p, t[0], t[1]);
         LoadPairInside<T, C>(p + (uint32_t)im.row, t[2], t[3]);
+        const float w00 = wx0 * wy0, w01 = wx1 * wy0, w10 = wx0 * wy1, w11 = wx1 * wy1;
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
-            float v = t[0][c] * wx0 * wy0;
-            v += t[1][c] * wx1 * wy0;
-            v += t[2][c] * wx0 * wy1;
-            v += t[3][c] * wx1 * wy1;
+            float v = t[0][c] * w00;
+            v += t[1][c] * w01;
+            v += t[2][c] * w10;
+            v += t[3][c] * w11;
             acc[c] = v;
         }
     }

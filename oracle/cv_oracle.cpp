@@ -752,6 +752,8 @@ void WarpOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_t 
                     }
                     else
                     {
+                        // the reference's device expression, tap * wx * wy (InterpolationWrap.hpp:429-447);
+                        // kept for comparison: the product library follows the golden's association above
                         o += (float)pix(y1, x1, k) * (x2 - sx) * (y2 - sy);
                         o += (float)pix(y1, x2, k) * (sx - x1) * (y2 - sy);
                         o += (float)pix(y2, x1, k) * (x2 - sx) * (sy - y1);
