@@ -509,60 +509,57 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     }
 }
 
-// Inverts one caller-supplied forward matrix (uniform per block).
+// Loads image `image`'s matrix from the caller's tensor and, unless it already maps destination to
+// source, inverts it (uniform per block). Straight-line selects instead of early exits: every m[i] is
+// assigned exactly once, which keeps the matrix in registers.
 __device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (&m)[9])
 {
     const float *p = reinterpret_cast<const float *>(a.xforms + image * a.xformStride);
-    const int    n = a.perspective ? 9 : 6;
+    const bool   persp = a.perspective != 0;
     float        f[9];
+#pragma unroll
+    for (int i = 0; i < 6; ++i)
+    {
+        f[i] = p[i];
+    }
+#pragma unroll
+    for (int i = 6; i < 9; ++i)
+    {
+        f[i] = persp ? p[i] : 0.f;
+    }
+    float r[9];
+    // affine inverse (reference: warp.cu:139-150, 1/det evaluated in double)
+    float den = f[0] * f[4] - f[1] * f[3];
+    den       = fabsf(den) > 1e-5 ? (float)(1. / (double)den) : 0.f;
+    r[0]      = f[4] * den;
+    r[1]      = -f[1] * den;
+    r[2]      = (f[1] * f[5] - f[4] * f[2]) * den;
+    r[3]      = -f[3] * den;
+    r[4]      = f[0] * den;
+    r[5]      = (f[3] * f[2] - f[0] * f[5]) * den;
+    r[6] = r[7] = r[8] = 0.f;
+    if (persp)
+    {
+        // 3x3 inverse by cofactors (reference: cuda_tools/math/LinAlg.hpp:1446-1450, 1640-1654); a singular
+        // matrix is left as given, like the reference's failed in-place inverse
+        const float d = f[0] * (f[4] * f[8] - f[5] * f[7]) + f[1] * (f[5] * f[6] - f[3] * f[8])
+                      + f[2] * (f[3] * f[7] - f[4] * f[6]);
+        const bool  ok = d != 0;
+        r[0]           = ok ? (f[4] * f[8] - f[5] * f[7]) / d : f[0];
+        r[1]           = ok ? -(f[1] * f[8] - f[2] * f[7]) / d : f[1];
+        r[2]           = ok ? (f[1] * f[5] - f[2] * f[4]) / d : f[2];
+        r[3]           = ok ? -(f[3] * f[8] - f[5] * f[6]) / d : f[3];
+        r[4]           = ok ? (f[0] * f[8] - f[2] * f[6]) / d : f[4];
+        r[5]           = ok ? -(f[0] * f[5] - f[2] * f[3]) / d : f[5];
+        r[6]           = ok ? (f[3] * f[7] - f[4] * f[6]) / d : f[6];
+        r[7]           = ok ? -(f[0] * f[7] - f[1] * f[6]) / d : f[7];
+        r[8]           = ok ? (f[0] * f[4] - f[1] * f[3]) / d : f[8];
+    }
+    const bool given = a.inverseGiven != 0;
 #pragma unroll
     for (int i = 0; i < 9; ++i)
     {
-        f[i] = i < n ? p[i] : 0.f;
-    }
-    if (a.inverseGiven)
-    {
-#pragma unroll
-        for (int i = 0; i < 9; ++i)
-        {
-            m[i] = f[i];
-        }
-        return;
-    }
-    if (!a.perspective)
-    {
-        float den = f[0] * f[4] - f[1] * f[3];
-        den       = fabsf(den) > 1e-5 ? (float)(1. / (double)den) : 0.f;
-        m[0]      = f[4] * den;
-        m[1]      = -f[1] * den;
-        m[2]      = (f[1] * f[5] - f[4] * f[2]) * den;
-        m[3]      = -f[3] * den;
-        m[4]      = f[0] * den;
-        m[5]      = (f[3] * f[2] - f[0] * f[5]) * den;
-        m[6] = m[7] = m[8] = 0.f;
-    }
-    else
-    {
-        const float d = f[0] * (f[4] * f[8] - f[5] * f[7]) + f[1] * (f[5] * f[6] - f[3] * f[8])
-                      + f[2] * (f[3] * f[7] - f[4] * f[6]);
-        if (d == 0)
-        {
-#pragma unroll
-            for (int i = 0; i < 9; ++i)
-            {
-                m[i] = f[i]; // singular: left as given, like the reference's failed in-place inverse
-            }
-            return;
-        }
-        m[0] = (f[4] * f[8] - f[5] * f[7]) / d;
-        m[1] = -(f[1] * f[8] - f[2] * f[7]) / d;
-        m[2] = (f[1] * f[5] - f[2] * f[4]) / d;
-        m[3] = -(f[3] * f[8] - f[5] * f[6]) / d;
-        m[4] = (f[0] * f[8] - f[2] * f[6]) / d;
-        m[5] = -(f[0] * f[5] - f[2] * f[3]) / d;
-        m[6] = (f[3] * f[7] - f[4] * f[6]) / d;
-        m[7] = -(f[0] * f[7] - f[1] * f[6]) / d;
-        m[8] = (f[0] * f[4] - f[1] * f[3]) / d;
+        m[i] = given ? f[i] : r[i];
     }
 }
 
