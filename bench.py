@@ -26,11 +26,12 @@ HBM_PEAK_GBS = 8000.0
 SEED_BASE = 0xC0FFEE00
 NEAREST, LINEAR, CUBIC = 0, 1, 2
 
-# HBM bytes one launch of the headline kernel moves, from hardware counters (rocprofv3 --pmc
+# HBM bytes one launch of a workload's kernel moves, from hardware counters (rocprofv3 --pmc
 # FETCH_SIZE and --pmc WRITE_SIZE in separate runs, each scaled by what the same counter reads for a
 # 128 MiB device copy: x1.99965 and x1.00000). It is a property of the kernel and the workload, not
-# of a run, so it is recorded here rather than re-measured: 84,436,703 read + 38,535,168 written.
-MEASURED_TRAFFIC_BYTES = {"fused": 122971871}
+# of a run, so it is recorded here rather than re-measured. fused: 84,436,703 read + 38,535,168
+# written; resize-cubic-4k: 1,415,442,526 read + 58,982,400 written.
+MEASURED_TRAFFIC_BYTES = {"fused": 122971871, "resize-cubic-4k": 1474424926}
 
 
 def span_bytes(n_out, crop, src, new, interp, pixel_bytes):
@@ -171,7 +172,7 @@ class ResizeC1:
 class CubicC5:
     key, config_id = "resize-cubic-4k", 5
     N, SRC_H, SRC_W, OUT_H, OUT_W = 16, 2160, 3840, 360, 640
-    kernel = "ResizeTensorKernel<float,4,CUBIC>"
+    kernel = "ResizeCubicStagedKernel<float,4>"
     dtype = "f32"
     workload = "Resize CUBIC: batch 16 f32 NHWC 3840x2160x4 -> 640x360x4"
 

@@ -332,10 +332,151 @@ __global__ __launch_bounds__(256) void ResizeVarShapeKernel(const ResizeArgs a, 
     ResizePixel<T, C, INTERP, true>(p, dx, dy);
 }
 
+// Bicubic for strong horizontal reductions. With one lane per output pixel the four taps of
+// neighbouring lanes lie scale*pixel bytes apart, so each of a wave's tap loads touches 64 separate
+// cache lines. Here the same 256 taps of a wave's row are fetched tap-major instead: lane l loads
+// tap l%4 of pixel 16k + l/4 (k = 0..3), four lanes covering 4 contiguous pixels, and the wave
+// hands the taps to their owners through LDS. Arithmetic and its order are those of ResizePixel.
+template<int BYTES>
+struct alignas(BYTES % 16 == 0 ? 16 : (BYTES % 8 == 0 ? 8 : 4)) LdsSlot
+{
+    uint32_t w[BYTES / 4];
+};
+
+// Orders a wave's LDS writes before its later LDS reads (and the reverse) where lanes of the same
+// wave exchange data: LDS instructions of one wave execute in order, so only the compiler has to
+// be kept from moving them.
+__device__ __forceinline__ void WaveExchangeFence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ __forceinline__ void CubicSourceX(int srcW, float scaleX, int dx, int &sx, float &fx)
+{
+    const float cx = (dx + .5f) * scaleX - .5f;
+    sx             = (int)floorf(cx);
+    fx             = cx - sx;
+    fx             = (sx < 1 || sx >= srcW - 3) ? 0.f : fx;
+    sx             = max(1, min(sx, srcW - 3));
+}
+
+template<class T, int C>
+__global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs a)
+{
+    using Px   = Pixel<T, C>;
+    using Slot = LdsSlot<sizeof(Px)>;
+    static_assert(sizeof(Px) % 4 == 0, "pixels are staged as whole dwords");
+    __shared__ Slot stage[kTileH][kTileW * 4];
+
+    const int   lane = threadIdx.x & 63;
+    const int   wave = threadIdx.x >> 6;
+    const Plane p    = GetPlanes<false>(a, blockIdx.z);
+    const int   dx   = blockIdx.x * kTileW + lane;
+    const int   dy   = blockIdx.y * kTileH + wave;
+
+    const float scaleX = static_cast<float>(p.srcW) / p.dstW;
+    const float scaleY = static_cast<float>(p.srcH) / p.dstH;
+
+    // lanes and rows past the output compute a duplicate of the last pixel and skip the store: every
+    // lane takes part in its wave's exchange (each wave owns one quarter of the staging array)
+    int   sx;
+    float fx;
+    CubicSourceX(p.srcW, scaleX, min(dx, p.dstW - 1), sx, fx);
+    const float cy = (min(dy, p.dstH - 1) + .5f) * scaleY - .5f;
+    int         sy = (int)floorf(cy);
+    const float fy = cy - sy;
+    sy             = max(1, min(sy, p.srcH - 3));
+    float wx[4], wy[4];
+    CubicCoeffs(fx, wx);
+    CubicCoeffs(fy, wy);
+
+    // loader role: column of the tap this lane fetches in each of the four instructions
+    int tapX[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        int   qsx;
+        float qfx;
+        CubicSourceX(p.srcW, scaleX, min(blockIdx.x * kTileW + 16 * k + (lane >> 2), p.dstW - 1), qsx, qfx);
+        tapX[k] = max(0, min(qsx - 1 + (lane & 3), p.srcW - 1));
+    }
+
+    Px   v[4];
+    auto loadRow = [&](int j)
+    {
+        const int      yy  = max(0, min(sy - 1 + j, p.srcH - 1));
+        const uint8_t *row = p.src + (int64_t)yy * p.srcRow;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            v[k] = LoadPx<T, C>(row, tapX[k]);
+        }
+    };
+
+    float sum[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        sum[c] = 0.f;
+    }
+    loadRow(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            __builtin_memcpy(&stage[wave][64 * k + lane], &v[k], sizeof(Px));
+        }
+        WaveExchangeFence();
+        if (j < 3)
+        {
+            loadRow(j + 1); // in flight while this row is summed
+        }
+        Px t[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            __builtin_memcpy(&t[i], &stage[wave][4 * lane + i], sizeof(Px));
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                sum[c] += (float)t[i].v[c] * (wx[i] * wy[j]);
+            }
+        }
+        WaveExchangeFence();
+    }
+    if (dx < p.dstW && dy < p.dstH)
+    {
+        Px out;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out.v[c] = SaturateCast<T>(fabsf(sum[c]));
+        }
+        StorePx<T, C>(p.dst + (int64_t)dy * p.dstRow, dx, out);
+    }
+}
+
 template<class T, int C, int INTERP>
 void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
 {
     dim3 grid(DivUp(a.dstW, kTileW), DivUp(a.dstH, kTileH), N);
+    if constexpr (INTERP == NVCV_INTERP_CUBIC && sizeof(Pixel<T, C>) % 4 == 0)
+    {
+        if (a.srcW >= 2 * a.dstW)
+        {
+            hipLaunchKernelGGL((ResizeCubicStagedKernel<T, C>), grid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeCubicStagedKernel");
+            return;
+        }
+    }
     hipLaunchKernelGGL((ResizeTensorKernel<T, C, INTERP>), grid, dim3(256), 0, stream, a);
     CheckLaunch("ResizeTensorKernel");
 }
