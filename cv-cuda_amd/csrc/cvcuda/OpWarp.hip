@@ -140,9 +140,9 @@ __device__ __forceinline__ int FloorToInt(float v)
     return (int)fminf(fmaxf(floorf(v), -1073741824.f), 1073741824.f);
 }
 
-// u8x3 taps are fetched with loads wider than the taps (4 bytes for one pixel, 8 for two), which
-// read 1-2 bytes past them. Inside the image that is harmless; the one tap after which the image
-// ends (last pixel of the last row) is kept off this path by TapsInside.
+// u8x3 taps are fetched through aligned dword windows (8 bytes for one pixel, 12 for two), which
+// read up to 6 bytes = 2 pixels past them. Inside the image that is harmless; taps within 2 pixels
+// of the end of the last row, after which the image ends, are kept off this path by TapsInside.
 template<class T, int C>
 constexpr bool kWideTapLoads = std::is_same_v<T, uint8_t> && C == 3;
 
@@ -174,7 +174,7 @@ __device__ __forceinline__ void LoadPairInside(const uint8_t *p, float (&p0)[C],
 {
     if constexpr (kWideTapLoads<T, C>)
     {
-        const uint64_t q  = LoadU64Unaligned(p);
+        const uint64_t q  = LoadU64Window(p);
         const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
         p0[0] = (float)(lo & 0xFF);
         p0[1] = (float)((lo >> 8) & 0xFF);
@@ -296,7 +296,7 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
 }
 
 // True when every tap of the sample at (sx, sy) lies inside the image (and, with WIDE loads, none of
-// them is the very last pixel of the image). Decided on the float coordinates: for an integer k,
+// them is among the last three pixels of the image's last row). Decided on the float coordinates: for an integer k,
 // floor(v) >= k <=> v >= k and floor(v) < k <=> v < k; a NaN coordinate fails every comparison.
 template<int INTERP, bool WIDE>
 __device__ __forceinline__ bool TapsInside(float wf, float hf, float sx, float sy)
@@ -313,7 +313,7 @@ __device__ __forceinline__ bool TapsInside(float wf, float hf, float sx, float s
     bool in = (sx >= lo) & (sy >= lo) & (sx < wf - hi) & (sy < hf - hi);
     if constexpr (WIDE)
     {
-        in = in & ((sx < wf - hi - 1.f) | (sy < hf - hi - 1.f));
+        in = in & ((sx < wf - hi - 2.f) | (sy < hf - hi - 1.f));
     }
     return in;
 }
