@@ -17,6 +17,7 @@
 #include <cvcuda/OpResize.h>
 
 #include <algorithm>
+#include <type_traits>
 
 namespace cvamd {
 
@@ -104,11 +105,10 @@ __device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
 }
 
 template<class T, int C, int INTERP, bool VARSHAPE>
-__device__ __forceinline__ void ResizePixel(const Plane &p, int dx, int dy)
+__device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int dy)
 {
     const float scaleX = static_cast<float>(p.srcW) / p.dstW;
     const float scaleY = static_cast<float>(p.srcH) / p.dstH;
-    uint8_t    *dstRow = p.dst + (int64_t)dy * p.dstRow;
     Pixel<T, C> out;
 
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
@@ -302,7 +302,13 @@ __device__ __forceinline__ void ResizePixel(const Plane &p, int dx, int dy)
             out.v[c] = SaturateCast<T>(fabsf(sum[c]));
         }
     }
-    StorePx<T, C>(dstRow, dx, out);
+    return out;
+}
+
+template<class T, int C, int INTERP, bool VARSHAPE>
+__device__ __forceinline__ void ResizePixel(const Plane &p, int dx, int dy)
+{
+    StorePx<T, C>(p.dst + (int64_t)dy * p.dstRow, dx, ResizeValue<T, C, INTERP, VARSHAPE>(p, dx, dy));
 }
 
 template<class T, int C, int INTERP>
@@ -330,6 +336,331 @@ __global__ __launch_bounds__(256) void ResizeVarShapeKernel(const ResizeArgs a, 
         return;
     }
     ResizePixel<T, C, INTERP, true>(p, dx, dy);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wave-patch form for small pixels. The per-pixel form above issues one load per tap and one store
+// per channel (8 tap loads and 3 byte stores per u8x3 bilinear pixel) and is bound by the number of
+// memory instructions, not by bytes or arithmetic. Here the horizontally adjacent taps of a sample
+// (2 for bilinear, 4 for bicubic) come from one load, and lanes exchange results so that each
+// stores 4 consecutive pixels as whole dwords. Arithmetic: the expressions of ResizeValue, term for
+// term.
+
+// N horizontally adjacent pixels at byte offset `off` of the source plane (all inside the image).
+// u8x3: 1 or 2 pixels are fetched with a 4- or 8-byte load that reads 1-2 bytes past them; where
+// that would cross the end of the plane (`planeBytes`) the load is moved back and the value shifted.
+template<class T, int C, int N>
+__device__ __forceinline__ void LoadTaps(const uint8_t *plane, int64_t off, int64_t planeBytes, float (&t)[N][C])
+{
+    if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 1)
+    {
+        const int      back = (int)max((int64_t)0, off - (planeBytes - 4));
+        const uint32_t q    = LoadU32Unaligned(plane + off - back) >> (8 * back);
+        t[0][0]             = (float)(q & 0xFF);
+        t[0][1]             = (float)((q >> 8) & 0xFF);
+        t[0][2]             = (float)((q >> 16) & 0xFF);
+    }
+    else if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 2)
+    {
+        const int      back = (int)max((int64_t)0, off - (planeBytes - 8));
+        const uint64_t q    = LoadU64Unaligned(plane + off - back) >> (8 * back);
+        const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
+        t[0][0] = (float)(lo & 0xFF);
+        t[0][1] = (float)((lo >> 8) & 0xFF);
+        t[0][2] = (float)((lo >> 16) & 0xFF);
+        t[1][0] = (float)(lo >> 24);
+        t[1][1] = (float)(hi & 0xFF);
+        t[1][2] = (float)((hi >> 8) & 0xFF);
+    }
+    else
+    {
+        const Pixel<T, N *C> v = *reinterpret_cast<const Pixel<T, N * C> *>(plane + off);
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                t[i][c] = (float)v.v[i * C + c];
+            }
+        }
+    }
+}
+
+// Requires srcW >= 4 (every tap group then lies inside a row without per-tap clamping).
+template<class T, int C, int INTERP, bool VARSHAPE>
+__device__ __forceinline__ Pixel<T, C> ResizeValueWide(const Plane &p, int64_t planeBytes, int dx, int dy)
+{
+    constexpr int PB     = sizeof(Pixel<T, C>);
+    const float   scaleX = static_cast<float>(p.srcW) / p.dstW;
+    const float   scaleY = static_cast<float>(p.srcH) / p.dstH;
+    Pixel<T, C>   out;
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        const int sx = min((int)floorf(scaleX * (dx + 0.5f)), p.srcW - 1);
+        const int sy = min((int)floorf(scaleY * (dy + 0.5f)), p.srcH - 1);
+        float     t[1][C];
+        LoadTaps<T, C, 1>(p.src, (int64_t)sy * p.srcRow + sx * PB, planeBytes, t);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out.v[c] = (T)t[0][c]; // exact: the value came from a T
+        }
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const float fx = (dx + .5f) * scaleX - .5f;
+        const float fy = (dy + .5f) * scaleY - .5f;
+        int         sx = (int)floorf(fx);
+        int         sy = (int)floorf(fy);
+        const float wx = (sx < 0) ? 0.f : ((sx > p.srcW - 2) ? 1.f : fx - sx);
+        const float wy = (sy < 0) ? 0.f : ((sy > p.srcH - 2) ? 1.f : fy - sy);
+        sx             = max(0, min(sx, p.srcW - 2));
+        sy             = max(0, min(sy, p.srcH - 2));
+        float t0[2][C], t1[2][C];
+        LoadTaps<T, C, 2>(p.src, (int64_t)sy * p.srcRow + sx * PB, planeBytes, t0);
+        LoadTaps<T, C, 2>(p.src, (int64_t)min(sy + 1, p.srcH - 1) * p.srcRow + sx * PB, planeBytes, t1);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            float v;
+            if constexpr (VARSHAPE)
+            {
+                v = (1.0f - wx) * (t0[0][c] * (1.0f - wy) + t1[0][c] * wy)
+                  + wx * (t0[1][c] * (1.0f - wy) + t1[1][c] * wy);
+            }
+            else
+            {
+                v = t0[0][c] * ((1.f - wx) * (1.f - wy)) + t0[1][c] * (wx * (1.f - wy)) + t1[0][c] * ((1.f - wx) * wy)
+                  + t1[1][c] * (wx * wy);
+            }
+            out.v[c] = SaturateCast<T>(v);
+        }
+    }
+    else
+    {
+        static_assert(INTERP == NVCV_INTERP_CUBIC);
+        const float cx = (dx + .5f) * scaleX - .5f;
+        const float cy = (dy + .5f) * scaleY - .5f;
+        int         sx = (int)floorf(cx);
+        int         sy = (int)floorf(cy);
+        float       fx = cx - sx;
+        const float fy = cy - sy;
+        fx             = (sx < 1 || sx >= p.srcW - 3) ? 0.f : fx;
+        sy             = max(1, min(sy, p.srcH - 3));
+        sx             = max(1, min(sx, p.srcW - 3)); // taps sx-1 .. sx+2 are inside for srcW >= 4
+        float wx[4], wy[4];
+        CubicCoeffs(fx, wx);
+        CubicCoeffs(fy, wy);
+        float sum[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            sum[c] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const int yy = max(0, min(sy - 1 + j, p.srcH - 1));
+            float     t[4][C];
+            LoadTaps<T, C, 4>(p.src, (int64_t)yy * p.srcRow + (sx - 1) * PB, planeBytes, t);
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                if constexpr (VARSHAPE)
+                {
+                    sum[c] += wy[j] * (wx[0] * t[0][c] + wx[1] * t[1][c] + wx[2] * t[2][c] + wx[3] * t[3][c]);
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        sum[c] += t[i][c] * (wx[i] * wy[j]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out.v[c] = SaturateCast<T>(fabsf(sum[c]));
+        }
+    }
+    return out;
+}
+
+struct __attribute__((packed, aligned(1))) UnalignedDword
+{
+    uint32_t w;
+};
+
+// Within every group of 4 adjacent lanes: r[k] of lane i <-> r[i] of lane k (i = lane & 3), as two
+// butterfly stages of cross-lane moves inside the group (no LDS).
+__device__ __forceinline__ uint32_t FromLaneXor1(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, false);
+}
+
+__device__ __forceinline__ uint32_t FromLaneXor2(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E /* quad_perm 2,3,0,1 */, 0xF, 0xF, false);
+}
+
+__device__ __forceinline__ void QuadTranspose(uint32_t (&r)[4], int i)
+{
+    const bool odd = (i & 1) != 0, upper = (i & 2) != 0;
+#pragma unroll
+    for (int b = 0; b < 4; b += 2) // 2x2 blocks (r0,r1) and (r2,r3) between lanes i and i^1
+    {
+        const uint32_t got = FromLaneXor1(odd ? r[b] : r[b + 1]);
+        r[b]               = odd ? got : r[b];
+        r[b + 1]           = odd ? r[b + 1] : got;
+    }
+#pragma unroll
+    for (int b = 0; b < 2; ++b) // (r0,r2) and (r1,r3) between lanes i and i^2
+    {
+        const uint32_t got = FromLaneXor2(upper ? r[b] : r[b + 2]);
+        r[b]               = upper ? got : r[b];
+        r[b + 2]           = upper ? r[b + 2] : got;
+    }
+}
+
+// 4 pixels of PB bytes, each held zero-extended in ceil(PB/4) dwords (q[d][k] = dword d of pixel k),
+// packed back to back into PB dwords.
+template<int PB>
+__device__ __forceinline__ void PackQuad(const uint32_t (&q)[(PB + 3) / 4][4], uint32_t (&w)[PB])
+{
+    if constexpr (PB % 4 == 0)
+    {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+#pragma unroll
+            for (int d = 0; d < PB / 4; ++d)
+            {
+                w[k * (PB / 4) + d] = q[d][k];
+            }
+        }
+    }
+    else if constexpr (PB == 1)
+    {
+        w[0] = q[0][0] | (q[0][1] << 8) | (q[0][2] << 16) | (q[0][3] << 24);
+    }
+    else if constexpr (PB == 2)
+    {
+        w[0] = q[0][0] | (q[0][1] << 16);
+        w[1] = q[0][2] | (q[0][3] << 16);
+    }
+    else if constexpr (PB == 3)
+    {
+        w[0] = q[0][0] | (q[0][1] << 24);
+        w[1] = (q[0][1] >> 8) | (q[0][2] << 16);
+        w[2] = (q[0][2] >> 16) | (q[0][3] << 8);
+    }
+    else
+    {
+        static_assert(PB == 6, "pixel sizes: 1, 2, 3, 4, 6, 8, 12, 16 bytes");
+        w[0] = q[0][0];
+        w[1] = q[1][0] | (q[0][1] << 16);
+        w[2] = (q[0][1] >> 16) | (q[1][1] << 16);
+        w[3] = q[0][2];
+        w[4] = q[1][2] | (q[0][3] << 16);
+        w[5] = (q[0][3] >> 16) | (q[1][3] << 16);
+    }
+}
+
+// One wave resizes a 64-column x 4-row patch of the output whose top left pixel is (x0, y0), both
+// wave-uniform. Sampling: lane l owns column x0 + l and computes its 4 rows (the column terms are
+// shared; neighbouring lanes read neighbouring source pixels whatever the scale). Storing: after
+// the 4x4 transposes lane l owns row y0 + (l & 3), columns x0 + 4 * (l >> 2) .. + 3.
+template<class T, int C, int INTERP, bool VARSHAPE>
+__device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
+{
+    constexpr int PB = sizeof(Pixel<T, C>), D = (PB + 3) / 4;
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    const int     lane       = threadIdx.x & 63;
+    const int64_t planeBytes = (int64_t)(p.srcH - 1) * p.srcRow + (int64_t)p.srcW * PB;
+    const bool    wide       = p.srcW >= 4; // uniform per image
+    // columns and rows past the output compute a duplicate of the last one: every lane takes part in
+    // the transposes
+    const int dx = min(x0 + lane, p.dstW - 1);
+    uint32_t  q[D][4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        const int         dy  = min(y0 + k, p.dstH - 1);
+        const Pixel<T, C> out = wide ? ResizeValueWide<T, C, INTERP, VARSHAPE>(p, planeBytes, dx, dy)
+                                     : ResizeValue<T, C, INTERP, VARSHAPE>(p, dx, dy);
+        uint32_t          w[D] = {};
+        __builtin_memcpy(w, &out, PB);
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+        {
+            q[d][k] = w[d];
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+    {
+        QuadTranspose(q[d], lane & 3);
+    }
+    const int dy = y0 + (lane & 3), dx0 = x0 + 4 * (lane >> 2);
+    if (dy >= p.dstH || dx0 >= p.dstW)
+    {
+        return;
+    }
+    uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * PB;
+    if (dx0 + 4 <= p.dstW)
+    {
+        uint32_t w[PB];
+        PackQuad<PB>(q, w);
+        UnalignedDword *ow = reinterpret_cast<UnalignedDword *>(to);
+#pragma unroll
+        for (int i = 0; i < PB; ++i)
+        {
+            __builtin_nontemporal_store(w[i], &ow[i].w); // streaming: the output is not read back
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+        {
+            if (dx0 + k < p.dstW)
+            {
+                uint32_t w[D];
+#pragma unroll
+                for (int d = 0; d < D; ++d)
+                {
+                    w[d] = q[d][k];
+                }
+                Pixel<T, C> px;
+                __builtin_memcpy(&px, w, PB);
+                reinterpret_cast<Pixel<T, C> *>(to)[k] = px;
+            }
+        }
+    }
+}
+
+constexpr int kPatchTileW = 64, kPatchTileH = 16; // block = 4 waves stacked vertically
+
+template<class T, int C, int INTERP>
+__global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs a)
+{
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizeWavePatch<T, C, INTERP, false>(p, blockIdx.x * kPatchTileW, blockIdx.y * kPatchTileH + (threadIdx.x >> 6) * 4);
+}
+
+template<class T, int C, int INTERP>
+__global__ __launch_bounds__(256) void ResizePatchVarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc = LocateTile(tiles, blockIdx.x);
+    const Plane     p  = GetPlanes<true>(a, tc.image);
+    ResizeWavePatch<T, C, INTERP, true>(p, tc.tx * kPatchTileW, tc.ty * kPatchTileH + (threadIdx.x >> 6) * 4);
 }
 
 // Bicubic for strong horizontal reductions. With one lane per output pixel the four taps of
@@ -464,6 +795,10 @@ __global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs 
     }
 }
 
+// Which (type, channels, interpolation) run as wave patches.
+template<class T, int C, int INTERP>
+constexpr bool kPatchForm = INTERP != NVCV_INTERP_AREA && sizeof(T) == 1;
+
 template<class T, int C, int INTERP>
 void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
 {
@@ -477,6 +812,13 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             return;
         }
     }
+    if constexpr (kPatchForm<T, C, INTERP>)
+    {
+        dim3 pgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, kPatchTileH), N);
+        hipLaunchKernelGGL((ResizePatchTensorKernel<T, C, INTERP>), pgrid, dim3(256), 0, stream, a);
+        CheckLaunch("ResizePatchTensorKernel");
+        return;
+    }
     hipLaunchKernelGGL((ResizeTensorKernel<T, C, INTERP>), grid, dim3(256), 0, stream, a);
     CheckLaunch("ResizeTensorKernel");
 }
@@ -486,8 +828,20 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, 
 {
     for (int first = 0; first < N; first += kMaxTileImages)
     {
-        VarTiles tiles;
-        int      total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kTileW, kTileH);
+        VarTiles  tiles;
+        const int count = std::min(kMaxTileImages, N - first);
+        if constexpr (kPatchForm<T, C, INTERP>)
+        {
+            int total = BuildVarTiles(tiles, dstHost, first, count, kPatchTileW, kPatchTileH);
+            if (total > 0)
+            {
+                hipLaunchKernelGGL((ResizePatchVarShapeKernel<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a,
+                                   tiles);
+                CheckLaunch("ResizePatchVarShapeKernel");
+            }
+            continue;
+        }
+        int total = BuildVarTiles(tiles, dstHost, first, count, kTileW, kTileH);
         if (total > 0)
         {
             hipLaunchKernelGGL((ResizeVarShapeKernel<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a, tiles);
