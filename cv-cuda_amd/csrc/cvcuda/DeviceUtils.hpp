@@ -21,9 +21,8 @@ __device__ __forceinline__ T SaturateCast(float v)
     }
     else if constexpr (std::is_same_v<T, uint8_t>)
     {
-        float r = rintf(v);
-        r       = fminf(fmaxf(r, 0.f), 255.f); // fmaxf(NaN, 0) == 0
-        return (uint8_t)(int)r;
+        // one instruction: round half to even, saturate to [0, 255], NaN -> 0
+        return (uint8_t)__builtin_amdgcn_cvt_pk_u8_f32(v, 0, 0);
     }
     else if constexpr (std::is_same_v<T, int8_t>)
     {

@@ -369,6 +369,11 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
     const float scaleH = static_cast<float>(srcH) / dstH;
     const float scaleW = static_cast<float>(srcW) / dstW;
     const double lo = (double)std::numeric_limits<T>::lowest(), hi = (double)std::numeric_limits<T>::max();
+    // Sources narrower or lower than the tap window (2 pixels for linear, 4 for cubic): the reference's
+    // golden and kernels index outside the image there (undefined values). This restatement defines
+    // those taps as clamped into the image, which changes nothing for larger sources.
+    auto tapX = [srcW](int x) { return std::max(0, std::min(x, srcW - 1)); };
+    auto tapY = [srcH](int y) { return std::max(0, std::min(y, srcH - 1)); };
 
     for (int dy = 0; dy < dstH; ++dy)
     {
@@ -399,10 +404,11 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                 double wy[2] = {1 - fy, fy}, wx[2] = {1 - fx, fx};
                 for (int c = 0; c < C; ++c)
                 {
-                    double res = std::rint(std::abs(src[(sy + 0) * srcStep + (int64_t)(sx + 0) * C + c] * wy[0] * wx[0]
-                                                    + src[(sy + 1) * srcStep + (int64_t)(sx + 0) * C + c] * wy[1] * wx[0]
-                                                    + src[(sy + 0) * srcStep + (int64_t)(sx + 1) * C + c] * wy[0] * wx[1]
-                                                    + src[(sy + 1) * srcStep + (int64_t)(sx + 1) * C + c] * wy[1] * wx[1]));
+                    const int y0 = tapY(sy), y1 = tapY(sy + 1), x0 = tapX(sx), x1 = tapX(sx + 1);
+                    double    res = std::rint(std::abs(src[y0 * srcStep + (int64_t)x0 * C + c] * wy[0] * wx[0]
+                                                       + src[y1 * srcStep + (int64_t)x0 * C + c] * wy[1] * wx[0]
+                                                       + src[y0 * srcStep + (int64_t)x1 * C + c] * wy[0] * wx[1]
+                                                       + src[y1 * srcStep + (int64_t)x1 * C + c] * wy[1] * wx[1]));
                     out[c]     = (T)(res < lo ? lo : (res > hi ? hi : res));
                 }
             }
@@ -418,10 +424,10 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                 sx        = std::max(0, std::min(sx, srcW - 2));
                 for (int c = 0; c < C; ++c)
                 {
-                    float p00 = src[(sy + 0) * srcStep + (int64_t)(sx + 0) * C + c];
-                    float p01 = src[(sy + 0) * srcStep + (int64_t)(sx + 1) * C + c];
-                    float p10 = src[(sy + 1) * srcStep + (int64_t)(sx + 0) * C + c];
-                    float p11 = src[(sy + 1) * srcStep + (int64_t)(sx + 1) * C + c];
+                    float p00 = src[tapY(sy) * srcStep + (int64_t)tapX(sx) * C + c];
+                    float p01 = src[tapY(sy) * srcStep + (int64_t)tapX(sx + 1) * C + c];
+                    float p10 = src[tapY(sy + 1) * srcStep + (int64_t)tapX(sx) * C + c];
+                    float p11 = src[tapY(sy + 1) * srcStep + (int64_t)tapX(sx + 1) * C + c];
                     float v   = p00 * ((1.f - wxv) * (1.f - wyv)) + p01 * (wxv * (1.f - wyv)) + p10 * ((1.f - wxv) * wyv)
                             + p11 * (wxv * wyv);
                     out[c] = SatF<T>(v);
@@ -439,10 +445,10 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                 sx       = std::max(0, std::min(sx, srcW - 2));
                 for (int c = 0; c < C; ++c)
                 {
-                    float a0 = src[(sy + 0) * srcStep + (int64_t)(sx + 0) * C + c];
-                    float a1 = src[(sy + 0) * srcStep + (int64_t)(sx + 1) * C + c];
-                    float b0 = src[(sy + 1) * srcStep + (int64_t)(sx + 0) * C + c];
-                    float b1 = src[(sy + 1) * srcStep + (int64_t)(sx + 1) * C + c];
+                    float a0 = src[tapY(sy) * srcStep + (int64_t)tapX(sx) * C + c];
+                    float a1 = src[tapY(sy) * srcStep + (int64_t)tapX(sx + 1) * C + c];
+                    float b0 = src[tapY(sy + 1) * srcStep + (int64_t)tapX(sx) * C + c];
+                    float b1 = src[tapY(sy + 1) * srcStep + (int64_t)tapX(sx + 1) * C + c];
                     float v  = (1.0f - fx) * (a0 * (1.0f - fy) + b0 * fy) + fx * (a1 * (1.0f - fy) + b1 * fy);
                     out[c]   = SatF<T>(v);
                 }
@@ -475,7 +481,7 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                     {
                         for (int iy = 0; iy < 4; ++iy)
                         {
-                            sum += src[(sy - 1 + iy) * srcStep + (int64_t)(sx - 1 + ix) * C + c] * wx[ix] * wy[iy];
+                            sum += src[tapY(sy - 1 + iy) * srcStep + (int64_t)tapX(sx - 1 + ix) * C + c] * wx[ix] * wy[iy];
                         }
                     }
                     double res = std::rint(std::abs(sum));
@@ -513,7 +519,7 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                         {
                             for (int cx = -1; cx <= 2; ++cx)
                             {
-                                sum += (float)src[(sy + cy) * srcStep + (int64_t)(sx + cx) * C + c]
+                                sum += (float)src[tapY(sy + cy) * srcStep + (int64_t)tapX(sx + cx) * C + c]
                                      * (wx[cx + 1] * wy[cy + 1]);
                             }
                         }
@@ -522,10 +528,11 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                     {
                         for (int row = 0; row < 4; ++row)
                         {
-                            const T *a = src + (sy + row - 1) * srcStep + (int64_t)(sx - 1) * C + c;
+                            const T *a = src + tapY(sy + row - 1) * srcStep + c;
                             sum += wy[row]
-                                 * (wx[0] * (float)a[0] + wx[1] * (float)a[C] + wx[2] * (float)a[2 * C]
-                                    + wx[3] * (float)a[3 * C]);
+                                 * (wx[0] * (float)a[(int64_t)tapX(sx - 1) * C] + wx[1] * (float)a[(int64_t)tapX(sx) * C]
+                                    + wx[2] * (float)a[(int64_t)tapX(sx + 1) * C]
+                                    + wx[3] * (float)a[(int64_t)tapX(sx + 2) * C]);
                         }
                     }
                     out[c] = SatF<T>(std::abs(sum));

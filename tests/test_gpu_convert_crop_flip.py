@@ -40,6 +40,23 @@ def test_convert_to_all_type_pairs(cv, orc, gpu, tin, tout):
             assert np.allclose(res, gold, rtol=1e-5, atol=1e-4)
 
 
+def test_float_to_u8_rounding_and_saturation_cases(cv, orc, gpu):
+    # every half-way case around the u8 range, their float neighbours, the range ends, non-finite values:
+    # round half to even, saturate, NaN -> 0 (cuda_tools/detail/SaturateCastImpl.hpp:41-50)
+    ties = np.arange(-4, 261, dtype=np.float32) + np.float32(0.5)
+    vals = np.concatenate([ties, np.nextafter(ties, np.float32(-1e9)), np.nextafter(ties, np.float32(1e9)),
+                           np.arange(-4, 261, dtype=np.float32),
+                           np.array([np.nan, np.inf, -np.inf, 1e9, -1e9, 3e38, -3e38, 1e-40, -1e-40, 0.0, -0.0,
+                                     254.5, 255.5, 255.49998, 256.0], np.float32)])
+    vals = np.resize(vals, (1, 1, -(-vals.size // 4), 4)).astype(np.float32)  # padded by repeating the start
+    out = cv.Tensor.alloc(list(vals.shape), np.uint8, "NHWC")
+    cv.ConvertTo()(None, cv.Tensor.from_numpy(vals, "NHWC"), out, 1.0, 0.0)
+    torch.cuda.synchronize()
+    with np.errstate(invalid="ignore"):
+        exp = np.clip(np.rint(np.nan_to_num(vals, nan=0.0, posinf=1e9, neginf=-1e9)), 0, 255).astype(np.uint8)
+    np.testing.assert_array_equal(out.numpy(), exp)
+
+
 def test_convert_to_reference_rows_and_pipeline_shape(cv, orc, gpu):
     # constant 0x10 images of the reference's table; expected value by its formula
     op = cv.ConvertTo()

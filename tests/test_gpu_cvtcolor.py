@@ -151,7 +151,7 @@ def test_negative_cases(cv, K, gpu):
         (cv.Tensor.alloc([1, 8, 8, 3], np.uint8, "NHWC"), cv.Tensor.alloc([1, 3, 8, 8], np.uint8, "NCHW"),
          K.COLOR_BGR2RGB),                                                                # layout
         (cv.Tensor.alloc([1, 8, 8, 3], np.uint8, "NHWC"), cv.Tensor.alloc([1, 8, 8, 3], np.uint8, "NHWC"),
-         K.COLOR_BGR2HSV),                                                                # code not provided
+         K.COLOR_BGR2Lab),                                                                # code not provided (by the reference either)
     ]
     for tin, tout, code in bad:
         with pytest.raises(cv.Error) as e:
