@@ -140,7 +140,7 @@ class ResizeC1:
         self.cv, self.orc, self.np, self.torch, self.interp = cv, orc, np, torch, interp
         name = "NEAREST" if interp == NEAREST else "LINEAR"
         self.key = "resize-" + name.lower()
-        self.kernel = "ResizeTensorKernel<uint8_t,3,%s>" % name
+        self.kernel = "ResizePatchTensorKernel<uint8_t,3,%s>" % name
         self.workload = "Resize %s: batch 8 u8 NHWC 1920x1080 -> 224x224" % name
         self.images = self.N
         rows, _ = span_bytes(self.OUT_H, 0, self.SRC_H, self.OUT_H, interp, 1)

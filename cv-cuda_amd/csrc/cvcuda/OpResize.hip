@@ -7,9 +7,12 @@
 // reference's CPU golden (tests/cvcuda/system/ResizeUtils.cpp:206-221) for every pixel, so results
 // are bit-exact against it also where the coordinate lands on an integer.
 //
-// Kernel shape: one lane per output pixel, a 256-thread block covers 64 columns x 4 rows; pixels
-// are moved as whole C-channel vectors (one load/store instruction each where the element size
-// allows), outputs use streaming stores. Var-shape batches run on a packed tile grid.
+// Three kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
+//  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
+//    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
+//  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
+//  * everything else (12/16-byte pixels, AREA): one lane per output pixel, a 256-thread block covers
+//    64 columns x 4 rows, pixels moved as whole C-channel vectors.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
@@ -346,24 +349,41 @@ __global__ __launch_bounds__(256) void ResizeVarShapeKernel(const ResizeArgs a, 
 // stores 4 consecutive pixels as whole dwords. Arithmetic: the expressions of ResizeValue, term for
 // term.
 
-// N horizontally adjacent pixels at byte offset `off` of the source plane (all inside the image).
-// u8x3: 1 or 2 pixels are fetched with a 4- or 8-byte load that reads 1-2 bytes past them; where
-// that would cross the end of the plane (`planeBytes`) the load is moved back and the value shifted.
+// N horizontally adjacent pixels at byte offset `xoff` of source row `row` (all inside the image).
+// u8x3: 1 or 2 pixels are fetched with a 4- or 8-byte load that reads 1-2 bytes past them, harmless
+// except behind the image's last row (`lastRow`, wave-uniform), where the load is moved back to end
+// with the row's `rowBytes` and the value shifted.
 template<class T, int C, int N>
-__device__ __forceinline__ void LoadTaps(const uint8_t *plane, int64_t off, int64_t planeBytes, float (&t)[N][C])
+__device__ __forceinline__ void LoadTaps(const uint8_t *row, int xoff, bool lastRow, int rowBytes, float (&t)[N][C])
 {
     if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 1)
     {
-        const int      back = (int)max((int64_t)0, off - (planeBytes - 4));
-        const uint32_t q    = LoadU32Unaligned(plane + off - back) >> (8 * back);
-        t[0][0]             = (float)(q & 0xFF);
-        t[0][1]             = (float)((q >> 8) & 0xFF);
-        t[0][2]             = (float)((q >> 16) & 0xFF);
+        uint32_t q;
+        if (lastRow)
+        {
+            const int back = max(0, xoff - (rowBytes - 4));
+            q              = LoadU32Unaligned(row + (xoff - back)) >> (8 * back);
+        }
+        else
+        {
+            q = LoadU32Unaligned(row + xoff);
+        }
+        t[0][0] = (float)(q & 0xFF);
+        t[0][1] = (float)((q >> 8) & 0xFF);
+        t[0][2] = (float)((q >> 16) & 0xFF);
     }
     else if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 2)
     {
-        const int      back = (int)max((int64_t)0, off - (planeBytes - 8));
-        const uint64_t q    = LoadU64Unaligned(plane + off - back) >> (8 * back);
+        uint64_t q;
+        if (lastRow)
+        {
+            const int back = max(0, xoff - (rowBytes - 8));
+            q              = LoadU64Unaligned(row + (xoff - back)) >> (8 * back);
+        }
+        else
+        {
+            q = LoadU64Unaligned(row + xoff);
+        }
         const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
         t[0][0] = (float)(lo & 0xFF);
         t[0][1] = (float)((lo >> 8) & 0xFF);
@@ -374,7 +394,7 @@ __device__ __forceinline__ void LoadTaps(const uint8_t *plane, int64_t off, int6
     }
     else
     {
-        const Pixel<T, N *C> v = *reinterpret_cast<const Pixel<T, N * C> *>(plane + off);
+        const Pixel<T, N *C> v = *reinterpret_cast<const Pixel<T, N * C> *>(row + xoff);
 #pragma unroll
         for (int i = 0; i < N; ++i)
         {
@@ -387,20 +407,70 @@ __device__ __forceinline__ void LoadTaps(const uint8_t *plane, int64_t off, int6
     }
 }
 
-// Requires srcW >= 4 (every tap group then lies inside a row without per-tap clamping).
-template<class T, int C, int INTERP, bool VARSHAPE>
-__device__ __forceinline__ Pixel<T, C> ResizeValueWide(const Plane &p, int64_t planeBytes, int dx, int dy)
+// Per-column and per-row terms of a sample: source index and weights, the expressions of
+// ResizeValue. W = number of weights (0 nearest, 1 linear, 4 cubic); sources are >= 4 pixels wide.
+template<int W>
+struct AxisTerms
 {
-    constexpr int PB     = sizeof(Pixel<T, C>);
-    const float   scaleX = static_cast<float>(p.srcW) / p.dstW;
-    const float   scaleY = static_cast<float>(p.srcH) / p.dstH;
+    int   s;                // nearest: source index; linear: first tap; cubic: second tap
+    float w[W > 0 ? W : 1]; // linear: weight of the second tap
+};
+
+template<int INTERP>
+constexpr int kWeights = INTERP == NVCV_INTERP_NEAREST ? 0 : (INTERP == NVCV_INTERP_LINEAR ? 1 : 4);
+
+template<int INTERP>
+__device__ __forceinline__ AxisTerms<kWeights<INTERP>> Axis(float scale, int d, int srcSize)
+{
+    AxisTerms<kWeights<INTERP>> a;
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        a.s = min((int)floorf(scale * (d + 0.5f)), srcSize - 1);
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const float f = (d + .5f) * scale - .5f;
+        const int   s = (int)floorf(f);
+        a.w[0]        = (s < 0) ? 0.f : ((s > srcSize - 2) ? 1.f : f - s);
+        a.s           = max(0, min(s, srcSize - 2));
+    }
+    else
+    {
+        const float c = (d + .5f) * scale - .5f;
+        const int   s = (int)floorf(c);
+        float       f = c - s;
+        a.s           = s;
+        a.w[0]        = f; // finished by the caller: the two axes treat the fraction differently
+    }
+    return a;
+}
+
+// Lane `from` (constant) of every field, as wave-uniform values.
+template<int W>
+__device__ __forceinline__ AxisTerms<W> FromLane(const AxisTerms<W> &a, int from)
+{
+    AxisTerms<W> r;
+    r.s = __builtin_amdgcn_readlane(a.s, from);
+#pragma unroll
+    for (int i = 0; i < (W > 0 ? W : 1); ++i)
+    {
+        r.w[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(a.w[i]), from));
+    }
+    return r;
+}
+
+// One output pixel from its column terms (per lane) and row terms (wave-uniform).
+template<class T, int C, int INTERP, bool VARSHAPE>
+__device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerms<kWeights<INTERP>> &col,
+                                                  const AxisTerms<kWeights<INTERP>> &row)
+{
+    constexpr int PB       = sizeof(Pixel<T, C>);
+    const int     rowBytes = p.srcW * PB;
     Pixel<T, C>   out;
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
     {
-        const int sx = min((int)floorf(scaleX * (dx + 0.5f)), p.srcW - 1);
-        const int sy = min((int)floorf(scaleY * (dy + 0.5f)), p.srcH - 1);
-        float     t[1][C];
-        LoadTaps<T, C, 1>(p.src, (int64_t)sy * p.srcRow + sx * PB, planeBytes, t);
+        float t[1][C];
+        LoadTaps<T, C, 1>(p.src + (int64_t)row.s * p.srcRow, col.s * PB, row.s == p.srcH - 1, rowBytes, t);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -409,17 +479,11 @@ __device__ __forceinline__ Pixel<T, C> ResizeValueWide(const Plane &p, int64_t p
     }
     else if constexpr (INTERP == NVCV_INTERP_LINEAR)
     {
-        const float fx = (dx + .5f) * scaleX - .5f;
-        const float fy = (dy + .5f) * scaleY - .5f;
-        int         sx = (int)floorf(fx);
-        int         sy = (int)floorf(fy);
-        const float wx = (sx < 0) ? 0.f : ((sx > p.srcW - 2) ? 1.f : fx - sx);
-        const float wy = (sy < 0) ? 0.f : ((sy > p.srcH - 2) ? 1.f : fy - sy);
-        sx             = max(0, min(sx, p.srcW - 2));
-        sy             = max(0, min(sy, p.srcH - 2));
-        float t0[2][C], t1[2][C];
-        LoadTaps<T, C, 2>(p.src, (int64_t)sy * p.srcRow + sx * PB, planeBytes, t0);
-        LoadTaps<T, C, 2>(p.src, (int64_t)min(sy + 1, p.srcH - 1) * p.srcRow + sx * PB, planeBytes, t1);
+        const int   y0 = row.s, y1 = min(row.s + 1, p.srcH - 1);
+        const float wx = col.w[0], wy = row.w[0];
+        float       t0[2][C], t1[2][C];
+        LoadTaps<T, C, 2>(p.src + (int64_t)y0 * p.srcRow, col.s * PB, y0 == p.srcH - 1, rowBytes, t0);
+        LoadTaps<T, C, 2>(p.src + (int64_t)y1 * p.srcRow, col.s * PB, y1 == p.srcH - 1, rowBytes, t1);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -439,19 +503,6 @@ __device__ __forceinline__ Pixel<T, C> ResizeValueWide(const Plane &p, int64_t p
     }
     else
     {
-        static_assert(INTERP == NVCV_INTERP_CUBIC);
-        const float cx = (dx + .5f) * scaleX - .5f;
-        const float cy = (dy + .5f) * scaleY - .5f;
-        int         sx = (int)floorf(cx);
-        int         sy = (int)floorf(cy);
-        float       fx = cx - sx;
-        const float fy = cy - sy;
-        fx             = (sx < 1 || sx >= p.srcW - 3) ? 0.f : fx;
-        sy             = max(1, min(sy, p.srcH - 3));
-        sx             = max(1, min(sx, p.srcW - 3)); // taps sx-1 .. sx+2 are inside for srcW >= 4
-        float wx[4], wy[4];
-        CubicCoeffs(fx, wx);
-        CubicCoeffs(fy, wy);
         float sum[C];
 #pragma unroll
         for (int c = 0; c < C; ++c)
@@ -461,22 +512,22 @@ __device__ __forceinline__ Pixel<T, C> ResizeValueWide(const Plane &p, int64_t p
 #pragma unroll
         for (int j = 0; j < 4; ++j)
         {
-            const int yy = max(0, min(sy - 1 + j, p.srcH - 1));
+            const int yy = max(0, min(row.s - 1 + j, p.srcH - 1));
             float     t[4][C];
-            LoadTaps<T, C, 4>(p.src, (int64_t)yy * p.srcRow + (sx - 1) * PB, planeBytes, t);
+            LoadTaps<T, C, 4>(p.src + (int64_t)yy * p.srcRow, (col.s - 1) * PB, yy == p.srcH - 1, rowBytes, t);
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
                 if constexpr (VARSHAPE)
                 {
-                    sum[c] += wy[j] * (wx[0] * t[0][c] + wx[1] * t[1][c] + wx[2] * t[2][c] + wx[3] * t[3][c]);
+                    sum[c] += row.w[j] * (col.w[0] * t[0][c] + col.w[1] * t[1][c] + col.w[2] * t[2][c] + col.w[3] * t[3][c]);
                 }
                 else
                 {
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
                     {
-                        sum[c] += t[i][c] * (wx[i] * wy[j]);
+                        sum[c] += t[i][c] * (col.w[i] * row.w[j]);
                     }
                 }
             }
@@ -488,6 +539,22 @@ __device__ __forceinline__ Pixel<T, C> ResizeValueWide(const Plane &p, int64_t p
         }
     }
     return out;
+}
+
+// Column (horizontal == true) or row terms of output index d, finished for sampling.
+template<int INTERP>
+__device__ __forceinline__ AxisTerms<kWeights<INTERP>> FinishedAxis(float scale, int d, int srcSize, bool horizontal)
+{
+    AxisTerms<kWeights<INTERP>> a = Axis<INTERP>(scale, d, srcSize);
+    if constexpr (INTERP == NVCV_INTERP_CUBIC)
+    {
+        // the reference zeroes the horizontal fraction next to the image border, not the vertical one
+        float f = a.w[0];
+        f       = (horizontal && (a.s < 1 || a.s >= srcSize - 3)) ? 0.f : f;
+        a.s     = max(1, min(a.s, srcSize - 3));
+        CubicCoeffs(f, a.w);
+    }
+    return a;
 }
 
 struct __attribute__((packed, aligned(1))) UnalignedDword
@@ -582,25 +649,48 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
     {
         return;
     }
-    const int     lane       = threadIdx.x & 63;
-    const int64_t planeBytes = (int64_t)(p.srcH - 1) * p.srcRow + (int64_t)p.srcW * PB;
-    const bool    wide       = p.srcW >= 4; // uniform per image
+    const int   lane   = threadIdx.x & 63;
+    const float scaleX = static_cast<float>(p.srcW) / p.dstW;
+    const float scaleY = static_cast<float>(p.srcH) / p.dstH;
+    const bool  wide   = p.srcW >= 4; // uniform per image
     // columns and rows past the output compute a duplicate of the last one: every lane takes part in
     // the transposes
     const int dx = min(x0 + lane, p.dstW - 1);
     uint32_t  q[D][4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
+    if (wide)
     {
-        const int         dy  = min(y0 + k, p.dstH - 1);
-        const Pixel<T, C> out = wide ? ResizeValueWide<T, C, INTERP, VARSHAPE>(p, planeBytes, dx, dy)
-                                     : ResizeValue<T, C, INTERP, VARSHAPE>(p, dx, dy);
-        uint32_t          w[D] = {};
-        __builtin_memcpy(w, &out, PB);
+        const auto col = FinishedAxis<INTERP>(scaleX, dx, p.srcW, true);
+        // the 4 rows' terms are computed side by side (lane l: row l & 3) and then read as uniform values
+        const auto rows = FinishedAxis<INTERP>(scaleY, min(y0 + (lane & 3), p.dstH - 1), p.srcH, false);
 #pragma unroll
-        for (int d = 0; d < D; ++d)
+        for (int k = 0; k < 4; ++k)
         {
-            q[d][k] = w[d];
+            const Pixel<T, C> out  = SampleWide<T, C, INTERP, VARSHAPE>(p, col, FromLane(rows, k));
+            uint32_t          w[D] = {};
+            __builtin_memcpy(w, &out, PB);
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+            {
+                q[d][k] = w[d];
+            }
+        }
+    }
+    else
+    {
+#pragma unroll 1
+        for (int k = 0; k < 4; ++k)
+        {
+            const Pixel<T, C> out  = ResizeValue<T, C, INTERP, VARSHAPE>(p, dx, min(y0 + k, p.dstH - 1));
+            uint32_t          w[D] = {};
+            __builtin_memcpy(w, &out, PB);
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+            {
+                q[d][0] = k == 0 ? w[d] : q[d][0];
+                q[d][1] = k == 1 ? w[d] : q[d][1];
+                q[d][2] = k == 2 ? w[d] : q[d][2];
+                q[d][3] = k == 3 ? w[d] : q[d][3];
+            }
         }
     }
 #pragma unroll
@@ -797,13 +887,13 @@ __global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs 
 
 // Which (type, channels, interpolation) run as wave patches.
 template<class T, int C, int INTERP>
-constexpr bool kPatchForm = INTERP != NVCV_INTERP_AREA && sizeof(T) == 1;
+constexpr bool kPatchForm = INTERP != NVCV_INTERP_AREA && sizeof(Pixel<T, C>) <= 8;
 
 template<class T, int C, int INTERP>
 void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
 {
     dim3 grid(DivUp(a.dstW, kTileW), DivUp(a.dstH, kTileH), N);
-    if constexpr (INTERP == NVCV_INTERP_CUBIC && sizeof(Pixel<T, C>) % 4 == 0)
+    if constexpr (INTERP == NVCV_INTERP_CUBIC && sizeof(Pixel<T, C>) % 4 == 0 && !kPatchForm<T, C, INTERP>)
     {
         if (a.srcW >= 2 * a.dstW)
         {
