@@ -45,6 +45,7 @@ struct ResizeArgs
     int64_t        srcSampleStride, dstSampleStride;
     int32_t        srcRowStride, dstRowStride;
     int32_t        srcW, srcH, dstW, dstH;
+    float          scaleX, scaleY; // srcW / dstW, srcH / dstH in float32 (var-shape: per image, in the kernel)
     // var-shape
     const NVCVImageBufferStrided *srcList;
     const NVCVImageBufferStrided *dstList;
@@ -55,6 +56,7 @@ struct Plane
     const uint8_t *src;
     uint8_t       *dst;
     int32_t        srcRow, dstRow, srcW, srcH, dstW, dstH;
+    float          scaleX, scaleY;
 };
 
 template<bool VARSHAPE>
@@ -65,7 +67,16 @@ __device__ __forceinline__ Plane GetPlanes(const ResizeArgs &a, int n)
     {
         const NVCVImagePlaneStrided &s = a.srcList[n].planes[0];
         const NVCVImagePlaneStrided &d = a.dstList[n].planes[0];
-        p = {s.basePtr, d.basePtr, s.rowStride, d.rowStride, s.width, s.height, d.width, d.height};
+        p = {s.basePtr,
+             d.basePtr,
+             s.rowStride,
+             d.rowStride,
+             s.width,
+             s.height,
+             d.width,
+             d.height,
+             static_cast<float>(s.width) / d.width,
+             static_cast<float>(s.height) / d.height};
     }
     else
     {
@@ -76,7 +87,9 @@ __device__ __forceinline__ Plane GetPlanes(const ResizeArgs &a, int n)
              a.srcW,
              a.srcH,
              a.dstW,
-             a.dstH};
+             a.dstH,
+             a.scaleX,
+             a.scaleY};
     }
     return p;
 }
@@ -110,8 +123,7 @@ __device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
 template<class T, int C, int INTERP, bool VARSHAPE>
 __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int dy)
 {
-    const float scaleX = static_cast<float>(p.srcW) / p.dstW;
-    const float scaleY = static_cast<float>(p.srcH) / p.dstH;
+    const float scaleX = p.scaleX, scaleY = p.scaleY;
     Pixel<T, C> out;
 
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
@@ -650,8 +662,7 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
         return;
     }
     const int   lane   = threadIdx.x & 63;
-    const float scaleX = static_cast<float>(p.srcW) / p.dstW;
-    const float scaleY = static_cast<float>(p.srcH) / p.dstH;
+    const float scaleX = p.scaleX, scaleY = p.scaleY;
     const bool  wide   = p.srcW >= 4; // uniform per image
     // columns and rows past the output compute a duplicate of the last one: every lane takes part in
     // the transposes
@@ -797,8 +808,7 @@ __global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs 
     const int   dx   = blockIdx.x * kTileW + lane;
     const int   dy   = blockIdx.y * kTileH + wave;
 
-    const float scaleX = static_cast<float>(p.srcW) / p.dstW;
-    const float scaleY = static_cast<float>(p.srcH) / p.dstH;
+    const float scaleX = p.scaleX, scaleY = p.scaleY;
 
     // lanes and rows past the output compute a duplicate of the last pixel and skip the store: every
     // lane takes part in its wave's exchange (each wave owns one quarter of the staging array)
@@ -1070,6 +1080,8 @@ public:
         {
             return;
         }
+        a.scaleX = static_cast<float>(in.W) / out.W; // IEEE float32 division, as the kernels would do it
+        a.scaleY = static_cast<float>(in.H) / out.H;
         DispatchType(in.elem, in.C, false, a, nullptr, in.N, interp, stream);
     }
 
