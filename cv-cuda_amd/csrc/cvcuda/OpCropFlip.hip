@@ -7,11 +7,13 @@
 //
 // Two kernels. Crops and row-mirroring flips keep the byte order inside a row, so they run as row
 // copies: every lane moves 16 bytes of a row with one unaligned 16-byte load and store whatever the
-// pixel type is (a wave covers 1 KiB of a row). Column-mirroring flips permute pixels and run with one
-// lane per pixel, the whole pixel as one vector access. Stores are streaming. Only the bytes of the
-// region are written; the rest of the output is left untouched.
+// pixel type is (a wave covers 1 KiB of a row). Column-mirroring flips permute pixels: a lane reads a
+// run of 4 source pixels with one vector load, reverses their order and writes them as whole dwords.
+// Stores are streaming. Only the bytes of the region are written; the rest of the output is left
+// untouched.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "RunIO.hpp"
 #include "VarShapeTiles.hpp"
 
 #include <cvcuda/OpCenterCrop.h>
@@ -99,18 +101,46 @@ __device__ __forceinline__ void CopyPixel(const uint8_t *srcRow, uint8_t *dstRow
     }
 }
 
+// dst pixels dx0 .. dx0+3 of a row  <-  src pixels sx, sx + step, .. (step = +1 / -1); the ragged end
+// of a row goes pixel by pixel
+template<class T, int C>
+__device__ __forceinline__ void CopyRun(const uint8_t *srcRow, uint8_t *dstRow, int w, int sx, int step, int dx0)
+{
+    if (dx0 + kRunPixels > w)
+    {
+        for (int k = 0; k < w - dx0; ++k)
+        {
+            CopyPixel<T, C>(srcRow, dstRow, sx + step * k, dx0 + k);
+        }
+        return;
+    }
+    T         in[kRunPixels * C], out[kRunPixels * C];
+    const int first = step > 0 ? sx : sx - (kRunPixels - 1);
+    LoadRun<T, kRunPixels * C>(srcRow + (int64_t)first * C * sizeof(T), in);
+#pragma unroll
+    for (int k = 0; k < kRunPixels; ++k)
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[k * C + c] = step > 0 ? in[k * C + c] : in[(kRunPixels - 1 - k) * C + c];
+        }
+    }
+    StoreRunNT<T, kRunPixels * C>(dstRow + (int64_t)dx0 * C * sizeof(T), out);
+}
+
 template<class T, int C>
 __global__ __launch_bounds__(256) void PixelMapTensor(const CopyArgs a)
 {
-    const int x = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int y = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int x = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int y = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x >= a.w || y >= a.h)
     {
         return;
     }
     const int n = blockIdx.z;
-    CopyPixel<T, C>(a.src + n * a.srcN + (int64_t)(a.y0 + a.stepY * y) * a.srcRow,
-                    a.dst + n * a.dstN + (int64_t)y * a.dstRow, a.x0 + a.stepX * x, x);
+    CopyRun<T, C>(a.src + n * a.srcN + (int64_t)(a.y0 + a.stepY * y) * a.srcRow, a.dst + n * a.dstN + (int64_t)y * a.dstRow,
+                  a.w, a.x0 + a.stepX * x, a.stepX, x);
 }
 
 template<class T, int C>
@@ -119,8 +149,8 @@ __global__ __launch_bounds__(256) void FlipVarShape(const CopyArgs a, const VarT
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x  = tc.tx * 64 + (threadIdx.x & 63);
-    const int                    y  = tc.ty * 4 + (threadIdx.x >> 6);
+    const int                    x  = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
     if (x >= d.width || y >= d.height)
     {
         return;
@@ -128,7 +158,8 @@ __global__ __launch_bounds__(256) void FlipVarShape(const CopyArgs a, const VarT
     const int  code    = *reinterpret_cast<const int32_t *>(a.codes + tc.image * a.codeStride);
     const bool mirrorX = code == 1 || code == -1, mirrorY = code == 0 || code == -1;
     const int  sx = mirrorX ? d.width - 1 - x : x, sy = mirrorY ? d.height - 1 - y : y;
-    CopyPixel<T, C>(s.basePtr + (int64_t)sy * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, sx, x);
+    CopyRun<T, C>(s.basePtr + (int64_t)sy * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, sx,
+                  mirrorX ? -1 : 1, x);
 }
 
 void LaunchRowCopy(const CopyArgs &a, int N, hipStream_t stream)
@@ -147,7 +178,7 @@ void LaunchPixelMap(const CopyArgs &a, int N, const NVCVImageBufferStrided *dstH
 {
     if (dstHost == nullptr)
     {
-        dim3 grid(DivUp(a.w, 64), DivUp(a.h, 4), N);
+        dim3 grid(DivUp(a.w, kRunTileW), DivUp(a.h, kRunTileH), N);
         hipLaunchKernelGGL((PixelMapTensor<T, C>), grid, dim3(256), 0, stream, a);
         CheckLaunch("PixelMapTensor");
         return;
@@ -155,7 +186,7 @@ void LaunchPixelMap(const CopyArgs &a, int N, const NVCVImageBufferStrided *dstH
     for (int first = 0; first < N; first += kMaxTileImages)
     {
         VarTiles tiles;
-        int      total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), 64, 4);
+        int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kRunTileW, kRunTileH);
         if (total > 0)
         {
             hipLaunchKernelGGL((FlipVarShape<T, C>), dim3(total), dim3(256), 0, stream, a, tiles);

@@ -13,6 +13,7 @@
 #include "CvtColorFamilies.hpp"
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "RunIO.hpp"
 #include "VarShapeTiles.hpp"
 
 #include <cvcuda/OpCvtColor.h>
@@ -234,18 +235,55 @@ __device__ __forceinline__ void SwizzlePixel(const uint8_t *srcRow, uint8_t *dst
     }
 }
 
+// Pixels x0 .. x0+3 of a row (a run per lane); the ragged end of a row goes pixel by pixel.
+template<class T, int SCH, int DCH>
+__device__ __forceinline__ void SwizzleRun(const uint8_t *srcRow, uint8_t *dstRow, int W, int x0, int bidx,
+                                           uint64_t alpha)
+{
+    if (x0 + kRunPixels > W)
+    {
+        for (int x = x0; x < W; ++x)
+        {
+            SwizzlePixel<T, SCH, DCH>(srcRow, dstRow, x, bidx, alpha);
+        }
+        return;
+    }
+    T in[kRunPixels * SCH], out[kRunPixels * DCH];
+    LoadRun<T, kRunPixels * SCH>(srcRow + (int64_t)x0 * SCH * sizeof(T), in);
+    const bool swap = bidx != 0;
+#pragma unroll
+    for (int k = 0; k < kRunPixels; ++k)
+    {
+        out[k * DCH + 0] = swap ? in[k * SCH + 2] : in[k * SCH + 0];
+        out[k * DCH + 1] = in[k * SCH + 1];
+        out[k * DCH + 2] = swap ? in[k * SCH + 0] : in[k * SCH + 2];
+        if constexpr (DCH == 4)
+        {
+            if constexpr (SCH == 4)
+            {
+                out[k * DCH + 3] = in[k * SCH + 3];
+            }
+            else
+            {
+                out[k * DCH + 3] = (T)alpha;
+            }
+        }
+    }
+    StoreRunNT<T, kRunPixels * DCH>(dstRow + (int64_t)x0 * DCH * sizeof(T), out);
+}
+
 template<class T, int SCH, int DCH>
 __global__ __launch_bounds__(256) void SwizzleTensor(const SwizzleArgs a)
 {
-    const int x = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int y = blockIdx.y * 4 + (threadIdx.x >> 6);
-    if (x >= a.W || y >= a.H)
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= a.W || y >= a.H)
     {
         return;
     }
     const int n = blockIdx.z;
-    SwizzlePixel<T, SCH, DCH>(a.srcBase + n * a.srcSampleStride + (int64_t)y * a.srcRowStride,
-                              a.dstBase + n * a.dstSampleStride + (int64_t)y * a.dstRowStride, x, a.bidx, a.alpha);
+    SwizzleRun<T, SCH, DCH>(a.srcBase + n * a.srcSampleStride + (int64_t)y * a.srcRowStride,
+                            a.dstBase + n * a.dstSampleStride + (int64_t)y * a.dstRowStride, a.W, x0, a.bidx, a.alpha);
 }
 
 template<class T, int SCH, int DCH>
@@ -254,14 +292,14 @@ __global__ __launch_bounds__(256) void SwizzleVarShape(const SwizzleArgs a, cons
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x  = tc.tx * 64 + (threadIdx.x & 63);
-    const int                    y  = tc.ty * 4 + (threadIdx.x >> 6);
-    if (x >= d.width || y >= d.height)
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= d.width || y >= d.height)
     {
         return;
     }
-    SwizzlePixel<T, SCH, DCH>(s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, x, a.bidx,
-                              a.alpha);
+    SwizzleRun<T, SCH, DCH>(s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, x0,
+                            a.bidx, a.alpha);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -358,7 +396,7 @@ void LaunchSwizzle(const SwizzleArgs &a, int N, const NVCVImageBufferStrided *ds
 {
     if (dstHost == nullptr)
     {
-        dim3 grid(DivUp(a.W, 64), DivUp(a.H, 4), N);
+        dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), N);
         hipLaunchKernelGGL((SwizzleTensor<T, SCH, DCH>), grid, dim3(256), 0, stream, a);
         CheckLaunch("SwizzleTensor");
         return;
@@ -366,7 +404,7 @@ void LaunchSwizzle(const SwizzleArgs &a, int N, const NVCVImageBufferStrided *ds
     for (int first = 0; first < N; first += kMaxTileImages)
     {
         VarTiles tiles;
-        int      total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), 64, 4);
+        int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kRunTileW, kRunTileH);
         if (total > 0)
         {
             hipLaunchKernelGGL((SwizzleVarShape<T, SCH, DCH>), dim3(total), dim3(256), 0, stream, a, tiles);

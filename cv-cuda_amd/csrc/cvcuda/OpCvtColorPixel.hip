@@ -16,6 +16,7 @@
 // vector access, streaming stores. Var-shape batches use the packed tile grid.
 #include "CvtColorFamilies.hpp"
 #include "DeviceUtils.hpp"
+#include "RunIO.hpp"
 #include "VarShapeTiles.hpp"
 
 #include <algorithm>
@@ -41,6 +42,8 @@ struct PixArgs
 template<class T, int C>
 struct __attribute__((packed, aligned(sizeof(T)))) Px
 {
+    using Elem              = T;
+    static constexpr int kC = C;
     T v[C];
 };
 
@@ -93,10 +96,10 @@ template<class T, int SCH>
 struct GrayFromBgr
 {
     static constexpr int kItemW = 1, kItemH = 1;
+    using Src = Px<T, SCH>;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int x, int y)
+    static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
-        const Px<T, SCH> s = reinterpret_cast<const Px<T, SCH> *>(v.src + (int64_t)y * v.srcRow)[x];
         const T          b = s.v[a.bidx], g = s.v[1], r = s.v[a.bidx ^ 2];
         Px<T, 1>         o;
         if constexpr (std::is_integral_v<T>)
@@ -107,7 +110,7 @@ struct GrayFromBgr
         {
             o.v[0] = b * 0.114f + g * 0.587f + r * 0.299f;
         }
-        StorePx<T, 1>(v.dst + (int64_t)y * v.dstRow, x, o);
+        return o;
     }
 };
 
@@ -115,17 +118,18 @@ template<class T, int DCH>
 struct BgrFromGray
 {
     static constexpr int kItemW = 1, kItemH = 1;
+    using Src = Px<T, 1>;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &, int x, int y)
+    static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &)
     {
-        const T    g = reinterpret_cast<const T *>(v.src + (int64_t)y * v.srcRow)[x];
+        const T    g = s.v[0];
         Px<T, DCH> o;
 #pragma unroll
         for (int c = 0; c < DCH; ++c)
         {
             o.v[c] = g;
         }
-        StorePx<T, DCH>(v.dst + (int64_t)y * v.dstRow, x, o);
+        return o;
     }
 };
 
@@ -133,10 +137,10 @@ template<class T>
 struct YuvFromBgr
 {
     static constexpr int kItemW = 1, kItemH = 1;
+    using Src = Px<T, 3>;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int x, int y)
+    static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
-        const Px<T, 3> s = reinterpret_cast<const Px<T, 3> *>(v.src + (int64_t)y * v.srcRow)[x];
         Px<T, 3>       o;
         if constexpr (std::is_integral_v<T>)
         {
@@ -157,7 +161,7 @@ struct YuvFromBgr
             o.v[2]        = (R - Y) * 0.877f + 0.5f;
             o.v[1]        = (B - Y) * 0.492f + 0.5f;
         }
-        StorePx<T, 3>(v.dst + (int64_t)y * v.dstRow, x, o);
+        return o;
     }
 };
 
@@ -165,10 +169,10 @@ template<class T>
 struct BgrFromYuv
 {
     static constexpr int kItemW = 1, kItemH = 1;
+    using Src = Px<T, 3>;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int x, int y)
+    static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
-        const Px<T, 3> s = reinterpret_cast<const Px<T, 3> *>(v.src + (int64_t)y * v.srcRow)[x];
         Px<T, 3>       o;
         T              b, g, r;
         if constexpr (std::is_integral_v<T>)
@@ -189,7 +193,7 @@ struct BgrFromYuv
         o.v[a.bidx]     = b;
         o.v[1]          = g;
         o.v[a.bidx ^ 2] = r;
-        StorePx<T, 3>(v.dst + (int64_t)y * v.dstRow, x, o);
+        return o;
     }
 };
 
@@ -197,10 +201,10 @@ template<class T>
 struct HsvFromBgr
 {
     static constexpr int kItemW = 1, kItemH = 1;
+    using Src = Px<T, 3>;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int x, int y)
+    static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
-        const Px<T, 3> s = reinterpret_cast<const Px<T, 3> *>(v.src + (int64_t)y * v.srcRow)[x];
         Px<T, 3>       o;
         if constexpr (std::is_integral_v<T>)
         {
@@ -249,7 +253,7 @@ struct HsvFromBgr
             o.v[1] = sat;
             o.v[2] = val;
         }
-        StorePx<T, 3>(v.dst + (int64_t)y * v.dstRow, x, o);
+        return o;
     }
 };
 
@@ -282,10 +286,10 @@ template<class T, int DCH>
 struct BgrFromHsv
 {
     static constexpr int kItemW = 1, kItemH = 1;
+    using Src = Px<T, 3>;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int x, int y)
+    static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
-        const Px<T, 3> s = reinterpret_cast<const Px<T, 3> *>(v.src + (int64_t)y * v.srcRow)[x];
         Px<T, DCH>     o;
         T              b, g, r;
         if constexpr (std::is_integral_v<T>)
@@ -308,7 +312,7 @@ struct BgrFromHsv
         {
             o.v[3] = AlphaOf<T>();
         }
-        StorePx<T, DCH>(v.dst + (int64_t)y * v.dstRow, x, o);
+        return o;
     }
 };
 
@@ -429,6 +433,74 @@ struct GrayFromYuv420
 };
 
 // ---- kernels -----------------------------------------------------------------------------------------
+// One pixel in, one pixel out (Op::Map): runs of 4 pixels per lane, one row per wave.
+template<class Op>
+__device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, int W, int x0, const PixArgs &a)
+{
+    using S  = typename Op::Src;
+    using D  = decltype(Op::Map(S{}, a));
+    using TS = typename S::Elem;
+    using TD = typename D::Elem;
+    if (x0 + kRunPixels > W)
+    {
+        for (int x = x0; x < W; ++x)
+        {
+            reinterpret_cast<D *>(dstRow)[x] = Op::Map(reinterpret_cast<const S *>(srcRow)[x], a);
+        }
+        return;
+    }
+    TS in[kRunPixels * S::kC];
+    TD out[kRunPixels * D::kC];
+    LoadRun<TS, kRunPixels * S::kC>(srcRow + (int64_t)x0 * sizeof(S), in);
+#pragma unroll
+    for (int k = 0; k < kRunPixels; ++k)
+    {
+        S s;
+#pragma unroll
+        for (int c = 0; c < S::kC; ++c)
+        {
+            s.v[c] = in[k * S::kC + c];
+        }
+        const D d = Op::Map(s, a);
+#pragma unroll
+        for (int c = 0; c < D::kC; ++c)
+        {
+            out[k * D::kC + c] = d.v[c];
+        }
+    }
+    StoreRunNT<TD, kRunPixels * D::kC>(dstRow + (int64_t)x0 * sizeof(D), out);
+}
+
+template<class Op>
+__global__ __launch_bounds__(256) void MapTensor(const PixArgs a)
+{
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= a.W || y >= a.H)
+    {
+        return;
+    }
+    const int n = blockIdx.z;
+    MapRun<Op>(a.src + n * a.srcN + (int64_t)y * a.srcRow, a.dst + n * a.dstN + (int64_t)y * a.dstRow, a.W, x0, a);
+}
+
+// var-shape: the size comes from the destination image
+template<class Op>
+__global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTiles tiles)
+{
+    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
+    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= d.width || y >= d.height)
+    {
+        return;
+    }
+    MapRun<Op>(s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, x0, a);
+}
+
+// Subsampled formats: one work item (Op::kItemW x Op::kItemH pixels) per lane, tensors only.
 template<class Op>
 __global__ __launch_bounds__(256) void PixelTensor(const PixArgs a)
 {
@@ -440,24 +512,6 @@ __global__ __launch_bounds__(256) void PixelTensor(const PixArgs a)
     }
     const int  n = blockIdx.z;
     const View v = {a.src + n * a.srcN, a.dst + n * a.dstN, a.srcRow, a.dstRow, a.W, a.H};
-    Op::Run(v, a, x, y);
-}
-
-// var-shape: one pixel per item only; the size comes from the destination image
-template<class Op>
-__global__ __launch_bounds__(256) void PixelVarShape(const PixArgs a, const VarTiles tiles)
-{
-    static_assert(Op::kItemW == 1 && Op::kItemH == 1);
-    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
-    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
-    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x  = tc.tx * 64 + (threadIdx.x & 63);
-    const int                    y  = tc.ty * 4 + (threadIdx.x >> 6);
-    if (x >= d.width || y >= d.height)
-    {
-        return;
-    }
-    const View v = {s.basePtr, d.basePtr, s.rowStride, d.rowStride, d.width, d.height};
     Op::Run(v, a, x, y);
 }
 
@@ -484,8 +538,38 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
     {
         return;
     }
-    if (io.dstHost == nullptr)
+    if constexpr (Op::kItemW == 1 && Op::kItemH == 1)
     {
+        if (io.dstHost == nullptr)
+        {
+            if (a.W == 0 || a.H == 0)
+            {
+                return;
+            }
+            dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), io.N);
+            hipLaunchKernelGGL((MapTensor<Op>), grid, dim3(256), 0, stream, a);
+            CheckLaunch("MapTensor");
+            return;
+        }
+        for (int first = 0; first < io.N; first += kMaxTileImages)
+        {
+            VarTiles tiles;
+            int      total = BuildVarTiles(tiles, io.dstHost, first, std::min(kMaxTileImages, io.N - first), kRunTileW,
+                                           kRunTileH);
+            if (total > 0)
+            {
+                hipLaunchKernelGGL((MapVarShape<Op>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("MapVarShape");
+            }
+        }
+    }
+    else
+    {
+        if (io.dstHost != nullptr)
+        {
+            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
+                          "Conversions to or from subsampled YUV formats are not available for image batches");
+        }
         a.itemsW = a.W / Op::kItemW;
         a.itemsH = a.H / Op::kItemH;
         if (a.itemsW == 0 || a.itemsH == 0)
@@ -495,25 +579,6 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
         dim3 grid(DivUp(a.itemsW, 64), DivUp(a.itemsH, 4), io.N);
         hipLaunchKernelGGL((PixelTensor<Op>), grid, dim3(256), 0, stream, a);
         CheckLaunch("PixelTensor");
-        return;
-    }
-    if constexpr (Op::kItemW == 1 && Op::kItemH == 1)
-    {
-        for (int first = 0; first < io.N; first += kMaxTileImages)
-        {
-            VarTiles tiles;
-            int      total = BuildVarTiles(tiles, io.dstHost, first, std::min(kMaxTileImages, io.N - first), 64, 4);
-            if (total > 0)
-            {
-                hipLaunchKernelGGL((PixelVarShape<Op>), dim3(total), dim3(256), 0, stream, a, tiles);
-                CheckLaunch("PixelVarShape");
-            }
-        }
-    }
-    else
-    {
-        throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
-                      "Conversions to or from subsampled YUV formats are not available for image batches");
     }
 }
 

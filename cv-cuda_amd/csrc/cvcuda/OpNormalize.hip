@@ -6,11 +6,13 @@
 // normalize_var_shape.cu:36-68, 227-308 for var-shape batches (there the output may be u8 or f32
 // whatever the input type, and base/scale are one value or one value per channel).
 //
-// Kernel shape: one lane per pixel (all channels of the pixel as one vector access on both sides),
-// 64 columns x 4 rows per block, streaming stores. base/scale are addressed with per-dimension
-// strides that are 0 along broadcast dimensions.
+// Kernel shapes: base/scale that vary per channel only (the usual mean/stddev vectors, and always
+// for var-shape batches) are read once per wave and the image is streamed in runs of 4 pixels per
+// lane; base/scale with extents along N, H or W go through the generic kernel, one lane per pixel,
+// which addresses them with per-dimension strides that are 0 along broadcast dimensions.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "RunIO.hpp"
 #include "VarShapeTiles.hpp"
 
 #include <cvcuda/OpNormalize.h>
@@ -103,9 +105,110 @@ __global__ __launch_bounds__(256) void NormVarShape(const NormArgs a, const VarT
     NormPixel<TI, TO, C>(a, s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, 0, 0, x);
 }
 
+// Per-channel base/scale: runs of 4 pixels per lane, one row per wave.
+template<class TI, class TO, int C>
+__device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow, uint8_t *dstRow, int W, int x0)
+{
+    float b[C], m[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        b[c]          = a.base.ptr[c * a.base.sC];
+        const float s = a.scale.ptr[c * a.scale.sC];
+        if (a.stddev)
+        {
+            const float t = s * s + a.eps;
+            m[c]          = 1.0f / sqrtf(t);
+        }
+        else
+        {
+            m[c] = s;
+        }
+    }
+    if (x0 + kRunPixels <= W)
+    {
+        TI in[kRunPixels * C];
+        TO out[kRunPixels * C];
+        LoadRun<TI, kRunPixels * C>(srcRow + (int64_t)x0 * C * sizeof(TI), in);
+#pragma unroll
+        for (int i = 0; i < kRunPixels * C; ++i)
+        {
+            out[i] = SaturateCast<TO>(((float)in[i] - b[i % C]) * m[i % C] * a.gscale + a.shift);
+        }
+        StoreRunNT<TO, kRunPixels * C>(dstRow + (int64_t)x0 * C * sizeof(TO), out);
+    }
+    else
+    {
+        for (int x = x0; x < W; ++x)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                const float v = ((float)reinterpret_cast<const TI *>(srcRow)[x * C + c] - b[c]) * m[c] * a.gscale + a.shift;
+                reinterpret_cast<TO *>(dstRow)[x * C + c] = SaturateCast<TO>(v);
+            }
+        }
+    }
+}
+
+template<class TI, class TO, int C>
+__global__ __launch_bounds__(256) void NormRunsTensor(const NormArgs a)
+{
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= a.W || y >= a.H)
+    {
+        return;
+    }
+    const int n = blockIdx.z;
+    NormRun<TI, TO, C>(a, a.src + n * a.srcN + (int64_t)y * a.srcRow, a.dst + n * a.dstN + (int64_t)y * a.dstRow, a.W,
+                       x0);
+}
+
+template<class TI, class TO, int C>
+__global__ __launch_bounds__(256) void NormRunsVarShape(const NormArgs a, const VarTiles tiles)
+{
+    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
+    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= d.width || y >= d.height)
+    {
+        return;
+    }
+    NormRun<TI, TO, C>(a, s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, x0);
+}
+
+inline bool PerChannelOnly(const ParamView &p)
+{
+    return p.sN == 0 && p.sH == 0 && p.sW == 0;
+}
+
 template<class TI, class TO, int C>
 void Launch(const NormArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
 {
+    if (PerChannelOnly(a.base) && PerChannelOnly(a.scale))
+    {
+        if (dstHost == nullptr)
+        {
+            dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), N);
+            hipLaunchKernelGGL((NormRunsTensor<TI, TO, C>), grid, dim3(256), 0, stream, a);
+            CheckLaunch("NormRunsTensor");
+            return;
+        }
+        for (int first = 0; first < N; first += kMaxTileImages)
+        {
+            VarTiles tiles;
+            int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kRunTileW, kRunTileH);
+            if (total > 0)
+            {
+                hipLaunchKernelGGL((NormRunsVarShape<TI, TO, C>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("NormRunsVarShape");
+            }
+        }
+        return;
+    }
     if (dstHost == nullptr)
     {
         dim3 grid(DivUp(a.W, 64), DivUp(a.H, 4), N);

@@ -4,11 +4,14 @@
 // element (n,y,x,c) of the output, whatever the two memory layouts are) and its validation (:118-197).
 // Only the bytes of real elements are written; row/plane padding of the output is left untouched.
 //
-// Kernel shape: one lane per pixel, 64 columns x 4 rows per block. The interleaved side of the
-// transfer moves all C channels of the pixel with one vector access, the planar side is one element
-// per lane per plane, i.e. contiguous across the wave on both sides. Stores are streaming.
+// Kernel shapes. Packed rows of 1- and 2-byte elements (interleaved: pixel stride C elements; planar:
+// pixel stride one element) move in runs of 4 pixels per lane: one vector load per lane on an
+// interleaved side, one 4-element access per plane on a planar side, whole-dword streaming stores.
+// Everything else: one lane per pixel, 64 columns x 4 rows per block, the interleaved side as one
+// vector access, the planar side one element per lane per plane.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "RunIO.hpp"
 
 #include <cvcuda/OpReformat.h>
 
@@ -76,9 +79,103 @@ __global__ __launch_bounds__(256) void ReformatKernel(const ReformatArgs a)
     }
 }
 
+// Runs of 4 pixels per lane; SRC_IL / DST_IL: interleaved packed rows, otherwise planar packed rows.
+template<class T, int C, bool SRC_IL, bool DST_IL>
+__global__ __launch_bounds__(256) void ReformatRunsKernel(const ReformatArgs a)
+{
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
+    if (x0 >= a.W || y >= a.H)
+    {
+        return;
+    }
+    const int      n = blockIdx.z;
+    const uint8_t *s = a.src + n * a.sN + y * a.sH + x0 * a.sW;
+    uint8_t       *d = a.dst + n * a.dN + y * a.dH + x0 * a.dW;
+    if (x0 + kRunPixels > a.W)
+    {
+        for (int x = 0; x < a.W - x0; ++x)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                *reinterpret_cast<T *>(d + x * a.dW + c * a.dC) = *reinterpret_cast<const T *>(s + x * a.sW + c * a.sC);
+            }
+        }
+        return;
+    }
+    T px[kRunPixels * C]; // pixel-major
+    if constexpr (SRC_IL)
+    {
+        LoadRun<T, kRunPixels * C>(s, px);
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            T t[kRunPixels];
+            LoadRun<T, kRunPixels>(s + c * a.sC, t);
+#pragma unroll
+            for (int k = 0; k < kRunPixels; ++k)
+            {
+                px[k * C + c] = t[k];
+            }
+        }
+    }
+    if constexpr (DST_IL)
+    {
+        StoreRunNT<T, kRunPixels * C>(d, px);
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            T t[kRunPixels];
+#pragma unroll
+            for (int k = 0; k < kRunPixels; ++k)
+            {
+                t[k] = px[k * C + c];
+            }
+            StoreRunNT<T, kRunPixels>(d + c * a.dC, t);
+        }
+    }
+}
+
 template<class T, int C>
 void LaunchC(const ReformatArgs &a, int N, bool srcIl, bool dstIl, hipStream_t stream)
 {
+    if constexpr (sizeof(T) <= 2)
+    {
+        const bool srcPlanar = a.sW == (int64_t)sizeof(T), dstPlanar = a.dW == (int64_t)sizeof(T);
+        const bool srcPacked = (srcIl && a.sW == (int64_t)(C * sizeof(T))) || srcPlanar;
+        const bool dstPacked = (dstIl && a.dW == (int64_t)(C * sizeof(T))) || dstPlanar;
+        if (srcPacked && dstPacked)
+        {
+            dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), N), block(256);
+            // C == 1: interleaved and planar coincide
+            const bool sIl = srcIl && !(C == 1), dIl = dstIl && !(C == 1);
+            if (sIl && dIl)
+            {
+                hipLaunchKernelGGL((ReformatRunsKernel<T, C, true, true>), grid, block, 0, stream, a);
+            }
+            else if (sIl)
+            {
+                hipLaunchKernelGGL((ReformatRunsKernel<T, C, true, false>), grid, block, 0, stream, a);
+            }
+            else if (dIl)
+            {
+                hipLaunchKernelGGL((ReformatRunsKernel<T, C, false, true>), grid, block, 0, stream, a);
+            }
+            else
+            {
+                hipLaunchKernelGGL((ReformatRunsKernel<T, C, false, false>), grid, block, 0, stream, a);
+            }
+            CheckLaunch("ReformatRunsKernel");
+            return;
+        }
+    }
     dim3 grid(DivUp(a.W, 64), DivUp(a.H, 4), N), block(256);
     if (srcIl && dstIl)
     {
