@@ -101,12 +101,13 @@ __device__ __forceinline__ void CopyPixel(const uint8_t *srcRow, uint8_t *dstRow
     }
 }
 
-// dst pixels dx0 .. dx0+3 of a row  <-  src pixels sx, sx + step, .. (step = +1 / -1); the ragged end
-// of a row goes pixel by pixel
+// a run of dst pixels from dx0 on  <-  src pixels sx, sx + step, .. (step = +1 / -1, wave-uniform); the
+// ragged end of a row goes pixel by pixel
 template<class T, int C>
 __device__ __forceinline__ void CopyRun(const uint8_t *srcRow, uint8_t *dstRow, int w, int sx, int step, int dx0)
 {
-    if (dx0 + kRunPixels > w)
+    constexpr int P = kRunPixelsFor<T, T>;
+    if (dx0 + P > w)
     {
         for (int k = 0; k < w - dx0; ++k)
         {
@@ -114,25 +115,30 @@ __device__ __forceinline__ void CopyRun(const uint8_t *srcRow, uint8_t *dstRow, 
         }
         return;
     }
-    T         in[kRunPixels * C], out[kRunPixels * C];
-    const int first = step > 0 ? sx : sx - (kRunPixels - 1);
-    LoadRun<T, kRunPixels * C>(srcRow + (int64_t)first * C * sizeof(T), in);
+    T         in[P * C], out[P * C];
+    const int first = step > 0 ? sx : sx - (P - 1);
+    LoadRun<T, P * C>(srcRow + (int64_t)first * C * sizeof(T), in);
+    if (step > 0)
+    {
+        StoreRunNT<T, P * C>(dstRow + (int64_t)dx0 * C * sizeof(T), in);
+        return;
+    }
 #pragma unroll
-    for (int k = 0; k < kRunPixels; ++k)
+    for (int k = 0; k < P; ++k)
     {
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
-            out[k * C + c] = step > 0 ? in[k * C + c] : in[(kRunPixels - 1 - k) * C + c];
+            out[k * C + c] = in[(P - 1 - k) * C + c];
         }
     }
-    StoreRunNT<T, kRunPixels * C>(dstRow + (int64_t)dx0 * C * sizeof(T), out);
+    StoreRunNT<T, P * C>(dstRow + (int64_t)dx0 * C * sizeof(T), out);
 }
 
 template<class T, int C>
 __global__ __launch_bounds__(256) void PixelMapTensor(const CopyArgs a)
 {
-    const int x = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int x = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixelsFor<T, T>;
     const int y = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x >= a.w || y >= a.h)
     {
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(256) void FlipVarShape(const CopyArgs a, const VarT
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x  = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    x  = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixelsFor<T, T>;
     const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
     if (x >= d.width || y >= d.height)
     {
@@ -178,7 +184,7 @@ void LaunchPixelMap(const CopyArgs &a, int N, const NVCVImageBufferStrided *dstH
 {
     if (dstHost == nullptr)
     {
-        dim3 grid(DivUp(a.w, kRunTileW), DivUp(a.h, kRunTileH), N);
+        dim3 grid(DivUp(a.w, 64 * kRunPixelsFor<T, T>), DivUp(a.h, kRunTileH), N);
         hipLaunchKernelGGL((PixelMapTensor<T, C>), grid, dim3(256), 0, stream, a);
         CheckLaunch("PixelMapTensor");
         return;
@@ -186,7 +192,8 @@ void LaunchPixelMap(const CopyArgs &a, int N, const NVCVImageBufferStrided *dstH
     for (int first = 0; first < N; first += kMaxTileImages)
     {
         VarTiles tiles;
-        int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kRunTileW, kRunTileH);
+        int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), 64 * kRunPixelsFor<T, T>,
+                                  kRunTileH);
         if (total > 0)
         {
             hipLaunchKernelGGL((FlipVarShape<T, C>), dim3(total), dim3(256), 0, stream, a, tiles);

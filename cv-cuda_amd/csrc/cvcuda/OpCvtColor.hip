@@ -235,12 +235,13 @@ __device__ __forceinline__ void SwizzlePixel(const uint8_t *srcRow, uint8_t *dst
     }
 }
 
-// Pixels x0 .. x0+3 of a row (a run per lane); the ragged end of a row goes pixel by pixel.
+// A run of pixels of a row from x0 on (one run per lane); the ragged end of a row goes pixel by pixel.
 template<class T, int SCH, int DCH>
 __device__ __forceinline__ void SwizzleRun(const uint8_t *srcRow, uint8_t *dstRow, int W, int x0, int bidx,
                                            uint64_t alpha)
 {
-    if (x0 + kRunPixels > W)
+    constexpr int P = kRunPixelsFor<T, T>;
+    if (x0 + P > W)
     {
         for (int x = x0; x < W; ++x)
         {
@@ -248,11 +249,11 @@ __device__ __forceinline__ void SwizzleRun(const uint8_t *srcRow, uint8_t *dstRo
         }
         return;
     }
-    T in[kRunPixels * SCH], out[kRunPixels * DCH];
-    LoadRun<T, kRunPixels * SCH>(srcRow + (int64_t)x0 * SCH * sizeof(T), in);
+    T in[P * SCH], out[P * DCH];
+    LoadRun<T, P * SCH>(srcRow + (int64_t)x0 * SCH * sizeof(T), in);
     const bool swap = bidx != 0;
 #pragma unroll
-    for (int k = 0; k < kRunPixels; ++k)
+    for (int k = 0; k < P; ++k)
     {
         out[k * DCH + 0] = swap ? in[k * SCH + 2] : in[k * SCH + 0];
         out[k * DCH + 1] = in[k * SCH + 1];
@@ -269,13 +270,13 @@ __device__ __forceinline__ void SwizzleRun(const uint8_t *srcRow, uint8_t *dstRo
             }
         }
     }
-    StoreRunNT<T, kRunPixels * DCH>(dstRow + (int64_t)x0 * DCH * sizeof(T), out);
+    StoreRunNT<T, P * DCH>(dstRow + (int64_t)x0 * DCH * sizeof(T), out);
 }
 
 template<class T, int SCH, int DCH>
 __global__ __launch_bounds__(256) void SwizzleTensor(const SwizzleArgs a)
 {
-    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixelsFor<T, T>;
     const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= a.W || y >= a.H)
     {
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(256) void SwizzleVarShape(const SwizzleArgs a, cons
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixelsFor<T, T>;
     const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= d.width || y >= d.height)
     {
@@ -396,7 +397,7 @@ void LaunchSwizzle(const SwizzleArgs &a, int N, const NVCVImageBufferStrided *ds
 {
     if (dstHost == nullptr)
     {
-        dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), N);
+        dim3 grid(DivUp(a.W, 64 * kRunPixelsFor<T, T>), DivUp(a.H, kRunTileH), N);
         hipLaunchKernelGGL((SwizzleTensor<T, SCH, DCH>), grid, dim3(256), 0, stream, a);
         CheckLaunch("SwizzleTensor");
         return;
@@ -404,7 +405,8 @@ void LaunchSwizzle(const SwizzleArgs &a, int N, const NVCVImageBufferStrided *ds
     for (int first = 0; first < N; first += kMaxTileImages)
     {
         VarTiles tiles;
-        int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kRunTileW, kRunTileH);
+        int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), 64 * kRunPixelsFor<T, T>,
+                                  kRunTileH);
         if (total > 0)
         {
             hipLaunchKernelGGL((SwizzleVarShape<T, SCH, DCH>), dim3(total), dim3(256), 0, stream, a, tiles);

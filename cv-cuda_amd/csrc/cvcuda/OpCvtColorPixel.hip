@@ -433,7 +433,11 @@ struct GrayFromYuv420
 };
 
 // ---- kernels -----------------------------------------------------------------------------------------
-// One pixel in, one pixel out (Op::Map): runs of 4 pixels per lane, one row per wave.
+// Pixels per lane of a one-in, one-out operation (input and output elements have the same type).
+template<class Op>
+constexpr int kMapRun = kRunPixelsFor<typename Op::Src::Elem, typename Op::Src::Elem>;
+
+// One pixel in, one pixel out (Op::Map): runs of kMapRun<Op> pixels per lane, one row per wave.
 template<class Op>
 __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, int W, int x0, const PixArgs &a)
 {
@@ -441,7 +445,8 @@ __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, i
     using D  = decltype(Op::Map(S{}, a));
     using TS = typename S::Elem;
     using TD = typename D::Elem;
-    if (x0 + kRunPixels > W)
+    constexpr int P = kRunPixelsFor<TS, TD>;
+    if (x0 + P > W)
     {
         for (int x = x0; x < W; ++x)
         {
@@ -449,11 +454,11 @@ __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, i
         }
         return;
     }
-    TS in[kRunPixels * S::kC];
-    TD out[kRunPixels * D::kC];
-    LoadRun<TS, kRunPixels * S::kC>(srcRow + (int64_t)x0 * sizeof(S), in);
+    TS in[P * S::kC];
+    TD out[P * D::kC];
+    LoadRun<TS, P * S::kC>(srcRow + (int64_t)x0 * sizeof(S), in);
 #pragma unroll
-    for (int k = 0; k < kRunPixels; ++k)
+    for (int k = 0; k < P; ++k)
     {
         S s;
 #pragma unroll
@@ -468,13 +473,13 @@ __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, i
             out[k * D::kC + c] = d.v[c];
         }
     }
-    StoreRunNT<TD, kRunPixels * D::kC>(dstRow + (int64_t)x0 * sizeof(D), out);
+    StoreRunNT<TD, P * D::kC>(dstRow + (int64_t)x0 * sizeof(D), out);
 }
 
 template<class Op>
 __global__ __launch_bounds__(256) void MapTensor(const PixArgs a)
 {
-    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kMapRun<Op>;
     const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= a.W || y >= a.H)
     {
@@ -491,7 +496,7 @@ __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTil
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kMapRun<Op>;
     const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= d.width || y >= d.height)
     {
@@ -546,7 +551,7 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
             {
                 return;
             }
-            dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), io.N);
+            dim3 grid(DivUp(a.W, 64 * kMapRun<Op>), DivUp(a.H, kRunTileH), io.N);
             hipLaunchKernelGGL((MapTensor<Op>), grid, dim3(256), 0, stream, a);
             CheckLaunch("MapTensor");
             return;
@@ -554,8 +559,8 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
         for (int first = 0; first < io.N; first += kMaxTileImages)
         {
             VarTiles tiles;
-            int      total = BuildVarTiles(tiles, io.dstHost, first, std::min(kMaxTileImages, io.N - first), kRunTileW,
-                                           kRunTileH);
+            int      total = BuildVarTiles(tiles, io.dstHost, first, std::min(kMaxTileImages, io.N - first),
+                                           64 * kMapRun<Op>, kRunTileH);
             if (total > 0)
             {
                 hipLaunchKernelGGL((MapVarShape<Op>), dim3(total), dim3(256), 0, stream, a, tiles);

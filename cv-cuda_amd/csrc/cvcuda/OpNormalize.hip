@@ -105,10 +105,11 @@ __global__ __launch_bounds__(256) void NormVarShape(const NormArgs a, const VarT
     NormPixel<TI, TO, C>(a, s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, 0, 0, x);
 }
 
-// Per-channel base/scale: runs of 4 pixels per lane, one row per wave.
+// Per-channel base/scale: runs of P pixels per lane, one row per wave.
 template<class TI, class TO, int C>
 __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow, uint8_t *dstRow, int W, int x0)
 {
+    constexpr int P = kRunPixelsFor<TI, TO>;
     float b[C], m[C];
 #pragma unroll
     for (int c = 0; c < C; ++c)
@@ -125,17 +126,17 @@ __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow
             m[c] = s;
         }
     }
-    if (x0 + kRunPixels <= W)
+    if (x0 + P <= W)
     {
-        TI in[kRunPixels * C];
-        TO out[kRunPixels * C];
-        LoadRun<TI, kRunPixels * C>(srcRow + (int64_t)x0 * C * sizeof(TI), in);
+        TI in[P * C];
+        TO out[P * C];
+        LoadRun<TI, P * C>(srcRow + (int64_t)x0 * C * sizeof(TI), in);
 #pragma unroll
-        for (int i = 0; i < kRunPixels * C; ++i)
+        for (int i = 0; i < P * C; ++i)
         {
             out[i] = SaturateCast<TO>(((float)in[i] - b[i % C]) * m[i % C] * a.gscale + a.shift);
         }
-        StoreRunNT<TO, kRunPixels * C>(dstRow + (int64_t)x0 * C * sizeof(TO), out);
+        StoreRunNT<TO, P * C>(dstRow + (int64_t)x0 * C * sizeof(TO), out);
     }
     else
     {
@@ -154,7 +155,7 @@ __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow
 template<class TI, class TO, int C>
 __global__ __launch_bounds__(256) void NormRunsTensor(const NormArgs a)
 {
-    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixelsFor<TI, TO>;
     const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= a.W || y >= a.H)
     {
@@ -171,7 +172,7 @@ __global__ __launch_bounds__(256) void NormRunsVarShape(const NormArgs a, const 
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixels;
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixelsFor<TI, TO>;
     const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= d.width || y >= d.height)
     {
@@ -192,7 +193,7 @@ void Launch(const NormArgs &a, int N, const NVCVImageBufferStrided *dstHost, hip
     {
         if (dstHost == nullptr)
         {
-            dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH), N);
+            dim3 grid(DivUp(a.W, 64 * kRunPixelsFor<TI, TO>), DivUp(a.H, kRunTileH), N);
             hipLaunchKernelGGL((NormRunsTensor<TI, TO, C>), grid, dim3(256), 0, stream, a);
             CheckLaunch("NormRunsTensor");
             return;
@@ -200,7 +201,8 @@ void Launch(const NormArgs &a, int N, const NVCVImageBufferStrided *dstHost, hip
         for (int first = 0; first < N; first += kMaxTileImages)
         {
             VarTiles tiles;
-            int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kRunTileW, kRunTileH);
+            int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first),
+                                      64 * kRunPixelsFor<TI, TO>, kRunTileH);
             if (total > 0)
             {
                 hipLaunchKernelGGL((NormRunsVarShape<TI, TO, C>), dim3(total), dim3(256), 0, stream, a, tiles);

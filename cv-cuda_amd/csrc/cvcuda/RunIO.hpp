@@ -12,9 +12,14 @@
 
 namespace cvamd {
 
-constexpr int kRunPixels = 4;                 // pixels per lane
-constexpr int kRunTileW  = 64 * kRunPixels;   // columns per wave
-constexpr int kRunTileH  = 4;                 // rows per 256-thread block (one per wave)
+constexpr int kRunPixels = 4;               // pixels per lane ...
+constexpr int kRunTileW  = 64 * kRunPixels; // ... columns per wave
+constexpr int kRunTileH  = 4;               // rows per 256-thread block (one per wave)
+
+// Pixels of 4-byte elements on both sides are whole dwords already: one pixel per lane keeps a
+// wave's accesses dense (4-pixel runs of 12-16 byte pixels would stride each load by 48-64 bytes).
+template<class TS, class TD>
+constexpr int kRunPixelsFor = (sizeof(TS) >= 4 && sizeof(TD) >= 4) ? 1 : kRunPixels;
 
 template<class T, int N>
 struct __attribute__((packed, aligned(sizeof(T)))) Run
