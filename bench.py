@@ -299,6 +299,111 @@ class WarpC4:
         return 8
 
 
+class Streaming:
+    """Operators either side of the five configurations, each on a 1080p batch: algorithmic bytes are
+    the input plus the output, the check is the oracle (or the numpy index map) on the first image."""
+    config_id = 0
+    H, W = 1080, 1920
+    SPECS = {
+        # key: (operator, batch, in dtype/channels, out dtype/channels/layout, kernel, arithmetic type, text)
+        "cvtcolor-bgr2rgb": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "SwizzleTensor<uint8_t,3,3>", "u8",
+                             "CvtColor BGR2RGB"),
+        "cvtcolor-bgr2gray": ("CvtColor", 32, ("uint8", 3), ("uint8", 1, "NHWC"), "MapTensor<GrayFromBgr<uint8_t,3>>",
+                              "int32", "CvtColor BGR2GRAY"),
+        "normalize-u8": ("Normalize", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "NormRunsTensor<uint8_t,uint8_t,3>",
+                         "f32", "Normalize (per-channel base/scale)"),
+        "normalize-f32": ("Normalize", 16, ("float32", 3), ("float32", 3, "NHWC"), "NormRunsTensor<float,float,3>",
+                          "f32", "Normalize (per-channel base/scale)"),
+        "reformat-nhwc-nchw": ("Reformat", 32, ("uint8", 3), ("uint8", 3, "NCHW"),
+                               "ReformatRunsKernel<uint8_t,3,true,false>", "u8", "Reformat NHWC -> NCHW"),
+        "convertto-u8-f32": ("ConvertTo", 32, ("uint8", 3), ("float32", 3, "NHWC"), "ConvertKernel<uint8_t,float>",
+                             "f32", "ConvertTo x 1/255"),
+        "flip-horizontal": ("Flip", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "PixelMapTensor<uint8_t,3>", "u8",
+                            "Flip (columns mirrored)"),
+        "resize-linear-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
+                               "ResizePatchTensorKernel<uint8_t,3,LINEAR>", "f32", "Resize LINEAR 1920x1080 -> 1280x720"),
+        "resize-linear-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
+                                  "ResizePatchTensorKernel<uint8_t,3,LINEAR>", "f32",
+                                  "Resize LINEAR 1280x720 -> 1920x1080"),
+    }
+
+    def __init__(self, cv, orc, np, torch, key):
+        self.cv, self.orc, self.np, self.torch, self.key = cv, orc, np, torch, key
+        opname, self.N, src, dst, self.kernel, self.dtype, text = self.SPECS[key]
+        self.images = self.N
+        self.sdt, self.sc = np.dtype(src[0]), src[1]
+        self.sh, self.sw = (src[2], src[3]) if len(src) > 2 else (self.H, self.W)
+        self.ddt, self.dc, self.dlayout = np.dtype(dst[0]), dst[1], dst[2]
+        self.dh, self.dw = (dst[3], dst[4]) if len(dst) > 3 else (self.sh, self.sw)
+        self.workload = "%s: batch %d %s NHWC %dx%dx%d -> %s %s %dx%dx%d" % (
+            text, self.N, self.sdt.name, self.sw, self.sh, self.sc, self.ddt.name, self.dlayout, self.dw, self.dh, self.dc)
+        self.alg_bytes = self.N * (self.sh * self.sw * self.sc * self.sdt.itemsize
+                                   + self.dh * self.dw * self.dc * self.ddt.itemsize)
+        one = orc.fill_u8((1, self.sh, self.sw, self.sc), SEED_BASE + 77)
+        self.host1 = one if self.sdt == np.uint8 else (one.astype(np.float32) / 255.0)
+        self.dev1 = torch.from_numpy(self.host1).cuda()
+        self.op = getattr(cv, opname)()
+        self.opname = opname
+        if opname == "Normalize":
+            self.base = np.array([[[[104.0, 117.0, 123.0]]]], np.float32) / (1.0 if self.sdt == np.uint8 else 255.0)
+            self.scale = np.array([[[[0.9, 1.1, 1.3]]]], np.float32)
+            self.tbase, self.tscale = cv.Tensor.from_numpy(self.base, "NHWC"), cv.Tensor.from_numpy(self.scale, "NHWC")
+
+    def make_set(self):
+        tin = self.cv.Tensor.alloc([self.N, self.sh, self.sw, self.sc], self.sdt, "NHWC")
+        tin.torch_view().copy_(self.dev1.expand(self.N, -1, -1, -1))
+        shape = [self.N, self.dc, self.dh, self.dw] if self.dlayout == "NCHW" else [self.N, self.dh, self.dw, self.dc]
+        return tin, self.cv.Tensor.alloc(shape, self.ddt, self.dlayout)
+
+    def submit(self, stream, s):
+        K = self.cv.K
+        if self.opname == "CvtColor":
+            self.op(stream, s[0], s[1], K.COLOR_BGR2RGB if self.dc == 3 else K.COLOR_BGR2GRAY)
+        elif self.opname == "Normalize":
+            self.op(stream, s[0], self.tbase, self.tscale, s[1], 1.0, 0.0, 0.0, 0)
+        elif self.opname == "Reformat":
+            self.op(stream, s[0], s[1])
+        elif self.opname == "ConvertTo":
+            self.op(stream, s[0], s[1], 1.0 / 255.0, 0.0)
+        elif self.opname == "Flip":
+            self.op(stream, s[0], s[1], 1)
+        else:
+            self.op(stream, s[0], s[1], LINEAR)
+
+    def _reference(self, a, threads=1):
+        np, orc = self.np, self.orc
+        if self.opname == "CvtColor":
+            if self.dc == 3:
+                return np.ascontiguousarray(a[..., ::-1])
+            b, g, r = (a[..., i].astype(np.int64) for i in range(3))
+            return ((b * 3735 + g * 19235 + r * 9798 + (1 << 14)) >> 15).astype(np.uint8)[..., None]
+        if self.opname == "Normalize":
+            return orc.normalize(a, self.base, self.scale, 1.0, 0.0, 0.0, False, threads=threads)
+        if self.opname == "Reformat":
+            return np.ascontiguousarray(a.transpose(0, 3, 1, 2))
+        if self.opname == "ConvertTo":
+            return orc.convert_to(a, np.float32, 1.0 / 255.0, 0.0, 1)
+        if self.opname == "Flip":
+            return np.ascontiguousarray(a[:, :, ::-1])
+        return orc.resize(a, (self.dh, self.dw), LINEAR, variant=1, threads=threads)
+
+    def check(self, s):
+        got = s[1].torch_view()[:1].cpu().numpy()
+        ref = self._reference(self.host1)
+        if self.ddt == self.np.float32:
+            assert (self.np.abs(got - ref) <= 1e-5 * self.np.maximum(1.0, self.np.abs(ref))).all()
+        else:
+            assert (got == ref).all(), "bench output differs from the oracle"
+
+    def cpu_cores(self, threads):
+        # the numpy index maps and the element-wise conversion run on one thread
+        return threads if self.opname in ("Normalize", "Resize") else 1
+
+    def cpu(self, threads):
+        self._reference(self.np.repeat(self.host1, 4, axis=0), threads)
+        return 4
+
+
 WORKLOADS = {
     "fused": Fused,
     "resize-nearest": lambda *a: ResizeC1(*a, NEAREST),
@@ -307,6 +412,7 @@ WORKLOADS = {
     "warp-affine-varshape": WarpC4,
     "resize-cubic-4k": CubicC5,
 }
+WORKLOADS.update({k: (lambda *a, k=k: Streaming(*a, k)) for k in Streaming.SPECS})
 
 
 def main():
@@ -419,9 +525,10 @@ def main():
             done += wl.cpu(threads)
             reps += 1
             tcpu = time.perf_counter() - c0
-        cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": threads, "kind": "port",
-               "sample": "%d images of this workload through the C++ oracle in %.1f s, %d threads"
-                         % (done, tcpu, threads)}
+        used = wl.cpu_cores(threads) if hasattr(wl, "cpu_cores") else threads
+        cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": used, "kind": "port",
+               "sample": "%d images of this workload through the CPU oracle in %.1f s, %d thread%s"
+                         % (done, tcpu, used, "" if used == 1 else "s")}
 
     out = {
         "metric": "images/sec and achieved HBM GB/s (% of roofline), 1 MI355X",
