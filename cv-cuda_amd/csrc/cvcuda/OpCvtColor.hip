@@ -213,9 +213,9 @@ __device__ __forceinline__ void SwizzlePixel(const uint8_t *srcRow, uint8_t *dst
 {
     const Px<T, SCH> s = reinterpret_cast<const Px<T, SCH> *>(srcRow)[x];
     Px<T, DCH>       d;
-    d.v[0] = s.v[bidx];
+    d.v[0] = bidx ? s.v[2] : s.v[0];
     d.v[1] = s.v[1];
-    d.v[2] = s.v[bidx ^ 2];
+    d.v[2] = bidx ? s.v[0] : s.v[2];
     if constexpr (DCH == 4)
     {
         if constexpr (SCH == 4)

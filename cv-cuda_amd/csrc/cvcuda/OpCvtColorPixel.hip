@@ -100,7 +100,7 @@ struct GrayFromBgr
 
     static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
-        const T          b = s.v[a.bidx], g = s.v[1], r = s.v[a.bidx ^ 2];
+        const T          b = a.bidx ? s.v[2] : s.v[0], g = s.v[1], r = a.bidx ? s.v[0] : s.v[2];
         Px<T, 1>         o;
         if constexpr (std::is_integral_v<T>)
         {
@@ -145,7 +145,7 @@ struct YuvFromBgr
         if constexpr (std::is_integral_v<T>)
         {
             constexpr int delta = ((int)(std::numeric_limits<T>::max() / 2 + 1)) << 14;
-            const int     B = s.v[a.bidx], G = s.v[1], R = s.v[a.bidx ^ 2];
+            const int     B = a.bidx ? s.v[2] : s.v[0], G = s.v[1], R = a.bidx ? s.v[0] : s.v[2];
             const int     Y  = Descale(R * 4899 + G * 9617 + B * 1868, 14);
             const int     Cr = Descale((R - Y) * 14369 + delta, 14);
             const int     Cb = Descale((B - Y) * 8061 + delta, 14);
@@ -155,7 +155,7 @@ struct YuvFromBgr
         }
         else
         {
-            const float B = s.v[a.bidx], G = s.v[1], R = s.v[a.bidx ^ 2];
+            const float B = a.bidx ? s.v[2] : s.v[0], G = s.v[1], R = a.bidx ? s.v[0] : s.v[2];
             const float Y = R * 0.299f + G * 0.587f + B * 0.114f;
             o.v[0]        = Y;
             o.v[2]        = (R - Y) * 0.877f + 0.5f;
@@ -190,9 +190,9 @@ struct BgrFromYuv
             g = Y + (Cb - 0.5f) * -0.395f + (Cr - 0.5f) * -0.581f;
             r = Y + (Cr - 0.5f) * 1.140f;
         }
-        o.v[a.bidx]     = b;
-        o.v[1]          = g;
-        o.v[a.bidx ^ 2] = r;
+        o.v[0] = a.bidx ? r : b;
+        o.v[1] = g;
+        o.v[2] = a.bidx ? b : r;
         return o;
     }
 };
@@ -209,7 +209,7 @@ struct HsvFromBgr
         if constexpr (std::is_integral_v<T>)
         {
             const int hrange = a.full ? 256 : 180;
-            const int b = s.v[a.bidx], g = s.v[1], r = s.v[a.bidx ^ 2];
+            const int b = a.bidx ? s.v[2] : s.v[0], g = s.v[1], r = a.bidx ? s.v[0] : s.v[2];
             const int vmin = min(b, min(g, r));
             const int val  = max(b, max(g, r));
             const int diff = val - vmin;
@@ -226,7 +226,7 @@ struct HsvFromBgr
         }
         else
         {
-            const float b = s.v[a.bidx], g = s.v[1], r = s.v[a.bidx ^ 2];
+            const float b = a.bidx ? s.v[2] : s.v[0], g = s.v[1], r = a.bidx ? s.v[0] : s.v[2];
             const float vmin = fminf(r, fminf(g, b));
             const float val  = fmaxf(r, fmaxf(g, b));
             float       diff = val - vmin;
@@ -257,29 +257,27 @@ struct HsvFromBgr
     }
 };
 
-__device__ __forceinline__ float Select4(const float (&tab)[4], int idx)
+__device__ __forceinline__ float Select4(float t0, float t1, float t2, float t3, int idx)
 {
-    float out = idx == 1 ? tab[1] : tab[0];
-    out       = idx == 2 ? tab[2] : out;
-    out       = idx == 3 ? tab[3] : out;
+    float out = idx == 1 ? t1 : t0;
+    out       = idx == 2 ? t2 : out;
+    out       = idx == 3 ? t3 : out;
     return out;
 }
 
 __device__ __forceinline__ void HsvToBgrFloat(float h, float s, float v, float &b, float &g, float &r)
 {
-    if (s == 0)
-    {
-        b = g = r = v;
-        return;
-    }
+    // the three constants say which of the four candidates each channel takes in each of the six hue
+    // sectors, 4 bits per sector; zero saturation gives grey whatever the hue
     h += 6 * (h < 0);
     int idx = (int)h; // sector
     h -= idx;         // fraction inside the sector
     idx = (idx % 6) << 2;
-    const float tab[4] = {v, v * (1 - s), v * (1 - s * h), v * (1 - s * (1 - h))};
-    b                  = Select4(tab, (0x00200311 >> idx) & 0xf);
-    g                  = Select4(tab, (0x00112003 >> idx) & 0xf);
-    r                  = Select4(tab, (0x00031120 >> idx) & 0xf);
+    const float t0 = v, t1 = v * (1 - s), t2 = v * (1 - s * h), t3 = v * (1 - s * (1 - h));
+    const bool  grey = s == 0;
+    b = grey ? v : Select4(t0, t1, t2, t3, (0x00200311 >> idx) & 0xf);
+    g = grey ? v : Select4(t0, t1, t2, t3, (0x00112003 >> idx) & 0xf);
+    r = grey ? v : Select4(t0, t1, t2, t3, (0x00031120 >> idx) & 0xf);
 }
 
 template<class T, int DCH>
@@ -305,9 +303,9 @@ struct BgrFromHsv
         {
             HsvToBgrFloat(s.v[0] * (6.0f / 360.0f), s.v[1], s.v[2], b, g, r);
         }
-        o.v[a.bidx]     = b;
-        o.v[1]          = g;
-        o.v[a.bidx ^ 2] = r;
+        o.v[0] = a.bidx ? r : b;
+        o.v[1] = g;
+        o.v[2] = a.bidx ? b : r;
         if constexpr (DCH == 4)
         {
             o.v[3] = AlphaOf<T>();
@@ -344,13 +342,13 @@ struct Yuv420FromBgr
             const Px<uint8_t, 2 * SCH> s
                 = *reinterpret_cast<const Px<uint8_t, 2 * SCH> *>(v.src + (int64_t)(y + r) * v.srcRow + x * SCH);
             uint8_t Y0, Y1, u, w;
-            BgrToYuv420(s.v[a.bidx], s.v[1], s.v[a.bidx ^ 2], Y0, u, w);
+            BgrToYuv420(a.bidx ? s.v[2] : s.v[0], s.v[1], a.bidx ? s.v[0] : s.v[2], Y0, u, w);
             if (r == 0)
             {
                 U = u;
                 V = w;
             }
-            BgrToYuv420(s.v[SCH + a.bidx], s.v[SCH + 1], s.v[SCH + (a.bidx ^ 2)], Y1, u, w);
+            BgrToYuv420(a.bidx ? s.v[SCH + 2] : s.v[SCH], s.v[SCH + 1], a.bidx ? s.v[SCH] : s.v[SCH + 2], Y1, u, w);
             __builtin_nontemporal_store((uint16_t)(Y0 | (Y1 << 8)),
                                         reinterpret_cast<uint16_t *>(v.dst + (int64_t)(y + r) * v.dstRow + x));
         }
@@ -396,9 +394,9 @@ struct BgrFromYuv422
         {
             uint8_t b, g, r;
             Yuv42xToBgr(k == 0 ? Y0 : Y1, U, V, b, g, r);
-            o.v[k * DCN + a.bidx]       = b;
-            o.v[k * DCN + 1]            = g;
-            o.v[k * DCN + (a.bidx ^ 2)] = r;
+            o.v[k * DCN + 0] = a.bidx ? r : b;
+            o.v[k * DCN + 1] = g;
+            o.v[k * DCN + 2] = a.bidx ? b : r;
             if constexpr (DCN == 4)
             {
                 o.v[k * DCN + 3] = 255;
