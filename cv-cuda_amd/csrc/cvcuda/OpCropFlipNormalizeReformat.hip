@@ -4,13 +4,17 @@
 // outside the rectangle :157-161, expression and its order :73-74, scale / stddev :45-59, type tables
 // :341-351 and :449-454, parameter checks :416-433, output layout :193-197.
 //
-// Kernel shape: one lane per output pixel, 64 columns x 4 rows per block, grid z = image. The crop
-// rectangle, the flip code and the per-channel base / scale values are uniform per block and read in
-// the prologue. Source and destination are addressed through per-channel strides, so interleaved and
-// planar images, NHWC and NCHW outputs all run through the same code; for an interleaved source the C
-// channel loads of a lane are adjacent bytes and coalesce in the memory pipeline. Streaming stores.
+// Two kernels, grid z = image; the crop rectangle, the flip code and the per-channel base / scale
+// values are uniform per block and read in the prologue; streaming stores.
+//  * The pipeline cases (interleaved u8 or f32 images to packed u8 / f32 NHWC or NCHW tensors): a
+//    lane produces a run of 4 output pixels. Where the 4 source pixels lie inside the image they are
+//    one vector load (reversed in registers for mirrored columns), otherwise they are fetched one by
+//    one through the border rule; the run is stored as whole dwords, per plane for NCHW.
+//  * Everything else: one lane per output pixel, source and destination addressed through
+//    per-channel strides, so planar images and any destination strides run through the same code.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "RunIO.hpp"
 
 #include <cvcuda/OpCropFlipNormalizeReformat.h>
 
@@ -123,9 +127,195 @@ __global__ __launch_bounds__(256) void CfnrKernel(const CfnrArgs a)
     }
 }
 
+// Runs of 4 output pixels per lane; interleaved source, destination rows packed (NHWC: pixel stride
+// C elements, NCHW: pixel stride one element).
+constexpr int kCfnrRowsPerWave = 1; // rows a wave works through (more per wave measured slower)
+
+template<class TS, class TD, int C>
+__global__ __launch_bounds__(256) void CfnrRunsKernel(const CfnrArgs a)
+{
+    constexpr int P  = kRunPixels;
+    const int     x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * P;
+    if (x0 >= a.W)
+    {
+        return;
+    }
+    const int      n    = blockIdx.z;
+    const int32_t *rect = reinterpret_cast<const int32_t *>(a.crop + n * a.cropStride);
+    const int      cx = rect[0], cy = rect[1], cw = rect[2], ch = rect[3];
+    const int      code    = *reinterpret_cast<const int32_t *>(a.flip + n * a.flipStride);
+    const bool     mirrorX = code == 1 || code == -1, mirrorY = code == 0 || code == -1;
+    const NVCVImagePlaneStrided &p0 = a.srcList[n].planes[0];
+    const uint8_t *srcBase = p0.basePtr;
+    const int      srcRow = p0.rowStride, srcW = p0.width, srcH = p0.height;
+    // every uniform value is loaded before the first use, so the loads share one round trip
+    float b[C], m[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        b[c] = a.base[a.baseC == 1 ? 0 : c];
+        m[c] = a.scale[a.scaleC == 1 ? 0 : c];
+    }
+    if (a.stddev)
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            m[c] = 1.0f / sqrtf(m[c] * m[c] + a.eps);
+        }
+    }
+    const int  first  = mirrorX ? cw - 1 - (x0 + P - 1) + cx : x0 + cx; // lowest source column of the run
+    const bool runIn  = x0 + P <= cw && first >= 0 && first + P <= srcW;
+    const bool planar = a.dW == (int64_t)sizeof(TD) && C > 1;
+
+#pragma unroll 2
+    for (int r = 0; r < kCfnrRowsPerWave; ++r)
+    {
+        const int y = (blockIdx.y * kCfnrRowsPerWave + r) * kRunTileH + (threadIdx.x >> 6);
+        if (y >= a.H)
+        {
+            break;
+        }
+        TD out[P * C];
+#pragma unroll
+        for (int i = 0; i < P * C; ++i)
+        {
+            out[i] = (TD)0; // outside the rectangle
+        }
+        if (x0 < cw && y < ch)
+        {
+            const int sy = (mirrorY ? ch - 1 - y : y) + cy;
+            TS        in[P * C];
+            if (runIn && sy >= 0 && sy < srcH)
+            {
+                // two branches with constant indices: a select between two indices would turn every
+                // element into a chain of compares over the whole run
+                TS raw[P * C];
+                LoadRun<TS, P * C>(srcBase + (int64_t)sy * srcRow + (int64_t)first * C * sizeof(TS), raw);
+                if (mirrorX)
+                {
+#pragma unroll
+                    for (int k = 0; k < P; ++k)
+                    {
+#pragma unroll
+                        for (int c = 0; c < C; ++c)
+                        {
+                            in[k * C + c] = raw[(P - 1 - k) * C + c];
+                        }
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < P * C; ++i)
+                    {
+                        in[i] = raw[i];
+                    }
+                }
+            }
+            else
+            {
+                const int syIn = a.border == NVCV_BORDER_CONSTANT ? sy : BorderIndex(a.border, sy, srcH);
+#pragma unroll
+                for (int k = 0; k < P; ++k)
+                {
+                    int        sx      = (mirrorX ? cw - 1 - (x0 + k) : x0 + k) + cx;
+                    const bool outside = a.border == NVCV_BORDER_CONSTANT && (sx < 0 || sx >= srcW || sy < 0 || sy >= srcH);
+                    if (a.border != NVCV_BORDER_CONSTANT)
+                    {
+                        sx = BorderIndex(a.border, sx, srcW);
+                    }
+                    // pixels of the run beyond the rectangle are computed from a clamped column and dropped below
+                    sx = outside ? 0 : min(max(sx, 0), srcW - 1);
+                    const TS *px = reinterpret_cast<const TS *>(srcBase + (int64_t)(outside ? 0 : syIn) * srcRow) + sx * C;
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                    {
+                        in[k * C + c] = outside ? BorderValueAs<TS>(a.borderValue) : px[c];
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < P; ++k)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    const float v  = ((float)in[k * C + c] - b[c]) * m[c] * a.gscale + a.shift;
+                    out[k * C + c] = x0 + k < cw ? SaturateCast<TD>(v) : (TD)0;
+                }
+            }
+        }
+        uint8_t *d = a.dst + n * a.dN + y * a.dH + x0 * a.dW;
+        if (x0 + P <= a.W)
+        {
+            if (planar)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    TD t[P];
+#pragma unroll
+                    for (int k = 0; k < P; ++k)
+                    {
+                        t[k] = out[k * C + c];
+                    }
+                    StoreRunNT<TD, P>(d + c * a.dC, t);
+                }
+            }
+            else
+            {
+                StoreRunNT<TD, P * C>(d, out);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int k = 0; k < P - 1; ++k)
+            {
+                if (x0 + k < a.W)
+                {
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                    {
+                        *reinterpret_cast<TD *>(d + k * a.dW + c * a.dC) = out[k * C + c];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template<class TS, class TD>
+constexpr bool kCfnrRuns = (std::is_same_v<TS, uint8_t> && (std::is_same_v<TD, uint8_t> || std::is_same_v<TD, float>))
+                        || (std::is_same_v<TS, float> && std::is_same_v<TD, float>);
+
 template<class TS, class TD>
 void Launch(const CfnrArgs &a, int N, hipStream_t stream)
 {
+    if constexpr (kCfnrRuns<TS, TD>)
+    {
+        const bool nchw = a.dW == (int64_t)sizeof(TD);
+        const bool nhwc = a.dC == (int64_t)sizeof(TD) && a.dW == (int64_t)(a.C * sizeof(TD));
+        if (!a.srcPlanar && (nchw || nhwc))
+        {
+            dim3 grid(DivUp(a.W, kRunTileW), DivUp(a.H, kRunTileH * kCfnrRowsPerWave), N);
+            switch (a.C)
+            {
+            case 1:
+                hipLaunchKernelGGL((CfnrRunsKernel<TS, TD, 1>), grid, dim3(256), 0, stream, a);
+                break;
+            case 3:
+                hipLaunchKernelGGL((CfnrRunsKernel<TS, TD, 3>), grid, dim3(256), 0, stream, a);
+                break;
+            default:
+                hipLaunchKernelGGL((CfnrRunsKernel<TS, TD, 4>), grid, dim3(256), 0, stream, a);
+                break;
+            }
+            CheckLaunch("CfnrRunsKernel");
+            return;
+        }
+    }
     dim3 grid(DivUp(a.W, 64), DivUp(a.H, 4), N);
     hipLaunchKernelGGL((CfnrKernel<TS, TD>), grid, dim3(256), 0, stream, a);
     CheckLaunch("CfnrKernel");
