@@ -92,7 +92,7 @@ class Fused:
     N, SRC_H, SRC_W = 64, 1080, 1920
     NEW_W, NEW_H, CROP_X, CROP_Y, OUT_H, OUT_W = 455, 256, 115, 16, 224, 224
     SCALE, OFFSET = 1.0 / (255.0 * 0.226), -0.449 / 0.226
-    kernel = "FusedBilinear<float,false,false>"
+    kernel = "FusedBilinear<float,false,false,false>"
     dtype = "f32"
     workload = ("fused ResizeCropConvertReformat: batch 64 u8 NHWC 1920x1080 -> bilinear 455x256 -> "
                 "crop 224x224 @(115,16) -> f32 NCHW, scale/offset")
