@@ -194,7 +194,112 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
                 }
             }
         };
-        if (ceilf(scaleX) == scaleX && ceilf(scaleY) == scaleY)
+        if constexpr (VARSHAPE)
+        {
+            // image batches follow the reference's separate kernel (legacy/resize_var_shape.cu:236-428):
+            // same sums for reductions, corners added last; enlargements are a bilinear variant whose
+            // fractions come from the inverse scale in double
+            const int  iscaleX = SaturateCast<int32_t>(scaleX), iscaleY = SaturateCast<int32_t>(scaleY);
+            const bool fast    = scaleX == (float)iscaleX && scaleY == (float)iscaleY;
+            if (scaleX >= 1.0f && scaleY >= 1.0f)
+            {
+                if (fast)
+                {
+                    const float scale = 1.f / (scaleX * scaleY);
+                    for (int cy = ymin; cy < ymax; ++cy)
+                    {
+                        for (int cx = xmin; cx < xmax; ++cx)
+                        {
+                            add(cx, cy, scale);
+                        }
+                    }
+                }
+                else
+                {
+                    const float scale = 1.f / (fminf(scaleX, p.srcW - fsx1) * fminf(scaleY, p.srcH - fsy1));
+                    for (int cy = ymin; cy < ymax; ++cy)
+                    {
+                        for (int cx = xmin; cx < xmax; ++cx)
+                        {
+                            add(cx, cy, scale);
+                        }
+                        if (xmin > fsx1)
+                        {
+                            add(xmin - 1, cy, (xmin - fsx1) * scale);
+                        }
+                        if (xmax < fsx2)
+                        {
+                            add(xmax, cy, (fsx2 - xmax) * scale);
+                        }
+                    }
+                    if (ymin > fsy1)
+                    {
+                        for (int cx = xmin; cx < xmax; ++cx)
+                        {
+                            add(cx, ymin - 1, (ymin - fsy1) * scale);
+                        }
+                    }
+                    if (ymax < fsy2)
+                    {
+                        for (int cx = xmin; cx < xmax; ++cx)
+                        {
+                            add(cx, ymax, (fsy2 - ymax) * scale);
+                        }
+                    }
+                    if (ymin > fsy1 && xmin > fsx1)
+                    {
+                        add(xmin - 1, ymin - 1, (ymin - fsy1) * (xmin - fsx1) * scale);
+                    }
+                    if (ymin > fsy1 && xmax < fsx2)
+                    {
+                        add(xmax, ymin - 1, (ymin - fsy1) * (fsx2 - xmax) * scale);
+                    }
+                    if (ymax < fsy2 && xmax < fsx2)
+                    {
+                        add(xmax, ymax, (fsy2 - ymax) * (fsx2 - xmax) * scale);
+                    }
+                    if (ymax < fsy2 && xmin > fsx1)
+                    {
+                        add(xmin - 1, ymax, (fsy2 - ymax) * (xmin - fsx1) * scale);
+                    }
+                }
+            }
+            else
+            {
+                const double invX = 1. / scaleX, invY = 1. / scaleY;
+                int          sy = (int)floorf(dy * scaleY);
+                float        fy = (float)((dy + 1) - (sy + 1) * invY);
+                fy              = fy <= 0 ? 0.f : fy - (int)floorf(fy);
+                int   sx = (int)floorf(dx * scaleX);
+                float fx = (float)((dx + 1) - (sx + 1) * invX);
+                fx       = fx < 0 ? 0.f : fx - (int)floorf(fx);
+                if (sx < 0)
+                {
+                    fx = 0, sx = 0;
+                }
+                if (sx >= p.srcW - 1)
+                {
+                    fx = 0, sx = p.srcW - 2;
+                }
+                if (sy >= p.srcH - 1)
+                {
+                    sy = p.srcH - 2;
+                }
+                // sources of one row or column: the reference indexes outside the image; taps clamped here
+                const int      x0 = max(sx, 0), x1 = min(sx + 1, p.srcW - 1), y0 = max(sy, 0), y1 = min(sy + 1, p.srcH - 1);
+                const uint8_t *r0 = p.src + (int64_t)y0 * p.srcRow, *r1 = p.src + (int64_t)y1 * p.srcRow;
+                const Pixel<T, C> p00 = LoadPx<T, C>(r0, x0), p10 = LoadPx<T, C>(r1, x0);
+                const Pixel<T, C> p01 = LoadPx<T, C>(r0, x1), p11 = LoadPx<T, C>(r1, x1);
+                const float       cx0 = 1.f - fx, cx1 = fx, cy0 = 1.f - fy, cy1 = fy;
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    sum[c] = (float)p00.v[c] * cx0 * cy0 + (float)p10.v[c] * cx0 * cy1 + (float)p01.v[c] * cx1 * cy0
+                           + (float)p11.v[c] * cx1 * cy1;
+                }
+            }
+        }
+        else if (ceilf(scaleX) == scaleX && ceilf(scaleY) == scaleY)
         {
             const float scale = 1.f / (scaleX * scaleY);
             for (int cy = ymin; cy < ymax; ++cy)
@@ -969,11 +1074,8 @@ void DispatchInterp(bool varshape, const ResizeArgs &a, const NVCVImageBufferStr
                  : LaunchTensor<T, C, NVCV_INTERP_CUBIC>(a, N, stream);
         break;
     case NVCV_INTERP_AREA:
-        if (varshape)
-        {
-            throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "AREA interpolation is available for tensors only");
-        }
-        LaunchTensor<T, C, NVCV_INTERP_AREA>(a, N, stream);
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_AREA>(a, dstHost, N, stream)
+                 : LaunchTensor<T, C, NVCV_INTERP_AREA>(a, N, stream);
         break;
     default:
         throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid interpolation (supported: NEAREST, LINEAR, CUBIC, AREA)");

@@ -13,6 +13,7 @@
 // Parity pinning status (see tests/test_oracle_*.py): every function below is pinned by closed
 // forms, brute force or library cross-checks; none is "parity unpinned".
 #include <algorithm>
+#include <cfloat>
 #include <cmath>
 #include <cstdint>
 #include <cstdlib>
@@ -279,7 +280,7 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
 {
     auto at = [&](int x, int y, int c) -> double
     { return (x < 0 || x >= srcW || y < 0 || y >= srcH) ? 0.0 : (double)src[y * srcStep + (int64_t)x * C + c]; };
-    if (variant == 0)
+    if (variant == 0 || variant == 3) // golden; 3 = its image-batch flavour (ResizeUtils.cpp:78, 136-176)
     {
         const double scaleH = static_cast<double>(srcH) / dstH, scaleW = static_cast<double>(srcW) / dstW;
         const double fsx1 = dx * scaleW, fsx2 = fsx1 + scaleW, fsy1 = dy * scaleH, fsy2 = fsy1 + scaleH;
@@ -294,6 +295,25 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
                 const double inv = 1.f / (scaleW * scaleH);
                 for (int y = sy1; y < sy2; ++y)
                     for (int x = sx1; x < sx2; ++x) o = o + at(x, y, c) * inv;
+            }
+            else if (variant == 3 && !(scaleH >= 1.0f && scaleW >= 1.0f))
+            {
+                // enlargement of image batches: a bilinear variant in mixed float / double
+                const double scaleHInv = 1.0 / scaleH, scaleWInv = 1.0 / scaleW;
+                int          y1 = (int)std::floor(fsy1), x1 = (int)std::floor(fsx1);
+                float        fy = (float)(float(dy + 1) - float(y1 + 1) * scaleHInv);
+                fy              = fy <= 0 ? 0.f : fy - (int)std::floor(fy);
+                float fx        = (float)(float(dx + 1) - float(x1 + 1) * scaleWInv);
+                fx              = fx <= 0 ? 0.f : fx - (int)std::floor(fx);
+                if (x1 < 0) { fx = 0; x1 = 0; }
+                if (x1 >= srcW - 1) { fx = 0; x1 = srcW - 2; }
+                if (y1 >= srcH - 1) { y1 = srcH - 2; }
+                // sources of one row or column: the reference indexes outside the image; taps clamped here
+                auto tap = [&](int x, int y) -> float // the golden's products and sums here are float
+                { return (float)src[std::max(0, std::min(y, srcH - 1)) * srcStep + (int64_t)std::max(0, std::min(x, srcW - 1)) * C + c]; };
+                const float cx0 = 1.f - fx, cx1 = fx, cy0 = 1.f - fy, cy1 = fy;
+                o = tap(x1, y1) * cx0 * cy0 + tap(x1, y1 + 1) * cx0 * cy1 + tap(x1 + 1, y1) * cx1 * cy0
+                  + tap(x1 + 1, y1 + 1) * cx1 * cy1;
             }
             else
             {
@@ -325,6 +345,63 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
     const float fsx1 = dx * scaleX, fsy1 = dy * scaleY, fsx2 = fsx1 + scaleX, fsy2 = fsy1 + scaleY;
     const int   xmin = (int)std::ceil(fsx1), xmax = (int)std::floor(fsx2);
     const int   ymin = (int)std::ceil(fsy1), ymax = (int)std::floor(fsy2);
+    if (variant == 2) // image-batch kernel: src/cvcuda/priv/legacy/resize_var_shape.cu:236-428
+    {
+        const int  iscaleX = (int)std::rint(scaleX), iscaleY = (int)std::rint(scaleY);
+        const bool fast = std::fabs(scaleX - iscaleX) < DBL_EPSILON && std::fabs(scaleY - iscaleY) < DBL_EPSILON;
+        for (int c = 0; c < C; ++c)
+        {
+            auto  v = [&](int x, int y) -> float { return (float)at(x, y, c); };
+            float o = 0.f;
+            if (scaleX >= 1.0f && scaleY >= 1.0f)
+            {
+                if (fast)
+                {
+                    const float scale = 1.f / (scaleX * scaleY);
+                    for (int cy = ymin; cy < ymax; ++cy)
+                        for (int cx = xmin; cx < xmax; ++cx) o = o + v(cx, cy) * scale;
+                }
+                else
+                {
+                    const float scale = 1.f / (std::fmin(scaleX, srcW - fsx1) * std::fmin(scaleY, srcH - fsy1));
+                    for (int cy = ymin; cy < ymax; ++cy)
+                    {
+                        for (int cx = xmin; cx < xmax; ++cx) o = o + v(cx, cy) * scale;
+                        if (xmin > fsx1) o = o + v(xmin - 1, cy) * ((xmin - fsx1) * scale);
+                        if (xmax < fsx2) o = o + v(xmax, cy) * ((fsx2 - xmax) * scale);
+                    }
+                    if (ymin > fsy1)
+                        for (int cx = xmin; cx < xmax; ++cx) o = o + v(cx, ymin - 1) * ((ymin - fsy1) * scale);
+                    if (ymax < fsy2)
+                        for (int cx = xmin; cx < xmax; ++cx) o = o + v(cx, ymax) * ((fsy2 - ymax) * scale);
+                    if (ymin > fsy1 && xmin > fsx1) o = o + v(xmin - 1, ymin - 1) * ((ymin - fsy1) * (xmin - fsx1) * scale);
+                    if (ymin > fsy1 && xmax < fsx2) o = o + v(xmax, ymin - 1) * ((ymin - fsy1) * (fsx2 - xmax) * scale);
+                    if (ymax < fsy2 && xmax < fsx2) o = o + v(xmax, ymax) * ((fsy2 - ymax) * (fsx2 - xmax) * scale);
+                    if (ymax < fsy2 && xmin > fsx1) o = o + v(xmin - 1, ymax) * ((fsy2 - ymax) * (xmin - fsx1) * scale);
+                }
+            }
+            else
+            {
+                const double invX = 1. / scaleX, invY = 1. / scaleY;
+                int          sy = (int)std::floor(dy * scaleY);
+                float        fy = (float)((dy + 1) - (sy + 1) * invY);
+                fy              = fy <= 0 ? 0.f : fy - (int)std::floor(fy);
+                int   sx = (int)std::floor(dx * scaleX);
+                float fx = (float)((dx + 1) - (sx + 1) * invX);
+                fx       = fx < 0 ? 0.f : fx - (int)std::floor(fx);
+                if (sx < 0) { fx = 0; sx = 0; }
+                if (sx >= srcW - 1) { fx = 0; sx = srcW - 2; }
+                if (sy >= srcH - 1) { sy = srcH - 2; }
+                auto tap = [&](int x, int y) -> float
+                { return (float)src[std::max(0, std::min(y, srcH - 1)) * srcStep + (int64_t)std::max(0, std::min(x, srcW - 1)) * C + c]; };
+                const float cx0 = 1.f - fx, cx1 = fx, cy0 = 1.f - fy, cy1 = fy;
+                o = tap(sx, sy) * cx0 * cy0 + tap(sx, sy + 1) * cx0 * cy1 + tap(sx + 1, sy) * cx1 * cy0
+                  + tap(sx + 1, sy + 1) * cx1 * cy1;
+            }
+            out[c] = SatF<T>(o);
+        }
+        return;
+    }
     const bool  integerArea = std::ceil(scaleX) == scaleX && std::ceil(scaleY) == scaleY;
     for (int c = 0; c < C; ++c)
     {

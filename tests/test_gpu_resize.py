@@ -201,6 +201,40 @@ def test_area_tensor(cv, orc, gpu, row):
         np.testing.assert_array_equal(res, device)
 
 
+@pytest.mark.parametrize("dt,c", [(np.uint8, 4), (np.uint8, 3), (np.uint16, 1), (np.int16, 3), (np.float32, 4)])
+def test_area_varshape(cv, K, orc, gpu, dt, c):
+    # image batches run the reference's separate AREA kernel (reductions: same sums, corners last;
+    # enlargements: a bilinear variant). Sizes: the reference's rows (TestOpResize.cpp:67-69) plus
+    # fractional factors in both directions and mixed reduce/enlarge.
+    fmt = _format_for(cv, K, dt, c)
+    sizes = [(44, 40, 22, 20), (30, 30, 20, 20), (30, 30, 60, 60), (97, 61, 13, 9), (50, 70, 75, 90), (64, 48, 32, 96),
+             (33, 21, 33, 21), (120, 90, 47, 31)]
+    n = len(sizes)
+    bin_, bout, hosts, outs = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], []
+    for i, (sw, sh, dw, dh) in enumerate(sizes):
+        a = make_input(orc, (sh, sw, c), dt, 0xA0EA + i)
+        hosts.append(a)
+        bin_.push_back(cv.Image.from_numpy(a, fmt))
+        o = cv.Image.alloc((dw, dh), fmt)
+        outs.append(o)
+        bout.push_back(o)
+    cv.Resize()(None, bin_, bout, AREA)
+    torch.cuda.synchronize()
+    for a, o, (sw, sh, dw, dh) in zip(hosts, outs, sizes):
+        res = o.plane_view(0, dt, c).cpu().numpy()[None]
+        golden = orc.resize(a[None], (dh, dw), AREA, variant=3)
+        device = orc.resize(a[None], (dh, dw), AREA, variant=2)
+        if dt == np.float32:
+            assert np.abs(res - device).max() <= 1e-5 and np.abs(res - golden).max() <= 1e-4
+        else:
+            np.testing.assert_array_equal(res, device)
+            # float32 source coordinates against the golden's double: a pixel whose box edge lands on an
+            # integer can take a different tap, so the 1-LSB bar is required of all but a few pixels
+            # (the reference's own rows have none)
+            bad = np.abs(res.astype(np.int64) - golden.astype(np.int64)) > 1
+            assert bad.mean() <= (0.0 if (sw, sh, dw, dh) in sizes[:3] else 0.02), (sw, sh, dw, dh, bad.mean())
+
+
 def test_negative_cases(cv, gpu):
     a = cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC")
     op = cv.Resize()

@@ -383,11 +383,11 @@ def test_resize_area_closed_forms(orc):
     # integer factors: the plain block mean
     for fy, fx in ((2, 2), (3, 4), (1, 6)):
         ref = a.reshape(1, 24 // fy, fy, 36 // fx, fx, 3).astype(np.float64).mean(axis=(2, 4))
-        for variant in (0, 1):
+        for variant in (0, 1, 2, 3):  # 2 / 3: the image-batch kernel and its golden
             r = orc.resize(a, (24 // fy, 36 // fx), 3, variant=variant)
             assert np.abs(r - ref).max() <= 0.5 + 1e-4
     # same size: identity; constant image: constant (weights sum to the covered area)
-    for variant in (0, 1):
+    for variant in (0, 1, 2, 3):
         np.testing.assert_array_equal(orc.resize(a, (24, 36), 3, variant=variant), a)
         k = np.full((1, 31, 47, 1), 200, np.uint8)
         r = orc.resize(k, (13, 10), 3, variant=variant)
@@ -396,6 +396,19 @@ def test_resize_area_closed_forms(orc):
     f = rng.random((1, 7, 9, 1)).astype(np.float32)
     fine = np.repeat(np.repeat(f, 60, axis=1), 60, axis=2)  # 420 x 540
     ref = fine.reshape(1, 5, 84, 6, 90, 1).mean(axis=(2, 4))  # 7 -> 5 rows, 9 -> 6 columns
-    for variant in (0, 1):
+    for variant in (0, 1, 2, 3):
         r = orc.resize(f, (5, 6), 3, variant=variant)
         assert np.abs(r - ref).max() < 1e-5
+    # image batches, enlargement by an integer factor: every fraction is 0, so the result is pixel
+    # replication -- except that the last source row and column are never reached (the reference steps
+    # back to the one before and takes that with weight 1)
+    for variant in (2, 3):
+        for k in (2, 3):
+            r = orc.resize(a, (24 * k, 36 * k), 3, variant=variant)
+            iy, ix = np.minimum(np.arange(24 * k) // k, 22), np.minimum(np.arange(36 * k) // k, 34)
+            np.testing.assert_array_equal(r, a[:, iy][:, :, ix])
+    # enlargement by 1.5: output pixel 1 lies half-way between source pixels 0 and 1
+    ramp = np.tile(np.arange(0, 80, 10, dtype=np.float32).reshape(1, 1, 8, 1), (1, 4, 1, 1))
+    for variant in (2, 3):
+        r = orc.resize(ramp, (6, 12), 3, variant=variant)
+        assert abs(float(r[0, 0, 1, 0]) - 5.0) < 1e-4 and float(r[0, 0, 0, 0]) == 0.0
