@@ -44,13 +44,14 @@ def last_error():
 _NP2DT = {
     np.dtype(np.uint8): K.DATA_TYPE_U8, np.dtype(np.int8): K.DATA_TYPE_S8,
     np.dtype(np.uint16): K.DATA_TYPE_U16, np.dtype(np.int16): K.DATA_TYPE_S16,
-    np.dtype(np.int32): K.DATA_TYPE_S32, np.dtype(np.float32): K.DATA_TYPE_F32,
+    np.dtype(np.int32): K.DATA_TYPE_S32, np.dtype(np.uint32): K.DATA_TYPE_U32, np.dtype(np.float32): K.DATA_TYPE_F32,
     np.dtype(np.float64): K.DATA_TYPE_F64, np.dtype(np.float16): K.DATA_TYPE_F16,
 }
 _DT2NP = {v: k for k, v in _NP2DT.items()}
 _NP2TORCH = {
     np.dtype(np.uint8): torch.uint8, np.dtype(np.int8): torch.int8, np.dtype(np.uint16): torch.uint16,
-    np.dtype(np.int16): torch.int16, np.dtype(np.int32): torch.int32, np.dtype(np.float32): torch.float32,
+    np.dtype(np.int16): torch.int16, np.dtype(np.int32): torch.int32, np.dtype(np.uint32): torch.uint32,
+    np.dtype(np.float32): torch.float32,
     np.dtype(np.float64): torch.float64, np.dtype(np.float16): torch.float16,
 }
 

@@ -42,6 +42,15 @@ __device__ __forceinline__ T SaturateCast(float v)
         r       = fminf(fmaxf(r, -32768.f), 32767.f);
         return (int16_t)(int)(v != v ? 0.f : r);
     }
+    else if constexpr (std::is_same_v<T, uint32_t>)
+    {
+        const float r = rintf(v);
+        if (!(r > 0.f)) // also NaN
+        {
+            return 0u;
+        }
+        return r >= 4294967296.f ? 0xFFFFFFFFu : (uint32_t)r;
+    }
     else if constexpr (std::is_same_v<T, int32_t>)
     {
         if (v != v)

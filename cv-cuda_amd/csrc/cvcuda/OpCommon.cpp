@@ -51,6 +51,7 @@ int ElemSize(ElemType t)
     case kF16:
         return 2;
     case kS32:
+    case kU32:
     case kF32:
         return 4;
     case kF64:
@@ -66,7 +67,7 @@ ElemType ElemFrom(NVCVDataKind kind, int bits)
     switch (kind)
     {
     case NVCV_DATA_KIND_UNSIGNED:
-        return bits == 8 ? kU8 : bits == 16 ? kU16 : kUnknown;
+        return bits == 8 ? kU8 : bits == 16 ? kU16 : bits == 32 ? kU32 : kUnknown;
     case NVCV_DATA_KIND_SIGNED:
         return bits == 8 ? kS8 : bits == 16 ? kS16 : bits == 32 ? kS32 : kUnknown;
     case NVCV_DATA_KIND_FLOAT:

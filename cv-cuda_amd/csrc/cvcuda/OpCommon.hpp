@@ -144,6 +144,7 @@ enum ElemType
     kF32     = 5,
     kF64     = 6,
     kF16     = 7,
+    kU32     = 8, // beyond the reference's enum: CropFlipNormalizeReformat and the byte-moving operators take it
     kUnknown = -1
 };
 

@@ -54,7 +54,7 @@ __device__ __forceinline__ T BorderValueAs(float v)
     {
         // truncation toward zero, saturated to the range of T
         const float lo = (float)std::numeric_limits<T>::min(), hi = (float)std::numeric_limits<T>::max();
-        return (T)(int)fminf(fmaxf(truncf(v), lo), hi);
+        return (T)(long long)fminf(fmaxf(truncf(v), lo), hi);
     }
 }
 
@@ -341,6 +341,9 @@ void DispatchDst(ElemType out, const CfnrArgs &a, int N, hipStream_t stream)
     case kS32:
         Launch<TS, int32_t>(a, N, stream);
         break;
+    case kU32:
+        Launch<TS, uint32_t>(a, N, stream);
+        break;
     case kF32:
         Launch<TS, float>(a, N, stream);
         break;
@@ -367,6 +370,9 @@ void DispatchSrc(ElemType in, ElemType out, const CfnrArgs &a, int N, hipStream_
         break;
     case kS32:
         DispatchDst<int32_t>(out, a, N, stream);
+        break;
+    case kU32:
+        DispatchDst<uint32_t>(out, a, N, stream);
         break;
     case kF32:
         DispatchDst<float>(out, a, N, stream);

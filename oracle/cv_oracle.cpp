@@ -37,6 +37,7 @@ enum DType
     S32 = 4,
     F32 = 5,
     F64 = 6,
+    U32 = 8, // not in the reference's legacy enum; used by CropFlipNormalizeReformat only
 };
 
 // ---- saturate cast: round-half-to-even then clamp ------------------------------------------------
@@ -920,6 +921,9 @@ int DispatchType(int dtype, F &&f)
         return 0;
     case F32:
         f(float{});
+        return 0;
+    case U32:
+        f(uint32_t{});
         return 0;
     default:
         return -1;

@@ -32,7 +32,7 @@ def lib():
 
 
 DTYPE_CODE = {np.dtype(np.uint8): 0, np.dtype(np.int8): 1, np.dtype(np.uint16): 2, np.dtype(np.int16): 3,
-              np.dtype(np.int32): 4, np.dtype(np.float32): 5, np.dtype(np.float64): 6}
+              np.dtype(np.int32): 4, np.dtype(np.float32): 5, np.dtype(np.float64): 6, np.dtype(np.uint32): 8}
 
 
 def _p(a):

@@ -32,8 +32,14 @@ ROWS = [
     # beyond the reference's table: the classification pipeline shape (u8 RGB -> f32 NCHW, mean/std)
     (320, 240, 6, False, False, STDDEV, 1.0, 0.0, 0.0, "RGB8", "RGBf32p", 0, np.uint8, np.float32),
     (64, 48, 4, False, False, 0, 0.5, 3.0, 0.0, "RGB8", "RGB8", 2, np.uint8, np.int8),
+    # 32-bit unsigned on either side (reference type tables OpCropFlipNormalizeReformat.cu:335-341, 449-454);
+    # the inputs span the whole range, so results saturate at both ends
+    (33, 21, 3, True, True, 0, 1.0, 0.0, 0.0, "U32", "U32", 0, np.uint32, np.uint32),
+    (33, 21, 3, True, True, 0, 1.5, -7.0e8, 0.0, "U32", "U32", 1, np.uint32, np.uint32),
+    (33, 21, 3, True, True, 0, 2.0e7, 0.0, 0.0, "U8", "U32", 0, np.uint8, np.uint32),
+    (33, 21, 3, True, True, 0, 1.0, 0.0, 0.0, "U32", "F32", 2, np.uint32, np.float32),
 ]
-CHANNELS = {"RGB8": 3, "RGB8p": 3, "RGBA8": 4, "RGBA8p": 4, "U8": 1, "F32": 1, "S32": 1, "RGBf32": 3, "RGBf32p": 3,
+CHANNELS = {"RGB8": 3, "RGB8p": 3, "RGBA8": 4, "RGBA8p": 4, "U8": 1, "F32": 1, "S32": 1, "U32": 1, "RGBf32": 3, "RGBf32p": 3,
             "RGBAf32": 4, "RGBAf32p": 4}
 
 
@@ -58,6 +64,8 @@ def test_reference_rows(cv, K, orc, gpu, row):
         iw = int(rng.integers(int(w * 0.8), int(w * 1.1) + 1))
         ih = int(rng.integers(int(h * 0.8), int(h * 1.1) + 1))
         a = orc.fill_u8((ih, iw, c), 900 + i).astype(ts)
+        if ts == np.uint32:
+            a = a * np.uint32(0x01010101)
         if ts == np.float32:
             a = a + orc.fill_f32((ih, iw, c), 950 + i)
         hosts.append(a)
@@ -73,7 +81,8 @@ def test_reference_rows(cv, K, orc, gpu, row):
     scale = orc.fill_f32((1, 1, 1, 1 if sscale else 4), 6)
     planar_out = dfmt.endswith("p")
     out = cv.Tensor.alloc([n, c, oh, ow] if planar_out else [n, oh, ow, c], td, "NCHW" if planar_out else "NHWC")
-    out.torch_view().fill_(77)
+    if td != np.uint32:  # torch has no fill for 32-bit unsigned tensors; every element is written anyway
+        out.torch_view().fill_(77)
     cv.CropFlipNormalizeReformat()(None, batch, out, cv.Tensor.from_numpy(crops, "NHWC"), border, 1.0,
                                    cv.Tensor.from_numpy(flips, "N"), cv.Tensor.from_numpy(base, "NHWC"),
                                    cv.Tensor.from_numpy(scale, "NHWC"), gscale, shift, eps, flags)
