@@ -3,9 +3,10 @@
  * src/cvcuda/priv/OpResize.cu:68-548 and src/cvcuda/priv/legacy/resize_var_shape.cu:92-548).
  *
  * in/out: [N]HWC tensors (or image batches) of u8 / u16 / s16 / f32 with 1, 3 or 4 channels, same
- * dtype, channel count and batch size. AREA (box filter over the covered source rectangle,
- * cuda_tools/InterpolationWrap.hpp:668-760) is available for tensors; image batches take NEAREST,
- * LINEAR and CUBIC. Status: INVALID_ARGUMENT for any mismatch or unsupported interpolation. */
+ * dtype, channel count and batch size. AREA is the box filter over the covered source rectangle
+ * (tensors: cuda_tools/InterpolationWrap.hpp:668-760; image batches: the reference's separate kernel,
+ * legacy/resize_var_shape.cu:236-428, whose enlargements are a bilinear variant).
+ * Status: INVALID_ARGUMENT for any mismatch or unsupported interpolation. */
 #ifndef CVCUDA_RESIZE_H
 #define CVCUDA_RESIZE_H
 
