@@ -858,7 +858,8 @@ template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeWavePatch<T, C, INTERP, false>(p, blockIdx.x * kPatchTileW, blockIdx.y * kPatchTileH + (threadIdx.x >> 6) * 4);
+    // blocks are 4 waves stacked vertically, or single waves when the whole launch is small
+    ResizeWavePatch<T, C, INTERP, false>(p, blockIdx.x * kPatchTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 4);
 }
 
 template<class T, int C, int INTERP>
@@ -1019,8 +1020,12 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     }
     if constexpr (kPatchForm<T, C, INTERP>)
     {
-        dim3 pgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, kPatchTileH), N);
-        hipLaunchKernelGGL((ResizePatchTensorKernel<T, C, INTERP>), pgrid, dim3(256), 0, stream, a);
+        // a launch of under 8 four-wave blocks per CU is spread as single-wave blocks: it is latency-bound
+        // and finishes sooner the more CUs take part
+        const int64_t blocks = (int64_t)DivUp(a.dstW, kPatchTileW) * DivUp(a.dstH, kPatchTileH) * N;
+        const int     waves  = blocks < 8 * 256 ? 1 : 4;
+        dim3          pgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, 4 * waves), N);
+        hipLaunchKernelGGL((ResizePatchTensorKernel<T, C, INTERP>), pgrid, dim3(64 * waves), 0, stream, a);
         CheckLaunch("ResizePatchTensorKernel");
         return;
     }
