@@ -79,6 +79,16 @@ __device__ __forceinline__ uint8_t SaturateU8(int v)
     return (uint8_t)min(max(v, 0), 255);
 }
 
+// A pointer read from memory (an image descriptor's base address) is generic to the compiler, and
+// every access through it becomes a flat instruction that also waits on the LDS counter. Image data
+// always lives in global memory: saying so turns those accesses into global loads and stores.
+template<class T>
+__device__ __forceinline__ T *AsGlobal(T *p)
+{
+    // through an integer: a plain pointer cast to the global address space and back is folded away
+    return (T *)(__attribute__((address_space(1))) T *)reinterpret_cast<uintptr_t>(p);
+}
+
 // Loads of 4 / 8 bytes from an address of arbitrary alignment. gfx950 global memory instructions
 // accept unaligned addresses, so these compile to a single global_load_dword / _dwordx2.
 struct __attribute__((packed, aligned(1))) UnalignedU32
@@ -113,10 +123,11 @@ __device__ __forceinline__ uint32_t LoadU32Window(const uint8_t *p)
     {
         uint32_t d[2];
     };
-    const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
-    const uint32_t  sh   = ((uint32_t)addr & 3u) * 8u;
-    const W2        w    = *reinterpret_cast<const W2 *>(addr & ~(uintptr_t)3);
-    return __builtin_amdgcn_alignbit(w.d[1], w.d[0], sh);
+    // the window's address is derived from p by pointer arithmetic (not through an integer), which
+    // keeps it a global-memory access instead of a generic (flat) one
+    const uint32_t off = (uint32_t)reinterpret_cast<uintptr_t>(p) & 3u;
+    const W2       w   = *reinterpret_cast<const W2 *>(p - off);
+    return __builtin_amdgcn_alignbit(w.d[1], w.d[0], off * 8u);
 }
 
 __device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *p)
@@ -125,11 +136,10 @@ __device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *p)
     {
         uint32_t d[3];
     };
-    const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
-    const uint32_t  sh   = ((uint32_t)addr & 3u) * 8u;
-    const W3        w    = *reinterpret_cast<const W3 *>(addr & ~(uintptr_t)3);
-    const uint32_t  lo   = __builtin_amdgcn_alignbit(w.d[1], w.d[0], sh);
-    const uint32_t  hi   = __builtin_amdgcn_alignbit(w.d[2], w.d[1], sh);
+    const uint32_t off = (uint32_t)reinterpret_cast<uintptr_t>(p) & 3u;
+    const W3       w   = *reinterpret_cast<const W3 *>(p - off);
+    const uint32_t lo  = __builtin_amdgcn_alignbit(w.d[1], w.d[0], off * 8u);
+    const uint32_t hi  = __builtin_amdgcn_alignbit(w.d[2], w.d[1], off * 8u);
     return ((uint64_t)hi << 32) | lo;
 }
 

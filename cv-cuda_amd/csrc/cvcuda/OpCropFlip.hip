@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void FlipVarShape(const CopyArgs a, const VarT
     const int  code    = *reinterpret_cast<const int32_t *>(a.codes + tc.image * a.codeStride);
     const bool mirrorX = code == 1 || code == -1, mirrorY = code == 0 || code == -1;
     const int  sx = mirrorX ? d.width - 1 - x : x, sy = mirrorY ? d.height - 1 - y : y;
-    CopyRun<T, C>(s.basePtr + (int64_t)sy * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, sx,
+    CopyRun<T, C>(AsGlobal(s.basePtr) + (int64_t)sy * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, sx,
                   mirrorX ? -1 : 1, x);
 }
 

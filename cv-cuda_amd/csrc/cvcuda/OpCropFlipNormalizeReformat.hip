@@ -112,11 +112,11 @@ __global__ __launch_bounds__(256) void CfnrKernel(const CfnrArgs a)
             else if (a.srcPlanar)
             {
                 const NVCVImagePlaneStrided &pl = img.planes[c];
-                v = reinterpret_cast<const TS *>(pl.basePtr + (int64_t)sy * pl.rowStride)[sx];
+                v = reinterpret_cast<const TS *>(AsGlobal(pl.basePtr) + (int64_t)sy * pl.rowStride)[sx];
             }
             else
             {
-                v = reinterpret_cast<const TS *>(p0.basePtr + (int64_t)sy * p0.rowStride)[sx * a.C + c];
+                v = reinterpret_cast<const TS *>(AsGlobal(p0.basePtr) + (int64_t)sy * p0.rowStride)[sx * a.C + c];
             }
             const float b = a.base[a.baseC == 1 ? 0 : c];
             const float s = a.scale[a.scaleC == 1 ? 0 : c];
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void CfnrRunsKernel(const CfnrArgs a)
     const int      code    = *reinterpret_cast<const int32_t *>(a.flip + n * a.flipStride);
     const bool     mirrorX = code == 1 || code == -1, mirrorY = code == 0 || code == -1;
     const NVCVImagePlaneStrided &p0 = a.srcList[n].planes[0];
-    const uint8_t *srcBase = p0.basePtr;
+    const uint8_t *srcBase = AsGlobal(p0.basePtr);
     const int      srcRow = p0.rowStride, srcW = p0.width, srcH = p0.height;
     // every uniform value is loaded before the first use, so the loads share one round trip
     float b[C], m[C];

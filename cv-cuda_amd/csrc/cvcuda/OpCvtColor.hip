@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256) void Yuv420ToRgbVarShape(const YuvArgs a, cons
     {
         return;
     }
-    ConvertBlock<DCN, SEMIPLANAR>(s.basePtr, s.rowStride, d.basePtr, d.rowStride, W, H, x, y, a.bidx, a.uidx);
+    ConvertBlock<DCN, SEMIPLANAR>(AsGlobal(s.basePtr), s.rowStride, AsGlobal(d.basePtr), d.rowStride, W, H, x, y, a.bidx, a.uidx);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void SwizzleVarShape(const SwizzleArgs a, cons
     {
         return;
     }
-    SwizzleRun<T, SCH, DCH>(s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, x0,
+    SwizzleRun<T, SCH, DCH>(AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0,
                             a.bidx, a.alpha);
 }
 

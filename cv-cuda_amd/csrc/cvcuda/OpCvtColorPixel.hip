@@ -500,7 +500,7 @@ __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTil
     {
         return;
     }
-    MapRun<Op>(s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, x0, a);
+    MapRun<Op>(AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0, a);
 }
 
 // Subsampled formats: one work item (Op::kItemW x Op::kItemH pixels) per lane, tensors only.

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void NormVarShape(const NormArgs a, const VarT
     {
         return;
     }
-    NormPixel<TI, TO, C>(a, s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, 0, 0, x);
+    NormPixel<TI, TO, C>(a, AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, 0, 0, x);
 }
 
 // Per-channel base/scale: runs of P pixels per lane, one row per wave.
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void NormRunsVarShape(const NormArgs a, const 
     {
         return;
     }
-    NormRun<TI, TO, C>(a, s.basePtr + (int64_t)y * s.rowStride, d.basePtr + (int64_t)y * d.rowStride, d.width, x0);
+    NormRun<TI, TO, C>(a, AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0);
 }
 
 inline bool PerChannelOnly(const ParamView &p)

@@ -14,6 +14,7 @@
 //  * everything else (12/16-byte pixels, AREA): one lane per output pixel, a 256-thread block covers
 //    64 columns x 4 rows, pixels moved as whole C-channel vectors.
 #include "DeviceUtils.hpp"
+#include "LaneExchange.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
 
@@ -67,8 +68,8 @@ __device__ __forceinline__ Plane GetPlanes(const ResizeArgs &a, int n)
     {
         const NVCVImagePlaneStrided &s = a.srcList[n].planes[0];
         const NVCVImagePlaneStrided &d = a.dstList[n].planes[0];
-        p = {s.basePtr,
-             d.basePtr,
+        p = {AsGlobal(s.basePtr),
+             AsGlobal(d.basePtr),
              s.rowStride,
              d.rowStride,
              s.width,
@@ -678,81 +679,6 @@ struct __attribute__((packed, aligned(1))) UnalignedDword
 {
     uint32_t w;
 };
-
-// Within every group of 4 adjacent lanes: r[k] of lane i <-> r[i] of lane k (i = lane & 3), as two
-// butterfly stages of cross-lane moves inside the group (no LDS).
-__device__ __forceinline__ uint32_t FromLaneXor1(uint32_t v)
-{
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, false);
-}
-
-__device__ __forceinline__ uint32_t FromLaneXor2(uint32_t v)
-{
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E /* quad_perm 2,3,0,1 */, 0xF, 0xF, false);
-}
-
-__device__ __forceinline__ void QuadTranspose(uint32_t (&r)[4], int i)
-{
-    const bool odd = (i & 1) != 0, upper = (i & 2) != 0;
-#pragma unroll
-    for (int b = 0; b < 4; b += 2) // 2x2 blocks (r0,r1) and (r2,r3) between lanes i and i^1
-    {
-        const uint32_t got = FromLaneXor1(odd ? r[b] : r[b + 1]);
-        r[b]               = odd ? got : r[b];
-        r[b + 1]           = odd ? r[b + 1] : got;
-    }
-#pragma unroll
-    for (int b = 0; b < 2; ++b) // (r0,r2) and (r1,r3) between lanes i and i^2
-    {
-        const uint32_t got = FromLaneXor2(upper ? r[b] : r[b + 2]);
-        r[b]               = upper ? got : r[b];
-        r[b + 2]           = upper ? r[b + 2] : got;
-    }
-}
-
-// 4 pixels of PB bytes, each held zero-extended in ceil(PB/4) dwords (q[d][k] = dword d of pixel k),
-// packed back to back into PB dwords.
-template<int PB>
-__device__ __forceinline__ void PackQuad(const uint32_t (&q)[(PB + 3) / 4][4], uint32_t (&w)[PB])
-{
-    if constexpr (PB % 4 == 0)
-    {
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-        {
-#pragma unroll
-            for (int d = 0; d < PB / 4; ++d)
-            {
-                w[k * (PB / 4) + d] = q[d][k];
-            }
-        }
-    }
-    else if constexpr (PB == 1)
-    {
-        w[0] = q[0][0] | (q[0][1] << 8) | (q[0][2] << 16) | (q[0][3] << 24);
-    }
-    else if constexpr (PB == 2)
-    {
-        w[0] = q[0][0] | (q[0][1] << 16);
-        w[1] = q[0][2] | (q[0][3] << 16);
-    }
-    else if constexpr (PB == 3)
-    {
-        w[0] = q[0][0] | (q[0][1] << 24);
-        w[1] = (q[0][1] >> 8) | (q[0][2] << 16);
-        w[2] = (q[0][2] >> 16) | (q[0][3] << 8);
-    }
-    else
-    {
-        static_assert(PB == 6, "pixel sizes: 1, 2, 3, 4, 6, 8, 12, 16 bytes");
-        w[0] = q[0][0];
-        w[1] = q[1][0] | (q[0][1] << 16);
-        w[2] = (q[0][1] >> 16) | (q[1][1] << 16);
-        w[3] = q[0][2];
-        w[4] = q[1][2] | (q[0][3] << 16);
-        w[5] = (q[0][3] >> 16) | (q[1][3] << 16);
-    }
-}
 
 // One wave resizes a 64-column x 4-row patch of the output whose top left pixel is (x0, y0), both
 // wave-uniform. Sampling: lane l owns column x0 + l and computes its 4 rows (the column terms are

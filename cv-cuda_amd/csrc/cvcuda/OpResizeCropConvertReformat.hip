@@ -95,7 +95,7 @@ __device__ __forceinline__ SrcImage GetSource(const FusedArgs &a, int n)
     if constexpr (VARSHAPE)
     {
         const NVCVImagePlaneStrided &pl = a.srcList[n].planes[0];
-        s.base                          = pl.basePtr;
+        s.base                          = AsGlobal(pl.basePtr);
         s.rowStride                     = pl.rowStride;
         s.w                             = pl.width;
         s.h                             = pl.height;

@@ -12,18 +12,20 @@
 // owns no device buffer and launches no separate inversion kernel; several var-shape submissions of
 // one operator handle may therefore be in flight at once. Var-shape batches run on a packed tile grid.
 //
-// Kernel shape. A 256-thread block produces a 64 x 16 pixel tile of the destination in two phases.
+// Kernel shape. A 256-thread block produces a 64 x 16 pixel tile of the destination; each of its four
+// waves works on its own 32 x 8 part, no LDS and no barrier.
 // Gather: the cost of the gather is set by how many distinct cache lines one wave-wide load touches,
 // and under a rotation every source row a wave's footprint crosses is another line; so a wave samples
 // compact 8 x 8 pixel patches (one lane per pixel, ~10 source rows per load where a 64 x 1 strip would
-// cross ~20), four patches per wave, i.e. kPxPerLane = 4 independent samples per lane whose loads are
-// in flight together. Taps that lie inside the source image - nearly all of them - skip the border
-// logic and fetch the horizontally adjacent taps of a row with one wide load (u8x3: the 6 bytes of two
-// pixels in one 8-byte load). Store: the results cross over through LDS so that each lane writes 4
-// consecutive pixels of one row as whole dwords (16 lanes cover a 64-pixel row segment); single-byte
-// stores scattered over 8 rows are several times slower. The block prologue (tile lookup, matrix
-// load / inversion) is paid once per 4 pixels.
+// cross ~20), four patches side by side per wave, i.e. kPxPerLane = 4 independent samples per lane
+// whose loads are in flight together. Taps that lie inside the source image - nearly all of them -
+// skip the border logic and fetch the horizontally adjacent taps of a row with one load (u8x3: the 6
+// bytes of two pixels from an aligned 12-byte window).
+// Store: a 4x4 transpose inside every group of 4 lanes (cross-lane moves) turns "one pixel in each of 4
+// patches" into "4 consecutive pixels of one row in one patch", which the lane writes as whole dwords;
+// single-byte stores scattered over 8 rows are several times slower.
 #include "DeviceUtils.hpp"
+#include "LaneExchange.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
 
@@ -403,15 +405,14 @@ template<class T, int C, int INTERP>
 __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dst, int dstRow,
                                          int dstW, int dstH, int tx, int ty)
 {
-    constexpr int PB       = C * sizeof(T);
-    constexpr int kLdsRow  = kTileW * PB + 4; // + 1 bank: the 8 rows of a patch start in different banks
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kTileH * kLdsRow];
+    constexpr int PB = C * sizeof(T), D = (PB + 3) / 4;
 
-    // ---- gather: lane (lx, ly) of wave w samples its pixel in patches 4w .. 4w+3
+    // ---- gather: lane (lx, ly) of wave w samples its pixel in patches 4w .. 4w+3 (side by side: a
+    // wave covers 32 columns x 8 rows)
     const int wave = threadIdx.x >> 6, lx = threadIdx.x & (kPatch - 1), ly = (threadIdx.x >> 3) & (kPatch - 1);
     const float wf = (float)im.w, hf = (float)im.h;
     float       sx[kPxPerLane], sy[kPxPerLane];
-    int         ldsAt[kPxPerLane];
+    uint32_t    q[D][kPxPerLane]; // q[d][k]: dword d of this lane's pixel in patch k
     // rows too long or too many for 24-bit offset arithmetic go through the generic path
     bool allInside = (im.row | im.h) < (1 << 23);
 #pragma unroll
@@ -419,7 +420,6 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     {
         const int patch = wave * kPxPerLane + k;
         const int px = (patch & 7) * kPatch + lx, py = (patch >> 3) * kPatch + ly;
-        ldsAt[k]     = py * kLdsRow + px * PB;
         // pixels of the tile beyond the image edge repeat the edge pixel's sample; they are never stored
         const int dx = min(tx * kTileW + px, dstW - 1), dy = min(ty * kTileH + py, dstH - 1);
         if (a.perspective)
@@ -443,10 +443,12 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
 #pragma unroll
         for (int k = 0; k < kPxPerLane; ++k)
         {
+            uint32_t w[D] = {};
+            __builtin_memcpy(w, v[k], PB);
 #pragma unroll
-            for (int c = 0; c < C; ++c)
+            for (int d = 0; d < D; ++d)
             {
-                reinterpret_cast<T *>(lds + ldsAt[k])[c] = v[k][c];
+                q[d][k] = w[d];
             }
         }
     }
@@ -455,8 +457,8 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
 #pragma nounroll
         for (int k = 0; k < kPxPerLane; ++k)
         {
-            // position and coordinates recomputed rather than indexed: a dynamic index would put the
-            // arrays in scratch memory
+            // position and coordinates recomputed rather than indexed, results placed by selects: a
+            // run-time index would put the arrays in scratch memory
             const int patch = wave * kPxPerLane + k;
             const int px = (patch & 7) * kPatch + lx, py = (patch >> 3) * kPatch + ly;
             const int dx = min(tx * kTileW + px, dstW - 1), dy = min(ty * kTileH + py, dstH - 1);
@@ -471,40 +473,64 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
             }
             T v[C];
             SampleWithBorder<T, C, INTERP>(im, a, bx, by, v);
+            uint32_t w[D] = {};
+            __builtin_memcpy(w, v, PB);
 #pragma unroll
-            for (int c = 0; c < C; ++c)
+            for (int d = 0; d < D; ++d)
             {
-                reinterpret_cast<T *>(lds + py * kLdsRow + px * PB)[c] = v[c];
+#pragma unroll
+                for (int j = 0; j < kPxPerLane; ++j)
+                {
+                    q[d][j] = k == j ? w[d] : q[d][j];
+                }
             }
         }
     }
-    __syncthreads();
 
-    // ---- store: thread t writes pixels 4*(t & 15) .. +3 of tile row t >> 4
-    const int row = threadIdx.x >> 4, x0 = (threadIdx.x & 15) * 4;
-    const int dy = ty * kTileH + row, dx0 = tx * kTileW + x0;
+    // ---- store: the 4 lanes lx & ~3 .. | 3 hold columns 4g .. 4g+3 (g = lx >> 2) of row ly in each of the
+    // wave's 4 patches; after a 4x4 transpose lane i = lx & 3 holds those 4 columns of patch 4w + i
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+    {
+        QuadTranspose(q[d], lx & 3);
+    }
+    const int patch = wave * kPxPerLane + (lx & 3);
+    const int px0 = (patch & 7) * kPatch + (lx & 4), py = (patch >> 3) * kPatch + ly;
+    const int dy = ty * kTileH + py, dx0 = tx * kTileW + px0;
     if (dy >= dstH || dx0 >= dstW)
     {
         return;
     }
-    const uint8_t *from  = lds + row * kLdsRow + x0 * PB;
-    uint8_t       *to    = dst + (int64_t)dy * dstRow + (int64_t)dx0 * PB;
-    const int      count = min(4, dstW - dx0);
-    if (count == 4)
+    uint8_t *to = dst + (int64_t)dy * dstRow + (int64_t)dx0 * PB;
+    if (dx0 + 4 <= dstW)
     {
+        uint32_t w[PB];
+        PackQuad<PB>(q, w);
         // streaming stores: the output is not read back by this kernel
         UnalignedWord *ow = reinterpret_cast<UnalignedWord *>(to);
 #pragma unroll
         for (int i = 0; i < PB; ++i) // 4 pixels = PB dwords
         {
-            __builtin_nontemporal_store(reinterpret_cast<const uint32_t *>(from)[i], &ow[i].w);
+            __builtin_nontemporal_store(w[i], &ow[i].w);
         }
     }
     else
     {
-        for (int i = 0; i < count * C; ++i)
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
         {
-            reinterpret_cast<T *>(to)[i] = reinterpret_cast<const T *>(from)[i];
+            if (dx0 + k < dstW)
+            {
+                uint32_t w[D];
+#pragma unroll
+                for (int d = 0; d < D; ++d)
+                {
+                    w[d] = q[d][k];
+                }
+                Vec<T, C> px;
+                __builtin_memcpy(&px, w, PB);
+                reinterpret_cast<Vec<T, C> *>(to)[k] = px;
+            }
         }
     }
 }
@@ -585,8 +611,8 @@ __global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarT
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
     float                        m[9];
     LoadMatrix(a, tc.image, m);
-    const Img im = {s.basePtr, s.rowStride, s.width, s.height};
-    WarpTile<T, C, INTERP>(im, a, m, d.basePtr, d.rowStride, d.width, d.height, tc.tx, tc.ty);
+    const Img im = {AsGlobal(s.basePtr), s.rowStride, s.width, s.height};
+    WarpTile<T, C, INTERP>(im, a, m, AsGlobal(d.basePtr), d.rowStride, d.width, d.height, tc.tx, tc.ty);
 }
 
 template<class T, int C, int INTERP>
