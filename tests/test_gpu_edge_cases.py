@@ -1,0 +1,100 @@
+"""Edge cases shared by the operators: empty image batches, one-pixel images, rows whose width is not
+a multiple of anything, odd base addresses and pitches (views into a larger buffer)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
+
+
+def test_empty_image_batches_are_rejected_like_the_reference(cv, K, gpu):
+    # nothing pushed: a batch without images has no format, which the reference reports as
+    # INVALID_ARGUMENT (e.g. legacy/resize_var_shape.cu:502-506); nothing is launched
+    a, b = cv.ImageBatchVarShape(4), cv.ImageBatchVarShape(4)
+    ident = cv.Tensor.from_numpy(np.tile(np.array([[1, 0, 0, 0, 1, 0]], np.float32), (4, 1)), "NW")
+    codes = cv.Tensor.from_numpy(np.zeros(4, np.int32), "N")
+    one = cv.Tensor.from_numpy(np.ones((1, 1, 1, 1), np.float32), "NHWC")
+    calls = [lambda: cv.Resize()(None, a, b, LINEAR),
+             lambda: cv.WarpAffine(4)(None, a, b, ident, LINEAR, 0, (0, 0, 0, 0)),
+             lambda: cv.Flip(4)(None, a, b, codes),
+             lambda: cv.Normalize()(None, a, one, one, b),
+             lambda: cv.CvtColor()(None, a, b, K.COLOR_BGR2RGB)]
+    for call in calls:
+        with pytest.raises(cv.Error) as e:
+            call()
+        assert e.value.status == 2
+    torch.cuda.synchronize()
+    assert len(a) == 0 and len(b) == 0
+
+
+@pytest.mark.parametrize("dt,c", [(np.uint8, 1), (np.uint8, 3), (np.uint8, 4), (np.uint16, 3), (np.float32, 1),
+                                  (np.float32, 4)])
+def test_one_pixel_and_one_row_images(cv, orc, gpu, dt, c):
+    rng = np.random.default_rng(11)
+    for (sh, sw), (dh, dw) in [((1, 1), (1, 1)), ((1, 1), (5, 7)), ((1, 9), (1, 4)), ((9, 1), (4, 1)), ((1, 9), (3, 13)),
+                               ((2, 2), (5, 5)), ((3, 3), (1, 1))]:
+        src = (rng.random((2, sh, sw, c)) * 200).astype(dt)
+        for interp in (NEAREST, LINEAR, CUBIC):
+            out = cv.Tensor.alloc([2, dh, dw, c], dt, "NHWC")
+            cv.Resize()(None, cv.Tensor.from_numpy(src, "NHWC"), out, interp)
+            torch.cuda.synchronize()
+            ref = orc.resize(src, (dh, dw), interp, variant=0 if interp == NEAREST else 1)
+            got = out.numpy()
+            if dt == np.float32:
+                assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max()), (sh, sw, dh, dw, interp)
+            else:
+                np.testing.assert_array_equal(got, ref, err_msg=str((sh, sw, dh, dw, interp)))
+
+
+def test_odd_base_addresses_and_pitches(cv, K, orc, gpu):
+    # operators on views that start at an odd byte of a larger buffer and have an odd row pitch: the
+    # run kernels' dword accesses must not assume alignment
+    n, h, w, c = 2, 19, 37, 3
+    pitch, plane = w * c + 5, (w * c + 5) * h + 3
+    src = orc.fill_u8((n, h, w, c), 77)
+    big_in = torch.zeros(n * plane + 64, dtype=torch.uint8, device="cuda")
+    big_out = torch.full((n * plane + 64,), 0xCD, dtype=torch.uint8, device="cuda")
+    view_in = torch.as_strided(big_in[1:], (n, h, w, c), (plane, pitch, c, 1))
+    view_in.copy_(torch.from_numpy(src).cuda())
+
+    def wrap(buf, elem=1, ch=c):
+        return cv.Tensor.wrap(buf.data_ptr() + 1, [n, h, w, ch], [plane, pitch, ch * elem, elem], np.uint8, "NHWC", keep=buf)
+
+    tin, tout = wrap(big_in), wrap(big_out)
+    out_view = torch.as_strided(big_out[1:], (n, h, w, c), (plane, pitch, c, 1))
+
+    def untouched():
+        mask = torch.ones_like(big_out, dtype=torch.bool)
+        torch.as_strided(mask[1:], (n, h, w * c), (plane, pitch, 1)).fill_(False)
+        return bool((big_out[mask] == 0xCD).all())
+
+    cv.CvtColor()(None, tin, tout, K.COLOR_BGR2RGB)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out_view.cpu().numpy(), src[..., ::-1])
+    assert untouched()
+
+    cv.Flip()(None, tin, tout, 1)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out_view.cpu().numpy(), src[:, :, ::-1])
+    assert untouched()
+
+    base = cv.Tensor.from_numpy(np.array([[[[3.0, 5.0, 7.0]]]], np.float32), "NHWC")
+    scale = cv.Tensor.from_numpy(np.array([[[[0.5, 1.5, 2.0]]]], np.float32), "NHWC")
+    cv.Normalize()(None, tin, base, scale, tout, 1.0, 0.0, 0.0, 0)
+    torch.cuda.synchronize()
+    ref = orc.normalize(src, np.array([[[[3.0, 5.0, 7.0]]]], np.float32), np.array([[[[0.5, 1.5, 2.0]]]], np.float32))
+    np.testing.assert_array_equal(out_view.cpu().numpy(), ref)
+    assert untouched()
+
+    cv.Resize()(None, tin, tout, LINEAR)  # same size: identity
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out_view.cpu().numpy(), src)
+    assert untouched()
+
+    ident = [1, 0, 0, 0, 1, 0]
+    cv.WarpAffine(0)(None, tin, tout, ident, LINEAR, 0, (0, 0, 0, 0))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out_view.cpu().numpy(), src)
+    assert untouched()
