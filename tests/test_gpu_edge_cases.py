@@ -98,3 +98,49 @@ def test_odd_base_addresses_and_pitches(cv, K, orc, gpu):
     torch.cuda.synchronize()
     np.testing.assert_array_equal(out_view.cpu().numpy(), src)
     assert untouched()
+
+
+def test_submits_captured_in_a_hip_graph_replay_correctly(cv, K, orc, gpu):
+    # a pipeline of Submits (fused resize -> Normalize -> Reformat, plus a warp) is captured once and
+    # replayed with new input contents and eager work in between; every replay must equal the eager result
+    n = 3
+    tin = cv.Tensor.alloc([n, 90, 160, 3], np.uint8, "NHWC")
+    t1 = cv.Tensor.alloc([n, 32, 32, 3], np.float32, "NHWC")
+    t2 = cv.Tensor.alloc([n, 32, 32, 3], np.float32, "NHWC")
+    t3 = cv.Tensor.alloc([n, 3, 32, 32], np.float32, "NCHW")
+    tw = cv.Tensor.alloc([n, 90, 160, 3], np.uint8, "NHWC")
+    base = cv.Tensor.from_numpy(np.array([[[[0.4, 0.5, 0.6]]]], np.float32), "NHWC")
+    scale = cv.Tensor.from_numpy(np.array([[[[0.2, 0.3, 0.4]]]], np.float32), "NHWC")
+    fused, norm, ref_, warp = cv.ResizeCropConvertReformat(), cv.Normalize(), cv.Reformat(), cv.WarpAffine(0)
+    mat = [0.9, -0.2, 7.0, 0.2, 0.9, -3.0]
+
+    def pipeline(stream):
+        fused(stream, tin, t1, (64, 36), LINEAR, (16, 2), 0, 1 / 255.0, 0.0, False)
+        norm(stream, t1, base, scale, t2, 1.0, 0.0, 0.0, K.CVCUDA_NORMALIZE_SCALE_IS_STDDEV)
+        ref_(stream, t2, t3)
+        warp(stream, tin, tw, mat, LINEAR, 0, (0, 0, 0, 0))
+
+    tin.torch_view().copy_(torch.from_numpy(orc.fill_u8((n, 90, 160, 3), 1)).cuda())
+    pipeline(torch.cuda.current_stream())  # warm up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pipeline(torch.cuda.current_stream())
+    for seed in (2, 3, 4):
+        src = orc.fill_u8((n, 90, 160, 3), seed)
+        tin.torch_view().copy_(torch.from_numpy(src).cuda())
+        t3.torch_view().zero_()
+        tw.torch_view().zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got3, gotw = t3.numpy().copy(), tw.numpy().copy()
+        t3.torch_view().zero_()
+        tw.torch_view().zero_()
+        pipeline(torch.cuda.current_stream())  # eager work between the replays
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(got3, t3.numpy())
+        np.testing.assert_array_equal(gotw, tw.numpy())
+        x = orc.fused_rccr(src, (32, 32), (64, 36), (16, 2), LINEAR, np.float32, False, 0, 1 / 255.0, 0.0, False)
+        want = orc.normalize(x, np.array([[[[0.4, 0.5, 0.6]]]], np.float32), np.array([[[[0.2, 0.3, 0.4]]]], np.float32),
+                             1.0, 0.0, 0.0, True).transpose(0, 3, 1, 2)
+        assert (np.abs(got3 - want) <= 1e-5 * np.maximum(1.0, np.abs(want))).all()
