@@ -7,9 +7,11 @@
 // reference's CPU golden (tests/cvcuda/system/ResizeUtils.cpp:206-221) for every pixel, so results
 // are bit-exact against it also where the coordinate lands on an integer.
 //
-// Three kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
+// Four kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
+//  * u8x3 bilinear at horizontal scales up to 2 (tensors): a lane owns 2 columns x 2 rows and fetches
+//    each source row once for both columns (one 12-byte load), lane pairs swap a pixel pair each;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
 //  * everything else (12/16-byte pixels, AREA): one lane per output pixel, a 256-thread block covers
 //    64 columns x 4 rows, pixels moved as whole C-channel vectors.
@@ -778,6 +780,131 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
     }
 }
 
+// u8x3 bilinear at horizontal scales up to 2 (tensors). The cost of the wave-patch form there is the
+// number of tap loads (the texture addresser is busy 76-90 % of the time). The taps of two neighbouring
+// output columns lie within 4 source pixels = 12 bytes, so here a lane owns 2 columns x 2 rows and
+// fetches each source row once for both columns: half the loads. A wave covers 128 columns x 2 rows;
+// lanes 2j and 2j+1 then swap a pixel pair each, so that lane 2j stores columns 4j .. 4j+3 of the
+// first row and lane 2j+1 those of the second. Arithmetic as in SampleWide.
+struct __attribute__((packed, aligned(1))) TapWindow
+{
+    uint32_t w[3];
+};
+
+__device__ __forceinline__ uint32_t BlendU8x3(uint64_t top, uint64_t bot, float wx, float wy)
+{
+    const uint32_t tl = (uint32_t)top, th = (uint32_t)(top >> 32), bl = (uint32_t)bot, bh = (uint32_t)(bot >> 32);
+    const float    t0[2][3] = {{(float)(tl & 0xFF), (float)((tl >> 8) & 0xFF), (float)((tl >> 16) & 0xFF)},
+                               {(float)(tl >> 24), (float)(th & 0xFF), (float)((th >> 8) & 0xFF)}};
+    const float    t1[2][3] = {{(float)(bl & 0xFF), (float)((bl >> 8) & 0xFF), (float)((bl >> 16) & 0xFF)},
+                               {(float)(bl >> 24), (float)(bh & 0xFF), (float)((bh >> 8) & 0xFF)}};
+    uint32_t       out      = 0;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+    {
+        const float v = t0[0][c] * ((1.f - wx) * (1.f - wy)) + t0[1][c] * (wx * (1.f - wy)) + t1[0][c] * ((1.f - wx) * wy)
+                      + t1[1][c] * (wx * wy);
+        out |= (uint32_t)SaturateCast<uint8_t>(v) << (8 * c);
+    }
+    return out;
+}
+
+// The 6 bytes of the pixel pair that starts `delta` (0, 1 or 2) pixels into a 12-byte window.
+__device__ __forceinline__ uint64_t PairFromWindow(const TapWindow &t, int delta)
+{
+    const bool     far = delta == 2;
+    const uint32_t a = far ? t.w[1] : t.w[0], b = far ? t.w[2] : t.w[1], c = far ? 0u : t.w[2];
+    const uint32_t sh = delta == 0 ? 0u : (far ? 16u : 24u);
+    return ((uint64_t)__builtin_amdgcn_alignbit(c, b, sh) << 32) | __builtin_amdgcn_alignbit(b, a, sh);
+}
+
+__device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    const int  lane = threadIdx.x & 63;
+    const bool odd  = (lane & 1) != 0;
+    // columns and rows past the output compute a duplicate of the last one: every lane takes part in the swap
+    const auto colA  = Axis<NVCV_INTERP_LINEAR>(p.scaleX, min(x0 + 2 * lane, p.dstW - 1), p.srcW);
+    const auto colB  = Axis<NVCV_INTERP_LINEAR>(p.scaleX, min(x0 + 2 * lane + 1, p.dstW - 1), p.srcW);
+    const int  delta = colB.s - colA.s; // 0 .. 2 at scales up to 2
+    // the 2 rows' terms are computed side by side (even lanes the first, odd lanes the second)
+    const auto rows = Axis<NVCV_INTERP_LINEAR>(p.scaleY, min(y0 + (lane & 1), p.dstH - 1), p.srcH);
+    uint32_t   pxA[2], pxB[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+    {
+        const auto row = FromLane(rows, k);
+        const int  ya = row.s, yb = min(row.s + 1, p.srcH - 1);
+        uint64_t   topA, topB, botA, botB;
+        auto       fetch = [&](int y, uint64_t &a, uint64_t &b)
+        {
+            const uint8_t *line = p.src + (int64_t)y * p.srcRow;
+            if (y == p.srcH - 1) // wave-uniform: nothing may be read past the end of the last row
+            {
+                const int rowBytes = p.srcW * 3;
+                const int offA = colA.s * 3, offB = colB.s * 3;
+                const int backA = max(0, offA - (rowBytes - 8)), backB = max(0, offB - (rowBytes - 8));
+                a = LoadU64Unaligned(line + (offA - backA)) >> (8 * backA);
+                b = LoadU64Unaligned(line + (offB - backB)) >> (8 * backB);
+            }
+            else
+            {
+                const TapWindow t = *reinterpret_cast<const TapWindow *>(line + colA.s * 3);
+                a                 = ((uint64_t)t.w[1] << 32) | t.w[0];
+                b                 = PairFromWindow(t, delta);
+            }
+        };
+        fetch(ya, topA, topB);
+        fetch(yb, botA, botB);
+        pxA[k] = BlendU8x3(topA, botA, colA.w[0], row.w[0]);
+        pxB[k] = BlendU8x3(topB, botB, colB.w[0], row.w[0]);
+    }
+    // even lanes keep their first-row pair and take the neighbour's, odd lanes the same for the second row
+    const uint32_t got0 = FromLaneXor1(odd ? pxA[0] : pxA[1]), got1 = FromLaneXor1(odd ? pxB[0] : pxB[1]);
+    const uint32_t q[1][4] = {{odd ? got0 : pxA[0], odd ? got1 : pxB[0], odd ? pxA[1] : got0, odd ? pxB[1] : got1}};
+    const int      dy = y0 + (lane & 1), dx0 = x0 + 2 * (lane & ~1);
+    if (dy >= p.dstH || dx0 >= p.dstW)
+    {
+        return;
+    }
+    uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * 3;
+    if (dx0 + 4 <= p.dstW)
+    {
+        uint32_t w[3];
+        PackQuad<3>(q, w);
+        UnalignedDword *ow = reinterpret_cast<UnalignedDword *>(to);
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+        {
+            __builtin_nontemporal_store(w[i], &ow[i].w);
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+        {
+            if (dx0 + k < p.dstW)
+            {
+                to[3 * k + 0] = (uint8_t)q[0][k];
+                to[3 * k + 1] = (uint8_t)(q[0][k] >> 8);
+                to[3 * k + 2] = (uint8_t)(q[0][k] >> 16);
+            }
+        }
+    }
+}
+
+constexpr int kPairsTileW = 128, kPairsTileH = 8; // block = 4 waves of 128 columns x 2 rows, stacked
+
+__global__ __launch_bounds__(256) void ResizeLinearPairsU8x3Kernel(const ResizeArgs a)
+{
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizeLinearPairsU8x3(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+}
+
 constexpr int kPatchTileW = 64, kPatchTileH = 16; // block = 4 waves stacked vertically
 
 template<class T, int C, int INTERP>
@@ -941,6 +1068,16 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         {
             hipLaunchKernelGGL((ResizeCubicStagedKernel<T, C>), grid, dim3(256), 0, stream, a);
             CheckLaunch("ResizeCubicStagedKernel");
+            return;
+        }
+    }
+    if constexpr (std::is_same_v<T, uint8_t> && C == 3 && INTERP == NVCV_INTERP_LINEAR)
+    {
+        if (a.srcW >= 4 && a.srcW <= 2 * a.dstW)
+        {
+            dim3 pgrid(DivUp(a.dstW, kPairsTileW), DivUp(a.dstH, kPairsTileH), N);
+            hipLaunchKernelGGL(ResizeLinearPairsU8x3Kernel, pgrid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeLinearPairsU8x3Kernel");
             return;
         }
     }
