@@ -791,6 +791,7 @@ struct __attribute__((packed, aligned(1))) TapWindow
     uint32_t w[3];
 };
 
+template<bool VARSHAPE>
 __device__ __forceinline__ uint32_t BlendU8x3(uint64_t top, uint64_t bot, float wx, float wy)
 {
     const uint32_t tl = (uint32_t)top, th = (uint32_t)(top >> 32), bl = (uint32_t)bot, bh = (uint32_t)(bot >> 32);
@@ -802,8 +803,16 @@ __device__ __forceinline__ uint32_t BlendU8x3(uint64_t top, uint64_t bot, float 
 #pragma unroll
     for (int c = 0; c < 3; ++c)
     {
-        const float v = t0[0][c] * ((1.f - wx) * (1.f - wy)) + t0[1][c] * (wx * (1.f - wy)) + t1[0][c] * ((1.f - wx) * wy)
-                      + t1[1][c] * (wx * wy);
+        float v;
+        if constexpr (VARSHAPE)
+        {
+            v = (1.0f - wx) * (t0[0][c] * (1.0f - wy) + t1[0][c] * wy) + wx * (t0[1][c] * (1.0f - wy) + t1[1][c] * wy);
+        }
+        else
+        {
+            v = t0[0][c] * ((1.f - wx) * (1.f - wy)) + t0[1][c] * (wx * (1.f - wy)) + t1[0][c] * ((1.f - wx) * wy)
+              + t1[1][c] * (wx * wy);
+        }
         out |= (uint32_t)SaturateCast<uint8_t>(v) << (8 * c);
     }
     return out;
@@ -818,6 +827,7 @@ __device__ __forceinline__ uint64_t PairFromWindow(const TapWindow &t, int delta
     return ((uint64_t)__builtin_amdgcn_alignbit(c, b, sh) << 32) | __builtin_amdgcn_alignbit(b, a, sh);
 }
 
+template<bool VARSHAPE>
 __device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, int y0)
 {
     if (x0 >= p.dstW || y0 >= p.dstH)
@@ -859,8 +869,8 @@ __device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, in
         };
         fetch(ya, topA, topB);
         fetch(yb, botA, botB);
-        pxA[k] = BlendU8x3(topA, botA, colA.w[0], row.w[0]);
-        pxB[k] = BlendU8x3(topB, botB, colB.w[0], row.w[0]);
+        pxA[k] = BlendU8x3<VARSHAPE>(topA, botA, colA.w[0], row.w[0]);
+        pxB[k] = BlendU8x3<VARSHAPE>(topB, botB, colB.w[0], row.w[0]);
     }
     // even lanes keep their first-row pair and take the neighbour's, odd lanes the same for the second row
     const uint32_t got0 = FromLaneXor1(odd ? pxA[0] : pxA[1]), got1 = FromLaneXor1(odd ? pxB[0] : pxB[1]);
@@ -902,7 +912,25 @@ constexpr int kPairsTileW = 128, kPairsTileH = 8; // block = 4 waves of 128 colu
 __global__ __launch_bounds__(256) void ResizeLinearPairsU8x3Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeLinearPairsU8x3(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+    ResizeLinearPairsU8x3<false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+}
+
+// Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
+// above 2 (or whose source is narrower than 4 pixels) is resized as four 64 x 4 wave patches instead.
+__global__ __launch_bounds__(256) void ResizeLinearPairsU8x3VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc   = LocateTile(tiles, blockIdx.x);
+    const Plane     p    = GetPlanes<true>(a, tc.image);
+    const int       wave = threadIdx.x >> 6;
+    if (p.srcW >= 4 && p.srcW <= 2 * p.dstW)
+    {
+        ResizeLinearPairsU8x3<true>(p, tc.tx * kPairsTileW, tc.ty * kPairsTileH + wave * 2);
+    }
+    else
+    {
+        ResizeWavePatch<uint8_t, 3, NVCV_INTERP_LINEAR, true>(p, tc.tx * kPairsTileW + (wave & 1) * 64,
+                                                             tc.ty * kPairsTileH + (wave >> 1) * 4);
+    }
 }
 
 constexpr int kPatchTileW = 64, kPatchTileH = 16; // block = 4 waves stacked vertically
@@ -1103,6 +1131,16 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, 
     {
         VarTiles  tiles;
         const int count = std::min(kMaxTileImages, N - first);
+        if constexpr (std::is_same_v<T, uint8_t> && C == 3 && INTERP == NVCV_INTERP_LINEAR)
+        {
+            int total = BuildVarTiles(tiles, dstHost, first, count, kPairsTileW, kPairsTileH);
+            if (total > 0)
+            {
+                hipLaunchKernelGGL(ResizeLinearPairsU8x3VarShapeKernel, dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeLinearPairsU8x3VarShapeKernel");
+            }
+            continue;
+        }
         if constexpr (kPatchForm<T, C, INTERP>)
         {
             int total = BuildVarTiles(tiles, dstHost, first, count, kPatchTileW, kPatchTileH);
