@@ -606,10 +606,12 @@ __global__ __launch_bounds__(256) void WarpTensor(const WarpArgs a)
 template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarTiles tiles)
 {
-    const TileCoord              tc = LocateTile(tiles, blockIdx.x);
-    const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
-    const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    float                        m[9];
+    const TileCoord tc = LocateTile(tiles, blockIdx.x);
+    // descriptors and matrix depend on the image index only: read by value here, ahead of the matrix
+    // arithmetic, so that all of these loads share one memory round trip
+    const NVCVImagePlaneStrided s = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided d = a.dstList[tc.image].planes[0];
+    float                       m[9];
     LoadMatrix(a, tc.image, m);
     const Img im = {AsGlobal(s.basePtr), s.rowStride, s.width, s.height};
     WarpTile<T, C, INTERP>(im, a, m, AsGlobal(d.basePtr), d.rowStride, d.width, d.height, tc.tx, tc.ty);
