@@ -110,20 +110,21 @@ template<class TI, class TO, int C>
 __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow, uint8_t *dstRow, int W, int x0)
 {
     constexpr int P = kRunPixelsFor<TI, TO>;
+    // every uniform value is loaded before the first use, so the loads share one round trip
     float b[C], m[C];
 #pragma unroll
     for (int c = 0; c < C; ++c)
     {
-        b[c]          = a.base.ptr[c * a.base.sC];
-        const float s = a.scale.ptr[c * a.scale.sC];
-        if (a.stddev)
+        b[c] = a.base.ptr[c * a.base.sC];
+        m[c] = a.scale.ptr[c * a.scale.sC];
+    }
+    if (a.stddev)
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
         {
-            const float t = s * s + a.eps;
+            const float t = m[c] * m[c] + a.eps;
             m[c]          = 1.0f / sqrtf(t);
-        }
-        else
-        {
-            m[c] = s;
         }
     }
     if (x0 + P <= W)
