@@ -321,9 +321,9 @@ class Streaming:
         "flip-horizontal": ("Flip", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "PixelMapTensor<uint8_t,3>", "u8",
                             "Flip (columns mirrored)"),
         "resize-linear-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
-                               "ResizeLinearPairsU8x3Kernel", "f32", "Resize LINEAR 1920x1080 -> 1280x720"),
+                               "ResizeLinearPairsU8Kernel<3>", "f32", "Resize LINEAR 1920x1080 -> 1280x720"),
         "resize-linear-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
-                                  "ResizeLinearPairsU8x3Kernel", "f32", "Resize LINEAR 1280x720 -> 1920x1080"),
+                                  "ResizeLinearPairsU8Kernel<3>", "f32", "Resize LINEAR 1280x720 -> 1920x1080"),
     }
 
     def __init__(self, cv, orc, np, torch, key):

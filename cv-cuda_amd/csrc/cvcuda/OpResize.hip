@@ -10,8 +10,8 @@
 // Four kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
-//  * u8x3 bilinear at horizontal scales up to 2 (tensors): a lane owns 2 columns x 2 rows and fetches
-//    each source row once for both columns (one 12-byte load), lane pairs swap a pixel pair each;
+//  * u8x3 bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows and fetches each source
+//    row once for both columns, lane pairs swap a pixel pair each;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
 //  * everything else (12/16-byte pixels, AREA): one lane per output pixel, a 256-thread block covers
 //    64 columns x 4 rows, pixels moved as whole C-channel vectors.
@@ -780,55 +780,66 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
     }
 }
 
-// u8x3 bilinear at horizontal scales up to 2 (tensors). The cost of the wave-patch form there is the
-// number of tap loads (the texture addresser is busy 76-90 % of the time). The taps of two neighbouring
-// output columns lie within 4 source pixels = 12 bytes, so here a lane owns 2 columns x 2 rows and
-// fetches each source row once for both columns: half the loads. A wave covers 128 columns x 2 rows;
-// lanes 2j and 2j+1 then swap a pixel pair each, so that lane 2j stores columns 4j .. 4j+3 of the
-// first row and lane 2j+1 those of the second. Arithmetic as in SampleWide.
+// 8-bit bilinear at horizontal scales up to 2. The cost of the wave-patch form there is the number
+// of tap loads (the texture addresser is busy 76-90 % of the time). The taps of two neighbouring
+// output columns lie within 4 source pixels, so here a lane owns 2 columns x 2 rows and fetches each
+// source row once for both columns (one 4-, 12- or 16-byte load): half the loads. A wave covers 128
+// columns x 2 rows; lanes 2j and 2j+1 then swap a pixel pair each, so that lane 2j stores columns
+// 4j .. 4j+3 of the first row and lane 2j+1 those of the second. Arithmetic as in SampleWide.
+// Pixels travel as one dword each (channel c in byte c; higher bytes are don't-care).
+template<int C>
 struct __attribute__((packed, aligned(1))) TapWindow
 {
-    uint32_t w[3];
+    uint32_t w[C]; // 4 pixels of C bytes
 };
 
-template<bool VARSHAPE>
-__device__ __forceinline__ uint32_t BlendU8x3(uint64_t top, uint64_t bot, float wx, float wy)
+// Pixel k (0 .. 3) of a window.
+template<int C>
+__device__ __forceinline__ uint32_t WindowPixel(const TapWindow<C> &t, int k)
 {
-    const uint32_t tl = (uint32_t)top, th = (uint32_t)(top >> 32), bl = (uint32_t)bot, bh = (uint32_t)(bot >> 32);
-    const float    t0[2][3] = {{(float)(tl & 0xFF), (float)((tl >> 8) & 0xFF), (float)((tl >> 16) & 0xFF)},
-                               {(float)(tl >> 24), (float)(th & 0xFF), (float)((th >> 8) & 0xFF)}};
-    const float    t1[2][3] = {{(float)(bl & 0xFF), (float)((bl >> 8) & 0xFF), (float)((bl >> 16) & 0xFF)},
-                               {(float)(bl >> 24), (float)(bh & 0xFF), (float)((bh >> 8) & 0xFF)}};
-    uint32_t       out      = 0;
-#pragma unroll
-    for (int c = 0; c < 3; ++c)
+    if constexpr (C == 4)
     {
-        float v;
+        return t.w[k];
+    }
+    else if constexpr (C == 1)
+    {
+        return t.w[0] >> (8 * k);
+    }
+    else
+    {
+        static_assert(C == 3);
+        return k == 0 ? t.w[0]
+             : k == 1 ? __builtin_amdgcn_alignbit(t.w[1], t.w[0], 24)
+             : k == 2 ? __builtin_amdgcn_alignbit(t.w[2], t.w[1], 16)
+                      : t.w[2] >> 8;
+    }
+}
+
+template<int C, bool VARSHAPE>
+__device__ __forceinline__ uint32_t BlendU8(uint32_t p00, uint32_t p01, uint32_t p10, uint32_t p11, float wx, float wy)
+{
+    uint32_t out = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        const float t00 = (float)((p00 >> (8 * c)) & 0xFF), t01 = (float)((p01 >> (8 * c)) & 0xFF);
+        const float t10 = (float)((p10 >> (8 * c)) & 0xFF), t11 = (float)((p11 >> (8 * c)) & 0xFF);
+        float       v;
         if constexpr (VARSHAPE)
         {
-            v = (1.0f - wx) * (t0[0][c] * (1.0f - wy) + t1[0][c] * wy) + wx * (t0[1][c] * (1.0f - wy) + t1[1][c] * wy);
+            v = (1.0f - wx) * (t00 * (1.0f - wy) + t10 * wy) + wx * (t01 * (1.0f - wy) + t11 * wy);
         }
         else
         {
-            v = t0[0][c] * ((1.f - wx) * (1.f - wy)) + t0[1][c] * (wx * (1.f - wy)) + t1[0][c] * ((1.f - wx) * wy)
-              + t1[1][c] * (wx * wy);
+            v = t00 * ((1.f - wx) * (1.f - wy)) + t01 * (wx * (1.f - wy)) + t10 * ((1.f - wx) * wy) + t11 * (wx * wy);
         }
         out |= (uint32_t)SaturateCast<uint8_t>(v) << (8 * c);
     }
     return out;
 }
 
-// The 6 bytes of the pixel pair that starts `delta` (0, 1 or 2) pixels into a 12-byte window.
-__device__ __forceinline__ uint64_t PairFromWindow(const TapWindow &t, int delta)
-{
-    const bool     far = delta == 2;
-    const uint32_t a = far ? t.w[1] : t.w[0], b = far ? t.w[2] : t.w[1], c = far ? 0u : t.w[2];
-    const uint32_t sh = delta == 0 ? 0u : (far ? 16u : 24u);
-    return ((uint64_t)__builtin_amdgcn_alignbit(c, b, sh) << 32) | __builtin_amdgcn_alignbit(b, a, sh);
-}
-
-template<bool VARSHAPE>
-__device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, int y0)
+template<int C, bool VARSHAPE>
+__device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int y0)
 {
     if (x0 >= p.dstW || y0 >= p.dstH)
     {
@@ -848,29 +859,44 @@ __device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, in
     {
         const auto row = FromLane(rows, k);
         const int  ya = row.s, yb = min(row.s + 1, p.srcH - 1);
-        uint64_t   topA, topB, botA, botB;
-        auto       fetch = [&](int y, uint64_t &a, uint64_t &b)
+        uint32_t   top[4], bot[4]; // A's two taps, then B's
+        auto       fetch = [&](int y, uint32_t (&t)[4])
         {
             const uint8_t *line = p.src + (int64_t)y * p.srcRow;
             if (y == p.srcH - 1) // wave-uniform: nothing may be read past the end of the last row
             {
-                const int rowBytes = p.srcW * 3;
-                const int offA = colA.s * 3, offB = colB.s * 3;
-                const int backA = max(0, offA - (rowBytes - 8)), backB = max(0, offB - (rowBytes - 8));
-                a = LoadU64Unaligned(line + (offA - backA)) >> (8 * backA);
-                b = LoadU64Unaligned(line + (offB - backB)) >> (8 * backB);
+                float a[2][C], b[2][C];
+                LoadTaps<uint8_t, C, 2>(line, colA.s * C, true, p.srcW * C, a);
+                LoadTaps<uint8_t, C, 2>(line, colB.s * C, true, p.srcW * C, b);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    t[i] = 0;
+                }
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    t[0] |= (uint32_t)a[0][c] << (8 * c);
+                    t[1] |= (uint32_t)a[1][c] << (8 * c);
+                    t[2] |= (uint32_t)b[0][c] << (8 * c);
+                    t[3] |= (uint32_t)b[1][c] << (8 * c);
+                }
             }
             else
             {
-                const TapWindow t = *reinterpret_cast<const TapWindow *>(line + colA.s * 3);
-                a                 = ((uint64_t)t.w[1] << 32) | t.w[0];
-                b                 = PairFromWindow(t, delta);
+                const TapWindow<C> win = *reinterpret_cast<const TapWindow<C> *>(line + colA.s * C);
+                const uint32_t     k0 = WindowPixel<C>(win, 0), k1 = WindowPixel<C>(win, 1), k2 = WindowPixel<C>(win, 2),
+                               k3 = WindowPixel<C>(win, 3);
+                t[0] = k0;
+                t[1] = k1;
+                t[2] = delta == 0 ? k0 : (delta == 1 ? k1 : k2);
+                t[3] = delta == 0 ? k1 : (delta == 1 ? k2 : k3);
             }
         };
-        fetch(ya, topA, topB);
-        fetch(yb, botA, botB);
-        pxA[k] = BlendU8x3<VARSHAPE>(topA, botA, colA.w[0], row.w[0]);
-        pxB[k] = BlendU8x3<VARSHAPE>(topB, botB, colB.w[0], row.w[0]);
+        fetch(ya, top);
+        fetch(yb, bot);
+        pxA[k] = BlendU8<C, VARSHAPE>(top[0], top[1], bot[0], bot[1], colA.w[0], row.w[0]);
+        pxB[k] = BlendU8<C, VARSHAPE>(top[2], top[3], bot[2], bot[3], colB.w[0], row.w[0]);
     }
     // even lanes keep their first-row pair and take the neighbour's, odd lanes the same for the second row
     const uint32_t got0 = FromLaneXor1(odd ? pxA[0] : pxA[1]), got1 = FromLaneXor1(odd ? pxB[0] : pxB[1]);
@@ -880,14 +906,14 @@ __device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, in
     {
         return;
     }
-    uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * 3;
+    uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * C;
     if (dx0 + 4 <= p.dstW)
     {
-        uint32_t w[3];
-        PackQuad<3>(q, w);
+        uint32_t w[C];
+        PackQuad<C>(q, w);
         UnalignedDword *ow = reinterpret_cast<UnalignedDword *>(to);
 #pragma unroll
-        for (int i = 0; i < 3; ++i)
+        for (int i = 0; i < C; ++i)
         {
             __builtin_nontemporal_store(w[i], &ow[i].w);
         }
@@ -899,36 +925,46 @@ __device__ __forceinline__ void ResizeLinearPairsU8x3(const Plane &p, int x0, in
         {
             if (dx0 + k < p.dstW)
             {
-                to[3 * k + 0] = (uint8_t)q[0][k];
-                to[3 * k + 1] = (uint8_t)(q[0][k] >> 8);
-                to[3 * k + 2] = (uint8_t)(q[0][k] >> 16);
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    to[C * k + c] = (uint8_t)(q[0][k] >> (8 * c));
+                }
             }
         }
     }
 }
 
+// Which (type, channels, interpolation) take the two-columns-per-lane form. The code is written for 1, 3
+// and 4 channels; with 1 and 4 it measured slower than the wave patches (u8x1 43 -> 58 us, u8x4 91 -> 104 us
+// on 1080p -> 720p: the column terms of two columns are amortised over 2 rows only), so 3 it is.
+template<class T, int C, int INTERP>
+constexpr bool kPairsForm = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_LINEAR && C == 3;
+
 constexpr int kPairsTileW = 128, kPairsTileH = 8; // block = 4 waves of 128 columns x 2 rows, stacked
 
-__global__ __launch_bounds__(256) void ResizeLinearPairsU8x3Kernel(const ResizeArgs a)
+template<int C>
+__global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeLinearPairsU8x3<false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+    ResizeLinearPairsU8<C, false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
 }
 
 // Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
 // above 2 (or whose source is narrower than 4 pixels) is resized as four 64 x 4 wave patches instead.
-__global__ __launch_bounds__(256) void ResizeLinearPairsU8x3VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+template<int C>
+__global__ __launch_bounds__(256) void ResizeLinearPairsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
 {
     const TileCoord tc   = LocateTile(tiles, blockIdx.x);
     const Plane     p    = GetPlanes<true>(a, tc.image);
     const int       wave = threadIdx.x >> 6;
     if (p.srcW >= 4 && p.srcW <= 2 * p.dstW)
     {
-        ResizeLinearPairsU8x3<true>(p, tc.tx * kPairsTileW, tc.ty * kPairsTileH + wave * 2);
+        ResizeLinearPairsU8<C, true>(p, tc.tx * kPairsTileW, tc.ty * kPairsTileH + wave * 2);
     }
     else
     {
-        ResizeWavePatch<uint8_t, 3, NVCV_INTERP_LINEAR, true>(p, tc.tx * kPairsTileW + (wave & 1) * 64,
+        ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, tc.tx * kPairsTileW + (wave & 1) * 64,
                                                              tc.ty * kPairsTileH + (wave >> 1) * 4);
     }
 }
@@ -1099,13 +1135,13 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             return;
         }
     }
-    if constexpr (std::is_same_v<T, uint8_t> && C == 3 && INTERP == NVCV_INTERP_LINEAR)
+    if constexpr (kPairsForm<T, C, INTERP>)
     {
         if (a.srcW >= 4 && a.srcW <= 2 * a.dstW)
         {
             dim3 pgrid(DivUp(a.dstW, kPairsTileW), DivUp(a.dstH, kPairsTileH), N);
-            hipLaunchKernelGGL(ResizeLinearPairsU8x3Kernel, pgrid, dim3(256), 0, stream, a);
-            CheckLaunch("ResizeLinearPairsU8x3Kernel");
+            hipLaunchKernelGGL((ResizeLinearPairsU8Kernel<C>), pgrid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeLinearPairsU8Kernel");
             return;
         }
     }
@@ -1131,13 +1167,13 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, 
     {
         VarTiles  tiles;
         const int count = std::min(kMaxTileImages, N - first);
-        if constexpr (std::is_same_v<T, uint8_t> && C == 3 && INTERP == NVCV_INTERP_LINEAR)
+        if constexpr (kPairsForm<T, C, INTERP>)
         {
             int total = BuildVarTiles(tiles, dstHost, first, count, kPairsTileW, kPairsTileH);
             if (total > 0)
             {
-                hipLaunchKernelGGL(ResizeLinearPairsU8x3VarShapeKernel, dim3(total), dim3(256), 0, stream, a, tiles);
-                CheckLaunch("ResizeLinearPairsU8x3VarShapeKernel");
+                hipLaunchKernelGGL((ResizeLinearPairsU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeLinearPairsU8VarShapeKernel");
             }
             continue;
         }

@@ -83,16 +83,17 @@ def test_tensor_cubic_reduction(cv, orc, gpu, row):
     test_tensor_table(cv, orc, gpu, row)
 
 
-# u8x3 bilinear at horizontal scales up to 2 takes the kernel in which a lane owns two columns: both
+# 8-bit bilinear at horizontal scales up to 2 takes the kernel in which a lane owns two columns: both
 # directions, the scale limit itself, ragged widths (1 - 3 columns left over), odd heights, tiny outputs
-PAIRS = [(sw, sh, dw, dh, LINEAR, n, np.uint8, 3)
+PAIRS = [(sw, sh, dw, dh, LINEAR, n, np.uint8, c)
+         for c in (3, 1, 4)
          for (sw, sh, dw, dh, n) in [(131, 37, 66, 19, 2), (100, 40, 50, 20, 1), (64, 48, 97, 71, 2), (640, 360, 431, 243, 1),
                                      (33, 9, 130, 30, 1), (5, 4, 7, 3, 3), (4, 4, 2, 2, 1), (257, 33, 129, 17, 1),
                                      (1280, 720, 1920, 1080, 1), (1920, 1080, 1280, 720, 1)]]
 
 
 @pytest.mark.parametrize("row", PAIRS, ids=lambda r: "%dx%d-%dx%d-i%d-n%d-%s%d" % (r[:6] + (np.dtype(r[6]).name, r[7])))
-def test_tensor_linear_u8x3_pair_columns(cv, orc, gpu, row):
+def test_tensor_linear_u8_pair_columns(cv, orc, gpu, row):
     test_tensor_table(cv, orc, gpu, row)
 
 
