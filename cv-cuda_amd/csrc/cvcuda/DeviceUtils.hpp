@@ -111,6 +111,19 @@ __device__ __forceinline__ uint64_t LoadU64Unaligned(const uint8_t *p)
     return reinterpret_cast<const UnalignedU64 *>(p)->v;
 }
 
+// N dwords to an address of arbitrary alignment, as streaming stores (for output that the kernel does
+// not read back).
+template<int N>
+__device__ __forceinline__ void StoreDwordsNT(uint8_t *p, const uint32_t (&w)[N])
+{
+    UnalignedU32 *o = reinterpret_cast<UnalignedU32 *>(p);
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+    {
+        __builtin_nontemporal_store(w[i], &o[i].v);
+    }
+}
+
 // 4 (or 8) bytes starting at an arbitrary byte address, fetched as 2 (or 3) ALIGNED dwords and funnel-
 // shifted into place. The texture path serves a misaligned multi-dword load at a fraction of the
 // rate of an aligned one (measured on a gather of u8x3 pixel pairs: 31 vs 22 cycles per wave-load),

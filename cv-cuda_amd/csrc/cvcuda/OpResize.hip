@@ -677,11 +677,6 @@ __device__ __forceinline__ AxisTerms<kWeights<INTERP>> FinishedAxis(float scale,
     return a;
 }
 
-struct __attribute__((packed, aligned(1))) UnalignedDword
-{
-    uint32_t w;
-};
-
 // One wave resizes a 64-column x 4-row patch of the output whose top left pixel is (x0, y0), both
 // wave-uniform. Sampling: lane l owns column x0 + l and computes its 4 rows (the column terms are
 // shared; neighbouring lanes read neighbouring source pixels whatever the scale). Storing: after
@@ -752,12 +747,7 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
     {
         uint32_t w[PB];
         PackQuad<PB>(q, w);
-        UnalignedDword *ow = reinterpret_cast<UnalignedDword *>(to);
-#pragma unroll
-        for (int i = 0; i < PB; ++i)
-        {
-            __builtin_nontemporal_store(w[i], &ow[i].w); // streaming: the output is not read back
-        }
+        StoreDwordsNT<PB>(to, w);
     }
     else
     {
@@ -911,12 +901,7 @@ __device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int 
     {
         uint32_t w[C];
         PackQuad<C>(q, w);
-        UnalignedDword *ow = reinterpret_cast<UnalignedDword *>(to);
-#pragma unroll
-        for (int i = 0; i < C; ++i)
-        {
-            __builtin_nontemporal_store(w[i], &ow[i].w);
-        }
+        StoreDwordsNT<C>(to, w);
     }
     else
     {

@@ -395,11 +395,6 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
     }
 }
 
-struct __attribute__((packed, aligned(1))) UnalignedWord
-{
-    uint32_t w;
-};
-
 // One 64 x 16 tile of the destination image `dst` (tile coordinates tx, ty), all 256 threads.
 template<class T, int C, int INTERP>
 __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dst, int dstRow,
@@ -506,13 +501,7 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     {
         uint32_t w[PB];
         PackQuad<PB>(q, w);
-        // streaming stores: the output is not read back by this kernel
-        UnalignedWord *ow = reinterpret_cast<UnalignedWord *>(to);
-#pragma unroll
-        for (int i = 0; i < PB; ++i) // 4 pixels = PB dwords
-        {
-            __builtin_nontemporal_store(w[i], &ow[i].w);
-        }
+        StoreDwordsNT<PB>(to, w); // 4 pixels = PB dwords
     }
     else
     {

@@ -6,6 +6,8 @@
 #ifndef CVCUDA_AMD_RUNIO_HPP
 #define CVCUDA_AMD_RUNIO_HPP
 
+#include "DeviceUtils.hpp"
+
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -25,11 +27,6 @@ template<class T, int N>
 struct __attribute__((packed, aligned(sizeof(T)))) Run
 {
     T v[N];
-};
-
-struct __attribute__((packed, aligned(1))) RunDword
-{
-    uint32_t w;
 };
 
 // N elements starting at p (aligned to one element).
@@ -53,12 +50,7 @@ __device__ __forceinline__ void StoreRunNT(uint8_t *p, const T (&v)[N])
     constexpr int D = N * sizeof(T) / 4;
     uint32_t      w[D];
     __builtin_memcpy(w, v, sizeof(w));
-    RunDword *o = reinterpret_cast<RunDword *>(p);
-#pragma unroll
-    for (int i = 0; i < D; ++i)
-    {
-        __builtin_nontemporal_store(w[i], &o[i].w);
-    }
+    StoreDwordsNT<D>(p, w);
 }
 
 } // namespace cvamd
