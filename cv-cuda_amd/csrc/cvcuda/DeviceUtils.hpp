@@ -10,6 +10,17 @@
 
 namespace cvamd {
 
+// N interleaved elements of type T, naturally aligned to one element only: the compiler may merge the
+// accesses into wider instructions (unaligned vector access is legal on gfx950). Pixels, runs of pixels
+// and groups of adjacent taps are all moved through this type.
+template<class T, int N>
+struct __attribute__((packed, aligned(sizeof(T)))) Packed
+{
+    using Elem              = T;
+    static constexpr int kC = N;
+    T v[N];
+};
+
 // float -> T with round-half-to-even and saturation; NaN -> 0 for integer targets
 // (semantics of the reference's SaturateCast, cuda_tools/detail/SaturateCastImpl.hpp:41-50, 125).
 template<class T>

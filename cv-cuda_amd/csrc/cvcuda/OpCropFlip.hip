@@ -84,10 +84,7 @@ __global__ __launch_bounds__(256) void RowCopyKernel(const CopyArgs a)
 }
 
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Vec
-{
-    T v[C];
-};
+using Vec = Packed<T, C>;
 
 template<class T, int C>
 __device__ __forceinline__ void CopyPixel(const uint8_t *srcRow, uint8_t *dstRow, int sx, int dx)

@@ -187,13 +187,8 @@ __global__ __launch_bounds__(256) void Yuv420ToRgbVarShape(const YuvArgs a, cons
     ConvertBlock<DCN, SEMIPLANAR>(AsGlobal(s.basePtr), s.rowStride, AsGlobal(d.basePtr), d.rowStride, W, H, x, y, a.bidx, a.uidx);
 }
 
-// ---------------------------------------------------------------------------------------------------
-// channel swizzle / alpha add / alpha drop
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Px
-{
-    T v[C];
-};
+using Px = Packed<T, C>;
 
 struct SwizzleArgs
 {
@@ -438,9 +433,6 @@ void DispatchSwizzle(int sch, int dch, const SwizzleArgs &a, int N, const NVCVIm
 }
 
 // The swizzle only moves bits: element types of equal size share a kernel. Alpha is passed as bits.
-template<>
-struct Px<double, 1>; // (no such instantiation; keeps the template from being used with C == 1)
-
 void RunSwizzle(NVCVColorConversionCode code, ElemType elem, int inC, int outC, SwizzleArgs &a, int N,
                 const NVCVImageBufferStrided *dstHost, hipStream_t stream)
 {

@@ -40,12 +40,7 @@ struct PixArgs
 };
 
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Px
-{
-    using Elem              = T;
-    static constexpr int kC = C;
-    T v[C];
-};
+using Px = Packed<T, C>;
 
 template<class T, int C>
 __device__ __forceinline__ void StorePx(uint8_t *row, int x, const Px<T, C> &p)

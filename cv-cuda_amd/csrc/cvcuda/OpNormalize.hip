@@ -44,10 +44,7 @@ struct NormArgs
 };
 
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Vec
-{
-    T v[C];
-};
+using Vec = Packed<T, C>;
 
 template<class TI, class TO, int C>
 __device__ __forceinline__ void NormPixel(const NormArgs &a, const uint8_t *srcRow, uint8_t *dstRow, int n, int y, int x)

@@ -29,10 +29,7 @@ struct ReformatArgs
 };
 
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Vec
-{
-    T v[C];
-};
+using Vec = Packed<T, C>;
 
 // C > 0: channel count known at compile time; SRC_IL / DST_IL: that side has its channels
 // interleaved and packed (stride of C == element size), so the whole pixel moves as one vector.

@@ -32,13 +32,8 @@ namespace {
 constexpr int kTileW = 64;
 constexpr int kTileH = 4;
 
-// C interleaved elements of type T, naturally aligned to one element: the compiler may merge the
-// accesses into wider instructions (unaligned vector access is legal on gfx950).
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Pixel
-{
-    T v[C];
-};
+using Pixel = Packed<T, C>;
 
 struct ResizeArgs
 {

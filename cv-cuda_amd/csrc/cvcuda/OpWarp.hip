@@ -64,10 +64,7 @@ struct WarpArgs
 };
 
 template<class T, int C>
-struct __attribute__((packed, aligned(sizeof(T)))) Vec
-{
-    T v[C];
-};
+using Vec = Packed<T, C>;
 
 struct Img
 {

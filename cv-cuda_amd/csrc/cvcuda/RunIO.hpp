@@ -24,10 +24,7 @@ template<class TS, class TD>
 constexpr int kRunPixelsFor = (sizeof(TS) >= 4 && sizeof(TD) >= 4) ? 1 : kRunPixels;
 
 template<class T, int N>
-struct __attribute__((packed, aligned(sizeof(T)))) Run
-{
-    T v[N];
-};
+using Run = Packed<T, N>;
 
 // N elements starting at p (aligned to one element).
 template<class T, int N>
