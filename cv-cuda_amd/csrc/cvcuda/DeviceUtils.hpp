@@ -6,6 +6,7 @@
 #include <nvcv/BorderType.h>
 
 #include <cstdint>
+#include <limits>
 #include <type_traits>
 
 namespace cvamd {
@@ -165,6 +166,22 @@ __device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *p)
     const uint32_t lo  = __builtin_amdgcn_alignbit(w.d[1], w.d[0], off * 8u);
     const uint32_t hi  = __builtin_amdgcn_alignbit(w.d[2], w.d[1], off * 8u);
     return ((uint64_t)hi << 32) | lo;
+}
+
+// The constant a caller gives for pixels outside the image, as an element of type T: truncated toward
+// zero and saturated to T's range (floats pass through).
+template<class T>
+__device__ __forceinline__ T BorderValueAs(float v)
+{
+    if constexpr (std::is_same_v<T, float>)
+    {
+        return v;
+    }
+    else
+    {
+        const float lo = (float)std::numeric_limits<T>::min(), hi = (float)std::numeric_limits<T>::max();
+        return (T)(long long)fminf(fmaxf(truncf(v), lo), hi);
+    }
 }
 
 // Coordinate c outside [0, s) -> the coordinate inside that the border mode stands for (every mode

@@ -43,21 +43,6 @@ struct CfnrArgs
     float          borderValue;
 };
 
-template<class T>
-__device__ __forceinline__ T BorderValueAs(float v)
-{
-    if constexpr (std::is_same_v<T, float>)
-    {
-        return v;
-    }
-    else
-    {
-        // truncation toward zero, saturated to the range of T
-        const float lo = (float)std::numeric_limits<T>::min(), hi = (float)std::numeric_limits<T>::max();
-        return (T)(long long)fminf(fmaxf(truncf(v), lo), hi);
-    }
-}
-
 template<class TS, class TD>
 __global__ __launch_bounds__(256) void CfnrKernel(const CfnrArgs a)
 {

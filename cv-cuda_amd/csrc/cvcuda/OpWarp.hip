@@ -72,21 +72,6 @@ struct Img
     int32_t        row, w, h;
 };
 
-template<class T>
-__device__ __forceinline__ T BorderCast(float v)
-{
-    if constexpr (std::is_same_v<T, float>)
-    {
-        return v;
-    }
-    else
-    {
-        // truncation toward zero, saturated to the range of T
-        const float lo = (float)std::numeric_limits<T>::min(), hi = (float)std::numeric_limits<T>::max();
-        return (T)(int)fminf(fmaxf(truncf(v), lo), hi);
-    }
-}
-
 template<class T, int C>
 __device__ __forceinline__ void Fetch(const Img &im, const WarpArgs &a, int x, int y, float (&out)[C])
 {
@@ -97,7 +82,7 @@ __device__ __forceinline__ void Fetch(const Img &im, const WarpArgs &a, int x, i
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
-                out[c] = (float)BorderCast<T>(a.bval[c]);
+                out[c] = (float)BorderValueAs<T>(a.bval[c]);
             }
             return;
         }
