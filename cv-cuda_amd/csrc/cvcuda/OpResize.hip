@@ -109,6 +109,64 @@ __device__ __forceinline__ void StorePx(uint8_t *row, int x, const Pixel<T, C> &
     }
 }
 
+// N horizontally adjacent pixels at byte offset `xoff` of source row `row` (all inside the image).
+// u8x3: 1 or 2 pixels are fetched with a 4- or 8-byte load that reads 1-2 bytes past them, harmless
+// except behind the image's last row (`lastRow`, wave-uniform), where the load is moved back to end
+// with the row's `rowBytes` and the value shifted.
+template<class T, int C, int N>
+__device__ __forceinline__ void LoadTaps(const uint8_t *row, int xoff, bool lastRow, int rowBytes, float (&t)[N][C])
+{
+    if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 1)
+    {
+        uint32_t q;
+        if (lastRow)
+        {
+            const int back = max(0, xoff - (rowBytes - 4));
+            q              = LoadU32Unaligned(row + (xoff - back)) >> (8 * back);
+        }
+        else
+        {
+            q = LoadU32Unaligned(row + xoff);
+        }
+        t[0][0] = (float)(q & 0xFF);
+        t[0][1] = (float)((q >> 8) & 0xFF);
+        t[0][2] = (float)((q >> 16) & 0xFF);
+    }
+    else if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 2)
+    {
+        uint64_t q;
+        if (lastRow)
+        {
+            const int back = max(0, xoff - (rowBytes - 8));
+            q              = LoadU64Unaligned(row + (xoff - back)) >> (8 * back);
+        }
+        else
+        {
+            q = LoadU64Unaligned(row + xoff);
+        }
+        const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
+        t[0][0] = (float)(lo & 0xFF);
+        t[0][1] = (float)((lo >> 8) & 0xFF);
+        t[0][2] = (float)((lo >> 16) & 0xFF);
+        t[1][0] = (float)(lo >> 24);
+        t[1][1] = (float)(hi & 0xFF);
+        t[1][2] = (float)((hi >> 8) & 0xFF);
+    }
+    else
+    {
+        const Pixel<T, N *C> v = *reinterpret_cast<const Pixel<T, N * C> *>(row + xoff);
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                t[i][c] = (float)v.v[i * C + c];
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
 {
     constexpr float A = -0.75f;
@@ -180,18 +238,28 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
         {
             sum[c] = 0.f;
         }
-        auto add = [&](int x, int y, float w)
+        // pixels [xa, xb) of row y, each with weight w, in ascending order; what lies outside the image
+        // contributes nothing, so the range is clipped once instead of testing every tap
+        auto addRun = [&](int xa, int xb, int y, float w)
         {
-            if (x >= 0 && x < p.srcW && y >= 0 && y < p.srcH)
+            if (y < 0 || y >= p.srcH)
             {
-                const Pixel<T, C> t = LoadPx<T, C>(p.src + (int64_t)y * p.srcRow, x);
+                return;
+            }
+            const uint8_t *row = p.src + (int64_t)y * p.srcRow;
+            xb                 = min(xb, p.srcW);
+            for (int x = max(xa, 0); x < xb; ++x)
+            {
+                float t[1][C];
+                LoadTaps<T, C, 1>(row, x * (int)sizeof(Pixel<T, C>), y == p.srcH - 1, p.srcW * (int)sizeof(Pixel<T, C>), t);
 #pragma unroll
                 for (int c = 0; c < C; ++c)
                 {
-                    sum[c] += (float)t.v[c] * w;
+                    sum[c] += t[0][c] * w;
                 }
             }
         };
+        auto add = [&](int x, int y, float w) { addRun(x, x + 1, y, w); };
         if constexpr (VARSHAPE)
         {
             // image batches follow the reference's separate kernel (legacy/resize_var_shape.cu:236-428):
@@ -206,10 +274,7 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
                     const float scale = 1.f / (scaleX * scaleY);
                     for (int cy = ymin; cy < ymax; ++cy)
                     {
-                        for (int cx = xmin; cx < xmax; ++cx)
-                        {
-                            add(cx, cy, scale);
-                        }
+                        addRun(xmin, xmax, cy, scale);
                     }
                 }
                 else
@@ -217,10 +282,7 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
                     const float scale = 1.f / (fminf(scaleX, p.srcW - fsx1) * fminf(scaleY, p.srcH - fsy1));
                     for (int cy = ymin; cy < ymax; ++cy)
                     {
-                        for (int cx = xmin; cx < xmax; ++cx)
-                        {
-                            add(cx, cy, scale);
-                        }
+                        addRun(xmin, xmax, cy, scale);
                         if (xmin > fsx1)
                         {
                             add(xmin - 1, cy, (xmin - fsx1) * scale);
@@ -232,17 +294,11 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
                     }
                     if (ymin > fsy1)
                     {
-                        for (int cx = xmin; cx < xmax; ++cx)
-                        {
-                            add(cx, ymin - 1, (ymin - fsy1) * scale);
-                        }
+                        addRun(xmin, xmax, ymin - 1, (ymin - fsy1) * scale);
                     }
                     if (ymax < fsy2)
                     {
-                        for (int cx = xmin; cx < xmax; ++cx)
-                        {
-                            add(cx, ymax, (fsy2 - ymax) * scale);
-                        }
+                        addRun(xmin, xmax, ymax, (fsy2 - ymax) * scale);
                     }
                     if (ymin > fsy1 && xmin > fsx1)
                     {
@@ -302,10 +358,7 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             const float scale = 1.f / (scaleX * scaleY);
             for (int cy = ymin; cy < ymax; ++cy)
             {
-                for (int cx = xmin; cx < xmax; ++cx)
-                {
-                    add(cx, cy, scale);
-                }
+                addRun(xmin, xmax, cy, scale);
             }
         }
         else
@@ -313,10 +366,7 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             const float scale = 1.f / (fminf(scaleX, p.srcW - fsx1) * fminf(scaleY, p.srcH - fsy1));
             for (int cy = ymin; cy < ymax; ++cy)
             {
-                for (int cx = xmin; cx < xmax; ++cx)
-                {
-                    add(cx, cy, scale);
-                }
+                addRun(xmin, xmax, cy, scale);
                 if (xmin > fsx1)
                 {
                     add(xmin - 1, cy, (xmin - fsx1) * scale);
@@ -328,10 +378,7 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             }
             if (ymin > fsy1)
             {
-                for (int cx = xmin; cx < xmax; ++cx)
-                {
-                    add(cx, ymin - 1, (ymin - fsy1) * scale);
-                }
+                addRun(xmin, xmax, ymin - 1, (ymin - fsy1) * scale);
                 if (xmin > fsx1)
                 {
                     add(xmin - 1, ymin - 1, (ymin - fsy1) * (xmin - fsx1) * scale);
@@ -343,10 +390,7 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             }
             if (ymax < fsy2)
             {
-                for (int cx = xmin; cx < xmax; ++cx)
-                {
-                    add(cx, ymax, (fsy2 - ymax) * scale);
-                }
+                addRun(xmin, xmax, ymax, (fsy2 - ymax) * scale);
                 if (xmax < fsx2)
                 {
                     add(xmax, ymax, (fsy2 - ymax) * (fsx2 - xmax) * scale);
@@ -463,64 +507,6 @@ __global__ __launch_bounds__(256) void ResizeVarShapeKernel(const ResizeArgs a, 
 // (2 for bilinear, 4 for bicubic) come from one load, and lanes exchange results so that each
 // stores 4 consecutive pixels as whole dwords. Arithmetic: the expressions of ResizeValue, term for
 // term.
-
-// N horizontally adjacent pixels at byte offset `xoff` of source row `row` (all inside the image).
-// u8x3: 1 or 2 pixels are fetched with a 4- or 8-byte load that reads 1-2 bytes past them, harmless
-// except behind the image's last row (`lastRow`, wave-uniform), where the load is moved back to end
-// with the row's `rowBytes` and the value shifted.
-template<class T, int C, int N>
-__device__ __forceinline__ void LoadTaps(const uint8_t *row, int xoff, bool lastRow, int rowBytes, float (&t)[N][C])
-{
-    if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 1)
-    {
-        uint32_t q;
-        if (lastRow)
-        {
-            const int back = max(0, xoff - (rowBytes - 4));
-            q              = LoadU32Unaligned(row + (xoff - back)) >> (8 * back);
-        }
-        else
-        {
-            q = LoadU32Unaligned(row + xoff);
-        }
-        t[0][0] = (float)(q & 0xFF);
-        t[0][1] = (float)((q >> 8) & 0xFF);
-        t[0][2] = (float)((q >> 16) & 0xFF);
-    }
-    else if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 2)
-    {
-        uint64_t q;
-        if (lastRow)
-        {
-            const int back = max(0, xoff - (rowBytes - 8));
-            q              = LoadU64Unaligned(row + (xoff - back)) >> (8 * back);
-        }
-        else
-        {
-            q = LoadU64Unaligned(row + xoff);
-        }
-        const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
-        t[0][0] = (float)(lo & 0xFF);
-        t[0][1] = (float)((lo >> 8) & 0xFF);
-        t[0][2] = (float)((lo >> 16) & 0xFF);
-        t[1][0] = (float)(lo >> 24);
-        t[1][1] = (float)(hi & 0xFF);
-        t[1][2] = (float)((hi >> 8) & 0xFF);
-    }
-    else
-    {
-        const Pixel<T, N *C> v = *reinterpret_cast<const Pixel<T, N * C> *>(row + xoff);
-#pragma unroll
-        for (int i = 0; i < N; ++i)
-        {
-#pragma unroll
-            for (int c = 0; c < C; ++c)
-            {
-                t[i][c] = (float)v.v[i * C + c];
-            }
-        }
-    }
-}
 
 // Per-column and per-row terms of a sample: source index and weights, the expressions of
 // ResizeValue. W = number of weights (0 nearest, 1 linear, 4 cubic); sources are >= 4 pixels wide.
