@@ -5,7 +5,7 @@
 // image needs and passes the running totals to the kernel BY VALUE in the kernel-argument segment.
 // Block b finds its image by a binary search over those totals (uniform per block, so it runs on
 // the scalar unit) and derives its tile coordinates. No device round trip, no host sync, no
-// operator-owned scratch; batches larger than kMaxImages are processed in several launches.
+// operator-owned scratch; batches larger than kMaxTileImages are processed in several launches.
 #ifndef CVCUDA_AMD_VARSHAPETILES_HPP
 #define CVCUDA_AMD_VARSHAPETILES_HPP
 

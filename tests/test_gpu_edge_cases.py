@@ -144,3 +144,89 @@ def test_submits_captured_in_a_hip_graph_replay_correctly(cv, K, orc, gpu):
         want = orc.normalize(x, np.array([[[[0.4, 0.5, 0.6]]]], np.float32), np.array([[[[0.2, 0.3, 0.4]]]], np.float32),
                              1.0, 0.0, 0.0, True).transpose(0, 3, 1, 2)
         assert (np.abs(got3 - want) <= 1e-5 * np.maximum(1.0, np.abs(want))).all()
+
+
+def test_image_batches_larger_than_one_launch(cv, K, orc, gpu):
+    # the image-batch operators pack at most a few hundred images' tiles into one launch and loop over
+    # the rest: 401 images make every operator issue a second launch, whose images must use their own
+    # descriptors, matrices and flip codes
+    rng = np.random.default_rng(401)
+    n = 401
+    bi, hosts = cv.ImageBatchVarShape(n), []
+    for i in range(n):
+        w, h = int(rng.integers(1, 40)), int(rng.integers(1, 24))
+        a = orc.fill_u8((h, w, 3), 9000 + i)
+        hosts.append(a)
+        bi.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_BGR8))
+
+    def outputs(fmt, size=lambda a: (a.shape[1], a.shape[0])):
+        batch, outs = cv.ImageBatchVarShape(n), []
+        for a in hosts:
+            o = cv.Image.alloc(size(a), fmt)
+            outs.append(o)
+            batch.push_back(o)
+        return batch, outs
+
+    bo, outs = outputs(K.IMAGE_FORMAT_RGB8)
+    cv.CvtColor()(None, bi, bo, K.COLOR_BGR2RGB)
+    torch.cuda.synchronize()
+    for a, o in zip(hosts, outs):
+        np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy(), a[..., ::-1])
+
+    bo, outs = outputs(K.IMAGE_FORMAT_BGR8)
+    codes = rng.integers(-1, 2, n).astype(np.int32)
+    cv.Flip(n)(None, bi, bo, cv.Tensor.from_numpy(codes, "N"))
+    torch.cuda.synchronize()
+    for a, o, code in zip(hosts, outs, codes):
+        ref = {1: a[:, ::-1], 0: a[::-1], -1: a[::-1, ::-1]}[int(code)]
+        np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy(), ref)
+
+    base, scale = np.array([[[[3.0, 5.0, 7.0]]]], np.float32), np.array([[[[0.5, 1.5, 2.0]]]], np.float32)
+    for b, s in ((base, scale), (base[..., :1], scale[..., :1])):
+        cv.Normalize()(None, bi, cv.Tensor.from_numpy(b, "NHWC"), cv.Tensor.from_numpy(s, "NHWC"), bo, 1.0, 0.0, 0.0, 0)
+        torch.cuda.synchronize()
+        for a, o in zip(hosts, outs):
+            np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy(), orc.normalize(a[None], b, s)[0])
+
+    shifts = rng.integers(-3, 4, (n, 2))
+    mats = np.array([[1, 0, sx, 0, 1, sy] for sx, sy in shifts], np.float32)
+    cv.WarpAffine(n)(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), NEAREST | 16, 0, (7, 8, 9, 0))  # 16: inverse map
+    torch.cuda.synchronize()
+    for a, o, m in zip(hosts, outs, mats):
+        ref = orc.warp(a[None], a.shape[:2], m, NEAREST, 0, (7, 8, 9, 0), variant=1)[0]
+        np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy(), ref)
+
+    bg, gouts = outputs(K.IMAGE_FORMAT_U8)
+    cv.CvtColor()(None, bi, bg, K.COLOR_BGR2GRAY)
+    torch.cuda.synchronize()
+    for a, o in zip(hosts, gouts):
+        b, g, r = (a[..., k].astype(np.int64) for k in range(3))
+        np.testing.assert_array_equal(o.plane_view(0, np.uint8, 1).cpu().numpy()[..., 0],
+                                      (b * 3735 + g * 19235 + r * 9798 + (1 << 14)) >> 15)
+
+    for interp in (LINEAR, AREA):
+        br, routs = outputs(K.IMAGE_FORMAT_BGR8, lambda a: (a.shape[1] * 2 // 3 + 1, a.shape[0] + 2))
+        cv.Resize()(None, bi, br, interp)
+        torch.cuda.synchronize()
+        for a, o in zip(hosts, routs):
+            w, h = o.size
+            ref = orc.resize(a[None], (h, w), interp, variant=2 if interp == AREA else 1)[0]
+            got = o.plane_view(0, np.uint8, 3).cpu().numpy()
+            assert np.abs(got.astype(np.int32) - ref).max() <= (1 if interp == LINEAR else 0), (interp, a.shape)
+
+    by, youts, yhosts = cv.ImageBatchVarShape(n), [], []
+    for i in range(n):
+        w, h = 2 * int(rng.integers(1, 20)), 2 * int(rng.integers(1, 12))
+        y = np.concatenate([orc.fill_u8((h, w), 100 + i, 16, 235), orc.fill_u8((h // 2, w), 600 + i, 16, 240)])[..., None]
+        yhosts.append(y)
+        by.push_back(cv.Image.from_numpy(y, K.IMAGE_FORMAT_U8))
+        o = cv.Image.alloc((w, h), K.IMAGE_FORMAT_RGB8)
+        youts.append(o)
+    byo = cv.ImageBatchVarShape(n)
+    for o in youts:
+        byo.push_back(o)
+    cv.CvtColor()(None, by, byo, K.COLOR_YUV2RGB_NV12)
+    torch.cuda.synchronize()
+    for y, o in zip(yhosts, youts):
+        np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy()[None],
+                                      orc.yuv420_to_rgb(y[None], 3, False, 0, True))
