@@ -136,35 +136,26 @@ __device__ __forceinline__ void StoreDwordsNT(uint8_t *p, const uint32_t (&w)[N]
     }
 }
 
-// 4 (or 8) bytes starting at an arbitrary byte address, fetched as 2 (or 3) ALIGNED dwords and funnel-
+// 8 bytes starting at the arbitrary byte address base + off, fetched as 3 ALIGNED dwords and funnel-
 // shifted into place. The texture path serves a misaligned multi-dword load at a fraction of the
 // rate of an aligned one (measured on a gather of u8x3 pixel pairs: 31 vs 22 cycles per wave-load),
-// which costs more than the two extra shifts. Reads the aligned window [p & ~3, (p & ~3) + 8 or 12):
-// up to 3 bytes before p (same dword as p, so never another page) and up to 7 (6) bytes after the
-// data; the caller keeps that tail inside its allocation.
-__device__ __forceinline__ uint32_t LoadU32Window(const uint8_t *p)
-{
-    struct alignas(4) W2
-    {
-        uint32_t d[2];
-    };
-    // the window's address is derived from p by pointer arithmetic (not through an integer), which
-    // keeps it a global-memory access instead of a generic (flat) one
-    const uint32_t off = (uint32_t)reinterpret_cast<uintptr_t>(p) & 3u;
-    const W2       w   = *reinterpret_cast<const W2 *>(p - off);
-    return __builtin_amdgcn_alignbit(w.d[1], w.d[0], off * 8u);
-}
-
-__device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *p)
+// which costs more than the two extra shifts. Reads the aligned window [p & ~3, (p & ~3) + 12) for
+// p = base + off: up to 3 bytes before p (same dword as p, so never another page) and up to 6 bytes
+// after the data; the caller keeps that tail inside its allocation. base must be uniform over the
+// wave: its misalignment is folded into the 32-bit offset, so the per-lane address arithmetic is one
+// mask (the load takes the aligned base from scalar registers plus a 32-bit lane offset) instead of
+// 64-bit adds per lane.
+__device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *base, uint32_t off)
 {
     struct alignas(4) W3
     {
         uint32_t d[3];
     };
-    const uint32_t off = (uint32_t)reinterpret_cast<uintptr_t>(p) & 3u;
-    const W3       w   = *reinterpret_cast<const W3 *>(p - off);
-    const uint32_t lo  = __builtin_amdgcn_alignbit(w.d[1], w.d[0], off * 8u);
-    const uint32_t hi  = __builtin_amdgcn_alignbit(w.d[2], w.d[1], off * 8u);
+    const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(base) & 3u;
+    const uint32_t o   = off + mis;
+    const W3       w   = *reinterpret_cast<const W3 *>((base - mis) + (o & ~3u));
+    const uint32_t lo  = __builtin_amdgcn_alignbit(w.d[1], w.d[0], o * 8u); // the shift uses bits 4:0
+    const uint32_t hi  = __builtin_amdgcn_alignbit(w.d[2], w.d[1], o * 8u);
     return ((uint64_t)hi << 32) | lo;
 }
 

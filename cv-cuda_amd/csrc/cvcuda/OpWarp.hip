@@ -152,13 +152,13 @@ __device__ __forceinline__ void LoadPixelInside(const uint8_t *p, T (&out)[C])
     }
 }
 
-// Two horizontally adjacent pixels starting at p, both known to be inside the image.
+// Two horizontally adjacent pixels starting at base + off, both known to be inside the image.
 template<class T, int C>
-__device__ __forceinline__ void LoadPairInside(const uint8_t *p, float (&p0)[C], float (&p1)[C])
+__device__ __forceinline__ void LoadPairInside(const uint8_t *base, uint32_t off, float (&p0)[C], float (&p1)[C])
 {
     if constexpr (kWideTapLoads<T, C>)
     {
-        const uint64_t q  = LoadU64Window(p);
+        const uint64_t q  = LoadU64Window(base, off);
         const uint32_t lo = (uint32_t)q, hi = (uint32_t)(q >> 32);
         p0[0] = (float)(lo & 0xFF);
         p0[1] = (float)((lo >> 8) & 0xFF);
@@ -169,7 +169,7 @@ __device__ __forceinline__ void LoadPairInside(const uint8_t *p, float (&p0)[C],
     }
     else
     {
-        const Vec<T, 2 * C> v = *reinterpret_cast<const Vec<T, 2 * C> *>(p);
+        const Vec<T, 2 * C> v = *reinterpret_cast<const Vec<T, 2 * C> *>(base + off);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -280,26 +280,30 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
 }
 
 // True when every tap of the sample at (sx, sy) lies inside the image (and, with WIDE loads, none of
-// them is among the last three pixels of the image's last row). Decided on the float coordinates: for an integer k,
-// floor(v) >= k <=> v >= k and floor(v) < k <=> v < k; a NaN coordinate fails every comparison.
-template<int INTERP, bool WIDE>
-__device__ __forceinline__ bool TapsInside(float wf, float hf, float sx, float sy)
+// them is among the image's last two columns: the window loads read 2 pixels past a tap pair, which
+// must not run off the end of the last row). limX / limY come from InsideLimits. For an integer k,
+// floor(v) < k <=> v < k, so the test is 0 <= v - lo < lim per axis, done as ONE unsigned comparison
+// of the float's bit pattern: non-negative floats order like their bits, negative ones and NaNs have
+// patterns above every finite positive limit (-0.0 fails too and takes the generic path, which
+// computes the same result).
+template<int INTERP>
+__device__ __forceinline__ bool TapsInside(float limX, float limY, float sx, float sy)
 {
-    // taps span [floor(v) - lo, floor(v) + hi] per axis
-    constexpr float lo = INTERP == NVCV_INTERP_CUBIC ? 1.f : 0.f;
-    constexpr float hi = INTERP == NVCV_INTERP_CUBIC ? 2.f : (INTERP == NVCV_INTERP_LINEAR ? 1.f : 0.f);
-    if constexpr (INTERP == NVCV_INTERP_NEAREST)
-    {
-        sx += .5f;
-        sy += .5f;
-    }
-    // bitwise on purpose: no short-circuit branches
-    bool in = (sx >= lo) & (sy >= lo) & (sx < wf - hi) & (sy < hf - hi);
-    if constexpr (WIDE)
-    {
-        in = in & ((sx < wf - hi - 2.f) | (sy < hf - hi - 1.f));
-    }
-    return in;
+    // taps span [floor(v) - lo, floor(v) + hi] per axis; NEAREST takes floor(v + .5)
+    constexpr float lo = INTERP == NVCV_INTERP_CUBIC ? 1.f : (INTERP == NVCV_INTERP_NEAREST ? -.5f : 0.f);
+    const bool inX = __float_as_uint(sx - lo) < __float_as_uint(limX);
+    const bool inY = __float_as_uint(sy - lo) < __float_as_uint(limY);
+    return inX & inY; // bitwise on purpose: no short-circuit branch
+}
+
+// Exclusive upper limit of floor(v) - lo along an axis of `size` pixels; 0 (no sample passes) when the
+// image is smaller than the tap span.
+template<int INTERP>
+__device__ __forceinline__ float InsideLimit(int size, bool wide)
+{
+    constexpr int lo = INTERP == NVCV_INTERP_CUBIC ? 1 : 0;
+    constexpr int hi = INTERP == NVCV_INTERP_CUBIC ? 2 : (INTERP == NVCV_INTERP_LINEAR ? 1 : 0);
+    return (float)max(size - hi - lo - (wide ? 2 : 0), 0);
 }
 
 // Same arithmetic as SampleWithBorder for a sample whose taps are all inside the image: no border
@@ -321,10 +325,10 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
         const float fx = floorf(sx), fy = floorf(sy);
         const float wx1 = sx - fx, wx0 = (fx + 1.f) - sx;
         const float wy1 = sy - fy, wy0 = (fy + 1.f) - sy;
-        const uint8_t *p = im.base + PixelOffset<PB>(im, (int)fx, (int)fy);
+        const uint32_t o = PixelOffset<PB>(im, (int)fx, (int)fy);
         float          t[4][C];
-        LoadPairInside<T, C>(p, t[0], t[1]);
-        LoadPairInside<T, C>(p + (uint32_t)im.row, t[2], t[3]);
+        LoadPairInside<T, C>(im.base, o, t[0], t[1]);
+        LoadPairInside<T, C>(im.base, o + (uint32_t)im.row, t[2], t[3]);
         const float w00 = wx0 * wy0, w01 = wx1 * wy0, w10 = wx0 * wy1, w11 = wx1 * wy1;
 #pragma unroll
         for (int c = 0; c < C; ++c)
@@ -342,14 +346,14 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
         float       wx[4], wy[4];
         CubicCoeffs(sx - fx, wx);
         CubicCoeffs(sy - fy, wy);
-        const uint8_t *p = im.base + PixelOffset<PB>(im, (int)fx - 1, (int)fy - 1);
-        float          t[4][4][C];
+        uint32_t o = PixelOffset<PB>(im, (int)fx - 1, (int)fy - 1);
+        float    t[4][4][C];
 #pragma unroll
         for (int cy = 0; cy < 4; ++cy)
         {
-            LoadPairInside<T, C>(p, t[cy][0], t[cy][1]);
-            LoadPairInside<T, C>(p + 2 * PB, t[cy][2], t[cy][3]);
-            p += (uint32_t)im.row;
+            LoadPairInside<T, C>(im.base, o, t[cy][0], t[cy][1]);
+            LoadPairInside<T, C>(im.base, o + 2 * PB, t[cy][2], t[cy][3]);
+            o += (uint32_t)im.row;
         }
 #pragma unroll
         for (int c = 0; c < C; ++c)
@@ -387,7 +391,7 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     // ---- gather: lane (lx, ly) of wave w samples its pixel in patches 4w .. 4w+3 (side by side: a
     // wave covers 32 columns x 8 rows)
     const int wave = threadIdx.x >> 6, lx = threadIdx.x & (kPatch - 1), ly = (threadIdx.x >> 3) & (kPatch - 1);
-    const float wf = (float)im.w, hf = (float)im.h;
+    const float limX = InsideLimit<INTERP>(im.w, kWideTapLoads<T, C>), limY = InsideLimit<INTERP>(im.h, false);
     float       sx[kPxPerLane], sy[kPxPerLane];
     uint32_t    q[D][kPxPerLane]; // q[d][k]: dword d of this lane's pixel in patch k
     // rows too long or too many for 24-bit offset arithmetic go through the generic path
@@ -407,7 +411,7 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
         {
             MapCoord<false>(m, dx, dy, sx[k], sy[k]);
         }
-        allInside = allInside & TapsInside<INTERP, kWideTapLoads<T, C>>(wf, hf, sx[k], sy[k]);
+        allInside = allInside & TapsInside<INTERP>(limX, limY, sx[k], sy[k]);
     }
     if (allInside)
     {
