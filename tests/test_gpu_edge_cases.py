@@ -230,3 +230,59 @@ def test_image_batches_larger_than_one_launch(cv, K, orc, gpu):
     for y, o in zip(yhosts, youts):
         np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy()[None],
                                       orc.yuv420_to_rgb(y[None], 3, False, 0, True))
+
+
+def test_concurrent_submits_on_shared_operator_handles(cv, K, orc, gpu):
+    # operators hold no per-call state: several host threads, each with its own stream and tensors,
+    # submit through the SAME handles at the same time (ctypes drops the GIL around each call), and
+    # create and destroy their tensors concurrently (handle pools). Every thread must get the result a
+    # lone thread gets, and an error raised in one thread must not show up in another's status.
+    import threading
+    resize, swz, norm, fused = cv.Resize(), cv.CvtColor(), cv.Normalize(), cv.ResizeCropConvertReformat()
+    b_host, s_host = np.array([[[[3.0, 5.0, 7.0]]]], np.float32), np.array([[[[0.5, 1.5, 2.0]]]], np.float32)
+    base, scale = cv.Tensor.from_numpy(b_host, "NHWC"), cv.Tensor.from_numpy(s_host, "NHWC")
+    torch.cuda.synchronize()
+    n_threads, rounds = 6, 25
+    failures, start = [], threading.Barrier(n_threads)
+
+    def worker(tid):
+        try:
+            torch.cuda.set_device(0)
+            stream = torch.cuda.Stream()
+            src = orc.fill_u8((2, 45 + tid, 70 + 3 * tid, 3), 700 + tid)
+            want_small = orc.resize(src, (23, 31), LINEAR, variant=1)
+            want_fused = orc.fused_rccr(src, (16, 16), (32, 24), (5, 3), LINEAR, np.float32, True, 0, 1 / 255.0, 0.0, False)
+            start.wait()
+            for r in range(rounds):
+                with torch.cuda.stream(stream):
+                    tin = cv.Tensor.from_numpy(src, "NHWC")
+                    t1 = cv.Tensor.alloc([2, 23, 31, 3], np.uint8, "NHWC")
+                    t2 = cv.Tensor.alloc([2, 23, 31, 3], np.uint8, "NHWC")
+                    t3 = cv.Tensor.alloc([2, 23, 31, 3], np.uint8, "NHWC")
+                    t4 = cv.Tensor.alloc([2, 3, 16, 16], np.float32, "NCHW")
+                    stream.synchronize()  # the uploads above ran on torch's streams
+                    resize(stream, tin, t1, LINEAR)
+                    swz(stream, t1, t2, K.COLOR_BGR2RGB)
+                    norm(stream, t2, base, scale, t3, 1.0, 0.0, 0.0, 0)
+                    fused(stream, tin, t4, (32, 24), LINEAR, (5, 3), 0, 1 / 255.0, 0.0, False)
+                    if r % 5 == tid % 5:  # a failing call in this thread only
+                        with pytest.raises(cv.Error) as e:
+                            resize(stream, tin, t4, LINEAR)
+                        assert e.value.status == 2
+                    stream.synchronize()
+                    got_small, got_norm, got_fused = t1.numpy(), t3.numpy(), t4.numpy()
+                assert np.abs(got_small.astype(np.int32) - want_small).max() <= 1
+                # the chain's later stages are exact functions of the first stage's output
+                np.testing.assert_array_equal(got_norm, orc.normalize(got_small[..., ::-1].copy(), b_host, s_host))
+                assert (np.abs(got_fused - want_fused) <= 1e-5 * np.maximum(1.0, np.abs(want_fused))).all()
+        except BaseException as exc:  # noqa: BLE001 - reported by the main thread
+            failures.append((tid, repr(exc)))
+            start.abort()
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(n_threads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not failures, failures
