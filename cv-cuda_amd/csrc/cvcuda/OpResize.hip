@@ -1023,7 +1023,7 @@ __global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs 
         tapX[k] = max(0, min(qsx - 1 + (lane & 3), p.srcW - 1));
     }
 
-    Px   v[4];
+    Px   v[4][4];
     auto loadRow = [&](int j)
     {
         const int      yy  = max(0, min(sy - 1 + j, p.srcH - 1));
@@ -1031,7 +1031,7 @@ __global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs 
 #pragma unroll
         for (int k = 0; k < 4; ++k)
         {
-            v[k] = LoadPx<T, C>(row, tapX[k]);
+            v[j][k] = LoadPx<T, C>(row, tapX[k]);
         }
     };
 
@@ -1041,20 +1041,20 @@ __global__ __launch_bounds__(256) void ResizeCubicStagedKernel(const ResizeArgs 
     {
         sum[c] = 0.f;
     }
-    loadRow(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        loadRow(j);
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
     {
 #pragma unroll
         for (int k = 0; k < 4; ++k)
         {
-            __builtin_memcpy(&stage[wave][64 * k + lane], &v[k], sizeof(Px));
+            __builtin_memcpy(&stage[wave][64 * k + lane], &v[j][k], sizeof(Px));
         }
         WaveExchangeFence();
-        if (j < 3)
-        {
-            loadRow(j + 1); // in flight while this row is summed
-        }
         Px t[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
