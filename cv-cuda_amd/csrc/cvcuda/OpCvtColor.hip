@@ -26,8 +26,9 @@ namespace {
 
 // ---------------------------------------------------------------------------------------------------
 // YUV 4:2:0 -> RGB
-constexpr int kYuvTileW = 256; // pixels per block row: 64 lanes x 4 pixels
-constexpr int kYuvTileH = 8;   // rows per block: 4 waves x 2 rows
+constexpr int kYuvBlockW = 8;               // pixels per lane and row (a lane converts a kYuvBlockW x 2 block)
+constexpr int kYuvTileW  = 64 * kYuvBlockW; // pixels per block row
+constexpr int kYuvTileH  = 8;               // rows per block: 4 waves x 2 rows
 
 struct YuvArgs
 {
@@ -157,18 +158,97 @@ __device__ __forceinline__ void ConvertBlock(const uint8_t *src, int srcRow, uin
     }
 }
 
+// A kYuvBlockW x 2 block that lies wholly inside the row (x + kYuvBlockW <= W): every access is a vector
+// of whole dwords (luma 8 bytes per row, chroma 8 or 4 + 4 bytes, 24 or 32 output bytes per row).
+template<int DCN, bool SEMIPLANAR>
+__device__ __forceinline__ void ConvertWideBlock(const uint8_t *src, int srcRow, uint8_t *dst, int dstRow, int W, int H,
+                                                 int x, int y, int bidx, int uidx)
+{
+    constexpr int BW = kYuvBlockW, NC = BW / 2;
+    int           uu[NC], vv[NC];
+    if constexpr (SEMIPLANAR)
+    {
+        uint8_t  c[BW];
+        uint32_t w[BW / 4];
+        LoadRun<uint8_t, BW>(src + (int64_t)(H + (y >> 1)) * srcRow + x, c);
+        __builtin_memcpy(w, c, sizeof(w));
+#pragma unroll
+        for (int k = 0; k < NC; ++k)
+        {
+            const int sh = 16 * (k & 1);
+            uu[k]        = (int)((w[k >> 1] >> (sh + 8 * uidx)) & 0xFF) - 128;
+            vv[k]        = (int)((w[k >> 1] >> (sh + 8 * (uidx ^ 1))) & 0xFF) - 128;
+        }
+    }
+    else
+    {
+        const int h4  = H >> 2;
+        const int uvx = (x >> 1) + ((W >> 1) & -((y >> 1) & 1));
+        uint8_t   pu[NC], pv[NC];
+        LoadRun<uint8_t, NC>(src + (int64_t)(H + (y >> 2) + h4 * uidx) * srcRow + uvx, pu);
+        LoadRun<uint8_t, NC>(src + (int64_t)(H + (y >> 2) + h4 * (uidx ^ 1)) * srcRow + uvx, pv);
+#pragma unroll
+        for (int k = 0; k < NC; ++k)
+        {
+            uu[k] = (int)pu[k] - 128;
+            vv[k] = (int)pv[k] - 128;
+        }
+    }
+#pragma unroll
+    for (int ry = 0; ry < 2; ++ry)
+    {
+        const int yy = y + ry;
+        if (yy >= H)
+        {
+            break;
+        }
+        uint8_t luma[BW], out[BW * DCN];
+        LoadRun<uint8_t, BW>(src + (int64_t)yy * srcRow + x, luma);
+#pragma unroll
+        for (int i = 0; i < BW; ++i)
+        {
+            uint32_t r, g, b;
+            YuvToRgb(luma[i], uu[i >> 1], vv[i >> 1], r, g, b);
+            out[i * DCN + 0] = (uint8_t)(bidx == 0 ? b : r);
+            out[i * DCN + 1] = (uint8_t)g;
+            out[i * DCN + 2] = (uint8_t)(bidx == 0 ? r : b);
+            if constexpr (DCN == 4)
+            {
+                out[i * DCN + 3] = 255;
+            }
+        }
+        StoreRunNT<uint8_t, BW * DCN>(dst + (int64_t)yy * dstRow + (int64_t)x * DCN, out);
+    }
+}
+
+// The lane's kYuvBlockW x 2 block at (x, y): the wide form inside the row, 4 x 2 blocks at its ragged end.
+template<int DCN, bool SEMIPLANAR>
+__device__ __forceinline__ void ConvertLaneBlock(const uint8_t *src, int srcRow, uint8_t *dst, int dstRow, int W, int H,
+                                                 int x, int y, int bidx, int uidx)
+{
+    if (x + kYuvBlockW <= W)
+    {
+        ConvertWideBlock<DCN, SEMIPLANAR>(src, srcRow, dst, dstRow, W, H, x, y, bidx, uidx);
+        return;
+    }
+    for (int xx = x; xx < W; xx += 4)
+    {
+        ConvertBlock<DCN, SEMIPLANAR>(src, srcRow, dst, dstRow, W, H, xx, y, bidx, uidx);
+    }
+}
+
 template<int DCN, bool SEMIPLANAR>
 __global__ __launch_bounds__(256) void Yuv420ToRgbTensor(const YuvArgs a)
 {
-    const int x = (blockIdx.x * 64 + (threadIdx.x & 63)) * 4;
+    const int x = (blockIdx.x * 64 + (threadIdx.x & 63)) * kYuvBlockW;
     const int y = (blockIdx.y * 4 + (threadIdx.x >> 6)) * 2;
     if (x >= a.W || y >= a.H)
     {
         return;
     }
     const int n = blockIdx.z;
-    ConvertBlock<DCN, SEMIPLANAR>(a.srcBase + n * a.srcSampleStride, a.srcRowStride, a.dstBase + n * a.dstSampleStride,
-                                  a.dstRowStride, a.W, a.H, x, y, a.bidx, a.uidx);
+    ConvertLaneBlock<DCN, SEMIPLANAR>(a.srcBase + n * a.srcSampleStride, a.srcRowStride, a.dstBase + n * a.dstSampleStride,
+                                      a.dstRowStride, a.W, a.H, x, y, a.bidx, a.uidx);
 }
 
 template<int DCN, bool SEMIPLANAR>
@@ -178,13 +258,14 @@ __global__ __launch_bounds__(256) void Yuv420ToRgbVarShape(const YuvArgs a, cons
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
     const int                    W = d.width, H = d.height;
-    const int                    x = (tc.tx * 64 + (threadIdx.x & 63)) * 4;
+    const int                    x = (tc.tx * 64 + (threadIdx.x & 63)) * kYuvBlockW;
     const int                    y = (tc.ty * 4 + (threadIdx.x >> 6)) * 2;
     if (x >= W || y >= H)
     {
         return;
     }
-    ConvertBlock<DCN, SEMIPLANAR>(AsGlobal(s.basePtr), s.rowStride, AsGlobal(d.basePtr), d.rowStride, W, H, x, y, a.bidx, a.uidx);
+    ConvertLaneBlock<DCN, SEMIPLANAR>(AsGlobal(s.basePtr), s.rowStride, AsGlobal(d.basePtr), d.rowStride, W, H, x, y, a.bidx,
+                                      a.uidx);
 }
 
 template<class T, int C>

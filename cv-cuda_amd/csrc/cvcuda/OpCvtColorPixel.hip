@@ -362,6 +362,53 @@ struct Yuv420FromBgr
             v.dst[(int64_t)(v.H + (y >> 2) + h4 * (a.uidx ^ 1)) * v.dstRow + uvx] = V;
         }
     }
+
+    // kGroup blocks side by side: 8 x 2 pixels, whole-dword stores on every plane
+    static constexpr int kGroup = 4;
+
+    static __device__ __forceinline__ void RunGroup(const View &v, const PixArgs &a, int ix, int iy)
+    {
+        constexpr int P = 2 * kGroup;
+        const int     x = ix * 2, y = iy * 2;
+        uint8_t       U[kGroup], V[kGroup];
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+        {
+            uint8_t s[P * SCH], Y[P];
+            LoadRun<uint8_t, P * SCH>(v.src + (int64_t)(y + r) * v.srcRow + x * SCH, s);
+#pragma unroll
+            for (int k = 0; k < P; ++k)
+            {
+                uint8_t u, w;
+                BgrToYuv420(a.bidx ? s[k * SCH + 2] : s[k * SCH], s[k * SCH + 1], a.bidx ? s[k * SCH] : s[k * SCH + 2],
+                            Y[k], u, w);
+                if (r == 0 && (k & 1) == 0)
+                {
+                    U[k >> 1] = u;
+                    V[k >> 1] = w;
+                }
+            }
+            StoreRunNT<uint8_t, P>(v.dst + (int64_t)(y + r) * v.dstRow + x, Y);
+        }
+        if constexpr (SEMIPLANAR)
+        {
+            uint8_t uv[P];
+#pragma unroll
+            for (int k = 0; k < kGroup; ++k)
+            {
+                uv[2 * k]     = a.uidx == 0 ? U[k] : V[k];
+                uv[2 * k + 1] = a.uidx == 0 ? V[k] : U[k];
+            }
+            StoreRunNT<uint8_t, P>(v.dst + (int64_t)(v.H + iy) * v.dstRow + x, uv);
+        }
+        else
+        {
+            const int h4  = v.H >> 2;
+            const int uvx = ix + ((v.W >> 1) & -(iy & 1));
+            StoreRunNT<uint8_t, kGroup>(v.dst + (int64_t)(v.H + (y >> 2) + h4 * a.uidx) * v.dstRow + uvx, U);
+            StoreRunNT<uint8_t, kGroup>(v.dst + (int64_t)(v.H + (y >> 2) + h4 * (a.uidx ^ 1)) * v.dstRow + uvx, V);
+        }
+    }
 };
 
 __device__ __forceinline__ void Yuv42xToBgr(int Y, int U, int V, uint8_t &b, uint8_t &g, uint8_t &r)
@@ -378,26 +425,50 @@ struct BgrFromYuv422
 {
     static constexpr int kItemW = 2, kItemH = 1;
 
-    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int ix, int y)
+    // the 2 pixels of source dword q to o[0 .. 2 * DCN)
+    static __device__ __forceinline__ void Convert(uint32_t q, const PixArgs &a, uint8_t *o)
     {
-        const uint32_t q  = *reinterpret_cast<const uint32_t *>(v.src + (int64_t)y * v.srcRow + ix * 4);
-        const int      Y0 = (q >> (8 * a.yidx)) & 0xFF, Y1 = (q >> (8 * (a.yidx + 2))) & 0xFF;
-        const int      U = (q >> (8 * ((a.yidx ^ 1) + a.uidx))) & 0xFF, V = (q >> (8 * ((a.yidx ^ 1) + (a.uidx ^ 2)))) & 0xFF;
-        Px<uint8_t, 2 * DCN> o;
+        const int Y0 = (q >> (8 * a.yidx)) & 0xFF, Y1 = (q >> (8 * (a.yidx + 2))) & 0xFF;
+        const int U = (q >> (8 * ((a.yidx ^ 1) + a.uidx))) & 0xFF, V = (q >> (8 * ((a.yidx ^ 1) + (a.uidx ^ 2)))) & 0xFF;
 #pragma unroll
         for (int k = 0; k < 2; ++k)
         {
             uint8_t b, g, r;
             Yuv42xToBgr(k == 0 ? Y0 : Y1, U, V, b, g, r);
-            o.v[k * DCN + 0] = a.bidx ? r : b;
-            o.v[k * DCN + 1] = g;
-            o.v[k * DCN + 2] = a.bidx ? b : r;
+            o[k * DCN + 0] = a.bidx ? r : b;
+            o[k * DCN + 1] = g;
+            o[k * DCN + 2] = a.bidx ? b : r;
             if constexpr (DCN == 4)
             {
-                o.v[k * DCN + 3] = 255;
+                o[k * DCN + 3] = 255;
             }
         }
+    }
+
+    static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int ix, int y)
+    {
+        const uint32_t       q = *reinterpret_cast<const uint32_t *>(v.src + (int64_t)y * v.srcRow + ix * 4);
+        Px<uint8_t, 2 * DCN> o;
+        Convert(q, a, o.v);
         StorePx<uint8_t, 2 * DCN>(v.dst + (int64_t)y * v.dstRow, ix, o);
+    }
+
+    // 4 pixels: 8 source bytes in, 12 or 16 bytes out as whole dwords
+    static constexpr int kGroup = 2;
+
+    static __device__ __forceinline__ void RunGroup(const View &v, const PixArgs &a, int ix, int y)
+    {
+        uint8_t  in[4 * kGroup];
+        uint32_t q[kGroup];
+        LoadRun<uint8_t, 4 * kGroup>(v.src + (int64_t)y * v.srcRow + ix * 4, in);
+        __builtin_memcpy(q, in, sizeof(q));
+        uint8_t o[kGroup * 2 * DCN];
+#pragma unroll
+        for (int g = 0; g < kGroup; ++g)
+        {
+            Convert(q[g], a, o + g * 2 * DCN);
+        }
+        StoreRunNT<uint8_t, kGroup * 2 * DCN>(v.dst + (int64_t)y * v.dstRow + (int64_t)ix * 2 * DCN, o);
     }
 };
 
@@ -411,6 +482,25 @@ struct GrayFromYuv422
         const uint32_t o = ((q >> (8 * a.yidx)) & 0xFF) | (((q >> (8 * (a.yidx + 2))) & 0xFF) << 8);
         __builtin_nontemporal_store((uint16_t)o, reinterpret_cast<uint16_t *>(v.dst + (int64_t)y * v.dstRow) + ix);
     }
+
+    // 8 pixels: 16 source bytes in, 8 bytes out
+    static constexpr int kGroup = 4;
+
+    static __device__ __forceinline__ void RunGroup(const View &v, const PixArgs &a, int ix, int y)
+    {
+        uint8_t  in[4 * kGroup];
+        uint32_t q[kGroup];
+        LoadRun<uint8_t, 4 * kGroup>(v.src + (int64_t)y * v.srcRow + ix * 4, in);
+        __builtin_memcpy(q, in, sizeof(q));
+        uint8_t o[2 * kGroup];
+#pragma unroll
+        for (int g = 0; g < kGroup; ++g)
+        {
+            o[2 * g]     = (uint8_t)(q[g] >> (8 * a.yidx));
+            o[2 * g + 1] = (uint8_t)(q[g] >> (8 * (a.yidx + 2)));
+        }
+        StoreRunNT<uint8_t, 2 * kGroup>(v.dst + (int64_t)y * v.dstRow + ix * 2, o);
+    }
 };
 
 // the luma rows of a 4:2:0 image are its gray image; 2 pixels per item (widths are even)
@@ -423,12 +513,36 @@ struct GrayFromYuv420
         const uint16_t q = reinterpret_cast<const uint16_t *>(v.src + (int64_t)y * v.srcRow)[ix];
         __builtin_nontemporal_store(q, reinterpret_cast<uint16_t *>(v.dst + (int64_t)y * v.dstRow) + ix);
     }
+
+    // 16 pixels: a 16-byte copy
+    static constexpr int kGroup = 8;
+
+    static __device__ __forceinline__ void RunGroup(const View &v, const PixArgs &, int ix, int y)
+    {
+        uint8_t q[2 * kGroup];
+        LoadRun<uint8_t, 2 * kGroup>(v.src + (int64_t)y * v.srcRow + ix * 2, q);
+        StoreRunNT<uint8_t, 2 * kGroup>(v.dst + (int64_t)y * v.dstRow + ix * 2, q);
+    }
 };
 
 // ---- kernels -----------------------------------------------------------------------------------------
-// Pixels per lane of a one-in, one-out operation (input and output elements have the same type).
+// Pixels per lane of a one-in, one-out operation. Byte pixels on both sides take runs of 8: measured
+// against 4 on 32 x 1080p, BGR2GRAY 53 -> 47 us (half as many of the narrow 1-byte-pixel stores), BGR2HSV
+// 82 -> 76 us, BGR2YUV 75 -> 73 us, swizzle-like maps unchanged; 16 and 32 were no better.
 template<class Op>
-constexpr int kMapRun = kRunPixelsFor<typename Op::Src::Elem, typename Op::Src::Elem>;
+constexpr int MapRunPixels()
+{
+    using S = typename Op::Src;
+    using D = decltype(Op::Map(S{}, PixArgs{}));
+    if (sizeof(typename D::Elem) == 1 && sizeof(typename S::Elem) == 1)
+    {
+        return 2 * kRunPixels;
+    }
+    return kRunPixelsFor<typename S::Elem, typename D::Elem>;
+}
+
+template<class Op>
+constexpr int kMapRun = MapRunPixels<Op>();
 
 // One pixel in, one pixel out (Op::Map): runs of kMapRun<Op> pixels per lane, one row per wave.
 template<class Op>
@@ -438,7 +552,7 @@ __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, i
     using D  = decltype(Op::Map(S{}, a));
     using TS = typename S::Elem;
     using TD = typename D::Elem;
-    constexpr int P = kRunPixelsFor<TS, TD>;
+    constexpr int P = kMapRun<Op>;
     if (x0 + P > W)
     {
         for (int x = x0; x < W; ++x)
@@ -498,19 +612,29 @@ __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTil
     MapRun<Op>(AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0, a);
 }
 
-// Subsampled formats: one work item (Op::kItemW x Op::kItemH pixels) per lane, tensors only.
+// Subsampled formats, tensors only: Op::kGroup work items (each Op::kItemW x Op::kItemH pixels) side by
+// side per lane, so that loads and stores are whole dwords; the items of a row's last, partial group
+// go one by one.
 template<class Op>
 __global__ __launch_bounds__(256) void PixelTensor(const PixArgs a)
 {
-    const int x = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int y = blockIdx.y * 4 + (threadIdx.x >> 6);
-    if (x >= a.itemsW || y >= a.itemsH)
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * Op::kGroup;
+    const int y  = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (x0 >= a.itemsW || y >= a.itemsH)
     {
         return;
     }
     const int  n = blockIdx.z;
     const View v = {a.src + n * a.srcN, a.dst + n * a.dstN, a.srcRow, a.dstRow, a.W, a.H};
-    Op::Run(v, a, x, y);
+    if (x0 + Op::kGroup <= a.itemsW)
+    {
+        Op::RunGroup(v, a, x0, y);
+        return;
+    }
+    for (int x = x0; x < a.itemsW; ++x)
+    {
+        Op::Run(v, a, x, y);
+    }
 }
 
 PixArgs MakeArgs(const ColorIO &io, int W, int H)
@@ -574,7 +698,7 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
         {
             return;
         }
-        dim3 grid(DivUp(a.itemsW, 64), DivUp(a.itemsH, 4), io.N);
+        dim3 grid(DivUp(a.itemsW, 64 * Op::kGroup), DivUp(a.itemsH, 4), io.N);
         hipLaunchKernelGGL((PixelTensor<Op>), grid, dim3(256), 0, stream, a);
         CheckLaunch("PixelTensor");
     }
