@@ -536,7 +536,7 @@ constexpr int MapRunPixels()
     using D = decltype(Op::Map(S{}, PixArgs{}));
     if (sizeof(typename D::Elem) == 1 && sizeof(typename S::Elem) == 1)
     {
-        return 2 * kRunPixels;
+        return 8;
     }
     return kRunPixelsFor<typename S::Elem, typename D::Elem>;
 }
