@@ -246,12 +246,32 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             {
                 return;
             }
+            // small pixels are fetched G at a time (one load of up to 16 bytes) and added in the same order
+            constexpr int  PB  = (int)sizeof(Pixel<T, C>), G = PB <= 4 ? 4 : (PB <= 8 ? 2 : 1);
             const uint8_t *row = p.src + (int64_t)y * p.srcRow;
             xb                 = min(xb, p.srcW);
-            for (int x = max(xa, 0); x < xb; ++x)
+            int x              = max(xa, 0);
+            if constexpr (G > 1)
+            {
+                for (; x + G <= xb; x += G)
+                {
+                    float t[G][C];
+                    LoadTaps<T, C, G>(row, x * PB, y == p.srcH - 1, p.srcW * PB, t);
+#pragma unroll
+                    for (int k = 0; k < G; ++k)
+                    {
+#pragma unroll
+                        for (int c = 0; c < C; ++c)
+                        {
+                            sum[c] += t[k][c] * w;
+                        }
+                    }
+                }
+            }
+            for (; x < xb; ++x)
             {
                 float t[1][C];
-                LoadTaps<T, C, 1>(row, x * (int)sizeof(Pixel<T, C>), y == p.srcH - 1, p.srcW * (int)sizeof(Pixel<T, C>), t);
+                LoadTaps<T, C, 1>(row, x * PB, y == p.srcH - 1, p.srcW * PB, t);
 #pragma unroll
                 for (int c = 0; c < C; ++c)
                 {
