@@ -212,17 +212,8 @@ __device__ __forceinline__ int BorderIndex(int border, int c, int s)
 }
 
 // MI355X hands the workgroups of a launch to its 8 XCDs round-robin (hardware id % 8) and every
-// XCD has an L2 of its own. This maps the hardware id of a 1-D launch of `total` workgroups to a
-// logical id such that each XCD works through ONE contiguous run of logical ids in launch order:
-// neighbouring logical ids then share an L2. Bijective for any `total`.
+// XCD has an L2 of its own.
 constexpr uint32_t kXcdCount = 8;
-
-__device__ __forceinline__ uint32_t XcdContiguousId(uint32_t hwId, uint32_t total)
-{
-    const uint32_t q = total / kXcdCount, r = total % kXcdCount;
-    const uint32_t xcd = hwId % kXcdCount, turn = hwId / kXcdCount;
-    return xcd * q + min(xcd, r) + turn;
-}
 
 } // namespace cvamd
 
