@@ -228,3 +228,36 @@ def test_varshape_per_pixel_families(cv, K, orc, col, gpu):
         bo.push_back(cv.Image.alloc((8, 12), K.IMAGE_FORMAT_U8))
         cv.CvtColor()(None, bi, bo, K.COLOR_RGB2YUV_NV12)
     assert e.value.status == 2
+
+
+def test_every_width_residue_of_the_grouped_kernels(cv, K, orc, col, gpu):
+    # the byte-pixel kernels move 8 or 16 pixels per lane and finish a row's ragged end item by item: every
+    # even width from 2 to 40 (all residues modulo 16, rows shorter than one group included) plus widths
+    # around a whole wave's 512 pixels, through each of those kernels
+    widths = list(range(2, 42, 2)) + [510, 512, 514, 516, 520, 526]
+    for w in widths:
+        h, n = 4, 2
+        nv = np.concatenate([orc.fill_u8((n, h, w), w, 16, 235), orc.fill_u8((n, h // 2, w), w + 1, 16, 240)], axis=1)[..., None]
+        for name, dcn, bgr, uidx, semi in [("COLOR_YUV2RGB_NV12", 3, False, 0, True), ("COLOR_YUV2BGRA_NV21", 4, True, 1, True),
+                                           ("COLOR_YUV2RGB_IYUV", 3, False, 0, False), ("COLOR_YUV2BGRA_YV12", 4, True, 1, False)]:
+            check(run(cv, nv, (n, h, w, dcn), np.uint8, getattr(K, name)), orc.yuv420_to_rgb(nv, dcn, bgr, uidx, semi, variant=0))
+        check(run(cv, nv, (n, h, w, 1), np.uint8, K.COLOR_YUV2GRAY_420), nv[:, :h])
+        a = image(orc, (n, h, w, 3), np.uint8, 3 * w)
+        a4 = image(orc, (n, h, w, 4), np.uint8, 5 * w)
+        check(run(cv, a, (n, h * 3 // 2, w, 1), np.uint8, K.COLOR_RGB2YUV_NV12), col.yuv420_from_bgr(a, False, 0, False))
+        check(run(cv, a4, (n, h * 3 // 2, w, 1), np.uint8, K.COLOR_BGRA2YUV_NV21), col.yuv420_from_bgr(a4, True, 1, False))
+        check(run(cv, a, (n, h * 3 // 2, w, 1), np.uint8, K.COLOR_BGR2YUV_I420), col.yuv420_from_bgr(a, True, 0, True))
+        check(run(cv, a4, (n, h * 3 // 2, w, 1), np.uint8, K.COLOR_RGBA2YUV_YV12), col.yuv420_from_bgr(a4, False, 1, True))
+        check(run(cv, a, (n, h, w, 1), np.uint8, K.COLOR_BGR2GRAY), col.gray_from_bgr(a, True))
+        check(run(cv, a, (n, h, w, 3), np.uint8, K.COLOR_RGB2HSV), col.hsv_from_bgr(a, False, False))
+        check(run(cv, a, (n, h, w, 3), np.uint8, K.COLOR_BGR2YUV), col.yuv_from_bgr(a, True))
+        y2 = image(orc, (n, h, 2 * w, 1), np.uint8, 7 * w)
+        check(run(cv, y2, (n, h, w, 3), np.uint8, K.COLOR_YUV2BGR_YUY2), col.bgr_from_yuv422(y2, True, 0, 0, 3))
+        check(run(cv, y2, (n, h, w, 4), np.uint8, K.COLOR_YUV2RGBA_UYVY), col.bgr_from_yuv422(y2, False, 1, 0, 4))
+        check(run(cv, y2, (n, h, w, 1), np.uint8, K.COLOR_YUV2GRAY_UYVY), col.gray_from_yuv422(y2, 1))
+    for w in (1, 3, 5, 7, 9, 15, 17, 511, 513):  # odd widths: the one-in, one-out maps only
+        a = image(orc, (2, 3, w, 3), np.uint8, 11 * w)
+        check(run(cv, a, (2, 3, w, 1), np.uint8, K.COLOR_RGB2GRAY), col.gray_from_bgr(a, False))
+        check(run(cv, a, (2, 3, w, 3), np.uint8, K.COLOR_BGR2HSV_FULL), col.hsv_from_bgr(a, True, True))
+        g = a[..., :1].copy()
+        check(run(cv, g, (2, 3, w, 3), np.uint8, K.COLOR_GRAY2BGR), col.bgr_from_gray(g))
