@@ -32,8 +32,7 @@ struct PixArgs
     uint8_t       *dst;
     int64_t        srcN, dstN;
     int32_t        srcRow, dstRow;
-    int32_t        itemsW, itemsH; // work items per image (tensor form)
-    int32_t        W, H;           // image size in pixels (tensor form)
+    int32_t        W, H; // size of the colour image in pixels (tensor form)
     const NVCVImageBufferStrided *srcList;
     const NVCVImageBufferStrided *dstList;
     int32_t bidx, uidx, yidx, full;
@@ -325,7 +324,8 @@ __device__ __forceinline__ void BgrToYuv420(int b, int g, int r, uint8_t &Y, uin
 template<int SCH, bool SEMIPLANAR>
 struct Yuv420FromBgr
 {
-    static constexpr int kItemW = 2, kItemH = 2;
+    static constexpr int  kItemW = 2, kItemH = 2;
+    static constexpr bool kSizeFromSrc = true; // the colour image is the input
 
     static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int ix, int iy)
     {
@@ -423,7 +423,8 @@ __device__ __forceinline__ void Yuv42xToBgr(int Y, int U, int V, uint8_t &b, uin
 template<int DCN>
 struct BgrFromYuv422
 {
-    static constexpr int kItemW = 2, kItemH = 1;
+    static constexpr int  kItemW = 2, kItemH = 1;
+    static constexpr bool kSizeFromSrc = false;
 
     // the 2 pixels of source dword q to o[0 .. 2 * DCN)
     static __device__ __forceinline__ void Convert(uint32_t q, const PixArgs &a, uint8_t *o)
@@ -474,7 +475,8 @@ struct BgrFromYuv422
 
 struct GrayFromYuv422
 {
-    static constexpr int kItemW = 2, kItemH = 1;
+    static constexpr int  kItemW = 2, kItemH = 1;
+    static constexpr bool kSizeFromSrc = false;
 
     static __device__ __forceinline__ void Run(const View &v, const PixArgs &a, int ix, int y)
     {
@@ -506,7 +508,8 @@ struct GrayFromYuv422
 // the luma rows of a 4:2:0 image are its gray image; 2 pixels per item (widths are even)
 struct GrayFromYuv420
 {
-    static constexpr int kItemW = 2, kItemH = 1;
+    static constexpr int  kItemW = 2, kItemH = 1;
+    static constexpr bool kSizeFromSrc = false;
 
     static __device__ __forceinline__ void Run(const View &v, const PixArgs &, int ix, int y)
     {
@@ -612,29 +615,48 @@ __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTil
     MapRun<Op>(AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0, a);
 }
 
-// Subsampled formats, tensors only: Op::kGroup work items (each Op::kItemW x Op::kItemH pixels) side by
-// side per lane, so that loads and stores are whole dwords; the items of a row's last, partial group
-// go one by one.
+// Subsampled formats: Op::kGroup work items (each Op::kItemW x Op::kItemH pixels) side by side per lane,
+// so that loads and stores are whole dwords; the items of a row's last, partial group go one by one.
+// Lane (tx, lane) of wave `ty` within the image whose view is v.
 template<class Op>
-__global__ __launch_bounds__(256) void PixelTensor(const PixArgs a)
+__device__ __forceinline__ void RunItems(const View &v, const PixArgs &a, int tx, int ty)
 {
-    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * Op::kGroup;
-    const int y  = blockIdx.y * 4 + (threadIdx.x >> 6);
-    if (x0 >= a.itemsW || y >= a.itemsH)
+    const int itemsW = v.W / Op::kItemW, itemsH = v.H / Op::kItemH;
+    const int x0 = (tx * 64 + (threadIdx.x & 63)) * Op::kGroup;
+    const int y  = ty * 4 + (threadIdx.x >> 6);
+    if (x0 >= itemsW || y >= itemsH)
     {
         return;
     }
-    const int  n = blockIdx.z;
-    const View v = {a.src + n * a.srcN, a.dst + n * a.dstN, a.srcRow, a.dstRow, a.W, a.H};
-    if (x0 + Op::kGroup <= a.itemsW)
+    if (x0 + Op::kGroup <= itemsW)
     {
         Op::RunGroup(v, a, x0, y);
         return;
     }
-    for (int x = x0; x < a.itemsW; ++x)
+    for (int x = x0; x < itemsW; ++x)
     {
         Op::Run(v, a, x, y);
     }
+}
+
+template<class Op>
+__global__ __launch_bounds__(256) void PixelTensor(const PixArgs a)
+{
+    const int  n = blockIdx.z;
+    const View v = {a.src + n * a.srcN, a.dst + n * a.dstN, a.srcRow, a.dstRow, a.W, a.H};
+    RunItems<Op>(v, a, blockIdx.x, blockIdx.y);
+}
+
+// Image batches: the size of the colour image comes from the input (Op::kSizeFromSrc) or the output.
+template<class Op>
+__global__ __launch_bounds__(256) void PixelVarShape(const PixArgs a, const VarTiles tiles)
+{
+    const TileCoord             tc = LocateTile(tiles, blockIdx.x);
+    const NVCVImagePlaneStrided s  = a.srcList[tc.image].planes[0];
+    const NVCVImagePlaneStrided d  = a.dstList[tc.image].planes[0];
+    const View v = {AsGlobal(s.basePtr), AsGlobal(d.basePtr), s.rowStride, d.rowStride,
+                    Op::kSizeFromSrc ? s.width : d.width, Op::kSizeFromSrc ? s.height : d.height};
+    RunItems<Op>(v, a, tc.tx, tc.ty);
 }
 
 PixArgs MakeArgs(const ColorIO &io, int W, int H)
@@ -687,18 +709,27 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
     }
     else
     {
+        constexpr int tileW = 64 * Op::kGroup * Op::kItemW, tileH = 4 * Op::kItemH; // pixels of the colour image
         if (io.dstHost != nullptr)
         {
-            throw OpError(NVCV_ERROR_INVALID_ARGUMENT,
-                          "Conversions to or from subsampled YUV formats are not available for image batches");
+            const NVCVImageBufferStrided *sizes = Op::kSizeFromSrc ? io.srcHost : io.dstHost;
+            for (int first = 0; first < io.N; first += kMaxTileImages)
+            {
+                VarTiles tiles;
+                int      total = BuildVarTiles(tiles, sizes, first, std::min(kMaxTileImages, io.N - first), tileW, tileH);
+                if (total > 0)
+                {
+                    hipLaunchKernelGGL((PixelVarShape<Op>), dim3(total), dim3(256), 0, stream, a, tiles);
+                    CheckLaunch("PixelVarShape");
+                }
+            }
+            return;
         }
-        a.itemsW = a.W / Op::kItemW;
-        a.itemsH = a.H / Op::kItemH;
-        if (a.itemsW == 0 || a.itemsH == 0)
+        if (a.W < Op::kItemW || a.H < Op::kItemH)
         {
             return;
         }
-        dim3 grid(DivUp(a.itemsW, 64 * Op::kGroup), DivUp(a.itemsH, 4), io.N);
+        dim3 grid(DivUp(a.W, tileW), DivUp(a.H, tileH), io.N);
         hipLaunchKernelGGL((PixelTensor<Op>), grid, dim3(256), 0, stream, a);
         CheckLaunch("PixelTensor");
     }
@@ -750,11 +781,19 @@ void RequireSameType(const ColorIO &io)
     }
 }
 
-void RequireTensors(const ColorIO &io)
+// check(srcW, srcH, dstW, dstH) on the tensor pair, or on every (input, output) image pair of a batch
+template<class F>
+void ForEachSizePair(const ColorIO &io, F check)
 {
-    if (io.dstHost != nullptr)
+    if (io.dstHost == nullptr)
     {
-        Bad("Conversions to or from subsampled YUV formats are not available for image batches");
+        check(io.srcW, io.srcH, io.dstW, io.dstH);
+        return;
+    }
+    for (int i = 0; i < io.N; ++i)
+    {
+        const NVCVImagePlaneStrided &s = io.srcHost[i].planes[0], &d = io.dstHost[i].planes[0];
+        check(s.width, s.height, d.width, d.height);
     }
 }
 
@@ -897,17 +936,20 @@ bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStr
     // ---- YUV 4:2:0 -> gray (106) ------------------------------------------------------------------------
     if (code == NVCV_COLOR_YUV2GRAY_420)
     {
-        RequireTensors(io);
         RequireChannels(io, 1, 1);
         RequireU8(io);
-        if (io.srcH % 3 != 0 || io.srcW % 2 != 0)
-        {
-            Bad("Invalid input shape: height must be a multiple of 3 and width a multiple of 2");
-        }
-        if (io.dstH != io.srcH * 2 / 3 || io.dstW != io.srcW)
-        {
-            Bad("Invalid output shape");
-        }
+        ForEachSizePair(io,
+                        [](int sw, int sh, int dw, int dh)
+                        {
+                            if (sh % 3 != 0 || sw % 2 != 0)
+                            {
+                                Bad("Invalid input shape: height must be a multiple of 3 and width a multiple of 2");
+                            }
+                            if (dh != sh * 2 / 3 || dw != sw)
+                            {
+                                Bad("Invalid output shape");
+                            }
+                        });
         Launch<GrayFromYuv420>(io, a, stream);
         return true;
     }
@@ -924,13 +966,8 @@ bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStr
         default:
             break;
         }
-        RequireTensors(io);
         RequireU8(io);
         const bool gray = code == NVCV_COLOR_YUV2GRAY_UYVY || code == NVCV_COLOR_YUV2GRAY_YUY2;
-        if (io.srcW % 4 != 0)
-        {
-            Bad("Invalid input shape -- width must be a multiple of 4");
-        }
         if (io.srcC != 1)
         {
             Bad("Invalid input channel number -- input must have 1 channel");
@@ -939,10 +976,18 @@ bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStr
         {
             throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid output channel number %d", io.dstC);
         }
-        if (io.dstH != io.srcH || 2 * io.dstW != io.srcW)
-        {
-            Bad("Invalid output shape");
-        }
+        ForEachSizePair(io,
+                        [](int sw, int sh, int dw, int dh)
+                        {
+                            if (sw % 4 != 0)
+                            {
+                                Bad("Invalid input shape -- width must be a multiple of 4");
+                            }
+                            if (dh != sh || 2 * dw != sw)
+                            {
+                                Bad("Invalid output shape");
+                            }
+                        });
         const bool bgrOrder = code == NVCV_COLOR_YUV2BGR_YUY2 || code == NVCV_COLOR_YUV2BGRA_YUY2
                            || code == NVCV_COLOR_YUV2BGR_YVYU || code == NVCV_COLOR_YUV2BGRA_YVYU
                            || code == NVCV_COLOR_YUV2BGR_UYVY || code == NVCV_COLOR_YUV2BGRA_UYVY;
@@ -973,7 +1018,6 @@ bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStr
     if ((c >= NVCV_COLOR_RGB2YUV_I420 && c <= NVCV_COLOR_BGRA2YUV_YV12)
         || (c >= NVCV_COLOR_RGB2YUV_NV12 && c <= NVCV_COLOR_BGRA2YUV_NV21))
     {
-        RequireTensors(io);
         const bool planar = c <= NVCV_COLOR_BGRA2YUV_YV12;
         const bool bgrOrder
             = code == NVCV_COLOR_BGR2YUV_NV12 || code == NVCV_COLOR_BGRA2YUV_NV12 || code == NVCV_COLOR_BGR2YUV_NV21
@@ -987,20 +1031,28 @@ bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStr
         {
             throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input channel number %d", io.srcC);
         }
-        if (io.srcH % 2 != 0 || io.srcW % 2 != 0)
-        {
-            Bad("Invalid input shape: width and height must be even");
-        }
-        if (planar && io.srcH % 4 != 0)
-        {
-            Bad("Invalid input shape: to convert to YUV 420 planar formats, the input tensor height must be a multiple "
-                "of 4");
-        }
         RequireU8(io);
-        if (io.dstC != 1 || io.dstH != io.srcH / 2 * 3 || io.dstW != io.srcW)
+        if (io.dstC != 1)
         {
             Bad("Invalid output shape");
         }
+        ForEachSizePair(io,
+                        [planar](int sw, int sh, int dw, int dh)
+                        {
+                            if (sh % 2 != 0 || sw % 2 != 0)
+                            {
+                                Bad("Invalid input shape: width and height must be even");
+                            }
+                            if (planar && sh % 4 != 0)
+                            {
+                                Bad("Invalid input shape: to convert to YUV 420 planar formats, the input height must "
+                                    "be a multiple of 4");
+                            }
+                            if (dh != sh / 2 * 3 || dw != sw)
+                            {
+                                Bad("Invalid output shape");
+                            }
+                        });
         a      = MakeArgs(io, io.srcW, io.srcH);
         a.bidx = bgrOrder ? 0 : 2;
         a.uidx = uFirst ? 0 : 1;

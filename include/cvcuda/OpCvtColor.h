@@ -13,8 +13,10 @@
  *   107, 108, 111, 112, 115..124 UYVY / YUY2 / YVYU -> RGB/BGR(A) or gray: u8, input 1-channel of width 2*W
  *   127..134, 140..147 RGB/BGR(A) -> I420 / YV12 / NV12 / NV21: u8, chroma from the top-left pixel of
  *            each 2x2 block
- * Image batches (VarShapeSubmit) take every code whose input and output have equal sizes, and the
- * 4:2:0 -> RGB codes. Any other code or combination -> INVALID_ARGUMENT. */
+ * Image batches (VarShapeSubmit) take the same codes (src/cvcuda/priv/legacy/cvt_color_var_shape.cu:
+ * 1324-1640); the 4:2:0 and 4:2:2 sides are single-plane u8 images of H*3/2 rows or 2*W columns, and
+ * every image pair is checked against the shape rules above. Any other code or combination ->
+ * INVALID_ARGUMENT. */
 #ifndef CVCUDA_CVTCOLOR_H
 #define CVCUDA_CVTCOLOR_H
 

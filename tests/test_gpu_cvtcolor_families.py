@@ -222,10 +222,64 @@ def test_varshape_per_pixel_families(cv, K, orc, col, gpu):
                 assert np.abs(res.astype(int) - r.astype(int)).max() <= 1
             else:
                 check(res, r, 1e-5)
-    with pytest.raises(cv.Error) as e:  # subsampled output: tensors only
-        bi, bo = cv.ImageBatchVarShape(1), cv.ImageBatchVarShape(1)
-        bi.push_back(cv.Image.alloc((8, 8), K.IMAGE_FORMAT_RGB8))
-        bo.push_back(cv.Image.alloc((8, 12), K.IMAGE_FORMAT_U8))
+
+
+def test_varshape_subsampled_families(cv, K, orc, col, gpu):
+    # image batches through the 4:2:0 encoders, the 4:2:2 decoders and the luma extractions (the
+    # reference: legacy/cvt_color_var_shape.cu:1416-1640): single-plane u8 images, every image its own size
+    rng = np.random.default_rng(21)
+    n = 7
+    sizes = [(2 * int(rng.integers(1, 150)), 4 * int(rng.integers(1, 30))) for _ in range(n)]
+    sizes[0], sizes[1] = (2, 4), (516, 8)
+
+    def batch_from(arrays, fmt):
+        b = cv.ImageBatchVarShape(len(arrays))
+        for a in arrays:
+            b.push_back(cv.Image.from_numpy(a, fmt))
+        return b
+
+    def batch_alloc(dims, fmt):
+        b, outs = cv.ImageBatchVarShape(len(dims)), []
+        for wh in dims:
+            outs.append(cv.Image.alloc(wh, fmt))
+            b.push_back(outs[-1])
+        return b, outs
+
+    def results(outs, c):
+        torch.cuda.synchronize()
+        return [o.plane_view(0, np.uint8, c).cpu().numpy() for o in outs]
+
+    for c, fmt in ((3, K.IMAGE_FORMAT_RGB8), (4, K.IMAGE_FORMAT_RGBA8)):
+        rgb = [image(orc, (h, w, c), np.uint8, 31 * i + c) for i, (w, h) in enumerate(sizes)]
+        bi = batch_from(rgb, fmt)
+        for name, bgr, uidx, planar in [("COLOR_RGB2YUV_NV12", False, 0, False), ("COLOR_BGR2YUV_NV21", True, 1, False),
+                                        ("COLOR_BGR2YUV_I420", True, 0, True), ("COLOR_RGB2YUV_YV12", False, 1, True)]:
+            name = name.replace("RGB2", "RGBA2").replace("BGR2", "BGRA2") if c == 4 else name
+            bo, outs = batch_alloc([(w, h * 3 // 2) for w, h in sizes], K.IMAGE_FORMAT_U8)
+            cv.CvtColor()(None, bi, bo, getattr(K, name))
+            for a, r in zip(rgb, results(outs, 1)):
+                check(r[None], col.yuv420_from_bgr(a[None], bgr, uidx, planar))
+    packed = [image(orc, (h, 2 * w, 1), np.uint8, 17 * i) for i, (w, h) in enumerate(sizes)]
+    bi = batch_from(packed, K.IMAGE_FORMAT_U8)
+    for name, bgr, yidx, uidx, dcn in [("COLOR_YUV2BGR_YUY2", True, 0, 0, 3), ("COLOR_YUV2RGBA_UYVY", False, 1, 0, 4),
+                                       ("COLOR_YUV2RGB_YVYU", False, 0, 2, 3)]:
+        bo, outs = batch_alloc(sizes, K.IMAGE_FORMAT_RGB8 if dcn == 3 else K.IMAGE_FORMAT_RGBA8)
+        cv.CvtColor()(None, bi, bo, getattr(K, name))
+        for a, r in zip(packed, results(outs, dcn)):
+            check(r[None], col.bgr_from_yuv422(a[None], bgr, yidx, uidx, dcn))
+    bo, outs = batch_alloc(sizes, K.IMAGE_FORMAT_U8)
+    cv.CvtColor()(None, bi, bo, K.COLOR_YUV2GRAY_YUY2)
+    for a, r in zip(packed, results(outs, 1)):
+        check(r[None], col.gray_from_yuv422(a[None], 0))
+    planes = [image(orc, (h * 3 // 2, w, 1), np.uint8, 13 * i) for i, (w, h) in enumerate(sizes)]
+    bo, outs = batch_alloc(sizes, K.IMAGE_FORMAT_U8)
+    cv.CvtColor()(None, batch_from(planes, K.IMAGE_FORMAT_U8), bo, K.COLOR_YUV2GRAY_420)
+    for a, r, (w, h) in zip(planes, results(outs, 1), sizes):
+        check(r, a[:h])
+    # one image of the batch with the wrong output height
+    bi = batch_from([image(orc, (8, 8, 3), np.uint8, 1), image(orc, (8, 16, 3), np.uint8, 2)], K.IMAGE_FORMAT_RGB8)
+    bo, _ = batch_alloc([(8, 12), (16, 8)], K.IMAGE_FORMAT_U8)
+    with pytest.raises(cv.Error) as e:
         cv.CvtColor()(None, bi, bo, K.COLOR_RGB2YUV_NV12)
     assert e.value.status == 2
 
