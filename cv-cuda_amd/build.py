@@ -24,11 +24,14 @@ COMMON = [
     "-std=c++17", "-O3", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wextra", "-Wno-unused-parameter",
     "-I" + INCLUDE, "-I" + CSRC,
 ]
-# Device code: no FMA contraction (results must match the CPU goldens' expression shapes) and no
-# packed-FP32 instruction selection.
+# Device code: no FMA contraction (results must match the CPU goldens' expression shapes), no
+# packed-FP32 instruction selection, and no v_ashr_pk_{u8,i8}_i32: the compiler treats the upper 16 bits
+# of that instruction's result as zero, on MI355X they held the destination's previous contents (seen
+# as wrong third bytes where two clamped shifts were OR-ed with a third in the 4:2:0 -> RGB kernel).
 DEVICE = [
     "--offload-arch=" + ARCH, "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Xclang", "-target-feature", "-Xclang", "-ashr-pk-insts",
 ]
 
 
@@ -52,7 +55,7 @@ def _compile(src, obj, extra, force, newest_header):
     cmd = ["hipcc"] + COMMON + extra + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     msgs = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
-                     if "packed-fp32-ops" not in l or "error" in l)
+                     if ("packed-fp32-ops" not in l and "ashr-pk-insts" not in l) or "error" in l)
     if r.returncode != 0:
         raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), msgs))
     return msgs

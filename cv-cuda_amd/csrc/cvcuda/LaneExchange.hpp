@@ -84,6 +84,16 @@ __device__ __forceinline__ void PackQuad(const uint32_t (&q)[(PB + 3) / 4][4], u
     }
 }
 
+// Orders a wave's LDS writes before its later LDS reads (and the reverse) where lanes of the same
+// wave exchange data: LDS instructions of one wave execute in order, so only the compiler has to
+// be kept from moving them.
+__device__ __forceinline__ void WaveExchangeFence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 } // namespace cvamd
 
 #endif // CVCUDA_AMD_LANEEXCHANGE_HPP

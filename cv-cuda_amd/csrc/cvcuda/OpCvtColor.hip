@@ -13,6 +13,7 @@
 #include "CvtColorFamilies.hpp"
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "LaneExchange.hpp"
 #include "RunIO.hpp"
 #include "VarShapeTiles.hpp"
 
@@ -165,7 +166,9 @@ __device__ __forceinline__ void ConvertWideBlock(const uint8_t *src, int srcRow,
                                                  int x, int y, int bidx, int uidx)
 {
     constexpr int BW = kYuvBlockW, NC = BW / 2;
-    int           uu[NC], vv[NC];
+    // lanes 0 .. lanes-1 of this wave take this path (the wave covers consecutive blocks of one row)
+    const int lane = threadIdx.x & 63, lanes = min(64, (W - (x - lane * BW)) / BW);
+    int       uu[NC], vv[NC];
     if constexpr (SEMIPLANAR)
     {
         uint8_t  c[BW];
@@ -194,6 +197,19 @@ __device__ __forceinline__ void ConvertWideBlock(const uint8_t *src, int srcRow,
             vv[k] = (int)pv[k] - 128;
         }
     }
+    // The chroma terms and the rounding constant of YuvToRgb's three sums, once per chroma sample (4
+    // pixels share them), already in output channel order; integer addition is associative, so the
+    // results are the same.
+    int c0[NC], c1[NC], c2[NC];
+#pragma unroll
+    for (int k = 0; k < NC; ++k)
+    {
+        const int rC = 1673527 * vv[k] + (1 << 19);
+        const int bC = 2116026 * uu[k] + (1 << 19);
+        c0[k]        = bidx == 0 ? bC : rC;
+        c1[k]        = -852492 * vv[k] - 409993 * uu[k] + (1 << 19);
+        c2[k]        = bidx == 0 ? rC : bC;
+    }
 #pragma unroll
     for (int ry = 0; ry < 2; ++ry)
     {
@@ -207,17 +223,46 @@ __device__ __forceinline__ void ConvertWideBlock(const uint8_t *src, int srcRow,
 #pragma unroll
         for (int i = 0; i < BW; ++i)
         {
-            uint32_t r, g, b;
-            YuvToRgb(luma[i], uu[i >> 1], vv[i >> 1], r, g, b);
-            out[i * DCN + 0] = (uint8_t)(bidx == 0 ? b : r);
-            out[i * DCN + 1] = (uint8_t)g;
-            out[i * DCN + 2] = (uint8_t)(bidx == 0 ? r : b);
+            const int t      = max(0, (int)luma[i] - 16) * 1220542;
+            out[i * DCN + 0] = (uint8_t)min(max((t + c0[i >> 1]) >> 20, 0), 255);
+            out[i * DCN + 1] = (uint8_t)min(max((t + c1[i >> 1]) >> 20, 0), 255);
+            out[i * DCN + 2] = (uint8_t)min(max((t + c2[i >> 1]) >> 20, 0), 255);
             if constexpr (DCN == 4)
             {
                 out[i * DCN + 3] = 255;
             }
         }
-        StoreRunNT<uint8_t, BW * DCN>(dst + (int64_t)yy * dstRow + (int64_t)x * DCN, out);
+        // The wave's lanes hold consecutive 24- (or 32-) byte pieces of one output row. Stored as they are,
+        // every 32-byte sector would be completed by two store instructions; handed round through LDS as
+        // 16-byte chunks (chunk c to lane c % lanes), every instruction writes one dense span.
+        constexpr int RB = BW * DCN; // bytes per lane and row
+        __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
+        uint8_t  *mine   = stage[threadIdx.x >> 6];
+        const int chunks = lanes * RB / 16;
+        __builtin_memcpy(mine + lane * RB, out, RB);
+        WaveExchangeFence();
+        uint8_t *rowOut = dst + (int64_t)yy * dstRow + (int64_t)(x - lane * BW) * DCN;
+#pragma unroll
+        for (int j = 0; j < (RB + 15) / 16; ++j)
+        {
+            const int c = j * lanes + lane;
+            if (c < chunks)
+            {
+                uint32_t w[4];
+                __builtin_memcpy(w, mine + c * 16, 16);
+                StoreDwordsNT<4>(rowOut + c * 16, w);
+            }
+        }
+        if constexpr (RB % 16 != 0)
+        {
+            if (lane == 0 && (lanes & 1)) // an odd number of 24-byte pieces ends with half a chunk
+            {
+                uint32_t w[2];
+                __builtin_memcpy(w, mine + chunks * 16, 8);
+                StoreDwordsNT<2>(rowOut + chunks * 16, w);
+            }
+        }
+        WaveExchangeFence();
     }
 }
 

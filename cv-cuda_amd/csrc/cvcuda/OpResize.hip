@@ -984,16 +984,6 @@ struct alignas(BYTES % 16 == 0 ? 16 : (BYTES % 8 == 0 ? 8 : 4)) LdsSlot
     uint32_t w[BYTES / 4];
 };
 
-// Orders a wave's LDS writes before its later LDS reads (and the reverse) where lanes of the same
-// wave exchange data: LDS instructions of one wave execute in order, so only the compiler has to
-// be kept from moving them.
-__device__ __forceinline__ void WaveExchangeFence()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 __device__ __forceinline__ void CubicSourceX(int srcW, float scaleX, int dx, int &sx, float &fx)
 {
     const float cx = (dx + .5f) * scaleX - .5f;
