@@ -845,50 +845,70 @@ __device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int 
     // the 2 rows' terms are computed side by side (even lanes the first, odd lanes the second)
     const auto rows = Axis<NVCV_INTERP_LINEAR>(p.scaleY, min(y0 + (lane & 1), p.dstH - 1), p.srcH);
     uint32_t   pxA[2], pxB[2];
-#pragma unroll
-    for (int k = 0; k < 2; ++k)
+    const auto row0 = FromLane(rows, 0), row1 = FromLane(rows, 1);
+    // taps of source row y for both columns: A's two, then B's
+    auto fetchLast = [&](int y, uint32_t (&t)[4]) // the image's last row: nothing may be read past its end
     {
-        const auto row = FromLane(rows, k);
-        const int  ya = row.s, yb = min(row.s + 1, p.srcH - 1);
-        uint32_t   top[4], bot[4]; // A's two taps, then B's
-        auto       fetch = [&](int y, uint32_t (&t)[4])
+        const uint8_t *line = p.src + (int64_t)y * p.srcRow;
+        float          a[2][C], b[2][C];
+        LoadTaps<uint8_t, C, 2>(line, colA.s * C, true, p.srcW * C, a);
+        LoadTaps<uint8_t, C, 2>(line, colB.s * C, true, p.srcW * C, b);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
         {
-            const uint8_t *line = p.src + (int64_t)y * p.srcRow;
-            if (y == p.srcH - 1) // wave-uniform: nothing may be read past the end of the last row
+            t[i] = 0;
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            t[0] |= (uint32_t)a[0][c] << (8 * c);
+            t[1] |= (uint32_t)a[1][c] << (8 * c);
+            t[2] |= (uint32_t)b[0][c] << (8 * c);
+            t[3] |= (uint32_t)b[1][c] << (8 * c);
+        }
+    };
+    auto window = [&](int y) { return *reinterpret_cast<const TapWindow<C> *>(p.src + (int64_t)y * p.srcRow + colA.s * C); };
+    auto unpack = [&](const TapWindow<C> &win, uint32_t (&t)[4])
+    {
+        const uint32_t k0 = WindowPixel<C>(win, 0), k1 = WindowPixel<C>(win, 1), k2 = WindowPixel<C>(win, 2),
+                       k3 = WindowPixel<C>(win, 3);
+        t[0] = k0;
+        t[1] = k1;
+        t[2] = delta == 0 ? k0 : (delta == 1 ? k1 : k2);
+        t[3] = delta == 0 ? k1 : (delta == 1 ? k2 : k3);
+    };
+    const int ya0 = row0.s, yb0 = min(row0.s + 1, p.srcH - 1), ya1 = row1.s, yb1 = min(row1.s + 1, p.srcH - 1);
+    uint32_t  top[2][4], bot[2][4];
+    if (max(yb0, yb1) < p.srcH - 1) // wave-uniform; the usual case: all four window loads go out together
+    {
+        const TapWindow<C> w0 = window(ya0), w1 = window(yb0), w2 = window(ya1), w3 = window(yb1);
+        unpack(w0, top[0]);
+        unpack(w1, bot[0]);
+        unpack(w2, top[1]);
+        unpack(w3, bot[1]);
+    }
+    else
+    {
+        auto fetch = [&](int y, uint32_t (&t)[4])
+        {
+            if (y == p.srcH - 1)
             {
-                float a[2][C], b[2][C];
-                LoadTaps<uint8_t, C, 2>(line, colA.s * C, true, p.srcW * C, a);
-                LoadTaps<uint8_t, C, 2>(line, colB.s * C, true, p.srcW * C, b);
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                {
-                    t[i] = 0;
-                }
-#pragma unroll
-                for (int c = 0; c < C; ++c)
-                {
-                    t[0] |= (uint32_t)a[0][c] << (8 * c);
-                    t[1] |= (uint32_t)a[1][c] << (8 * c);
-                    t[2] |= (uint32_t)b[0][c] << (8 * c);
-                    t[3] |= (uint32_t)b[1][c] << (8 * c);
-                }
+                fetchLast(y, t);
             }
             else
             {
-                const TapWindow<C> win = *reinterpret_cast<const TapWindow<C> *>(line + colA.s * C);
-                const uint32_t     k0 = WindowPixel<C>(win, 0), k1 = WindowPixel<C>(win, 1), k2 = WindowPixel<C>(win, 2),
-                               k3 = WindowPixel<C>(win, 3);
-                t[0] = k0;
-                t[1] = k1;
-                t[2] = delta == 0 ? k0 : (delta == 1 ? k1 : k2);
-                t[3] = delta == 0 ? k1 : (delta == 1 ? k2 : k3);
+                unpack(window(y), t);
             }
         };
-        fetch(ya, top);
-        fetch(yb, bot);
-        pxA[k] = BlendU8<C, VARSHAPE>(top[0], top[1], bot[0], bot[1], colA.w[0], row.w[0]);
-        pxB[k] = BlendU8<C, VARSHAPE>(top[2], top[3], bot[2], bot[3], colB.w[0], row.w[0]);
+        fetch(ya0, top[0]);
+        fetch(yb0, bot[0]);
+        fetch(ya1, top[1]);
+        fetch(yb1, bot[1]);
     }
+    pxA[0] = BlendU8<C, VARSHAPE>(top[0][0], top[0][1], bot[0][0], bot[0][1], colA.w[0], row0.w[0]);
+    pxB[0] = BlendU8<C, VARSHAPE>(top[0][2], top[0][3], bot[0][2], bot[0][3], colB.w[0], row0.w[0]);
+    pxA[1] = BlendU8<C, VARSHAPE>(top[1][0], top[1][1], bot[1][0], bot[1][1], colA.w[0], row1.w[0]);
+    pxB[1] = BlendU8<C, VARSHAPE>(top[1][2], top[1][3], bot[1][2], bot[1][3], colB.w[0], row1.w[0]);
     // even lanes keep their first-row pair and take the neighbour's, odd lanes the same for the second row
     const uint32_t got0 = FromLaneXor1(odd ? pxA[0] : pxA[1]), got1 = FromLaneXor1(odd ? pxB[0] : pxB[1]);
     const uint32_t q[1][4] = {{odd ? got0 : pxA[0], odd ? got1 : pxB[0], odd ? pxA[1] : got0, odd ? pxB[1] : got1}};
