@@ -232,37 +232,10 @@ __device__ __forceinline__ void ConvertWideBlock(const uint8_t *src, int srcRow,
                 out[i * DCN + 3] = 255;
             }
         }
-        // The wave's lanes hold consecutive 24- (or 32-) byte pieces of one output row. Stored as they are,
-        // every 32-byte sector would be completed by two store instructions; handed round through LDS as
-        // 16-byte chunks (chunk c to lane c % lanes), every instruction writes one dense span.
-        constexpr int RB = BW * DCN; // bytes per lane and row
+        constexpr int RB = BW * DCN; // bytes per lane and row: more than one store, so the row is regrouped
         __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
-        uint8_t  *mine   = stage[threadIdx.x >> 6];
-        const int chunks = lanes * RB / 16;
-        __builtin_memcpy(mine + lane * RB, out, RB);
-        WaveExchangeFence();
-        uint8_t *rowOut = dst + (int64_t)yy * dstRow + (int64_t)(x - lane * BW) * DCN;
-#pragma unroll
-        for (int j = 0; j < (RB + 15) / 16; ++j)
-        {
-            const int c = j * lanes + lane;
-            if (c < chunks)
-            {
-                uint32_t w[4];
-                __builtin_memcpy(w, mine + c * 16, 16);
-                StoreDwordsNT<4>(rowOut + c * 16, w);
-            }
-        }
-        if constexpr (RB % 16 != 0)
-        {
-            if (lane == 0 && (lanes & 1)) // an odd number of 24-byte pieces ends with half a chunk
-            {
-                uint32_t w[2];
-                __builtin_memcpy(w, mine + chunks * 16, 8);
-                StoreDwordsNT<2>(rowOut + chunks * 16, w);
-            }
-        }
-        WaveExchangeFence();
+        StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], dst + (int64_t)yy * dstRow + (int64_t)(x - lane * BW) * DCN, out, lane,
+                             lanes);
     }
 }
 
