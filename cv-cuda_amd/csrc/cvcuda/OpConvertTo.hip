@@ -9,6 +9,7 @@
 // 16-byte store per lane). A wave covers 256 scalars of a row, a block 4 rows. Streaming stores.
 #include "DeviceUtils.hpp"
 #include "OpCommon.hpp"
+#include "RunIO.hpp"
 
 #include <cvcuda/OpConvertTo.h>
 
@@ -27,12 +28,6 @@ struct ConvertArgs
     int32_t        srcRow, dstRow;
     int32_t        rowElems, H;
     double         alpha, beta;
-};
-
-template<int WORDS>
-struct __attribute__((packed, aligned(1))) Words
-{
-    uint32_t w[WORDS];
 };
 
 // double -> T with round-half-to-even and saturation; NaN -> 0 for integer targets
@@ -79,11 +74,18 @@ __device__ __forceinline__ TD ConvertOne(TS s, const ConvertArgs &a)
     }
 }
 
+// Scalars per lane: 4 (one 4- to 32-byte access per side). Byte inputs widened to 4-byte outputs take 8, so
+// that the load is 8 bytes instead of 4; their 32 output bytes per lane leave through the row-regrouped
+// stores (stored directly they measured 235 us against 175 us with 4 scalars on 32 x 1080p x 3).
+template<class TS, class TD>
+constexpr int kConvertRun = (sizeof(TS) == 1 && sizeof(TD) == 4) ? 8 : 4;
+
 template<class TS, class TD>
 __global__ __launch_bounds__(256) void ConvertKernel(const ConvertArgs a)
 {
-    const int y = blockIdx.y * 4 + (threadIdx.x >> 6);
-    const int e = (blockIdx.x * 64 + (threadIdx.x & 63)) * 4;
+    constexpr int E = kConvertRun<TS, TD>;
+    const int     y = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int     lane = threadIdx.x & 63, e0 = blockIdx.x * 64 * E, e = e0 + lane * E;
     if (y >= a.H || e >= a.rowElems)
     {
         return;
@@ -91,29 +93,28 @@ __global__ __launch_bounds__(256) void ConvertKernel(const ConvertArgs a)
     const int      n = blockIdx.z;
     const uint8_t *s = a.src + n * a.srcN + (int64_t)y * a.srcRow + (int64_t)e * sizeof(TS);
     uint8_t       *d = a.dst + n * a.dstN + (int64_t)y * a.dstRow + (int64_t)e * sizeof(TD);
-    if (e + 4 <= a.rowElems)
+    if (e + E <= a.rowElems)
     {
-        union
-        {
-            Words<sizeof(TS)> w;
-            TS                v[4];
-        } in;
-        union
-        {
-            Words<sizeof(TD)> w;
-            TD                v[4];
-        } out;
-        in.w = *reinterpret_cast<const Words<sizeof(TS)> *>(s);
+        TS in[E];
+        TD out[E];
+        LoadRun<TS, E>(s, in);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < E; ++i)
         {
-            out.v[i] = ConvertOne<TS, TD>(in.v[i], a);
+            out[i] = ConvertOne<TS, TD>(in[i], a);
         }
-        Words<sizeof(TD)> *o = reinterpret_cast<Words<sizeof(TD)> *>(d);
-#pragma unroll
-        for (int i = 0; i < (int)sizeof(TD); ++i)
+        if constexpr (E * sizeof(TD) > 16)
         {
-            __builtin_nontemporal_store(out.w.w[i], &o->w[i]);
+            constexpr int RB = E * sizeof(TD);
+            __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
+            uint8_t piece[RB];
+            __builtin_memcpy(piece, out, RB);
+            StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], d - (int64_t)lane * RB, piece, lane,
+                                 min(64, (a.rowElems - e0) / E));
+        }
+        else
+        {
+            StoreRunNT<TD, E>(d, out);
         }
     }
     else
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void ConvertKernel(const ConvertArgs a)
 template<class TS, class TD>
 void Launch(const ConvertArgs &a, int N, hipStream_t stream)
 {
-    dim3 grid(DivUp(a.rowElems, 256), DivUp(a.H, 4), N);
+    dim3 grid(DivUp(a.rowElems, 64 * kConvertRun<TS, TD>), DivUp(a.H, 4), N);
     hipLaunchKernelGGL((ConvertKernel<TS, TD>), grid, dim3(256), 0, stream, a);
     CheckLaunch("ConvertKernel");
 }
