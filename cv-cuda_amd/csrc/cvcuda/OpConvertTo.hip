@@ -103,19 +103,7 @@ __global__ __launch_bounds__(256) void ConvertKernel(const ConvertArgs a)
         {
             out[i] = ConvertOne<TS, TD>(in[i], a);
         }
-        if constexpr (E * sizeof(TD) > 16)
-        {
-            constexpr int RB = E * sizeof(TD);
-            __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
-            uint8_t piece[RB];
-            __builtin_memcpy(piece, out, RB);
-            StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], d - (int64_t)lane * RB, piece, lane,
-                                 min(64, (a.rowElems - e0) / E));
-        }
-        else
-        {
-            StoreRunNT<TD, E>(d, out);
-        }
+        StoreRowRunNT<TD, E>(d - (int64_t)lane * E * sizeof(TD), out, lane, min(64, (a.rowElems - e0) / E));
     }
     else
     {

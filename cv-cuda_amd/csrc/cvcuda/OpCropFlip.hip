@@ -108,15 +108,16 @@ __device__ __forceinline__ void CopyRuns(const uint8_t *srcRow, uint8_t *dstRow,
 {
     constexpr int P = kRunPixelsFor<T, T>, PB = C * sizeof(T), D = P * PB / 4;
     static_assert((P * PB) % 4 == 0, "runs are whole dwords");
-    const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63, lanes = min(64, max(0, w - run0 * P) / P); // lanes with a whole run
     const int dx0  = (run0 + lane) * P;
+    uint8_t  *out0 = dstRow + (int64_t)run0 * P * PB; // where lane 0's run goes
     T         in[P * C];
     if (step > 0)
     {
         if (dx0 + P <= w)
         {
             LoadRun<T, P * C>(srcRow + (int64_t)(sx0 + dx0) * PB, in);
-            StoreRunNT<T, P * C>(dstRow + (int64_t)dx0 * PB, in);
+            StoreRowRunNT<T, P * C>(out0, in, lane, lanes);
             return;
         }
     }
@@ -147,7 +148,7 @@ __device__ __forceinline__ void CopyRuns(const uint8_t *srcRow, uint8_t *dstRow,
                     out[k * C + c] = in[(P - 1 - k) * C + c];
                 }
             }
-            StoreRunNT<T, P * C>(dstRow + (int64_t)dx0 * PB, out);
+            StoreRowRunNT<T, P * C>(out0, out, lane, lanes);
             return;
         }
     }

@@ -250,20 +250,8 @@ __global__ __launch_bounds__(256) void CfnrRunsKernel(const CfnrArgs a)
             }
             else
             {
-                constexpr int RB = P * C * (int)sizeof(TD); // output bytes per lane
-                if constexpr (RB > 16 && RB % 8 == 0)
-                {
-                    // more than one store per lane: the wave's lanes 0 .. lanes-1 hold consecutive pieces of the row
-                    __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
-                    const int lane = threadIdx.x & 63, lanes = min(64, (a.W - (x0 - lane * P)) / P);
-                    uint8_t   piece[RB];
-                    __builtin_memcpy(piece, out, RB);
-                    StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], d - (int64_t)lane * RB, piece, lane, lanes);
-                }
-                else
-                {
-                    StoreRunNT<TD, P * C>(d, out);
-                }
+                const int lane = threadIdx.x & 63, lanes = min(64, (a.W - (x0 - lane * P)) / P);
+                StoreRowRunNT<TD, P * C>(d - (int64_t)lane * P * C * sizeof(TD), out, lane, lanes);
             }
         }
         else

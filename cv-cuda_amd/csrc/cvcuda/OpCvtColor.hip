@@ -232,10 +232,7 @@ __device__ __forceinline__ void ConvertWideBlock(const uint8_t *src, int srcRow,
                 out[i * DCN + 3] = 255;
             }
         }
-        constexpr int RB = BW * DCN; // bytes per lane and row: more than one store, so the row is regrouped
-        __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
-        StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], dst + (int64_t)yy * dstRow + (int64_t)(x - lane * BW) * DCN, out, lane,
-                             lanes);
+        StoreRowRunNT<uint8_t, BW * DCN>(dst + (int64_t)yy * dstRow + (int64_t)(x - lane * BW) * DCN, out, lane, lanes);
     }
 }
 
@@ -364,7 +361,8 @@ __device__ __forceinline__ void SwizzleRun(const uint8_t *srcRow, uint8_t *dstRo
             }
         }
     }
-    StoreRunNT<T, P * DCH>(dstRow + (int64_t)x0 * DCH * sizeof(T), out);
+    const int lane = threadIdx.x & 63, lanes = min(64, (W - (x0 - lane * P)) / P);
+    StoreRowRunNT<T, P * DCH>(dstRow + (int64_t)(x0 - lane * P) * DCH * sizeof(T), out, lane, lanes);
 }
 
 template<class T, int SCH, int DCH>

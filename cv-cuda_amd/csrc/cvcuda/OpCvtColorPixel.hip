@@ -583,18 +583,9 @@ __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, i
             out[k * D::kC + c] = d.v[c];
         }
     }
-    constexpr int RB = P * (int)sizeof(D);
-    if constexpr (RB > 16 && RB % 8 == 0 && sizeof(TD) == 1)
-    {
-        // the wave's lanes 0 .. lanes-1 hold consecutive pieces of this row (the ragged run returned above)
-        __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
-        const int lane = threadIdx.x & 63, lanes = min(64, (W - (x0 - lane * P)) / P);
-        StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], dstRow + (int64_t)(x0 - lane * P) * sizeof(D), out, lane, lanes);
-    }
-    else
-    {
-        StoreRunNT<TD, P * D::kC>(dstRow + (int64_t)x0 * sizeof(D), out);
-    }
+    // the wave's lanes 0 .. lanes-1 hold consecutive pieces of this row (the ragged run returned above)
+    const int lane = threadIdx.x & 63, lanes = min(64, (W - (x0 - lane * P)) / P);
+    StoreRowRunNT<TD, P * D::kC>(dstRow + (int64_t)(x0 - lane * P) * sizeof(D), out, lane, lanes);
 }
 
 template<class Op>

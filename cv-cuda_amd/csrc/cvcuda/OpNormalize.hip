@@ -134,21 +134,9 @@ __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow
         {
             out[i] = SaturateCast<TO>(((float)in[i] - b[i % C]) * m[i % C] * a.gscale + a.shift);
         }
-        constexpr int RB = P * C * (int)sizeof(TO); // output bytes per lane
-        if constexpr (RB > 16 && RB % 8 == 0)
-        {
-            // more than one store per lane: the wave's lanes 0 .. lanes-1 hold consecutive pieces of the row
-            __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
-            const int lane = threadIdx.x & 63, lanes = min(64, (W - (x0 - lane * P)) / P);
-            uint8_t   piece[RB];
-            __builtin_memcpy(piece, out, RB);
-            StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], dstRow + (int64_t)(x0 - lane * P) * C * sizeof(TO), piece, lane,
-                                 lanes);
-        }
-        else
-        {
-            StoreRunNT<TO, P * C>(dstRow + (int64_t)x0 * C * sizeof(TO), out);
-        }
+        // the wave's lanes 0 .. lanes-1 hold consecutive pieces of the row
+        const int lane = threadIdx.x & 63, lanes = min(64, (W - (x0 - lane * P)) / P);
+        StoreRowRunNT<TO, P * C>(dstRow + (int64_t)(x0 - lane * P) * C * sizeof(TO), out, lane, lanes);
     }
     else
     {

@@ -89,6 +89,26 @@ __device__ __forceinline__ void StoreRowPiecesNT(uint8_t *stage, uint8_t *rowOut
     WaveExchangeFence(); // the next row may overwrite the staging area
 }
 
+// N elements per lane as one piece of an output row: lanes 0 .. lanes-1 of the wave hold consecutive
+// pieces, lane 0's at row0. Pieces of up to 16 bytes are one dense store instruction already; longer
+// ones go through StoreRowPiecesNT (blocks of 4 waves; the staging area is this function's own).
+template<class T, int N>
+__device__ __forceinline__ void StoreRowRunNT(uint8_t *row0, const T (&v)[N], int lane, int lanes)
+{
+    constexpr int RB = N * (int)sizeof(T);
+    if constexpr (RB > 16 && RB % 8 == 0)
+    {
+        __shared__ __attribute__((aligned(16))) uint8_t stage[4][64 * RB];
+        uint8_t                                         piece[RB];
+        __builtin_memcpy(piece, v, RB);
+        StoreRowPiecesNT<RB>(stage[threadIdx.x >> 6], row0, piece, lane, lanes);
+    }
+    else
+    {
+        StoreRunNT<T, N>(row0 + (int64_t)lane * RB, v);
+    }
+}
+
 } // namespace cvamd
 
 #endif // CVCUDA_AMD_RUNIO_HPP
