@@ -129,10 +129,21 @@ __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow
         TI in[P * C];
         TO out[P * C];
         LoadRun<TI, P * C>(srcRow + (int64_t)x0 * C * sizeof(TI), in);
-#pragma unroll
-        for (int i = 0; i < P * C; ++i)
+        if (a.gscale == 1.f && a.shift == 0.f) // wave-uniform; x * 1 + 0 == x, two operations per element saved
         {
-            out[i] = SaturateCast<TO>(((float)in[i] - b[i % C]) * m[i % C] * a.gscale + a.shift);
+#pragma unroll
+            for (int i = 0; i < P * C; ++i)
+            {
+                out[i] = SaturateCast<TO>(((float)in[i] - b[i % C]) * m[i % C]);
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int i = 0; i < P * C; ++i)
+            {
+                out[i] = SaturateCast<TO>(((float)in[i] - b[i % C]) * m[i % C] * a.gscale + a.shift);
+            }
         }
         // the wave's lanes 0 .. lanes-1 hold consecutive pieces of the row
         const int lane = threadIdx.x & 63, lanes = min(64, (W - (x0 - lane * P)) / P);
