@@ -172,21 +172,30 @@ __global__ __launch_bounds__(256) void PixelMapTensor(const CopyArgs a)
 }
 
 template<class T, int C>
+constexpr int kFlipVarRows = kVarShapeRows<kRunPixelsFor<T, T> * C * (int)sizeof(T)>;
+
+template<class T, int C>
 __global__ __launch_bounds__(256) void FlipVarShape(const CopyArgs a, const VarTiles tiles)
 {
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
-    if (y >= d.height)
-    {
-        return;
-    }
     const int  code    = *reinterpret_cast<const int32_t *>(a.codes + tc.image * a.codeStride);
     const bool mirrorX = code == 1 || code == -1, mirrorY = code == 0 || code == -1;
-    const int  sy      = mirrorY ? d.height - 1 - y : y;
-    CopyRuns<T, C>(AsGlobal(s.basePtr) + (int64_t)sy * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width,
-                   mirrorX ? d.width - 1 : 0, mirrorX ? -1 : 1, tc.tx * 64);
+    const uint8_t *src = AsGlobal(s.basePtr);
+    uint8_t       *dst = AsGlobal(d.basePtr);
+    const int      W = d.width, H = d.height, srcRow = s.rowStride, dstRow = d.rowStride;
+    constexpr int  R = kFlipVarRows<T, C>;
+    for (int r = 0; r < R; ++r)
+    {
+        const int y = (tc.ty * R + r) * kRunTileH + (threadIdx.x >> 6);
+        if (y >= H)
+        {
+            return;
+        }
+        const int sy = mirrorY ? H - 1 - y : y;
+        CopyRuns<T, C>(src + (int64_t)sy * srcRow, dst + (int64_t)y * dstRow, W, mirrorX ? W - 1 : 0, mirrorX ? -1 : 1, tc.tx * 64);
+    }
 }
 
 void LaunchRowCopy(const CopyArgs &a, int N, hipStream_t stream)
@@ -214,7 +223,7 @@ void LaunchPixelMap(const CopyArgs &a, int N, const NVCVImageBufferStrided *dstH
     {
         VarTiles tiles;
         int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), 64 * kRunPixelsFor<T, T>,
-                                  kRunTileH);
+                                  kRunTileH * kFlipVarRows<T, C>);
         if (total > 0)
         {
             hipLaunchKernelGGL((FlipVarShape<T, C>), dim3(total), dim3(256), 0, stream, a, tiles);

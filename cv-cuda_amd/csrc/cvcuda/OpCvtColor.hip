@@ -379,6 +379,9 @@ __global__ __launch_bounds__(256) void SwizzleTensor(const SwizzleArgs a)
                             a.dstBase + n * a.dstSampleStride + (int64_t)y * a.dstRowStride, a.W, x0, a.bidx, a.alpha);
 }
 
+template<class T, int DCH>
+constexpr int kSwizzleVarRows = kVarShapeRows<kRunPixelsFor<T, T> * DCH * (int)sizeof(T)>;
+
 template<class T, int SCH, int DCH>
 __global__ __launch_bounds__(256) void SwizzleVarShape(const SwizzleArgs a, const VarTiles tiles)
 {
@@ -386,13 +389,23 @@ __global__ __launch_bounds__(256) void SwizzleVarShape(const SwizzleArgs a, cons
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
     const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixelsFor<T, T>;
-    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
-    if (x0 >= d.width || y >= d.height)
+    const uint8_t *src = AsGlobal(s.basePtr);
+    uint8_t       *dst = AsGlobal(d.basePtr);
+    const int      W = d.width, H = d.height, srcRow = s.rowStride, dstRow = d.rowStride;
+    if (x0 >= W)
     {
         return;
     }
-    SwizzleRun<T, SCH, DCH>(AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0,
-                            a.bidx, a.alpha);
+    constexpr int R = kSwizzleVarRows<T, DCH>;
+    for (int r = 0; r < R; ++r)
+    {
+        const int y = (tc.ty * R + r) * kRunTileH + (threadIdx.x >> 6);
+        if (y >= H)
+        {
+            return;
+        }
+        SwizzleRun<T, SCH, DCH>(src + (int64_t)y * srcRow, dst + (int64_t)y * dstRow, W, x0, a.bidx, a.alpha);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -498,7 +511,7 @@ void LaunchSwizzle(const SwizzleArgs &a, int N, const NVCVImageBufferStrided *ds
     {
         VarTiles tiles;
         int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), 64 * kRunPixelsFor<T, T>,
-                                  kRunTileH);
+                                  kRunTileH * kSwizzleVarRows<T, DCH>);
         if (total > 0)
         {
             hipLaunchKernelGGL((SwizzleVarShape<T, SCH, DCH>), dim3(total), dim3(256), 0, stream, a, tiles);

@@ -601,6 +601,17 @@ __global__ __launch_bounds__(256) void MapTensor(const PixArgs a)
     MapRun<Op>(a.src + n * a.srcN + (int64_t)y * a.srcRow, a.dst + n * a.dstN + (int64_t)y * a.dstRow, a.W, x0, a);
 }
 
+template<class Op>
+constexpr int MapPieceBytes()
+{
+    using S = typename Op::Src;
+    using D = decltype(Op::Map(S{}, PixArgs{}));
+    return kMapRun<Op> * (int)sizeof(D);
+}
+
+template<class Op>
+constexpr int kMapVarRows = kVarShapeRows<MapPieceBytes<Op>()>;
+
 // var-shape: the size comes from the destination image
 template<class Op>
 __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTiles tiles)
@@ -609,12 +620,23 @@ __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTil
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
     const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kMapRun<Op>;
-    const int                    y  = tc.ty * kRunTileH + (threadIdx.x >> 6);
-    if (x0 >= d.width || y >= d.height)
+    const uint8_t *src = AsGlobal(s.basePtr);
+    uint8_t       *dst = AsGlobal(d.basePtr);
+    const int      W = d.width, H = d.height, srcRow = s.rowStride, dstRow = d.rowStride;
+    if (x0 >= W)
     {
         return;
     }
-    MapRun<Op>(AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, d.width, x0, a);
+    constexpr int R = kMapVarRows<Op>;
+    for (int r = 0; r < R; ++r)
+    {
+        const int y = (tc.ty * R + r) * kRunTileH + (threadIdx.x >> 6);
+        if (y >= H)
+        {
+            return;
+        }
+        MapRun<Op>(src + (int64_t)y * srcRow, dst + (int64_t)y * dstRow, W, x0, a);
+    }
 }
 
 // Subsampled formats: Op::kGroup work items (each Op::kItemW x Op::kItemH pixels) side by side per lane,
@@ -701,7 +723,7 @@ void Launch(const ColorIO &io, PixArgs a, hipStream_t stream)
         {
             VarTiles tiles;
             int      total = BuildVarTiles(tiles, io.dstHost, first, std::min(kMaxTileImages, io.N - first),
-                                           64 * kMapRun<Op>, kRunTileH);
+                                           64 * kMapRun<Op>, kRunTileH * kMapVarRows<Op>);
             if (total > 0)
             {
                 hipLaunchKernelGGL((MapVarShape<Op>), dim3(total), dim3(256), 0, stream, a, tiles);

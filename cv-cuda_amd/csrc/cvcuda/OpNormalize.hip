@@ -177,12 +177,8 @@ __global__ __launch_bounds__(256) void NormRunsTensor(const NormArgs a)
                        x0);
 }
 
-// Rows a wave of the image-batch kernel works through: the tile search and the descriptor loads are a
-// dependent chain of memory round trips before the first pixel load, a quarter of a one-row wave's life
-// (32 x 1080p u8x3: 94 -> 71 us with 4 rows). Outputs that go through the row-regrouped stores keep 1
-// (u8x3 -> f32x3: 171 us with 1 row, 190 us with 4).
 template<class TI, class TO, int C>
-constexpr int kVarRows = (kRunPixelsFor<TI, TO> * C * (int)sizeof(TO) > 16) ? 1 : 4;
+constexpr int kVarRows = kVarShapeRows<kRunPixelsFor<TI, TO> * C * (int)sizeof(TO)>;
 
 template<class TI, class TO, int C>
 __global__ __launch_bounds__(256) void NormRunsVarShape(const NormArgs a, const VarTiles tiles)

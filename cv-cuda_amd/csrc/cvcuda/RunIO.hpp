@@ -109,6 +109,13 @@ __device__ __forceinline__ void StoreRowRunNT(uint8_t *row0, const T (&v)[N], in
     }
 }
 
+// Rows a wave of an image-batch run kernel works through. The tile search and the descriptor loads are a
+// dependent chain of memory round trips before the first pixel load, a quarter of a one-row wave's life
+// (Normalize, 32 x 1080p u8x3: 94 -> 71 us with 4 rows). Outputs that go through the row-regrouped stores
+// keep 1 (Normalize u8x3 -> f32x3: 171 us with 1 row, 190 us with 4).
+template<int PIECE_BYTES>
+constexpr int kVarShapeRows = PIECE_BYTES > 16 ? 1 : 4;
+
 } // namespace cvamd
 
 #endif // CVCUDA_AMD_RUNIO_HPP
