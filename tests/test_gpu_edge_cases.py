@@ -286,3 +286,31 @@ def test_concurrent_submits_on_shared_operator_handles(cv, K, orc, gpu):
         t.join()
     torch.cuda.synchronize()
     assert not failures, failures
+
+
+def test_row_pieces_longer_than_one_store_with_odd_lane_counts(cv, K, orc, gpu):
+    # 2-byte pixels give 24- or 32-byte pieces per lane, which the run kernels hand round the wave as
+    # 16-byte chunks; an odd number of 24-byte pieces ends with half a chunk. Widths chosen so that the
+    # number of whole runs per row is 1, 3, 5, 63, 64, 65 (plus a ragged end).
+    rng = np.random.default_rng(24)
+    for w in (4, 6, 13, 22, 254, 256, 259, 262):
+        for c in (3, 4):
+            a = rng.integers(0, 65536, (2, 5, w, c)).astype(np.uint16)
+            tin = cv.Tensor.from_numpy(a, "NHWC")
+            out = cv.Tensor.alloc([2, 5, w, c], np.uint16, "NHWC")
+            for code, ref in ((1, a[:, :, ::-1]), (0, a[:, ::-1]), (-1, a[:, ::-1, ::-1])):
+                out.torch_view().zero_()
+                cv.Flip()(None, tin, out, code)
+                torch.cuda.synchronize()
+                np.testing.assert_array_equal(out.numpy(), ref, err_msg="flip %d w=%d c=%d" % (code, w, c))
+            swapped = cv.Tensor.alloc([2, 5, w, c], np.uint16, "NHWC")
+            cv.CvtColor()(None, tin, swapped, K.COLOR_BGR2RGB if c == 3 else K.COLOR_BGRA2RGBA)
+            torch.cuda.synchronize()
+            want = a.copy()
+            want[..., :3] = a[..., 2::-1]
+            np.testing.assert_array_equal(swapped.numpy(), want, err_msg="swizzle w=%d c=%d" % (w, c))
+        a8 = orc.fill_u8((2, 5, w, 3), 90 + w)
+        f = cv.Tensor.alloc([2, 5, w, 3], np.float64, "NHWC")
+        cv.ConvertTo()(None, cv.Tensor.from_numpy(a8, "NHWC"), f, 0.5, 1.0)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(f.numpy(), a8.astype(np.float64) * 0.5 + 1.0)
