@@ -94,17 +94,34 @@ def polygon_clip_area(poly, w, h):
 # (per step), make_set() -> buffer set, submit(stream, set), check(set) (oracle spot check of what
 # the GPU produced), cpu(threads) -> images the oracle processed.
 class Fused:
-    key, config_id = "fused", 2
+    """Configuration 2 in four forms (`form`):
+    fused            one cvcudaResizeCropConvertReformatSubmit, normalisation as one scale/offset pair
+    fused-normalize  one cvcudaxResizeCropConvertReformatNormalizeSubmit (extension): per-channel mean/std
+    fused-chain      what the reference needs for per-channel mean/std: fused (x 1/255, f32 NHWC) ->
+                     Normalize (scale is stddev) -> Reformat (NCHW), three Submits per step
+    fused-copy-bound not an operator: a kernel with the fused kernel's grid, tap loads and stores but no
+                     arithmetic (libcvamd_bench.so), i.e. what the memory system allows this access pattern
+    """
+    config_id = 2
     N, SRC_H, SRC_W = 64, 1080, 1920
     NEW_W, NEW_H, CROP_X, CROP_Y, OUT_H, OUT_W = 455, 256, 115, 16, 224, 224
     SCALE, OFFSET = 1.0 / (255.0 * 0.226), -0.449 / 0.226
-    kernel = "FusedBilinear<float,false,false,false>"
+    MEAN, STD = (0.485, 0.456, 0.406), (0.229, 0.224, 0.225)
     dtype = "f32"
-    workload = ("fused ResizeCropConvertReformat: batch 64 u8 NHWC 1920x1080 -> bilinear 455x256 -> "
-                "crop 224x224 @(115,16) -> f32 NCHW, scale/offset")
+    KERNELS = {"fused": "FusedBilinear<float,false,false,false>",
+               "fused-normalize": "FusedBilinear<float,false,false,true>",
+               "fused-chain": "FusedBilinear<float,false,false,false> + NormRunsTensor<float,float,3> + "
+                              "ReformatRunsKernel<float,3,true,false>",
+               "fused-copy-bound": "FusedCopyBound"}
+    TEXT = {"fused": "scale/offset", "fused-normalize": "per-channel mean/std in the same kernel (extension entry point)",
+            "fused-chain": "per-channel mean/std as the three-operator chain fused -> Normalize -> Reformat",
+            "fused-copy-bound": "copy-bound twin of the fused kernel (same grid, loads and stores, no arithmetic)"}
 
-    def __init__(self, cv, orc, np, torch):
-        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+    def __init__(self, cv, orc, np, torch, form="fused"):
+        self.cv, self.orc, self.np, self.torch, self.form = cv, orc, np, torch, form
+        self.key, self.kernel = form, self.KERNELS[form]
+        self.workload = ("fused ResizeCropConvertReformat: batch 64 u8 NHWC 1920x1080 -> bilinear 455x256 -> "
+                         "crop 224x224 @(115,16) -> f32 NCHW, " + self.TEXT[form])
         self.images = self.N
         rows, _ = span_bytes(self.OUT_H, self.CROP_Y, self.SRC_H, self.NEW_H, LINEAR, 1)
         _, span = span_bytes(self.OUT_W, self.CROP_X, self.SRC_W, self.NEW_W, LINEAR, 3)
@@ -112,24 +129,69 @@ class Fused:
         self.host = orc.fill_u8((self.N, self.SRC_H, self.SRC_W, 3), SEED_BASE + self.config_id)
         self.dev = torch.from_numpy(self.host).cuda()
         self.op = cv.ResizeCropConvertReformat()
+        if form == "fused-chain":
+            self.norm, self.reformat = cv.Normalize(), cv.Reformat()
+            self.tmean = cv.Tensor.from_numpy(np.asarray(self.MEAN, np.float32).reshape(1, 1, 1, 3), "NHWC")
+            self.tstd = cv.Tensor.from_numpy(np.asarray(self.STD, np.float32).reshape(1, 1, 1, 3), "NHWC")
+        if form == "fused-copy-bound":
+            import ctypes as C
+            lib = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(cv.__file__)), "lib", "libcvamd_bench.so"))
+            self.copy_fn = lib.cvamdBenchFusedCopyBound
+            self.copy_fn.restype = C.c_int
+            self.copy_fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64] + [C.c_int32] * 3 + [C.c_void_p] + [C.c_int32] * 7
 
     def make_set(self):
-        tin = self.cv.Tensor.alloc([self.N, self.SRC_H, self.SRC_W, 3], self.np.uint8, "NHWC")
+        cv, np = self.cv, self.np
+        tin = cv.Tensor.alloc([self.N, self.SRC_H, self.SRC_W, 3], np.uint8, "NHWC")
         tin.torch_view().copy_(self.dev)
-        return tin, self.cv.Tensor.alloc([self.N, 3, self.OUT_H, self.OUT_W], self.np.float32, "NCHW")
+        out = cv.Tensor.alloc([self.N, 3, self.OUT_H, self.OUT_W], np.float32, "NCHW")
+        if self.form == "fused-chain":
+            return (tin, out, cv.Tensor.alloc([self.N, self.OUT_H, self.OUT_W, 3], np.float32, "NHWC"),
+                    cv.Tensor.alloc([self.N, self.OUT_H, self.OUT_W, 3], np.float32, "NHWC"))
+        return tin, out
 
     def submit(self, stream, s):
-        self.op(stream, s[0], s[1], (self.NEW_W, self.NEW_H), LINEAR, (self.CROP_X, self.CROP_Y), 0, self.SCALE,
-                self.OFFSET, False)
+        geom = ((self.NEW_W, self.NEW_H), LINEAR, (self.CROP_X, self.CROP_Y))
+        if self.form == "fused":
+            self.op(stream, s[0], s[1], *geom, 0, self.SCALE, self.OFFSET, False)
+        elif self.form == "fused-normalize":
+            self.op.normalized(stream, s[0], s[1], *geom, self.MEAN, self.STD, 0, 1 / 255.0, 0.0, False, 1.0, 0.0, 0.0,
+                               self.cv.K.CVCUDA_NORMALIZE_SCALE_IS_STDDEV)
+        elif self.form == "fused-chain":
+            self.op(stream, s[0], s[2], *geom, 0, 1 / 255.0, 0.0, False)
+            self.norm(stream, s[2], self.tmean, self.tstd, s[3], 1.0, 0.0, 0.0, self.cv.K.CVCUDA_NORMALIZE_SCALE_IS_STDDEV)
+            self.reformat(stream, s[3], s[1])
+        else:
+            tv = s[0].torch_view()
+            rc = self.copy_fn(self.cv.stream_ptr(stream), tv.data_ptr(), tv.stride(0), tv.stride(1), self.SRC_W,
+                              self.SRC_H, s[1].torch_view().data_ptr(), self.N, self.OUT_W, self.OUT_H, self.NEW_W,
+                              self.NEW_H, self.CROP_X, self.CROP_Y)
+            assert rc == 0, "cvamdBenchFusedCopyBound failed: hipError %d" % rc
 
     def _oracle(self, src, threads=1):
-        return self.orc.fused_rccr(src, (self.OUT_H, self.OUT_W), (self.NEW_W, self.NEW_H), (self.CROP_X, self.CROP_Y),
-                                   LINEAR, self.np.float32, True, 0, self.SCALE, self.OFFSET, False, threads=threads)
+        np, orc = self.np, self.orc
+        size, geom = (self.OUT_H, self.OUT_W), ((self.NEW_W, self.NEW_H), (self.CROP_X, self.CROP_Y), LINEAR)
+        if self.form in ("fused", "fused-copy-bound"):
+            return orc.fused_rccr(src, size, *geom, np.float32, True, 0, self.SCALE, self.OFFSET, False, threads=threads)
+        x = orc.fused_rccr(src, size, *geom, np.float32, False, 0, 1 / 255.0, 0.0, False, threads=threads)
+        mean = np.asarray(self.MEAN, np.float32).reshape(1, 1, 1, 3)
+        std = np.asarray(self.STD, np.float32).reshape(1, 1, 1, 3)
+        return np.ascontiguousarray(orc.normalize(x, mean, std, 1.0, 0.0, 0.0, True, threads=threads).transpose(0, 3, 1, 2))
 
     def check(self, s):
         np = self.np
-        ref = self._oracle(self.host[:2])
         got = s[1].torch_view()[:2].cpu().numpy()
+        if self.form == "fused-copy-bound":
+            # plane 0 holds the 3 bytes of the upper row's first tap: the same place the operator reads
+            f32 = np.float32
+            dx, dy = np.arange(self.OUT_W, dtype=f32), np.arange(self.OUT_H, dtype=f32)
+            sx = np.maximum(np.floor((dx + f32(self.CROP_X) + f32(0.5)) * (f32(self.SRC_W) / f32(self.NEW_W)) - f32(0.5)), 0)
+            sy = np.maximum(np.floor((dy + f32(self.CROP_Y) + f32(0.5)) * (f32(self.SRC_H) / f32(self.NEW_H)) - f32(0.5)), 0)
+            px = self.host[:2][:, sy.astype(int)][:, :, sx.astype(int)].astype(np.uint32)
+            want = px[..., 0] | (px[..., 1] << 8) | (px[..., 2] << 16)
+            assert (got[:, 0].view(np.uint32) == want).all(), "copy-bound kernel read other pixels than the operator"
+            return
+        ref = self._oracle(self.host[:2])
         assert (np.abs(got - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all(), "bench output differs from oracle"
 
     def cpu(self, threads):
@@ -411,6 +473,9 @@ class Streaming:
 
 WORKLOADS = {
     "fused": Fused,
+    "fused-normalize": lambda *a: Fused(*a, "fused-normalize"),
+    "fused-chain": lambda *a: Fused(*a, "fused-chain"),
+    "fused-copy-bound": lambda *a: Fused(*a, "fused-copy-bound"),
     "resize-nearest": lambda *a: ResizeC1(*a, NEAREST),
     "resize-linear": lambda *a: ResizeC1(*a, LINEAR),
     "nv12-to-rgb": Nv12C3,
@@ -429,6 +494,8 @@ def main():
     ap.add_argument("--rotate", type=int, default=0,
                     help="distinct buffer sets cycled through (0 = at least 3 and enough for 1.5 GB of algorithmic bytes, 1 = cache-resident)")
     ap.add_argument("--no-graph", action="store_true", help="time eager Submits instead of a HIP-graph replay")
+    ap.add_argument("--min-seconds", type=float, default=0.3,
+                    help="the K steps are repeated until the timed region holds at least this much device work")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget of the CPU-oracle leg (0 = skip)")
     ap.add_argument("--streams", type=int, default=1,
                     help="independent streams the K steps are dealt to inside the captured graph (default 1: every "
@@ -490,21 +557,37 @@ def main():
             sys.stderr.write("bench.py: graph capture failed (%s), timing eager submits\n" % e)
             graph = None
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def run_steps():
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(args.steps):
+                wl.submit(stream, sets[i % nsets])
+
+    # One untimed pass sizes the timed region: the K steps are repeated `replays` times so that the timed
+    # region holds at least --min-seconds of device work whatever K is. With a few dozen steps of a ~20 us
+    # kernel the clocks would otherwise mostly see the host's launch and synchronisation latency, and the
+    # device would still be ramping its memory clocks up.
     torch.cuda.synchronize()
+    e0.record(stream)
+    run_steps()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    est_s = max(e0.elapsed_time(e1) * 1e-3, 1e-6)
+    replays = max(1, min(100000, math.ceil(args.min_seconds / est_s)))
     t0 = time.perf_counter()
     e0.record(stream)
-    if graph is not None:
-        graph.replay()
-    else:
-        for i in range(args.steps):
-            wl.submit(stream, sets[i % nsets])
+    for _ in range(replays):
+        run_steps()
     e1.record(stream)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     wall = t1 - t0
-    # mean launch-to-launch duration of the kernel over the timed region (includes the gap between
+    timed_steps = args.steps * replays
+    # mean launch-to-launch duration of a step on the device over the timed region (includes the gap between
     # dependent launches, so it is an upper bound of the pure kernel time)
-    mean_kernel_ms = e0.elapsed_time(e1) / args.steps
+    mean_kernel_ms = e0.elapsed_time(e1) / timed_steps
 
     if args.copy_probe > 0:
         a = torch.full((args.copy_probe << 20,), 7, dtype=torch.uint8, device="cuda")
@@ -523,26 +606,34 @@ def main():
     # ---- CPU oracle on the same workload (bounded sample)
     cpu = None
     if args.cpu_seconds > 0:
+        def cpu_leg(threads, budget):
+            reps, done, tcpu = 0, 0, 0.0
+            c0 = time.perf_counter()
+            while reps < 2 or tcpu < budget:
+                done += wl.cpu(threads)
+                reps += 1
+                tcpu = time.perf_counter() - c0
+            return done, tcpu
+
         threads = min(os.cpu_count() or 1, 16)
-        reps, done, tcpu = 0, 0, 0.0
-        c0 = time.perf_counter()
-        while reps < 2 or tcpu < args.cpu_seconds:
-            done += wl.cpu(threads)
-            reps += 1
-            tcpu = time.perf_counter() - c0
+        done, tcpu = cpu_leg(threads, args.cpu_seconds)
         used = wl.cpu_cores(threads) if hasattr(wl, "cpu_cores") else threads
+        done1, tcpu1 = cpu_leg(1, args.cpu_seconds / 2)
         cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": used, "kind": "port",
                "sample": "%d images of this workload through the CPU oracle in %.1f s, %d thread%s"
-                         % (done, tcpu, used, "" if used == 1 else "s")}
+                         % (done, tcpu, used, "" if used == 1 else "s"),
+               "single_thread": {"value": round(done1 / tcpu1, 1), "unit": "images/s", "cores": 1,
+                                 "sample": "%d images in %.1f s, 1 thread" % (done1, tcpu1)}}
 
     out = {
         "metric": "images/sec and achieved HBM GB/s (% of roofline), 1 MI355X",
-        "value": round(wl.images * args.steps / wall, 1),
+        "value": round(wl.images * timed_steps / wall, 1),
         "unit": "images/s",
         "n_gpus": 1,
         "steps": args.steps,
+        "replays": replays,
         "warmup": args.warmup,
-        "ms_per_step": round(wall / args.steps * 1e3, 5),
+        "ms_per_step": round(wall / timed_steps * 1e3, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -2,6 +2,8 @@
 
   lib/libnvcv_types.so  -- NVCV core objects (host C++ on the HIP runtime)
   lib/libcvcuda.so      -- operators: host validation/dispatch + HIP kernels
+  lib/libcvamd_bench.so -- kernels the benchmark times beside the operators (a copy-bound twin of the
+                           fused kernel); nothing in the two libraries above uses it
 
 Usage: python cv-cuda_amd/build.py [--force] [-j N]
 Objects are cached under build/ next to this file and rebuilt when a source or header is newer.
@@ -67,9 +69,10 @@ def build(force=False, jobs=8, verbose=True):
     newest_header = max(os.path.getmtime(h) for h in _headers())
     core = [(s, []) for s in _sources("nvcv", (".cpp",))]
     ops = [(s, DEVICE if s.endswith(".hip") else []) for s in _sources("cvcuda", (".cpp", ".hip"))]
+    bench = [(s, DEVICE) for s in _sources("bench", (".hip",))]
     tasks = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        for group, items in (("nvcv", core), ("cvcuda", ops)):
+        for group, items in (("nvcv", core), ("cvcuda", ops), ("bench", bench)):
             for src, extra in items:
                 obj = os.path.join(OBJDIR, group + "_" + os.path.basename(src) + ".o")
                 tasks.append((group, obj, ex.submit(_compile, src, obj, extra, force, newest_header)))
@@ -89,7 +92,9 @@ def build(force=False, jobs=8, verbose=True):
     subprocess.run(link + ops_objs + ["-o", cvcuda_so, "-Wl,-soname,libcvcuda.so", "-L" + LIBDIR, "-lnvcv_types",
                                       "-Wl,-rpath,$ORIGIN",
                                       "-Wl,--version-script=" + os.path.join(maps, "cvcuda.map")], check=True)
-    return nvcv_so, cvcuda_so
+    bench_so = os.path.join(LIBDIR, "libcvamd_bench.so")
+    subprocess.run(link + [o for g, o, _ in tasks if g == "bench"] + ["-o", bench_so], check=True)
+    return nvcv_so, cvcuda_so, bench_so
 
 
 if __name__ == "__main__":

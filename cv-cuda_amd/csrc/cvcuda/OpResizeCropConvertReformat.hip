@@ -5,116 +5,26 @@
 // follow its operator() (:418-683).
 //
 // Kernel shape (gfx950, wave64): one lane per output column, each wave produces kRowsPerWave output
-// rows, a 256-thread block covers 64 columns x 4*kRowsPerWave rows. The x-dependent terms (source column, weight)
+// rows (one: see FusedTiles.hpp), a 256-thread block covers 64 columns x 4*kRowsPerWave rows. The x-dependent terms (source column, weight)
 // are computed once per lane and reused for all its rows. Source taps are two adjacent u8x3 pixels,
 // i.e. 6 contiguous bytes, fetched with ONE unaligned 8-byte load per source row; consecutive lanes
 // read addresses ~3*scale bytes apart, so a wave touches a dense run of cache lines and the HBM
 // traffic equals the row span the output needs. Output stores are one element per lane per plane
 // (planar: 256 contiguous bytes per wave).
 #include "DeviceUtils.hpp"
+#include "FusedTiles.hpp"
 #include "LaneExchange.hpp"
 #include "OpCommon.hpp"
 
 #include <cvcuda/OpNormalize.h>
 #include <cvcuda/OpResizeCropConvertReformat.h>
 
+#include <algorithm>
 #include <cmath>
 
 namespace cvamd {
 
 namespace {
-
-constexpr int kRowsPerWave  = 2;
-constexpr int kWavesPerBlk  = 4;
-constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlk;
-
-struct FusedArgs
-{
-    // source: tensor (base + n*sampleStride) or var-shape descriptor list
-    const uint8_t                *srcBase;
-    int64_t                       srcSampleStride;
-    int32_t                       srcRowStride;
-    int32_t                       srcW, srcH;
-    const NVCVImageBufferStrided *srcList;
-    // destination, strides in elements
-    void   *dstBase;
-    int64_t dstStrideN;
-    int32_t dstStrideY, dstStrideX;
-    int64_t dstOffC[3]; // element offset of source channel c in the destination (mapping applied)
-    int32_t interleaved; // 0: any strides; 1 / 2: pixels are 3 adjacent elements in source / reversed channel order
-    int32_t dstW, dstH;
-    // geometry
-    int32_t newW, newH;
-    int32_t cropX, cropY;
-    float   scaleX, scaleY; // tensor path: srcW/newW, srcH/newH
-    float   scale, offset;
-    int32_t srcCast;
-    // launch shape: column tiles and row tiles per image; the grid is 1-D
-    uint32_t tilesX, tilesY;
-    uint32_t rowTiles; // tilesY * N
-    // per-channel normalisation of the extension entry points, indexed by source channel:
-    // ((scale*v + offset) - normBase) * normMul * normGlobal + normShift
-    float normBase[3], normMul[3];
-    float normGlobal, normShift;
-};
-
-struct TilePos
-{
-    int n, tx, ty;
-};
-
-// Hardware workgroup id -> (image, row tile, column tile).
-// The column tiles of one row tile read overlapping cache lines (a 128-byte line straddles each
-// tile boundary). MI355X deals workgroups to its 8 XCDs round-robin and each XCD has its own L2, so
-// with the natural order both neighbours would fetch the shared line from memory. Here the column
-// tiles of a row tile go to ONE XCD on consecutive turns (the second hits in L2), while consecutive
-// row tiles still go to consecutive XCDs, so that all XCDs stream through the same region of the
-// batch at the same time. The launch is padded to a multiple of 8 row tiles; padding workgroups
-// get an out-of-range column and leave at once.
-__device__ __forceinline__ TilePos LocateFusedTile(const FusedArgs &a)
-{
-    const uint32_t xcd = blockIdx.x % kXcdCount, turn = blockIdx.x / kXcdCount;
-    const uint32_t inRow   = turn % a.tilesX;
-    const uint32_t rowTile = (turn / a.tilesX) * kXcdCount + xcd; // over all images
-    TilePos        p;
-    p.n  = (int)(rowTile / a.tilesY);
-    p.ty = (int)(rowTile - (uint32_t)p.n * a.tilesY);
-    p.tx = rowTile < a.rowTiles ? (int)inRow : (1 << 24);
-    return p;
-}
-
-struct SrcImage
-{
-    const uint8_t *base;
-    int32_t        rowStride, w, h;
-    float          scaleX, scaleY;
-};
-
-template<bool VARSHAPE>
-__device__ __forceinline__ SrcImage GetSource(const FusedArgs &a, int n)
-{
-    SrcImage s;
-    if constexpr (VARSHAPE)
-    {
-        const NVCVImagePlaneStrided &pl = a.srcList[n].planes[0];
-        s.base                          = AsGlobal(pl.basePtr);
-        s.rowStride                     = pl.rowStride;
-        s.w                             = pl.width;
-        s.h                             = pl.height;
-        s.scaleX                        = static_cast<float>(s.w) / a.newW;
-        s.scaleY                        = static_cast<float>(s.h) / a.newH;
-    }
-    else
-    {
-        s.base      = a.srcBase + n * a.srcSampleStride;
-        s.rowStride = a.srcRowStride;
-        s.w         = a.srcW;
-        s.h         = a.srcH;
-        s.scaleX    = a.scaleX;
-        s.scaleY    = a.scaleY;
-    }
-    return s;
-}
 
 template<class DstT, bool NORM>
 __device__ __forceinline__ DstT Finish(const FusedArgs &a, float v, int c)
@@ -138,16 +48,16 @@ __device__ __forceinline__ DstT Finish(const FusedArgs &a, float v, int c)
 // three separate element stores per lane complete every 32-byte sector in three instructions, which
 // costs write traffic (f32 NHWC: 29.7 -> 24 us per batch). f32 pixels are one 12-byte store; u8 pixels
 // are packed into dwords across the wave through LDS first.
-template<class DstT, bool NORM>
+template<class DstT, bool NORM, bool PLANAR = false>
 __device__ __forceinline__ void StorePixel(const FusedArgs &a, DstT *rowOut, int dx, float v0, float v1, float v2)
 {
     const DstT f0 = Finish<DstT, NORM>(a, v0, 0), f1 = Finish<DstT, NORM>(a, v1, 1), f2 = Finish<DstT, NORM>(a, v2, 2);
-    if (a.interleaved == 0)
+    if (PLANAR || a.interleaved == 0)
     {
         DstT *out = rowOut + dx * a.dstStrideX;
-        __builtin_nontemporal_store(f0, out + a.dstOffC[0]);
-        __builtin_nontemporal_store(f1, out + a.dstOffC[1]);
-        __builtin_nontemporal_store(f2, out + a.dstOffC[2]);
+        StoreStreamThrough(f0, out + a.dstOffC[0]);
+        StoreStreamThrough(f1, out + a.dstOffC[1]);
+        StoreStreamThrough(f2, out + a.dstOffC[2]);
         return;
     }
     const bool rev   = a.interleaved == 2;
@@ -218,12 +128,11 @@ __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
     }
 }
 
-// BYTEWISE=false: each source row is fetched with one unaligned 8-byte load per lane (the two taps
-// are 6 contiguous bytes). The load may extend up to 5 bytes past the taps; inside the image that
-// is harmless, at the very end of the image buffer the load is moved back so that it ends with the
-// buffer and the value is shifted into place (no divergent branch). Needs an image of >= 8 bytes.
-// BYTEWISE=true: plain byte loads, used for images smaller than 8 bytes.
-template<class DstT, bool VARSHAPE, bool BYTEWISE, bool NORM>
+// BYTEWISE=false: each source row is fetched with one unaligned 8-byte load per lane (LoadTapPairs; needs
+// an image of >= 8 bytes). BYTEWISE=true: plain byte loads, used for images smaller than 8 bytes.
+// PLANAR=true: the caller knows that the output is not pixel-interleaved (a.interleaved == 0), which takes the
+// interleaved store paths and their branch out of the kernel.
+template<class DstT, bool VARSHAPE, bool BYTEWISE, bool NORM, bool PLANAR>
 __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
@@ -238,18 +147,9 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
     const SrcImage s   = GetSource<VARSHAPE>(a, n);
     DstT          *dst = static_cast<DstT *>(a.dstBase) + n * a.dstStrideN;
 
-    // x terms, shared by all rows of this lane
-    float fx  = (dx + a.cropX + 0.5f) * s.scaleX - 0.5f;
-    int   sx0 = (int)floorf(fx);
-    int   sx1 = min(sx0 + 1, s.w - 1);
-    fx -= sx0;
-    sx0               = max(0, sx0);
-    const bool  twoTap = sx1 > sx0; // second tap is the next pixel, otherwise the same pixel
-    const int   xoff   = sx0 * 3;
-    const float wx0    = 1 - fx;
-
-    // last byte offset at which an 8-byte load still ends inside the image
-    const int64_t lastLoad = (int64_t)(s.h - 1) * s.rowStride + (int64_t)s.w * 3 - 8;
+    const FusedColumn col = ColumnTerms(a, s, dx); // shared by all rows of this lane
+    const float       fx = col.fx, wx0 = 1 - col.fx;
+    const int64_t     lastLoad = LastTapLoad(s);
 
 #pragma unroll
     for (int r = 0; r < kRowsPerWave; ++r)
@@ -259,20 +159,14 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
         {
             break;
         }
-        float fy  = (dy + a.cropY + 0.5f) * s.scaleY - 0.5f;
-        int   sy0 = (int)floorf(fy);
-        int   sy1 = min(sy0 + 1, s.h - 1);
-        fy -= sy0;
-        sy0 = max(0, sy0);
-
-        const int64_t off0 = (int64_t)sy0 * s.rowStride + xoff;
-        const int64_t off1 = (int64_t)sy1 * s.rowStride + xoff;
+        const FusedRow row = RowTerms(a, s, dy, col.xoff);
+        const float    fy  = row.fy;
 
         uint32_t a0, a1, b0, b1; // bytes 0..2 of a0/b0: first tap of the upper/lower row; a1/b1: second tap
         if constexpr (BYTEWISE)
         {
-            const int      x1 = twoTap ? 3 : 0;
-            const uint8_t *p0 = s.base + off0, *p1 = s.base + off1;
+            const int      x1 = col.twoTap ? 3 : 0;
+            const uint8_t *p0 = s.base + row.off0, *p1 = s.base + row.off1;
             a0 = p0[0] | (p0[1] << 8) | (p0[2] << 16);
             a1 = p0[x1] | (p0[x1 + 1] << 8) | (p0[x1 + 2] << 16);
             b0 = p1[0] | (p1[1] << 8) | (p1[2] << 16);
@@ -280,14 +174,7 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
         }
         else
         {
-            const int      back0 = (int)max((int64_t)0, off0 - lastLoad);
-            const int      back1 = (int)max((int64_t)0, off1 - lastLoad);
-            const uint64_t q0    = LoadU64Unaligned(s.base + off0 - back0) >> (8 * back0);
-            const uint64_t q1    = LoadU64Unaligned(s.base + off1 - back1) >> (8 * back1);
-            a0                   = (uint32_t)q0;
-            b0                   = (uint32_t)q1;
-            a1 = twoTap ? __builtin_amdgcn_alignbyte((uint32_t)(q0 >> 32), a0, 3) : a0;
-            b1 = twoTap ? __builtin_amdgcn_alignbyte((uint32_t)(q1 >> 32), b0, 3) : b0;
+            LoadTapPairs(s, row, lastLoad, col.twoTap, a0, a1, b0, b1);
         }
         float v[3];
 #pragma unroll
@@ -304,7 +191,7 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
             }
             v[c] = t;
         }
-        StorePixel<DstT, NORM>(a, dst + (int64_t)dy * a.dstStrideY, dx, v[0], v[1], v[2]);
+        StorePixel<DstT, NORM, PLANAR>(a, dst + (int64_t)dy * a.dstStrideY, dx, v[0], v[1], v[2]);
     }
 }
 
@@ -315,33 +202,36 @@ void LaunchKernels(FusedArgs a, int N, NVCVInterpolationType interp, bool tinyIm
     {
         return;
     }
-    a.tilesX            = DivUp(a.dstW, 64);
-    a.tilesY            = DivUp(a.dstH, kRowsPerBlock);
-    a.rowTiles          = a.tilesY * N;
-    const int64_t total = (int64_t)a.tilesX * DivUp(a.rowTiles, kXcdCount) * kXcdCount;
-    if (total > INT32_MAX)
+    if ((a.dstW + 63) / 64 > (INT32_MAX / (int)kXcdCount) || (a.dstH + kRowsPerBlock - 1) / kRowsPerBlock / (int)kXcdCount >= 65535)
     {
-        throw OpError(NVCV_ERROR_OVERFLOW, "Output of %d images of %d x %d needs too many tiles for one launch", N,
-                      a.dstW, a.dstH);
+        throw OpError(NVCV_ERROR_OVERFLOW, "Output of %d x %d needs too many tiles for one launch", a.dstW, a.dstH);
     }
-    dim3 block(256);
-    dim3 grid((uint32_t)total);
-    if (interp == NVCV_INTERP_NEAREST)
+    const dim3 block(256);
+    for (int first = 0; first < N; first += kFusedImagesPerLaunch)
     {
-        hipLaunchKernelGGL((FusedNearest<DstT, VARSHAPE, NORM>), grid, block, 0, stream, a);
-        CheckLaunch("FusedNearest");
-    }
-    else
-    {
-        if (tinyImages)
+        a.firstImage    = (uint32_t)first;
+        const dim3 grid = SetFusedGrid(a, std::min(N - first, kFusedImagesPerLaunch));
+        if (interp == NVCV_INTERP_NEAREST)
         {
-            hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, true, NORM>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((FusedNearest<DstT, VARSHAPE, NORM>), grid, block, 0, stream, a);
+            CheckLaunch("FusedNearest");
         }
         else
         {
-            hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, false, NORM>), grid, block, 0, stream, a);
+            if (tinyImages)
+            {
+                hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, true, NORM, false>), grid, block, 0, stream, a);
+            }
+            else if (a.interleaved == 0)
+            {
+                hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, false, NORM, true>), grid, block, 0, stream, a);
+            }
+            else
+            {
+                hipLaunchKernelGGL((FusedBilinear<DstT, VARSHAPE, false, NORM, false>), grid, block, 0, stream, a);
+            }
+            CheckLaunch("FusedBilinear");
         }
-        CheckLaunch("FusedBilinear");
     }
 }
 
