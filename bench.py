@@ -367,6 +367,56 @@ class WarpC4:
         return 8
 
 
+class WarpTensor:
+    """WarpAffine on a tensor: 32 u8 RGB images of 1280x780 rotated by 17 degrees about the centre at scale 1.05
+    (forward map), constant border 0. Algorithmic bytes: the part of the source the destination's inverse image
+    covers, plus the output."""
+    config_id = 0
+    N, H, W = 32, 780, 1280
+    dtype = "f32"
+
+    def __init__(self, cv, orc, np, torch, interp):
+        self.cv, self.orc, self.np, self.torch, self.interp = cv, orc, np, torch, interp
+        name = {NEAREST: "NEAREST", LINEAR: "LINEAR", CUBIC: "CUBIC"}[interp]
+        self.key = "warp-affine-tensor-" + name.lower()
+        self.kernel = "WarpTensor<uint8_t,3,%s>" % name
+        self.workload = "WarpAffine %s: batch 32 u8 NHWC 1280x780x3, rotation 17 deg x scale 1.05, constant border 0" % name
+        self.images = self.N
+        w, h = self.W, self.H
+        t, sc = math.radians(17.0), 1.05
+        c, sn, cx, cy = sc * math.cos(t), sc * math.sin(t), (w - 1) / 2.0, (h - 1) / 2.0
+        self.m = [c, -sn, cx - c * cx + sn * cy, sn, c, cy - sn * cx - c * cy]
+        inv = orc.invert_affine(self.m).astype(np.float64)
+        corners = [(inv[0] * x + inv[1] * y + inv[2], inv[3] * x + inv[4] * y + inv[5])
+                   for x, y in ((0, 0), (w, 0), (w, h), (0, h))]
+        self.alg_bytes = self.N * (min(w * h * 3, int(3 * polygon_clip_area(corners, w, h))) + w * h * 3)
+        self.host = orc.fill_u8((1, h, w, 3), SEED_BASE + 55)
+        self.dev = torch.from_numpy(self.host).cuda()
+        self.op = cv.WarpAffine(0)
+
+    def make_set(self):
+        tin = self.cv.Tensor.alloc([self.N, self.H, self.W, 3], self.np.uint8, "NHWC")
+        tin.torch_view().copy_(self.dev.expand(self.N, -1, -1, -1))
+        return tin, self.cv.Tensor.alloc([self.N, self.H, self.W, 3], self.np.uint8, "NHWC")
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], self.m, self.interp, 0, (0, 0, 0, 0))
+
+    def _oracle(self, src, threads=1):
+        return self.orc.warp(src, (self.H, self.W), self.orc.invert_affine(self.m), self.interp, 0, (0, 0, 0, 0),
+                             variant=0, threads=threads)
+
+    def check(self, s):
+        np = self.np
+        got = s[1].torch_view()[:1].cpu().numpy()
+        ref = self._oracle(self.host)
+        assert np.abs(got.astype(np.int16) - ref.astype(np.int16)).max() <= (0 if self.interp == NEAREST else 1)
+
+    def cpu(self, threads):
+        self._oracle(self.host, threads)
+        return 1
+
+
 class Streaming:
     """Operators either side of the five configurations, each on a 1080p batch: algorithmic bytes are
     the input plus the output, the check is the oracle (or the numpy index map) on the first image."""
@@ -480,6 +530,9 @@ WORKLOADS = {
     "resize-linear": lambda *a: ResizeC1(*a, LINEAR),
     "nv12-to-rgb": Nv12C3,
     "warp-affine-varshape": WarpC4,
+    "warp-affine-tensor-nearest": lambda *a: WarpTensor(*a, NEAREST),
+    "warp-affine-tensor-linear": lambda *a: WarpTensor(*a, LINEAR),
+    "warp-affine-tensor-cubic": lambda *a: WarpTensor(*a, CUBIC),
     "resize-cubic-4k": CubicC5,
 }
 WORKLOADS.update({k: (lambda *a, k=k: Streaming(*a, k)) for k in Streaming.SPECS})

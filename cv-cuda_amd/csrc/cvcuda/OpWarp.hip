@@ -381,6 +381,86 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
     }
 }
 
+// True when every tap of the sample at (sx, sy) lies outside the image. For an integer k,
+// floor(v) < k <=> v < k and floor(v) >= k <=> v >= k; NaN coordinates fail every comparison.
+template<int INTERP>
+__device__ __forceinline__ bool TapsOutside(const Img &im, float sx, float sy)
+{
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+        // the tap is floor(v + .5)
+        return (sx + .5f < 0.f) | (sx + .5f >= (float)im.w) | (sy + .5f < 0.f) | (sy + .5f >= (float)im.h);
+    }
+    constexpr float lo = INTERP == NVCV_INTERP_CUBIC ? 1.f : 0.f;
+    constexpr float hi = INTERP == NVCV_INTERP_CUBIC ? 2.f : 1.f;
+    return (sx < -hi) | (sx >= (float)im.w + lo) | (sy < -hi) | (sy >= (float)im.h + lo);
+}
+
+// SampleWithBorder for a sample whose taps all lie outside the image under NVCV_BORDER_CONSTANT: every tap is
+// the border value, the weights and the order of the sum are the general sampler's, nothing is loaded.
+template<class T, int C, int INTERP>
+__device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, float sy, T (&out)[C])
+{
+    float t[C], acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        t[c]   = (float)BorderValueAs<T>(a.bval[c]);
+        acc[c] = 0.f;
+    }
+    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[c] = (T)t[c];
+        }
+        return;
+    }
+    else if constexpr (INTERP == NVCV_INTERP_LINEAR)
+    {
+        const int x1 = FloorToInt(sx), y1 = FloorToInt(sy);
+        const int x2 = x1 + 1, y2 = y1 + 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            const float wx = (i & 1) ? (sx - x1) : (x2 - sx);
+            const float wy = (i >> 1) ? (sy - y1) : (y2 - sy);
+            const float w  = wx * wy;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                acc[c] += t[c] * w;
+            }
+        }
+    }
+    else
+    {
+        const int ix = FloorToInt(sx), iy = FloorToInt(sy);
+        float     wx[4], wy[4];
+        CubicCoeffs(sx - ix, wx);
+        CubicCoeffs(sy - iy, wy);
+#pragma unroll
+        for (int cy = 0; cy < 4; ++cy)
+        {
+#pragma unroll
+            for (int cx = 0; cx < 4; ++cx)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    acc[c] += t[c] * (wx[cx] * wy[cy]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        out[c] = SaturateCast<T>(acc[c]);
+    }
+}
+
 // One 64 x 16 tile of the destination image `dst` (tile coordinates tx, ty), all 256 threads.
 template<class T, int C, int INTERP>
 __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dst, int dstRow,
@@ -453,7 +533,14 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
                 MapCoord<false>(m, dx, dy, bx, by);
             }
             T v[C];
-            SampleWithBorder<T, C, INTERP>(im, a, bx, by, v);
+            if (a.border == NVCV_BORDER_CONSTANT && TapsOutside<INTERP>(im, bx, by))
+            {
+                SampleAllOutside<T, C, INTERP>(a, bx, by, v);
+            }
+            else
+            {
+                SampleWithBorder<T, C, INTERP>(im, a, bx, by, v);
+            }
             uint32_t w[D] = {};
             __builtin_memcpy(w, v, PB);
 #pragma unroll
