@@ -6,8 +6,10 @@
  * which case it is used as the dst->src map directly; the low bits of `flags` hold the interpolation.
  * in/out: [N]HWC tensors (or image batches) of u8/u16/s16/f32 with 1, 3 or 4 channels.
  * The var-shape variant takes one matrix per image from an f32 tensor of shape [N,6] and needs
- * N <= maxVarShapeBatchSize given at creation (else INVALID_ARGUMENT); one operator handle may
- * have at most one var-shape submission in flight per stream ordering (it owns the matrix buffer). */
+ * N <= maxVarShapeBatchSize given at creation (else INVALID_ARGUMENT). The kernel reads each matrix from
+ * that tensor and inverts it itself: the operator owns no device buffer, so var-shape submissions of one
+ * handle may be in flight on several streams at once (the reference serialises them on an operator-owned
+ * matrix buffer); the matrix tensor must stay unchanged until the submitted work has run. */
 #ifndef CVCUDA_WARP_AFFINE_H
 #define CVCUDA_WARP_AFFINE_H
 

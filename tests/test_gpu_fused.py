@@ -155,18 +155,17 @@ def test_varshape(cv, K, orc, gpu):
 
 
 def test_benchmark_config_full_size(cv, orc, gpu):
-    # BASELINE config 2 at full size: batch 64 of 1080p; oracle on 4 threads over a subset of images,
-    # plus a size-independent property on the whole batch: identical images give identical outputs.
+    # BASELINE config 2 at full size: batch 64 of 1080p, every image different (one random image rolled by
+    # 7 * n columns and n rows, so an image index that aliases would show), the oracle on all 64.
     N = 64
-    one = orc.fill_u8((4, 1080, 1920, 3), 0xC0FFEE02)
-    src = np.concatenate([one] * (N // 4))
+    one = orc.fill_u8((1080, 1920, 3), 0xC0FFEE02)
+    src = np.stack([np.roll(one, (n, 7 * n), axis=(0, 1)) for n in range(N)])
     res = run_tensor(cv, src, (224, 224), (455, 256), (115, 16), LINEAR, np.float32, True, 0,
                      1 / (255 * 0.226), -0.449 / 0.226, False)
-    ref = orc.fused_rccr(one, (224, 224), (455, 256), (115, 16), LINEAR, np.float32, True, 0,
-                         1 / (255 * 0.226), -0.449 / 0.226, False, threads=4)
-    compare(res[:4], ref, LINEAR, np.float32)
-    for k in range(1, N // 4):
-        np.testing.assert_array_equal(res[4 * k:4 * k + 4], res[:4])
+    ref = orc.fused_rccr(src, (224, 224), (455, 256), (115, 16), LINEAR, np.float32, True, 0,
+                         1 / (255 * 0.226), -0.449 / 0.226, False, threads=8)
+    compare(res, ref, LINEAR, np.float32)
+    assert not (res[1] == res[0]).all()
 
 
 # ---- extension: fused + per-channel normalisation in one kernel -------------------------------------

@@ -311,6 +311,56 @@ def test_warp_cubic_golden_vs_device_and_perspective(orc):
     np.testing.assert_array_equal(a, p)
 
 
+def _homography(src_pts, dst_pts):
+    """3x3 matrix H (float64, H[2,2] = 1) with H @ (x, y, 1) ~ (u, v, 1) for the four pairs (x, y) -> (u, v):
+    the textbook direct linear solve."""
+    A, b = [], []
+    for (x, y), (u, v) in zip(src_pts, dst_pts):
+        A.append([x, y, 1, 0, 0, 0, -u * x, -u * y])
+        b.append(u)
+        A.append([0, 0, 0, x, y, 1, -v * x, -v * y])
+        b.append(v)
+    h = np.linalg.solve(np.asarray(A, np.float64), np.asarray(b, np.float64))
+    return np.append(h, 1.0).reshape(3, 3)
+
+
+def test_warp_true_homography_against_float64_coordinates(orc):
+    # Pins the projective branch (reference: src/cvcuda/priv/legacy/CvCudaLegacy.h:157-183) with a matrix whose
+    # last row is not (0, 0, 1) and has m6 != m7: a dropped "coeff *" on one axis, m6 and m7 swapped or a
+    # transposed matrix all fail here. The matrix maps destination pixels to source positions (what the
+    # oracle takes); it is built from four corner correspondences in float64.
+    W, H, w, h = 40, 32, 36, 28
+    dst_corners = [(0, 0), (w - 1, 0), (w - 1, h - 1), (0, h - 1)]
+    src_points = [(2, 3), (37, 1), (33, 29), (5, 24)]
+    M = _homography(dst_corners, src_points)
+    assert abs(M[2, 0]) > 1e-4 and abs(M[2, 1]) > 1e-4 and abs(M[2, 0] - M[2, 1]) > 1e-4
+    xs, ys = np.meshgrid(np.arange(w, dtype=np.float64), np.arange(h, dtype=np.float64))
+    den = M[2, 0] * xs + M[2, 1] * ys + M[2, 2]
+    u = (M[0, 0] * xs + M[0, 1] * ys + M[0, 2]) / den
+    v = (M[1, 0] * xs + M[1, 1] * ys + M[1, 2]) / den
+    # NEAREST on an image that holds its own pixel index: the output names the pixel that was read
+    index = (np.arange(H)[:, None] * W + np.arange(W)[None, :]).astype(np.float32)[None, :, :, None]
+    iu, iv = np.floor(u + 0.5), np.floor(v + 0.5)
+    inside = (iu >= 0) & (iu < W) & (iv >= 0) & (iv < H)
+    # away from the half-integer coordinates, where float32 and float64 may round to different pixels
+    safe = inside & (np.abs(u + 0.5 - np.round(u + 0.5)) > 1e-3) & (np.abs(v + 0.5 - np.round(v + 0.5)) > 1e-3)
+    assert safe.mean() > 0.9
+    for variant in (0, 1):
+        got = orc.warp(index, (h, w), M.reshape(9), NEAREST, border=0, border_value=(-1, 0, 0, 0), perspective=True,
+                       variant=variant)[0, :, :, 0]
+        np.testing.assert_array_equal(got[safe], (iv * W + iu)[safe].astype(np.float32))
+        # the four corners land on the stated source points
+        for (x, y), (px, py) in zip(dst_corners, src_points):
+            assert got[y, x] == py * W + px
+    # LINEAR reproduces an image that is linear in (x, y) at the float64 coordinates
+    ramp = (0.25 * np.arange(W)[None, :] + 1.5 * np.arange(H)[:, None] + 3.0).astype(np.float32)[None, :, :, None]
+    well_inside = (u >= 0) & (u <= W - 1) & (v >= 0) & (v <= H - 1)
+    assert well_inside.mean() > 0.9
+    for variant in (0, 1):
+        got = orc.warp(ramp, (h, w), M.reshape(9), LINEAR, border=1, perspective=True, variant=variant)[0, :, :, 0]
+        np.testing.assert_allclose(got[well_inside], (0.25 * u + 1.5 * v + 3.0)[well_inside], rtol=0, atol=2e-3)
+
+
 # ------------------------------------------------------------------------------------------ generator
 def test_seeded_generators(orc):
     a = orc.fill_u8((1000,), 42)
