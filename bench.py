@@ -120,7 +120,7 @@ class Fused:
     def __init__(self, cv, orc, np, torch, form="fused"):
         self.cv, self.orc, self.np, self.torch, self.form = cv, orc, np, torch, form
         self.key, self.kernel = form, self.KERNELS[form]
-        self.workload = ("fused ResizeCropConvertReformat: batch 64 u8 NHWC 1920x1080 -> bilinear 455x256 -> "
+        self.workload = ("fused ResizeCropConvertReformat: batch %d u8 NHWC 1920x1080 -> bilinear 455x256 -> " % self.N +
                          "crop 224x224 @(115,16) -> f32 NCHW, " + self.TEXT[form])
         self.images = self.N
         rows, _ = span_bytes(self.OUT_H, self.CROP_Y, self.SRC_H, self.NEW_H, LINEAR, 1)
@@ -195,8 +195,9 @@ class Fused:
         assert (np.abs(got - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all(), "bench output differs from oracle"
 
     def cpu(self, threads):
-        self._oracle(self.host[:8], threads)
-        return 8
+        n = min(8, self.N)
+        self._oracle(self.host[:n], threads)
+        return n
 
 
 class ResizeC1:
@@ -209,7 +210,7 @@ class ResizeC1:
         name = "NEAREST" if interp == NEAREST else "LINEAR"
         self.key = "resize-" + name.lower()
         self.kernel = "ResizePatchTensorKernel<uint8_t,3,%s>" % name
-        self.workload = "Resize %s: batch 8 u8 NHWC 1920x1080 -> 224x224" % name
+        self.workload = "Resize %s: batch %d u8 NHWC 1920x1080 -> 224x224" % (name, self.N)
         self.images = self.N
         rows, _ = span_bytes(self.OUT_H, 0, self.SRC_H, self.OUT_H, interp, 1)
         _, span = span_bytes(self.OUT_W, 0, self.SRC_W, self.OUT_W, interp, 3)
@@ -417,6 +418,32 @@ class WarpTensor:
         return 1
 
 
+class EmptyLaunch:
+    """Not an operator: one launch of a kernel that does nothing (libcvamd_bench.so), i.e. what a dependent
+    launch costs in the same timed region as the operators. No bytes, so no roofline fraction."""
+    key, config_id, kernel, dtype = "empty-launch", 0, "EmptyKernel", "none"
+    workload = "one empty kernel launch per step (64 threads)"
+    images, alg_bytes = 0, 0
+
+    def __init__(self, cv, orc, np, torch):
+        import ctypes as C
+        lib = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(cv.__file__)), "lib", "libcvamd_bench.so"))
+        self.fn, self.cv = lib.cvamdBenchEmptyLaunch, cv
+        self.fn.restype, self.fn.argtypes = C.c_int, [C.c_void_p]
+
+    def make_set(self):
+        return ()
+
+    def submit(self, stream, s):
+        assert self.fn(self.cv.stream_ptr(stream)) == 0
+
+    def check(self, s):
+        pass
+
+    def cpu(self, threads):
+        return 0
+
+
 class Streaming:
     """Operators either side of the five configurations, each on a 1080p batch: algorithmic bytes are
     the input plus the output, the check is the oracle (or the numpy index map) on the first image."""
@@ -522,6 +549,7 @@ class Streaming:
 
 
 WORKLOADS = {
+    "empty-launch": EmptyLaunch,
     "fused": Fused,
     "fused-normalize": lambda *a: Fused(*a, "fused-normalize"),
     "fused-chain": lambda *a: Fused(*a, "fused-chain"),
@@ -550,6 +578,9 @@ def main():
     ap.add_argument("--min-seconds", type=float, default=0.3,
                     help="the K steps are repeated until the timed region holds at least this much device work")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget of the CPU-oracle leg (0 = skip)")
+    ap.add_argument("--batch", type=int, default=0,
+                    help="images per step for the fused and resize-nearest / resize-linear workloads (0 = the "
+                         "configuration's own batch size); for fits of launch time against batch size")
     ap.add_argument("--streams", type=int, default=1,
                     help="independent streams the K steps are dealt to inside the captured graph (default 1: every "
                          "step waits for the one before, as consecutive Submits on one stream do)")
@@ -575,8 +606,15 @@ def main():
     torch.cuda.set_device(0)
 
     # ---- inputs resident in HBM ----------------------------------------------------------------
+    if args.batch > 0:
+        if args.workload.startswith("fused"):
+            Fused.N = args.batch
+        elif args.workload in ("resize-nearest", "resize-linear"):
+            ResizeC1.N = args.batch
+        else:
+            sys.exit("bench.py: --batch applies to the fused and resize-nearest / resize-linear workloads")
     wl = WORKLOADS[args.workload](cv, orc, np, torch)
-    nsets = args.rotate if args.rotate > 0 else max(3, math.ceil(1.5e9 / wl.alg_bytes))
+    nsets = args.rotate if args.rotate > 0 else max(3, math.ceil(1.5e9 / max(wl.alg_bytes, 1)) if wl.alg_bytes else 1)
     sets = [wl.make_set() for _ in range(nsets)]
     stream = torch.cuda.current_stream()
     torch.cuda.synchronize()
@@ -658,7 +696,7 @@ def main():
 
     # ---- CPU oracle on the same workload (bounded sample)
     cpu = None
-    if args.cpu_seconds > 0:
+    if args.cpu_seconds > 0 and wl.images > 0:
         def cpu_leg(threads, budget):
             reps, done, tcpu = 0, 0, 0.0
             c0 = time.perf_counter()

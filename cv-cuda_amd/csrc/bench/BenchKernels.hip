@@ -1,5 +1,5 @@
-// Copy-bound twin of the fused bilinear kernel, for the benchmark only (libcvamd_bench.so, not part of
-// the operator libraries): the same grid, the same workgroup -> tile map, the same four 8-byte tap
+// Kernels the benchmark times beside the operators (libcvamd_bench.so, not part of the operator
+// libraries). FusedCopyBound is the copy-bound twin of the fused bilinear kernel: the same grid, the same workgroup -> tile map, the same four 8-byte tap
 // loads per lane and the same three streaming stores per lane into an f32 NCHW batch, but no blend,
 // no conversion and no scale/offset: the stored values are the loaded bytes. Its launch time is what
 // the memory system allows a kernel of this access pattern; the fused kernel's time is compared with it.
@@ -44,7 +44,16 @@ __global__ __launch_bounds__(256) void FusedCopyBound(const FusedArgs a)
     }
 }
 
+__global__ void EmptyKernel() {}
+
 } // namespace
+
+// One launch of a kernel that does nothing: the cost of a dependent launch as the benchmark's clocks see it.
+extern "C" __attribute__((visibility("default"))) int cvamdBenchEmptyLaunch(hipStream_t stream)
+{
+    hipLaunchKernelGGL(EmptyKernel, dim3(1), dim3(64), 0, stream);
+    return (int)hipGetLastError();
+}
 
 // src: u8 NHWC batch of N images (srcW x srcH x 3, given row and sample strides in bytes); dst: packed
 // f32 NCHW batch N x 3 x dstH x dstW. Geometry as cvcudaResizeCropConvertReformatSubmit computes it for a

@@ -1,7 +1,7 @@
 // Launch geometry and source addressing of the fused resize-crop-convert-reformat kernels: the argument
 // block, the workgroup -> tile map and the tap loads. Shared by the operator
 // (OpResizeCropConvertReformat.hip) and by the benchmark's copy-bound twin of its bilinear kernel
-// (csrc/bench/FusedCopyBound.hip), which must read the same bytes through the same grid.
+// (csrc/bench/BenchKernels.hip), which must read the same bytes through the same grid.
 #ifndef CVCUDA_AMD_FUSEDTILES_HPP
 #define CVCUDA_AMD_FUSEDTILES_HPP
 
