@@ -112,14 +112,18 @@ __device__ __forceinline__ void StorePx(uint8_t *row, int x, const Pixel<T, C> &
 // N horizontally adjacent pixels at byte offset `xoff` of source row `row` (all inside the image).
 // u8x3: 1 or 2 pixels are fetched with a 4- or 8-byte load that reads 1-2 bytes past them, harmless
 // except behind the image's last row (`lastRow`, wave-uniform), where the load is moved back to end
-// with the row's `rowBytes` and the value shifted.
+// with the row's `rowBytes` and the value shifted; rows shorter than the load are read byte by byte.
 template<class T, int C, int N>
 __device__ __forceinline__ void LoadTaps(const uint8_t *row, int xoff, bool lastRow, int rowBytes, float (&t)[N][C])
 {
     if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 1)
     {
         uint32_t q;
-        if (lastRow)
+        if (lastRow && rowBytes < 4) // a 1-pixel-wide image: moving the load back would leave the row (and a 1 x 1 image)
+        {
+            q = row[xoff] | (row[xoff + 1] << 8) | (row[xoff + 2] << 16);
+        }
+        else if (lastRow)
         {
             const int back = max(0, xoff - (rowBytes - 4));
             q              = LoadU32Unaligned(row + (xoff - back)) >> (8 * back);
@@ -135,7 +139,16 @@ __device__ __forceinline__ void LoadTaps(const uint8_t *row, int xoff, bool last
     else if constexpr (std::is_same_v<T, uint8_t> && C == 3 && N == 2)
     {
         uint64_t q;
-        if (lastRow)
+        if (lastRow && rowBytes < 8) // a 2-pixel-wide image (the two taps are all of the row)
+        {
+            q = 0;
+#pragma unroll
+            for (int i = 0; i < 6; ++i)
+            {
+                q |= (uint64_t)row[xoff + i] << (8 * i);
+            }
+        }
+        else if (lastRow)
         {
             const int back = max(0, xoff - (rowBytes - 8));
             q              = LoadU64Unaligned(row + (xoff - back)) >> (8 * back);

@@ -107,6 +107,22 @@ public:
         buf.hostFormatList                        = m_hostFormats;
         if (m_dirtyFrom < m_num)
         {
+            // A stream under graph capture would record the upload and the event below into the graph: every
+            // replay would then copy whatever the host mirror holds at that time, and the captured event could
+            // no longer be waited on by the next push. Descriptors must be on the device before capture starts.
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &capture) != hipSuccess)
+            {
+                (void)hipGetLastError(); // e.g. the legacy stream while another stream captures: not this stream's capture
+                capture = hipStreamCaptureStatusNone;
+            }
+            if (capture != hipStreamCaptureStatusNone)
+            {
+                throw Error(NVCV_ERROR_INVALID_OPERATION,
+                            "Image batch has %d image descriptor(s) not yet uploaded and the stream is capturing a graph: "
+                            "submit the batch once (or export its data) on a stream that is not capturing first",
+                            m_num - m_dirtyFrom);
+            }
             // Order after any earlier upload (possibly issued on another stream), then copy the tail
             // of the arrays that changed since the last export.
             CheckHip(hipStreamWaitEvent(stream, m_uploaded, 0), "hipStreamWaitEvent");

@@ -146,6 +146,34 @@ def test_submits_captured_in_a_hip_graph_replay_correctly(cv, K, orc, gpu):
         assert (np.abs(got3 - want) <= 1e-5 * np.maximum(1.0, np.abs(want))).all()
 
 
+def test_image_batch_descriptors_must_be_uploaded_before_graph_capture(cv, K, orc, gpu):
+    # A var-shape Submit uploads the descriptors of images pushed since the last Submit on the caller's stream.
+    # Under graph capture that copy would be recorded into the graph (and replay whatever the host mirror holds
+    # later), so it is refused with INVALID_OPERATION; after one Submit outside the capture the same call captures.
+    imgs = [orc.fill_u8((20 + 2 * i, 30 + i, 3), 40 + i) for i in range(3)]
+    bi, bo, outs = cv.ImageBatchVarShape(3), cv.ImageBatchVarShape(3), []
+    for a in imgs:
+        bi.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_RGB8))
+        outs.append(cv.Image.alloc((a.shape[1], a.shape[0]), K.IMAGE_FORMAT_RGB8))
+        bo.push_back(outs[-1])
+    op = cv.CvtColor()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        with pytest.raises(cv.Error) as e:
+            op(torch.cuda.current_stream(), bi, bo, K.COLOR_BGR2RGB)
+    assert e.value.status == 4  # NVCV_ERROR_INVALID_OPERATION
+    op(None, bi, bo, K.COLOR_BGR2RGB)  # uploads the descriptors
+    torch.cuda.synchronize()
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2, stream=side):
+        op(torch.cuda.current_stream(), bi, bo, K.COLOR_BGR2RGB)
+    graph2.replay()
+    torch.cuda.synchronize()
+    for a, o in zip(imgs, outs):
+        np.testing.assert_array_equal(o.plane_view(0, np.uint8, 3).cpu().numpy(), a[:, :, ::-1])
+
+
 def test_image_batches_larger_than_one_launch(cv, K, orc, gpu):
     # the image-batch operators pack at most a few hundred images' tiles into one launch and loop over
     # the rest: 401 images make every operator issue a second launch, whose images must use their own

@@ -217,6 +217,20 @@ def test_area_tensor(cv, orc, gpu, row):
         np.testing.assert_array_equal(res, device)
 
 
+def test_area_sources_one_and_two_pixels_wide(cv, orc, gpu):
+    # u8x3 rows shorter than the 4- and 8-byte tap loads: 1 x 1, 1 x H, 2 x 1 and W x 1 sources, every
+    # interpolation (the tap loads of the last row must not be moved in front of the row)
+    for (sw, sh) in ((1, 1), (1, 7), (2, 1), (2, 5), (9, 1)):
+        src = make_input(orc, (2, sh, sw, 3), np.uint8, 31 * sw + sh)
+        for interp in (NEAREST, LINEAR, CUBIC, AREA):
+            for (dw, dh) in ((1, 1), (3, 2), (5, 9)):
+                tout = cv.Tensor.alloc([2, dh, dw, 3], np.uint8, "NHWC")
+                cv.Resize()(None, cv.Tensor.from_numpy(src, "NHWC"), tout, interp)
+                torch.cuda.synchronize()
+                device = orc.resize(src, (dh, dw), interp, variant=0 if interp == NEAREST else 1)
+                np.testing.assert_array_equal(tout.numpy(), device, err_msg=str((sw, sh, dw, dh, interp)))
+
+
 @pytest.mark.parametrize("dt,c", [(np.uint8, 4), (np.uint8, 3), (np.uint16, 1), (np.int16, 3), (np.float32, 4)])
 def test_area_varshape(cv, K, orc, gpu, dt, c):
     # image batches run the reference's separate AREA kernel (reductions: same sums, corners last;
