@@ -10,7 +10,8 @@ import os
 import torch  # noqa: F401  (loads the HIP runtime once, before our libraries resolve it)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIBDIR = os.path.join(_HERE, "lib")
+# CVCUDA_AMD_LIBDIR selects another build of the same libraries (the host-sanitizer build in lib_san/)
+_LIBDIR = os.environ.get("CVCUDA_AMD_LIBDIR") or os.path.join(_HERE, "lib")
 
 
 def _load(name):

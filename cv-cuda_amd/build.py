@@ -5,8 +5,19 @@
   lib/libcvamd_bench.so -- kernels the benchmark times beside the operators (a copy-bound twin of the
                            fused kernel); nothing in the two libraries above uses it
 
-Usage: python cv-cuda_amd/build.py [--force] [-j N]
+Usage: python cv-cuda_amd/build.py [--force] [-j N] [--sanitize]
 Objects are cached under build/ next to this file and rebuilt when a source or header is newer.
+
+--sanitize builds the same libraries into lib_san/ (objects in build_san/) with AddressSanitizer and
+UndefinedBehaviorSanitizer on the HOST code only (device code is compiled as usual). The host logic -
+handle pools, reference counts, stride rules, operator validation - can then be run under the sanitizers
+without a GPU:
+
+  LD_PRELOAD=$(python cv-cuda_amd/build.py --asan-runtime) ASAN_OPTIONS=detect_leaks=0 \
+  CVCUDA_AMD_LIBDIR=cv-cuda_amd/lib_san python -m pytest tests/test_core.py tests/test_op_validation.py -q
+
+(the interpreter itself is not instrumented, so the sanitizer runtime has to be loaded first; leak detection is
+off because the interpreter's own allocations would drown the report).
 """
 import argparse
 import concurrent.futures
@@ -63,13 +74,27 @@ def _compile(src, obj, extra, force, newest_header):
     return msgs
 
 
-def build(force=False, jobs=8, verbose=True):
+def asan_runtime():
+    """Path of the AddressSanitizer runtime of hipcc's clang (to LD_PRELOAD into an uninstrumented python)."""
+    r = subprocess.run(["hipcc", "-print-file-name=libclang_rt.asan-x86_64.so"], capture_output=True, text=True)
+    return r.stdout.strip()
+
+
+def build(force=False, jobs=8, verbose=True, sanitize=False):
+    global LIBDIR, OBJDIR
+    host_extra, hip_extra, link_extra = [], [], []
+    if sanitize:
+        LIBDIR, OBJDIR = os.path.join(HERE, "lib_san"), os.path.join(HERE, "build_san")
+        # on a hipcc line every -fsanitize= goes directly after -Xarch_host: the device pass must not see it
+        hip_extra = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-fno-omit-frame-pointer", "-g"]
+        host_extra = hip_extra # hipcc compiles the plain .cpp sources as HIP too
+        link_extra = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-shared-libsan"]
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     newest_header = max(os.path.getmtime(h) for h in _headers())
-    core = [(s, []) for s in _sources("nvcv", (".cpp",))]
-    ops = [(s, DEVICE if s.endswith(".hip") else []) for s in _sources("cvcuda", (".cpp", ".hip"))]
-    bench = [(s, DEVICE) for s in _sources("bench", (".hip",))]
+    core = [(s, host_extra) for s in _sources("nvcv", (".cpp",))]
+    ops = [(s, DEVICE + hip_extra if s.endswith(".hip") else host_extra) for s in _sources("cvcuda", (".cpp", ".hip"))]
+    bench = [(s, DEVICE + hip_extra) for s in _sources("bench", (".hip",))]
     tasks = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         for group, items in (("nvcv", core), ("cvcuda", ops), ("bench", bench)):
@@ -84,7 +109,7 @@ def build(force=False, jobs=8, verbose=True):
     ops_objs = [o for g, o, _ in tasks if g == "cvcuda"]
     nvcv_so = os.path.join(LIBDIR, "libnvcv_types.so")
     cvcuda_so = os.path.join(LIBDIR, "libcvcuda.so")
-    link = ["hipcc", "-shared", "-fPIC", "--offload-arch=" + ARCH, "-Wl,--no-undefined"]
+    link = ["hipcc", "-shared", "-fPIC", "--offload-arch=" + ARCH] + (link_extra if sanitize else ["-Wl,--no-undefined"])
     # ELF symbol versions of the reference's ABI (FUNC@@NVCV_x.y / FUNC@@CVCUDA_x.y), see csrc/abi
     maps = os.path.join(CSRC, "abi")
     subprocess.run(link + core_objs + ["-o", nvcv_so, "-Wl,-soname,libnvcv_types.so",
@@ -101,5 +126,10 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
     ap.add_argument("-j", type=int, default=8)
+    ap.add_argument("--sanitize", action="store_true", help="ASan + UBSan build of the host code into lib_san/")
+    ap.add_argument("--asan-runtime", action="store_true", help="print the sanitizer runtime to LD_PRELOAD and exit")
     a = ap.parse_args()
-    print("\n".join(build(a.force, a.j)))
+    if a.asan_runtime:
+        print(asan_runtime())
+    else:
+        print("\n".join(build(a.force, a.j, sanitize=a.sanitize)))

@@ -27,7 +27,7 @@ struct ColorIO
 };
 
 // Validates and launches; false when `code` belongs to none of these families.
-bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStream_t stream);
+bool RunPixelColorFamily(ColorCode code, const ColorIO &io, hipStream_t stream);
 
 } // namespace cvamd
 

@@ -78,6 +78,22 @@ NVCVStatus Protect(F &&fn) noexcept
     }
 }
 
+// The bits of an enumeration argument as an int. A C caller can pass any integer where the C API names an
+// enum; reading such a value THROUGH the enum type is undefined in C++ when it lies outside the range the
+// enumerators span (the undefined-behaviour sanitizer reports every such read), so arguments that are
+// validated - and may be invalid - are carried as plain ints from the entry point on.
+template<class E>
+inline int EnumBits(const E &e)
+{
+    static_assert(sizeof(E) == sizeof(int), "C enums of this API are int-sized");
+    int v;
+    __builtin_memcpy(&v, &e, sizeof(v));
+    return v;
+}
+
+// A colour conversion code as callers pass it (an NVCVColorConversionCode, possibly not a valid one).
+using ColorCode = int;
+
 // Calls a core-library function and rethrows its status (with its message) as an OpError.
 void CheckCore(NVCVStatus st);
 void CheckHip(hipError_t e, const char *what);

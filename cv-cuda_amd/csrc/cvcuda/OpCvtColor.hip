@@ -416,7 +416,7 @@ enum class Family
     Unsupported
 };
 
-Family FamilyOf(NVCVColorConversionCode code)
+Family FamilyOf(ColorCode code)
 {
     const int c = (int)code;
     if (c >= NVCV_COLOR_BGR2BGRA && c <= NVCV_COLOR_BGRA2RGBA)
@@ -436,7 +436,7 @@ struct YuvCode
     bool planar;
 };
 
-YuvCode DecodeYuvCode(NVCVColorConversionCode code)
+YuvCode DecodeYuvCode(ColorCode code)
 {
     YuvCode y;
     switch (code)
@@ -543,7 +543,7 @@ void DispatchSwizzle(int sch, int dch, const SwizzleArgs &a, int N, const NVCVIm
 }
 
 // The swizzle only moves bits: element types of equal size share a kernel. Alpha is passed as bits.
-void RunSwizzle(NVCVColorConversionCode code, ElemType elem, int inC, int outC, SwizzleArgs &a, int N,
+void RunSwizzle(ColorCode code, ElemType elem, int inC, int outC, SwizzleArgs &a, int N,
                 const NVCVImageBufferStrided *dstHost, hipStream_t stream)
 {
     const int sch = (code == NVCV_COLOR_BGRA2BGR || code == NVCV_COLOR_RGBA2BGR || code == NVCV_COLOR_BGRA2RGBA) ? 4 : 3;
@@ -627,7 +627,7 @@ void RunYuv(const YuvCode &yc, int dcn, const YuvArgs &a, int N, const NVCVImage
 class CvtColor final : public IOperator
 {
 public:
-    void submit(hipStream_t stream, NVCVTensorHandle hin, NVCVTensorHandle hout, NVCVColorConversionCode code) const
+    void submit(hipStream_t stream, NVCVTensorHandle hin, NVCVTensorHandle hout, ColorCode code) const
     {
         NVCVTensorData din, dout;
         ExportTensor(hin, din, "Input");
@@ -747,7 +747,7 @@ public:
     }
 
     void submit(hipStream_t stream, NVCVImageBatchHandle hin, NVCVImageBatchHandle hout,
-                NVCVColorConversionCode code) const
+                ColorCode code) const
     {
         VarShapeView in  = ExportVarShape(hin, stream, "Input");
         VarShapeView out = ExportVarShape(hout, stream, "Output");
@@ -847,13 +847,15 @@ CVCUDA_PUBLIC NVCVStatus cvcudaCvtColorCreate(NVCVOperatorHandle *handle)
 CVCUDA_PUBLIC NVCVStatus cvcudaCvtColorSubmit(NVCVOperatorHandle handle, hipStream_t stream, NVCVTensorHandle in,
                                               NVCVTensorHandle out, NVCVColorConversionCode code)
 {
-    return Protect([&] { ToOperator<CvtColor>(handle).submit(stream, in, out, code); });
+    const ColorCode value = EnumBits(code);
+    return Protect([&] { ToOperator<CvtColor>(handle).submit(stream, in, out, value); });
 }
 
 CVCUDA_PUBLIC NVCVStatus cvcudaCvtColorVarShapeSubmit(NVCVOperatorHandle handle, hipStream_t stream,
                                                       NVCVImageBatchHandle in, NVCVImageBatchHandle out,
                                                       NVCVColorConversionCode code)
 {
-    return Protect([&] { ToOperator<CvtColor>(handle).submit(stream, in, out, code); });
+    const ColorCode value = EnumBits(code);
+    return Protect([&] { ToOperator<CvtColor>(handle).submit(stream, in, out, value); });
 }
 }

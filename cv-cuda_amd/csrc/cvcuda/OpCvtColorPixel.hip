@@ -831,7 +831,7 @@ void RequireU8(const ColorIO &io)
 
 } // namespace
 
-bool RunPixelColorFamily(NVCVColorConversionCode code, const ColorIO &io, hipStream_t stream)
+bool RunPixelColorFamily(ColorCode code, const ColorIO &io, hipStream_t stream)
 {
     const int c = (int)code;
     PixArgs   a = MakeArgs(io, io.dstW, io.dstH);

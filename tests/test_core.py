@@ -354,7 +354,8 @@ def test_custom_allocator(cv, capi):
 
     def alloc(ctx, size, align):
         log.append(("alloc", size, align))
-        return libc.aligned_alloc(max(align, 8), max(size, max(align, 8)))
+        a = max(align, 8)
+        return libc.aligned_alloc(a, (max(size, a) + a - 1) // a * a)  # C11: size is a multiple of the alignment
 
     def free(ctx, ptr, size, align):
         log.append(("free", size, align))
