@@ -421,6 +421,33 @@ NVCVStatus MakeFormat(NVCVImageFormat *out, NVCVColorModel model, uint32_t spec,
         });
 }
 
+template<class E>
+NVCVStatus GetSpecField(NVCVColorSpec cspec, int off, int len, E *out, const char *what)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(out, what);
+            *out = (E)Get((uint64_t)(uint32_t)EnumValue(cspec), off, len);
+        });
+}
+
+NVCVStatus SetSpecField(NVCVColorSpec *cspec, int off, int len, uint64_t value)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(cspec, "Pointer to input colorspec");
+            const uint64_t mask = ((1ULL << len) - 1) << off;
+            *cspec = (NVCVColorSpec)(int32_t)((((uint64_t)(uint32_t)EnumValue(*cspec)) & ~mask) | Put(value, off, len));
+        });
+}
+
+const char *EnumName(int v, const char *const *names, int count, const char *type)
+{
+    return (v >= 0 && v < count) ? names[v] : ThreadName("%s(%d)", type, v);
+}
+
 } // namespace
 } // namespace nvcvamd
 
@@ -536,6 +563,10 @@ NVCVStatus nvcvChromaSubsamplingGetNumSamples(NVCVChromaSubsampling css, int32_t
     return Protect(
         [&]
         {
+            if (outSamplesHoriz == nullptr && outSamplesVert == nullptr)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "At least one of the two sample-count outputs must be non-NULL");
+            }
             if ((int)css < 0 || (int)css > 7)
             {
                 throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid chroma subsampling: %d", (int)css);
@@ -583,9 +614,246 @@ const char *nvcvColorModelGetName(NVCVColorModel cmodel)
 
 const char *nvcvChromaSubsamplingGetName(NVCVChromaSubsampling css)
 {
-    static const char *const names[] = {"NVCV_CSS_444", "NVCV_CSS_422",  "NVCV_CSS_422R", "NVCV_CSS_411",
-                                        "NVCV_CSS_411R", "NVCV_CSS_420", "NVCV_CSS_410",  "NVCV_CSS_410R"};
+    // J:a:b notation (reference: src/nvcv/src/priv/ColorSpec.cpp:447-478)
+    static const char *const names[] = {"4:4:4", "4:2:2", "4:2:2R", "4:1:1", "4:1:1R", "4:2:0", "4:1:0", "4:1:0R"};
     return ((int)css >= 0 && (int)css < 8) ? names[(int)css] : ThreadName("NVCVChromaSubsampling(%d)", (int)css);
+}
+
+NVCVStatus nvcvMakeChromaSubsampling(NVCVChromaSubsampling *outCSS, int32_t samplesHoriz, int32_t samplesVert)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outCSS, "Pointer to output chroma subsampling");
+            // samples per 4 luma samples -> code (reference: priv/ColorSpec.cpp:99-143); 1 x 1 is 4:4:4 as well
+            static const struct
+            {
+                int                   h, v;
+                NVCVChromaSubsampling css;
+            } table[] = {{4, 4, NVCV_CSS_444}, {4, 2, NVCV_CSS_422R}, {4, 1, NVCV_CSS_411R}, {2, 4, NVCV_CSS_422},
+                         {2, 2, NVCV_CSS_420}, {2, 1, NVCV_CSS_410R}, {1, 1, NVCV_CSS_444},  {1, 2, NVCV_CSS_410},
+                         {1, 4, NVCV_CSS_411}};
+            for (const auto &e : table)
+            {
+                if (e.h == samplesHoriz && e.v == samplesVert)
+                {
+                    *outCSS = e.css;
+                    return;
+                }
+            }
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT,
+                        "%d horizontal and %d vertical samples doesn't correspond to any supported chroma subsampling scheme",
+                        samplesHoriz, samplesVert);
+        });
+}
+
+// Colour spec word: space [0,3) xfer [3,7) encoding [7,10) horizontal / vertical chroma location [10,12) [12,14)
+// range [14,15) (reference: detail/FormatUtils.h:34-37, priv/ColorSpec.cpp:41-95). No value is range-checked,
+// here or there: components are truncated to their fields.
+NVCVStatus nvcvMakeColorSpec(NVCVColorSpec *outColorSpec, NVCVColorSpace cspace, NVCVYCbCrEncoding encoding,
+                             NVCVColorTransferFunction xferFunc, NVCVColorRange range, NVCVChromaLocation locHoriz,
+                             NVCVChromaLocation locVert)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outColorSpec, "Pointer to output colorspec");
+            *outColorSpec = (NVCVColorSpec)(int32_t)NVCV_DETAIL_COLOR_SPEC_WORD(
+                EnumValue(cspace), EnumValue(encoding), EnumValue(xferFunc), EnumValue(range), EnumValue(locHoriz),
+                EnumValue(locVert));
+        });
+}
+
+NVCVStatus nvcvColorSpecGetChromaLoc(NVCVColorSpec cspec, NVCVChromaLocation *outLocHoriz, NVCVChromaLocation *outLocVert)
+{
+    return Protect(
+        [&]
+        {
+            if (outLocHoriz == nullptr && outLocVert == nullptr)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT,
+                            "Pointer to output horizontal and vertical chroma location cannot both be NULL");
+            }
+            const uint64_t w = (uint32_t)EnumValue(cspec);
+            if (outLocHoriz != nullptr)
+            {
+                *outLocHoriz = (NVCVChromaLocation)Get(w, 10, 2);
+            }
+            if (outLocVert != nullptr)
+            {
+                *outLocVert = (NVCVChromaLocation)Get(w, 12, 2);
+            }
+        });
+}
+
+NVCVStatus nvcvColorSpecSetChromaLoc(NVCVColorSpec *cspec, NVCVChromaLocation locHoriz, NVCVChromaLocation locVert)
+{
+    return SetSpecField(cspec, 10, 4, Put((uint64_t)EnumValue(locHoriz), 0, 2) | Put((uint64_t)EnumValue(locVert), 2, 2));
+}
+
+NVCVStatus nvcvColorSpecGetColorSpace(NVCVColorSpec cspec, NVCVColorSpace *outColorSpace)
+{
+    return GetSpecField(cspec, 0, 3, outColorSpace, "Pointer to output color space");
+}
+
+NVCVStatus nvcvColorSpecSetColorSpace(NVCVColorSpec *cspec, NVCVColorSpace cspace)
+{
+    return SetSpecField(cspec, 0, 3, (uint64_t)EnumValue(cspace));
+}
+
+NVCVStatus nvcvColorSpecGetYCbCrEncoding(NVCVColorSpec cspec, NVCVYCbCrEncoding *outEncoding)
+{
+    return GetSpecField(cspec, 7, 3, outEncoding, "Pointer to output YCbCr encoding");
+}
+
+NVCVStatus nvcvColorSpecSetYCbCrEncoding(NVCVColorSpec *cspec, NVCVYCbCrEncoding encoding)
+{
+    return SetSpecField(cspec, 7, 3, (uint64_t)EnumValue(encoding));
+}
+
+NVCVStatus nvcvColorSpecGetColorTransferFunction(NVCVColorSpec cspec, NVCVColorTransferFunction *outXferFunc)
+{
+    return GetSpecField(cspec, 3, 4, outXferFunc, "Pointer to output color transfer function");
+}
+
+NVCVStatus nvcvColorSpecSetColorTransferFunction(NVCVColorSpec *cspec, NVCVColorTransferFunction xferFunc)
+{
+    return SetSpecField(cspec, 3, 4, (uint64_t)EnumValue(xferFunc));
+}
+
+NVCVStatus nvcvColorSpecGetRange(NVCVColorSpec cspec, NVCVColorRange *outColorRange)
+{
+    return GetSpecField(cspec, 14, 1, outColorRange, "Pointer to output color range");
+}
+
+NVCVStatus nvcvColorSpecSetRange(NVCVColorSpec *cspec, NVCVColorRange range)
+{
+    return SetSpecField(cspec, 14, 1, (uint64_t)EnumValue(range));
+}
+
+NVCVStatus nvcvColorModelNeedsColorspec(NVCVColorModel cmodel, int8_t *outBool)
+{
+    return Protect(
+        [&]
+        {
+            NotNull(outBool, "Pointer to output boolean");
+            switch (EnumValue(cmodel))
+            {
+            case NVCV_COLOR_MODEL_YCbCr:
+            case NVCV_COLOR_MODEL_RGB:
+                *outBool = 1;
+                return;
+            case NVCV_COLOR_MODEL_UNDEFINED:
+            case NVCV_COLOR_MODEL_RAW:
+            case NVCV_COLOR_MODEL_XYZ:
+            case NVCV_COLOR_MODEL_HSV:
+            case NVCV_COLOR_MODEL_CMYK:
+            case NVCV_COLOR_MODEL_YCCK:
+                *outBool = 0;
+                return;
+            }
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid color model: %s", nvcvColorModelGetName(cmodel));
+        });
+}
+
+const char *nvcvColorSpaceGetName(NVCVColorSpace cspace)
+{
+    static const char *const n[] = {"NVCV_COLOR_SPACE_BT601", "NVCV_COLOR_SPACE_BT709", "NVCV_COLOR_SPACE_BT2020",
+                                    "NVCV_COLOR_SPACE_DCIP3"};
+    return EnumName(EnumValue(cspace), n, 4, "NVCVColorSpace");
+}
+
+const char *nvcvWhitePointGetName(NVCVWhitePoint wpoint)
+{
+    static const char *const n[] = {"NVCV_WHITE_POINT_D65"};
+    return EnumName(EnumValue(wpoint), n, 1, "NVCVWhitePoint");
+}
+
+const char *nvcvYCbCrEncodingGetName(NVCVYCbCrEncoding enc)
+{
+    static const char *const n[] = {"NVCV_YCbCr_ENC_UNDEFINED", "NVCV_YCbCr_ENC_BT601",   "NVCV_YCbCr_ENC_BT709",
+                                    "NVCV_YCbCr_ENC_BT2020",    "NVCV_YCbCr_ENC_BT2020c", "NVCV_YCbCr_ENC_SMPTE240M"};
+    return EnumName(EnumValue(enc), n, 6, "NVCVYCbCrEncoding");
+}
+
+const char *nvcvColorTransferFunctionGetName(NVCVColorTransferFunction xfer)
+{
+    static const char *const n[] = {"NVCV_COLOR_XFER_LINEAR", "NVCV_COLOR_XFER_sRGB",  "NVCV_COLOR_XFER_sYCC",
+                                    "NVCV_COLOR_XFER_PQ",     "NVCV_COLOR_XFER_BT709", "NVCV_COLOR_XFER_BT2020",
+                                    "NVCV_COLOR_XFER_SMPTE240M"};
+    return EnumName(EnumValue(xfer), n, 7, "NVCVColorTransferFunction");
+}
+
+const char *nvcvColorRangeGetName(NVCVColorRange range)
+{
+    static const char *const n[] = {"NVCV_COLOR_RANGE_FULL", "NVCV_COLOR_RANGE_LIMITED"};
+    return EnumName(EnumValue(range), n, 2, "NVCVColorRange");
+}
+
+const char *nvcvChromaLocationGetName(NVCVChromaLocation loc)
+{
+    static const char *const n[] = {"NVCV_CHROMA_LOC_BOTH", "NVCV_CHROMA_LOC_EVEN", "NVCV_CHROMA_LOC_CENTER",
+                                    "NVCV_CHROMA_LOC_ODD"};
+    return EnumName(EnumValue(loc), n, 4, "NVCVChromaLocation");
+}
+
+const char *nvcvRawPatternGetName(NVCVRawPattern raw)
+{
+    static const char *const n[]
+        = {"NVCV_RAW_BAYER_RGGB", "NVCV_RAW_BAYER_BGGR", "NVCV_RAW_BAYER_GRBG", "NVCV_RAW_BAYER_GBRG", "NVCV_RAW_BAYER_RCCB",
+           "NVCV_RAW_BAYER_BCCR", "NVCV_RAW_BAYER_CRBC", "NVCV_RAW_BAYER_CBRC", "NVCV_RAW_BAYER_RCCC", "NVCV_RAW_BAYER_CRCC",
+           "NVCV_RAW_BAYER_CCRC", "NVCV_RAW_BAYER_CCCR", "NVCV_RAW_BAYER_CCCC"};
+    return EnumName(EnumValue(raw), n, 13, "NVCVRawPattern");
+}
+
+const char *nvcvColorSpecGetName(NVCVColorSpec cspec)
+{
+    // predefined specs by name; anything else by its components with the enumerators' common prefixes
+    // shortened (reference: priv/ColorSpec.cpp:179-262). The reserved all-ones value gets both.
+    static const struct
+    {
+        NVCVColorSpec spec;
+        const char   *name;
+    } predefined[] = {
+#define CVAMD_SPEC(x) {x, #x}
+        CVAMD_SPEC(NVCV_COLOR_SPEC_UNDEFINED),     CVAMD_SPEC(NVCV_COLOR_SPEC_MPEG2_BT601),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_MPEG2_BT709),   CVAMD_SPEC(NVCV_COLOR_SPEC_MPEG2_SMPTE240M),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_BT601),         CVAMD_SPEC(NVCV_COLOR_SPEC_BT601_ER),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_BT709),         CVAMD_SPEC(NVCV_COLOR_SPEC_BT709_ER),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_BT709_LINEAR),  CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020_ER),     CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020_LINEAR),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020_PQ),     CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020_PQ_ER),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020c),       CVAMD_SPEC(NVCV_COLOR_SPEC_BT2020c_ER),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_SMPTE240M),     CVAMD_SPEC(NVCV_COLOR_SPEC_sRGB),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_sYCC),          CVAMD_SPEC(NVCV_COLOR_SPEC_DISPLAYP3),
+        CVAMD_SPEC(NVCV_COLOR_SPEC_DISPLAYP3_LINEAR),
+#undef CVAMD_SPEC
+    };
+    const int value = EnumValue(cspec);
+    for (const auto &e : predefined)
+    {
+        if ((int)e.spec == value)
+        {
+            return e.name;
+        }
+    }
+    const uint64_t w = (uint32_t)value;
+    auto           part = [](const char *full, const char *prefix, const char *shortened)
+    {
+        const size_t n = strlen(prefix);
+        return strncmp(full, prefix, n) == 0 ? ThreadName("%s%s", shortened, full + n) : full;
+    };
+    // the ring behind ThreadName holds fewer strings than are needed here at once: copy each part
+    char space[64], enc[64], xfer[64], range[64], loch[64], locv[64];
+    snprintf(space, sizeof(space), "%s", part(nvcvColorSpaceGetName((NVCVColorSpace)Get(w, 0, 3)), "NVCV_COLOR_SPACE_", "SPACE_"));
+    snprintf(enc, sizeof(enc), "%s", part(nvcvYCbCrEncodingGetName((NVCVYCbCrEncoding)Get(w, 7, 3)), "NVCV_YCbCr_", ""));
+    snprintf(xfer, sizeof(xfer), "%s",
+             part(nvcvColorTransferFunctionGetName((NVCVColorTransferFunction)Get(w, 3, 4)), "NVCV_COLOR_XFER_", "XFER_"));
+    snprintf(range, sizeof(range), "%s", part(nvcvColorRangeGetName((NVCVColorRange)Get(w, 14, 1)), "NVCV_COLOR_RANGE_", "RANGE_"));
+    snprintf(loch, sizeof(loch), "%s", part(nvcvChromaLocationGetName((NVCVChromaLocation)Get(w, 10, 2)), "NVCV_CHROMA_LOC_", "LOC_"));
+    snprintf(locv, sizeof(locv), "%s", part(nvcvChromaLocationGetName((NVCVChromaLocation)Get(w, 12, 2)), "NVCV_CHROMA_LOC_", "LOC_"));
+    return ThreadName("%sNVCVColorSpec(%s,%s,%s,%s,%s,%s)", value == (int)NVCV_COLOR_SPEC_FORCE32 ? "NVCVColorSpec(invalid)" : "",
+                      space, enc, xfer, range, loch, locv);
 }
 
 // ---- data type ---------------------------------------------------------------------------------

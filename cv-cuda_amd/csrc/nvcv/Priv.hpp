@@ -66,6 +66,17 @@ NVCVStatus Protect(F &&fn) noexcept
     }
 }
 
+// The value of an enumeration argument as an int, read through its bytes: C callers may pass any integer where
+// the API names an enum, and reading a value outside the enumerators' range through the enum type is undefined.
+template<class E>
+inline int EnumValue(const E &e)
+{
+    static_assert(sizeof(E) == sizeof(int), "C enums of this API are int-sized");
+    int v;
+    __builtin_memcpy(&v, &e, sizeof(v));
+    return v;
+}
+
 template<class T>
 T *NotNull(T *p, const char *what)
 {

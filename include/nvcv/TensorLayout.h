@@ -6,6 +6,7 @@
 
 #include "Export.h"
 #include "Status.h"
+#include "detail/CompilerUtils.h"
 
 #include <stdint.h>
 #include <string.h>
@@ -114,13 +115,15 @@ static inline int32_t nvcvTensorLayoutFindDimIndex(NVCVTensorLayout layout, char
     return -1;
 }
 
-static inline char nvcvTensorLayoutGetLabel(NVCVTensorLayout layout, int idx)
+/* The three accessors below are constant expressions in C++ (the C++ wrappers evaluate them at compile time). */
+NVCV_CONSTEXPR static inline char nvcvTensorLayoutGetLabel(NVCVTensorLayout layout, int idx)
 {
-    int i = idx < 0 ? layout.rank + idx : idx;
-    return (i >= 0 && i < layout.rank) ? layout.data[i] : '\0';
+    return ((idx < 0 ? layout.rank + idx : idx) >= 0 && (idx < 0 ? layout.rank + idx : idx) < layout.rank)
+             ? layout.data[idx < 0 ? layout.rank + idx : idx]
+             : '\0';
 }
 
-static inline int32_t nvcvTensorLayoutGetNumDim(NVCVTensorLayout layout)
+NVCV_CONSTEXPR static inline int32_t nvcvTensorLayoutGetNumDim(NVCVTensorLayout layout)
 {
     return layout.rank;
 }
@@ -142,7 +145,7 @@ static inline int32_t nvcvTensorLayoutEndsWith(NVCVTensorLayout layout, NVCVTens
         && memcmp(test.data, layout.data + layout.rank - test.rank, (size_t)test.rank) == 0;
 }
 
-static inline const char *nvcvTensorLayoutGetName(const NVCVTensorLayout *layout)
+NVCV_CONSTEXPR static inline const char *nvcvTensorLayoutGetName(const NVCVTensorLayout *layout)
 {
     return layout ? layout->data : "";
 }

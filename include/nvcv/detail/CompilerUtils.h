@@ -1,5 +1,5 @@
 /* Language-level helper macros used by the C headers and by the reference's header-only C++ wrappers
- * (nvcv/*.hpp include this file by name).
+ * (the nvcv .hpp files include this file by name).
  * Replaces: src/nvcv/src/include/nvcv/detail/CompilerUtils.h:17-35. */
 #ifndef NVCV_DETAIL_COMPILERUTILS_H
 #define NVCV_DETAIL_COMPILERUTILS_H

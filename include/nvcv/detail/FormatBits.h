@@ -48,6 +48,9 @@
     (NVCV_DETAIL_BITS_PUT(space, 0, 3) | NVCV_DETAIL_BITS_PUT(xfer, 3, 4) | NVCV_DETAIL_BITS_PUT(enc, 7, 3)   \
      | NVCV_DETAIL_BITS_PUT(loch, 10, 2) | NVCV_DETAIL_BITS_PUT(locv, 12, 2) | NVCV_DETAIL_BITS_PUT(range, 14, 1))
 
+#define NVCV_DETAIL_MAKE_COLOR_SPEC(CSpace, Encoding, XferFunc, Range, LocHoriz, LocVert) \
+    NVCV_DETAIL_COLOR_SPEC_WORD(CSpace, Encoding, XferFunc, Range, LocHoriz, LocVert)
+
 /* Colour block [16,35) for a model / spec (or raw pattern) / chroma-subsampling triple. */
 #define NVCV_DETAIL_COLOR_BLOCK(model, spec, css)                                                       \
     ((model) == 1 /* YCbCr */                                                                           \
