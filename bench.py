@@ -30,14 +30,19 @@ NEAREST, LINEAR, CUBIC = 0, 1, 2
 
 # HBM bytes one launch of a workload's kernel moves, from hardware counters (rocprofv3 --pmc
 # FETCH_SIZE and --pmc WRITE_SIZE in separate runs, each scaled by what the same counter reads for a
-# 128 MiB device copy: x1.99965 and x1.00000). It is a property of the kernel and the workload, not
-# of a run, so it is recorded here rather than re-measured. fused: 84,436,703 read + 38,535,168
-# written; resize-cubic-4k: 1,415,442,526 read + 58,982,400 written; resize-nearest: 11,031,874 +
-# 1,204,224; resize-linear: 22,084,429 + 1,204,224; nv12-to-rgb: 99,581,316 + 199,067,341;
-# warp-affine-varshape: 186,479,540 + 117,211,648 (the counters sit between the L2s and the fabric:
-# this batch fits the memory-side cache, so part of those reads never reaches HBM).
-MEASURED_TRAFFIC_BYTES = {"fused": 122971871, "resize-cubic-4k": 1474424926, "resize-nearest": 12236098,
-                          "resize-linear": 23288653, "nv12-to-rgb": 298648657, "warp-affine-varshape": 303691188}
+# plain device copy of known size appended to the same run by --copy-probe). It is a property of the
+# kernel and the workload, not of a run, so it is recorded here rather than re-measured; read and
+# write parts are in the summary files named below. The counters sit between the L2s and the fabric:
+# a batch that fits the memory-side cache (warp-affine-varshape) has part of those reads served there.
+MEASURED_TRAFFIC_BYTES = {"fused": 122961076, "resize-cubic-4k": 1474461132, "resize-nearest": 12234391,
+                          "resize-linear": 23284857, "nv12-to-rgb": 298659913, "warp-affine-varshape": 301970150}
+# The rocprofv3 counter summary each figure above is the "total" line of (a CPU test compares them).
+TRAFFIC_PROFILES = {"fused": "FusedBilinear_batch64_1080p_to_224",
+                    "resize-cubic-4k": "ResizeCubicStagedKernel_f32x4_batch16_4k_to_640x360",
+                    "resize-nearest": "ResizePatchTensorKernel_u8x3_NEAREST_batch8_1080p_to_224",
+                    "resize-linear": "ResizePatchTensorKernel_u8x3_LINEAR_batch8_1080p_to_224",
+                    "nv12-to-rgb": "Yuv420ToRgbTensor_NV12_batch32_1080p",
+                    "warp-affine-varshape": "WarpVarShape_u8x3_LINEAR_batch32_varshape"}
 
 
 def span_bytes(n_out, crop, src, new, interp, pixel_bytes):
@@ -108,10 +113,10 @@ class Fused:
     SCALE, OFFSET = 1.0 / (255.0 * 0.226), -0.449 / 0.226
     MEAN, STD = (0.485, 0.456, 0.406), (0.229, 0.224, 0.225)
     dtype = "f32"
-    KERNELS = {"fused": "FusedBilinear<float,false,false,false>",
-               "fused-normalize": "FusedBilinear<float,false,false,true>",
-               "fused-chain": "FusedBilinear<float,false,false,false> + NormRunsTensor<float,float,3> + "
-                              "ReformatRunsKernel<float,3,true,false>",
+    KERNELS = {"fused": "FusedBilinear<float,false,false,false,true>",
+               "fused-normalize": "FusedBilinear<float,false,false,true,true>",
+               "fused-chain": "FusedBilinear<float,false,false,false,false> + NormRunsTensor<float,float,3> + "
+                              "ReformatKernel<unsigned int,3,true,false>",
                "fused-copy-bound": "FusedCopyBound"}
     TEXT = {"fused": "scale/offset", "fused-normalize": "per-channel mean/std in the same kernel (extension entry point)",
             "fused-chain": "per-channel mean/std as the three-operator chain fused -> Normalize -> Reformat",
