@@ -10,15 +10,10 @@ namespace nvcvamd {
 
 namespace {
 
-struct PackingRow
-{
-    NVCVPacking packing;
-    int32_t     bits[4];
-};
-
 const PackingRow kPackings[] = {
 #include "PackingTable.inc"
 };
+constexpr int kNumPackings = sizeof(kPackings) / sizeof(kPackings[0]);
 
 const char *const kSwizzles[] = {
 #include "SwizzleTable.inc"
@@ -27,12 +22,12 @@ constexpr int kNumSwizzles = sizeof(kSwizzles) / sizeof(kSwizzles[0]);
 
 inline uint64_t Get(uint64_t v, int off, int len)
 {
-    return NVCV_DETAIL_BITS_GET(v, off, len);
+    return FieldGet(v, off, len);
 }
 
 inline uint64_t Put(uint64_t v, int off, int len)
 {
-    return NVCV_DETAIL_BITS_PUT(v, off, len);
+    return FieldPut(v, off, len);
 }
 
 int BppFromCode(int code, int sub, int nch)
@@ -63,6 +58,24 @@ uint64_t PackSlot(NVCVPacking p, int nsub, int nch, int nbpp)
 
 } // namespace
 
+const PackingRow *FindPacking(NVCVPacking p)
+{
+    for (const PackingRow &row : kPackings)
+    {
+        if (row.packing == p)
+        {
+            return &row;
+        }
+    }
+    return nullptr;
+}
+
+const PackingRow *PackingTable(int *count)
+{
+    *count = kNumPackings;
+    return kPackings;
+}
+
 PackingInfo DecodePacking(NVCVPacking p)
 {
     PackingInfo info = {};
@@ -71,16 +84,14 @@ PackingInfo DecodePacking(NVCVPacking p)
         info.known = true;
         return info;
     }
-    info.numChannels  = (int)Get(p, 4, 2) + 1;
-    info.bitsPerPixel = BppFromCode((int)Get(p, 6, 4), (int)Get(p, 0, 4), info.numChannels);
-    for (const PackingRow &row : kPackings)
+    info.numComponents = (int)Get(p, 4, 2) + 1;
+    // a 4:2:2 pixel pair stores four components for three channels (luma twice)
+    info.numChannels  = (p == NVCV_PACKING_X8_Y8__X8_Z8 || p == NVCV_PACKING_Y8_X8__Z8_X8) ? 3 : info.numComponents;
+    info.bitsPerPixel = BppFromCode((int)Get(p, 6, 4), (int)Get(p, 0, 4), info.numComponents);
+    if (const PackingRow *row = FindPacking(p))
     {
-        if (row.packing == p)
-        {
-            std::memcpy(info.bits, row.bits, sizeof(info.bits));
-            info.known = true;
-            break;
-        }
+        std::memcpy(info.bits, row->bits, sizeof(info.bits));
+        info.known = true;
     }
     return info;
 }
@@ -260,33 +271,125 @@ int FormatPlanePixelStrideBytes(uint64_t fmt, int plane)
 
 uint64_t MakeFormatWord(NVCVColorModel model, uint32_t specOrRaw, NVCVChromaSubsampling css, NVCVMemLayout layout,
                         NVCVDataKind kind, NVCVSwizzle swizzle, NVCVAlphaType alpha, NVCVPacking p0, NVCVPacking p1,
-                        NVCVPacking p2, NVCVPacking p3)
+                        NVCVPacking p2, NVCVPacking p3, const NVCVExtraChannelInfo *ex)
 {
-    uint64_t color;
-    int      m = (int)model;
-    if (m == NVCV_COLOR_MODEL_YCbCr)
+    const bool extra = ex != nullptr && ex->numChannels > 0;
+    return NVCV_DETAIL_FORMAT_WORD_EX((int)model, specOrRaw, (int)css, (int)layout, (int)kind, (int)swizzle, (int)alpha,
+                                      extra ? ex->numChannels : 0, extra ? ex->bitsPerPixel : 0,
+                                      extra ? (int)ex->datakind : 0, extra ? (int)ex->channelType : 0, (uint64_t)p0,
+                                      (uint64_t)p1, (uint64_t)p2, (uint64_t)p3);
+}
+
+NVCVAlphaType FormatAlphaType(uint64_t fmt)
+{
+    return (NVCVAlphaType)Get(fmt, 6, 1);
+}
+
+int FormatRawPattern(uint64_t fmt)
+{
+    return FormatColorModel(fmt) == NVCV_COLOR_MODEL_RAW ? (int)Get(fmt, 21, 6) : -1;
+}
+
+NVCVExtraChannelInfo FormatExtraChannels(uint64_t fmt)
+{
+    NVCVExtraChannelInfo info = {0, 0, NVCV_DATA_KIND_UNSPECIFIED, NVCV_EXTRA_CHANNEL_U};
+    // bit 7 clear = the bits above plane 0's packing describe extra channels, not planes 1..3
+    if (fmt != 0 && Get(fmt, 7, 1) == 0 && Get(fmt, 47, 3) > 0)
     {
-        color = Put(specOrRaw, 20, 15) | Put(css, 17, 3);
+        info.numChannels  = (int32_t)Get(fmt, 47, 3);
+        info.bitsPerPixel = BppFromCode((int)Get(fmt, 50, 3), 4, 2);
+        info.datakind     = (NVCVDataKind)Get(fmt, 53, 3);
+        info.channelType  = (NVCVExtraChannel)Get(fmt, 44, 3);
     }
-    else if (m == NVCV_COLOR_MODEL_UNDEFINED)
+    return info;
+}
+
+NVCVSwizzle MakeSwizzle(NVCVChannel x, NVCVChannel y, NVCVChannel z, NVCVChannel w)
+{
+    const NVCVChannel want[4] = {x, y, z, w};
+    for (int i = 0; i < kNumSwizzles; ++i)
     {
-        color = Put((1u << 19) - 1, 16, 19);
+        NVCVChannel have[4];
+        SwizzleChannels((NVCVSwizzle)i, have);
+        if (std::memcmp(have, want, sizeof(want)) == 0)
+        {
+            return (NVCVSwizzle)i;
+        }
     }
-    else if (m - 2 < 7)
+    return NVCV_SWIZZLE_UNSUPPORTED;
+}
+
+// Argument rules of the reference's format constructors (src/nvcv/src/priv/ImageFormat.cpp:36-235).
+uint64_t MakeCheckedFormat(NVCVColorModel model, uint32_t specOrRaw, NVCVChromaSubsampling css, NVCVMemLayout layout,
+                           NVCVDataKind kind, NVCVSwizzle swizzle, NVCVPacking p0, NVCVPacking p1, NVCVPacking p2,
+                           NVCVPacking p3, NVCVAlphaType alpha, const NVCVExtraChannelInfo *ex)
+{
+    const NVCVPacking pk[4] = {p0, p1, p2, p3};
+    if (p0 == NVCV_PACKING_0)
     {
-        color = Put(1, 16, 1) | Put(specOrRaw, 20, 15) | Put(m - 2, 17, 3);
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Packing of the first plane must not be 0");
     }
-    else if (m == NVCV_COLOR_MODEL_RAW)
+    // plane slots keep 3 bits of the packing's sub-code (planes 0..2) or none (plane 3)
+    for (int i = 0; i < 3; ++i)
     {
-        color = Put(1, 16, 1) | Put(7, 17, 3) | Put(specOrRaw, 21, 6);
+        if (((uint64_t)pk[i] & 8) != 0)
+        {
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Packing %s cannot be stored for plane %d", nvcvPackingGetName(pk[i]), i);
+        }
     }
-    else
+    if (((uint64_t)p3 & 15) != 0)
     {
-        color = Put(1, 16, 1) | Put(7, 17, 3) | Put(1, 20, 1) | Put(m - 10, 21, 6);
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Packing %s cannot be stored for plane 3", nvcvPackingGetName(p3));
     }
-    return Put(kind, 61, 3) | Put(swizzle, 0, 6) | Put(alpha, 6, 1) | Put(layout, 12, 3) | color | Put(1, 7, 1)
-         | Put(PackSlot(p0, 3, 2, 4), 35, 9) | Put(PackSlot(p1, 3, 1, 3), 44, 7) | Put(PackSlot(p2, 3, 1, 3), 51, 7)
-         | Put(PackSlot(p3, 0, 0, 3), 58, 3);
+    int channels = 0;
+    for (int i = 0; i < 4; ++i)
+    {
+        const PackingInfo pi = DecodePacking(pk[i]);
+        if (i >= 1 && pi.bitsPerPixel > (i == 3 ? 64 : 128))
+        {
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Plane %d may have at most %d bits per pixel, not %d", i, i == 3 ? 64 : 128,
+                        pi.bitsPerPixel);
+        }
+        if (i == 1 && pi.numChannels > 2)
+        {
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Plane 1 may have at most 2 channels, not %d", pi.numChannels);
+        }
+        channels += pi.numChannels;
+    }
+    if (SwizzleNumChannels(swizzle) != channels)
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Swizzle %s names %d channels, the packings hold %d", nvcvSwizzleGetName(swizzle),
+                    SwizzleNumChannels(swizzle), channels);
+    }
+    if (model == NVCV_COLOR_MODEL_UNDEFINED && (specOrRaw != (uint32_t)NVCV_COLOR_SPEC_UNDEFINED || css != NVCV_CSS_NONE))
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Without a colour model, colour spec must be undefined and chroma subsampling NONE");
+    }
+    if (model != NVCV_COLOR_MODEL_RAW && model != NVCV_COLOR_MODEL_RGB && model != NVCV_COLOR_MODEL_YCbCr
+        && model != NVCV_COLOR_MODEL_CMYK && model != NVCV_COLOR_MODEL_YCCK && specOrRaw != (uint32_t)NVCV_COLOR_SPEC_UNDEFINED)
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Colour model %s takes no colour spec", nvcvColorModelGetName(model));
+    }
+    if (ex != nullptr)
+    {
+        if (ex->numChannels > NVCV_MAX_EXTRA_CHANNEL_COUNT)
+        {
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "At most %d extra channels, not %d", NVCV_MAX_EXTRA_CHANNEL_COUNT, ex->numChannels);
+        }
+        if (ex->numChannels > 0 && (p1 != NVCV_PACKING_0 || p2 != NVCV_PACKING_0 || p3 != NVCV_PACKING_0))
+        {
+            throw Error(NVCV_ERROR_INVALID_IMAGE_FORMAT, "Extra channels need a single-plane format");
+        }
+        if (ex->bitsPerPixel > 128)
+        {
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Extra channels may have at most 128 bits, not %d", ex->bitsPerPixel);
+        }
+    }
+    if (model != NVCV_COLOR_MODEL_YCbCr && css != NVCV_CSS_NONE)
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Only YCbCr formats have chroma subsampling");
+    }
+    return MakeFormatWord(model, specOrRaw, css, layout, kind, swizzle, alpha, p0, p1, p2, p3, ex);
 }
 
 NVCVDataType FormatPlaneDataType(uint64_t fmt, int plane)
@@ -295,6 +398,10 @@ NVCVDataType FormatPlaneDataType(uint64_t fmt, int plane)
     if (p == NVCV_PACKING_0)
     {
         return NVCV_DATA_TYPE_NONE;
+    }
+    if (p == NVCV_PACKING_X8_Y8__X8_Z8 || p == NVCV_PACKING_Y8_X8__Z8_X8)
+    {
+        p = NVCV_PACKING_X8_Y8; // one pixel of the pair: a luma and a chroma sample
     }
     return NVCV_DETAIL_MAKE_DATA_TYPE(FormatDataKind(fmt), (uint64_t)p);
 }
@@ -344,28 +451,21 @@ int DataTypeStrideBytes(NVCVDataType t)
 
 int DataTypeAlignment(NVCVDataType t)
 {
-    // Machine-word size of one stored component group: for the "_"-separated packings this is the
-    // component size, for sub-word packings the whole pixel.
-    PackingInfo pi = DecodePacking(DataTypePacking(t));
-    if (pi.numChannels == 0)
+    // Machine-word size of one stored component group: for the "_"-separated packings the component size, for
+    // sub-word packings the whole pixel (table column; sub-byte packings count as one byte).
+    const NVCVPacking p = DataTypePacking(t);
+    if (const PackingRow *row = FindPacking(p))
     {
-        return 1;
+        return row->alignment > 0 ? row->alignment : 1;
     }
-    bool uniform = pi.known && pi.bits[0] >= 8;
-    for (int i = 1; uniform && i < pi.numChannels; ++i)
-    {
-        uniform = pi.bits[i] == pi.bits[0];
-    }
-    int bytes = uniform && pi.bits[0] * pi.numChannels == pi.bitsPerPixel ? pi.bits[0] / 8 : (pi.bitsPerPixel + 7) / 8;
-    return (int)NextPow2(bytes);
+    PackingInfo pi = DecodePacking(p);
+    return pi.numComponents == 0 ? 1 : (int)NextPow2((pi.bitsPerPixel + 7) / 8);
 }
-
-namespace {
 
 const char *ThreadName(const char *fmt, ...)
 {
     // Small ring so that a name built from other generated names does not overwrite its inputs.
-    static thread_local char ring[4][256];
+    static thread_local char ring[4][512];
     static thread_local int  next = 0;
     char                    *buf  = ring[next];
     next                          = (next + 1) % 4;
@@ -375,6 +475,13 @@ const char *ThreadName(const char *fmt, ...)
     va_end(va);
     return buf;
 }
+
+const char *EnumName(int v, const char *const *names, int count, const char *type)
+{
+    return (v >= 0 && v < count) ? names[v] : ThreadName("%s(%d)", type, v);
+}
+
+namespace {
 
 const char *KindLetter(NVCVDataKind k)
 {
@@ -393,14 +500,6 @@ const char *KindLetter(NVCVDataKind k)
     }
 }
 
-void CheckPlane(int plane)
-{
-    if (plane < 0 || plane >= 4)
-    {
-        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Plane index must be in [0,4), not %d", plane);
-    }
-}
-
 NVCVStatus MakeFormat(NVCVImageFormat *out, NVCVColorModel model, uint32_t spec, NVCVChromaSubsampling css,
                       NVCVMemLayout layout, NVCVDataKind kind, NVCVSwizzle swizzle, NVCVPacking p0, NVCVPacking p1,
                       NVCVPacking p2, NVCVPacking p3, NVCVAlphaType alpha, const NVCVExtraChannelInfo *ex)
@@ -409,15 +508,7 @@ NVCVStatus MakeFormat(NVCVImageFormat *out, NVCVColorModel model, uint32_t spec,
         [&]
         {
             NotNull(out, "Pointer to output format");
-            if (ex != nullptr && ex->numChannels > 0)
-            {
-                throw Error(NVCV_ERROR_NOT_IMPLEMENTED, "Formats with extra channels are not supported");
-            }
-            if (p0 == NVCV_PACKING_0 && (p1 != NVCV_PACKING_0 || p2 != NVCV_PACKING_0 || p3 != NVCV_PACKING_0))
-            {
-                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Plane packings must be given without gaps");
-            }
-            *out = MakeFormatWord(model, spec, css, layout, kind, swizzle, alpha, p0, p1, p2, p3);
+            *out = MakeCheckedFormat(model, spec, css, layout, kind, swizzle, p0, p1, p2, p3, alpha, ex);
         });
 }
 
@@ -441,11 +532,6 @@ NVCVStatus SetSpecField(NVCVColorSpec *cspec, int off, int len, uint64_t value)
             const uint64_t mask = ((1ULL << len) - 1) << off;
             *cspec = (NVCVColorSpec)(int32_t)((((uint64_t)(uint32_t)EnumValue(*cspec)) & ~mask) | Put(value, off, len));
         });
-}
-
-const char *EnumName(int v, const char *const *names, int count, const char *type)
-{
-    return (v >= 0 && v < count) ? names[v] : ThreadName("%s(%d)", type, v);
 }
 
 } // namespace
@@ -472,16 +558,11 @@ NVCVStatus nvcvMakeSwizzle(NVCVSwizzle *outSwizzle, NVCVChannel x, NVCVChannel y
         [&]
         {
             NotNull(outSwizzle, "Pointer to output swizzle");
-            NVCVChannel want[4] = {x, y, z, w};
-            for (int i = 0; i < kNumSwizzles; ++i)
+            const NVCVSwizzle sw = MakeSwizzle(x, y, z, w);
+            if (sw != NVCV_SWIZZLE_UNSUPPORTED)
             {
-                NVCVChannel have[4];
-                SwizzleChannels((NVCVSwizzle)i, have);
-                if (std::memcmp(have, want, sizeof(want)) == 0)
-                {
-                    *outSwizzle = (NVCVSwizzle)i;
-                    return;
-                }
+                *outSwizzle = sw;
+                return;
             }
             throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Channel combination has no swizzle code");
         });
@@ -489,7 +570,7 @@ NVCVStatus nvcvMakeSwizzle(NVCVSwizzle *outSwizzle, NVCVChannel x, NVCVChannel y
 
 NVCVStatus nvcvPackingGetNumComponents(NVCVPacking packing, int32_t *outNumComponents)
 {
-    return Protect([&] { *NotNull(outNumComponents, "Pointer to output") = DecodePacking(packing).numChannels; });
+    return Protect([&] { *NotNull(outNumComponents, "Pointer to output") = DecodePacking(packing).numComponents; });
 }
 
 NVCVStatus nvcvPackingGetBitsPerComponent(NVCVPacking packing, int32_t *outBits)
@@ -524,36 +605,25 @@ NVCVStatus nvcvPackingGetAlignment(NVCVPacking packing, int32_t *outAlignment)
 
 const char *nvcvDataKindGetName(NVCVDataKind kind)
 {
-    switch (kind)
-    {
-    case NVCV_DATA_KIND_UNSPECIFIED:
-        return "NVCV_DATA_KIND_UNSPECIFIED";
-    case NVCV_DATA_KIND_UNSIGNED:
-        return "NVCV_DATA_KIND_UNSIGNED";
-    case NVCV_DATA_KIND_SIGNED:
-        return "NVCV_DATA_KIND_SIGNED";
-    case NVCV_DATA_KIND_FLOAT:
-        return "NVCV_DATA_KIND_FLOAT";
-    case NVCV_DATA_KIND_COMPLEX:
-        return "NVCV_DATA_KIND_COMPLEX";
-    }
-    return "Unexpected error retrieving NVCVDataKind string representation";
+    static const char *const names[] = {"NVCV_DATA_KIND_UNSPECIFIED", "NVCV_DATA_KIND_UNSIGNED", "NVCV_DATA_KIND_SIGNED",
+                                        "NVCV_DATA_KIND_FLOAT", "NVCV_DATA_KIND_COMPLEX"};
+    const int v = EnumValue(kind);
+    return (v >= -1 && v <= 3) ? names[v + 1] : ThreadName("NVCVDataKind(%d)", v);
 }
 
 const char *nvcvMemLayoutGetName(NVCVMemLayout memlayout)
 {
-    return memlayout == NVCV_MEM_LAYOUT_PITCH_LINEAR ? "NVCV_MEM_LAYOUT_PITCH_LINEAR"
-                                                     : ThreadName("NVCV_MEM_LAYOUT_BLOCK%d_LINEAR",
-                                                                  1 << ((int)memlayout - 1));
+    static const char *const names[] = {"NVCV_MEM_LAYOUT_PITCH_LINEAR",   "NVCV_MEM_LAYOUT_BLOCK1_LINEAR", "NVCV_MEM_LAYOUT_BLOCK2_LINEAR",
+                                        "NVCV_MEM_LAYOUT_BLOCK4_LINEAR",  "NVCV_MEM_LAYOUT_BLOCK8_LINEAR", "NVCV_MEM_LAYOUT_BLOCK16_LINEAR",
+                                        "NVCV_MEM_LAYOUT_BLOCK32_LINEAR"};
+    return EnumName(EnumValue(memlayout), names, 7, "NVCVMemLayout");
 }
 
+// The four channel selectors spelled out, e.g. "XYZ1".
 const char *nvcvSwizzleGetName(NVCVSwizzle swizzle)
 {
-    if ((int)swizzle >= 0 && (int)swizzle < kNumSwizzles)
-    {
-        return ThreadName("NVCV_SWIZZLE_%s", kSwizzles[(int)swizzle]);
-    }
-    return "NVCV_SWIZZLE_UNSUPPORTED";
+    const int v = EnumValue(swizzle);
+    return (v >= 0 && v < kNumSwizzles) ? kSwizzles[v] : ThreadName("NVCVSwizzle(%d)", v);
 }
 
 // ---- colour spec -------------------------------------------------------------------------------
@@ -567,12 +637,13 @@ NVCVStatus nvcvChromaSubsamplingGetNumSamples(NVCVChromaSubsampling css, int32_t
             {
                 throw Error(NVCV_ERROR_INVALID_ARGUMENT, "At least one of the two sample-count outputs must be non-NULL");
             }
-            if ((int)css < 0 || (int)css > 7)
+            const int code = EnumValue(css);
+            if (code < 0 || code > 7)
             {
-                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid chroma subsampling: %d", (int)css);
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid chroma subsampling: %d", code);
             }
             // Evaluate the plane-size rule on a 4x4 luma block of a synthetic YCbCr format.
-            uint64_t fmt = MakeFormatWord(NVCV_COLOR_MODEL_YCbCr, NVCV_COLOR_SPEC_BT601, css, NVCV_MEM_LAYOUT_PL,
+            uint64_t fmt = MakeFormatWord(NVCV_COLOR_MODEL_YCbCr, NVCV_COLOR_SPEC_BT601, (NVCVChromaSubsampling)code, NVCV_MEM_LAYOUT_PL,
                                           NVCV_DATA_KIND_UNSIGNED, NVCV_SWIZZLE_XYZ0, NVCV_ALPHA_ASSOCIATED,
                                           NVCV_PACKING_X8, NVCV_PACKING_X8_Y8, NVCV_PACKING_0, NVCV_PACKING_0);
             int32_t  w, h;
@@ -590,7 +661,8 @@ NVCVStatus nvcvChromaSubsamplingGetNumSamples(NVCVChromaSubsampling css, int32_t
 
 const char *nvcvColorModelGetName(NVCVColorModel cmodel)
 {
-    switch (cmodel)
+    const int value = EnumValue(cmodel);
+    switch (value)
     {
     case NVCV_COLOR_MODEL_UNDEFINED:
         return "NVCV_COLOR_MODEL_UNDEFINED";
@@ -609,14 +681,14 @@ const char *nvcvColorModelGetName(NVCVColorModel cmodel)
     case NVCV_COLOR_MODEL_YCCK:
         return "NVCV_COLOR_MODEL_YCCK";
     }
-    return ThreadName("NVCVColorModel(%d)", (int)cmodel);
+    return ThreadName("NVCVColorModel(%d)", value);
 }
 
 const char *nvcvChromaSubsamplingGetName(NVCVChromaSubsampling css)
 {
     // J:a:b notation (reference: src/nvcv/src/priv/ColorSpec.cpp:447-478)
     static const char *const names[] = {"4:4:4", "4:2:2", "4:2:2R", "4:1:1", "4:1:1R", "4:2:0", "4:1:0", "4:1:0R"};
-    return ((int)css >= 0 && (int)css < 8) ? names[(int)css] : ThreadName("NVCVChromaSubsampling(%d)", (int)css);
+    return EnumName(EnumValue(css), names, 8, "NVCVChromaSubsampling");
 }
 
 NVCVStatus nvcvMakeChromaSubsampling(NVCVChromaSubsampling *outCSS, int32_t samplesHoriz, int32_t samplesVert)
@@ -752,7 +824,7 @@ NVCVStatus nvcvColorModelNeedsColorspec(NVCVColorModel cmodel, int8_t *outBool)
                 *outBool = 0;
                 return;
             }
-            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid color model: %s", nvcvColorModelGetName(cmodel));
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid color model: %d", EnumValue(cmodel));
         });
 }
 
@@ -969,15 +1041,9 @@ NVCVStatus nvcvMakeColorImageFormat(NVCVImageFormat *outFormat, NVCVColorModel c
                                     NVCVPacking packing3, NVCVAlphaType alphaType,
                                     const NVCVExtraChannelInfo *exChannelInfo)
 {
-    if (colorModel == NVCV_COLOR_MODEL_YCbCr || colorModel == NVCV_COLOR_MODEL_UNDEFINED
-        || colorModel == NVCV_COLOR_MODEL_RAW)
+    if (colorModel == NVCV_COLOR_MODEL_RAW)
     {
-        return Protect(
-            [&] {
-                throw Error(NVCV_ERROR_INVALID_ARGUMENT,
-                            "Use the YCbCr / non-colour / raw constructors for colour model %s",
-                            nvcvColorModelGetName(colorModel));
-            });
+        return Protect([&] { throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Raw formats are made by nvcvMakeRawImageFormat"); });
     }
     return MakeFormat(outFormat, colorModel, colorSpec, NVCV_CSS_NONE, memLayout, dataKind, swizzle, packing0,
                       packing1, packing2, packing3, alphaType, exChannelInfo);
@@ -988,7 +1054,7 @@ NVCVStatus nvcvMakeNonColorImageFormat(NVCVImageFormat *outFormat, NVCVMemLayout
                                        NVCVPacking packing2, NVCVPacking packing3, NVCVAlphaType alphaType,
                                        const NVCVExtraChannelInfo *exChannelInfo)
 {
-    return MakeFormat(outFormat, NVCV_COLOR_MODEL_UNDEFINED, 0, NVCV_CSS_NONE, memLayout, dataKind, swizzle, packing0,
+    return MakeFormat(outFormat, NVCV_COLOR_MODEL_UNDEFINED, NVCV_COLOR_SPEC_UNDEFINED, NVCV_CSS_NONE, memLayout, dataKind, swizzle, packing0,
                       packing1, packing2, packing3, alphaType, exChannelInfo);
 }
 
@@ -1042,7 +1108,6 @@ NVCVStatus nvcvImageFormatGetPlanePacking(NVCVImageFormat fmt, int32_t plane, NV
     return Protect(
         [&]
         {
-            CheckPlane(plane);
             *NotNull(outPacking, "Pointer to output") = FormatPlanePacking(fmt, plane);
         });
 }
@@ -1052,7 +1117,6 @@ NVCVStatus nvcvImageFormatGetPlaneNumChannels(NVCVImageFormat fmt, int32_t plane
     return Protect(
         [&]
         {
-            CheckPlane(plane);
             *NotNull(outPlaneNumChannels, "Pointer to output") = DecodePacking(FormatPlanePacking(fmt, plane)).numChannels;
         });
 }
@@ -1062,7 +1126,6 @@ NVCVStatus nvcvImageFormatGetPlaneBitsPerPixel(NVCVImageFormat fmt, int32_t plan
     return Protect(
         [&]
         {
-            CheckPlane(plane);
             *NotNull(outBPP, "Pointer to output") = DecodePacking(FormatPlanePacking(fmt, plane)).bitsPerPixel;
         });
 }
@@ -1072,7 +1135,6 @@ NVCVStatus nvcvImageFormatGetPlanePixelStrideBytes(NVCVImageFormat fmt, int32_t 
     return Protect(
         [&]
         {
-            CheckPlane(plane);
             *NotNull(outStrideBytes, "Pointer to output") = FormatPlanePixelStrideBytes(fmt, plane);
         });
 }
@@ -1082,7 +1144,6 @@ NVCVStatus nvcvImageFormatGetPlaneDataType(NVCVImageFormat fmt, int32_t plane, N
     return Protect(
         [&]
         {
-            CheckPlane(plane);
             *NotNull(outDataType, "Pointer to output") = FormatPlaneDataType(fmt, plane);
         });
 }
@@ -1093,7 +1154,10 @@ NVCVStatus nvcvImageFormatGetPlaneSize(NVCVImageFormat fmt, int32_t plane, int32
     return Protect(
         [&]
         {
-            CheckPlane(plane);
+            if (outPlaneWidth == nullptr && outPlaneHeight == nullptr)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "At least one of the two size outputs must be non-NULL");
+            }
             int32_t w, h;
             FormatPlaneSize(fmt, plane, imgWidth, imgHeight, &w, &h);
             if (outPlaneWidth)
@@ -1160,21 +1224,23 @@ NVCVStatus nvcvImageFormatHasSameDataLayout(NVCVImageFormat a, NVCVImageFormat b
 
 const char *nvcvImageFormatGetName(NVCVImageFormat fmt)
 {
-    if (fmt == NVCV_IMAGE_FORMAT_NONE)
-    {
-        return "NVCV_IMAGE_FORMAT_NONE";
-    }
+    // The formats the reference names (src/nvcv/src/priv/ImageFormat.cpp:1218-1290); every other value, other named
+    // constants included, is spelled out field by field.
     static const struct
     {
         NVCVImageFormat fmt;
         const char     *name;
     } known[] = {
 #define F(x) {NVCV_IMAGE_FORMAT_##x, "NVCV_IMAGE_FORMAT_" #x}
-        F(U8),     F(S8),     F(U16),     F(S16),     F(U32),     F(S32),    F(F16),    F(F32),     F(F64),
-        F(2S16),   F(2F32),   F(Y8),      F(Y8_ER),   F(NV12),    F(NV12_ER), F(UYVY),  F(YUYV),    F(YUV8),
-        F(YUV8p),  F(RGB8),   F(BGR8),    F(RGBA8),   F(BGRA8),   F(RGBf32), F(BGRf32), F(RGBAf32), F(BGRAf32),
-        F(RGBf16), F(BGRf16), F(RGBAf16), F(BGRAf16), F(HSV8),    F(RGB8p),  F(BGR8p),  F(RGBA8p),  F(BGRA8p),
-        F(RGBf32p), F(BGRf32p), F(RGBAf32p), F(BGRAf32p), F(RGBf16p), F(BGRf16p),
+        F(NONE),       F(U8),         F(U8_BL),      F(S8),         F(U16),        F(S16),      F(S16_BL),
+        F(U32),        F(S32),        F(Y8),         F(Y8_BL),      F(Y8_ER),      F(Y8_ER_BL), F(Y16),
+        F(Y16_BL),     F(Y16_ER),     F(Y16_ER_BL),  F(NV12),       F(NV12_BL),    F(NV12_ER),  F(NV12_ER_BL),
+        F(NV24),       F(NV24_BL),    F(NV24_ER),    F(NV24_ER_BL), F(RGB8),       F(RGBA8),    F(BGR8),
+        F(BGRA8),      F(F32),        F(F64),        F(2S16),       F(2S16_BL),    F(2F32),     F(C64),
+        F(2C64),       F(C128),       F(2C128),      F(UYVY),       F(UYVY_BL),    F(UYVY_ER),  F(UYVY_ER_BL),
+        F(VYUY),       F(VYUY_BL),    F(VYUY_ER),    F(VYUY_ER_BL), F(YUYV),       F(YUYV_BL),  F(YUYV_ER),
+        F(YUYV_ER_BL), F(YUV8p),      F(YUV8p_ER),   F(RGB8_1U_U8), F(RGB8_7U_U8), F(RGBA8_3U_U16),
+        F(RGBA8_3POS3D_U32), F(RGB8_3D_F32), F(YCCK8), F(CMYK8),   F(HSV8),       F(RGBAf32),  F(RGBAf32p),
 #undef F
     };
     for (const auto &k : known)
@@ -1184,8 +1250,56 @@ const char *nvcvImageFormatGetName(NVCVImageFormat fmt)
             return k.name;
         }
     }
-    return ThreadName("NVCVImageFormat(%s,%s,%s,%s,planes=%d)", nvcvColorModelGetName(FormatColorModel(fmt)),
-                      nvcvChromaSubsamplingGetName(FormatCSS(fmt)), nvcvDataKindGetName(FormatDataKind(fmt)),
-                      nvcvSwizzleGetName(FormatSwizzle(fmt)), FormatNumPlanes(fmt));
+    std::string          text  = "NVCVImageFormat(";
+    const NVCVColorModel model = FormatColorModel(fmt);
+    text += nvcvColorModelGetName(model);
+    text += ",";
+    if (model == NVCV_COLOR_MODEL_RAW)
+    {
+        text += nvcvRawPatternGetName((NVCVRawPattern)FormatRawPattern(fmt));
+        text += ",";
+    }
+    else if (model != NVCV_COLOR_MODEL_UNDEFINED)
+    {
+        text += nvcvColorSpecGetName(FormatColorSpec(fmt));
+        text += ",";
+        if (model == NVCV_COLOR_MODEL_YCbCr)
+        {
+            text += nvcvChromaSubsamplingGetName(FormatCSS(fmt));
+            text += ",";
+        }
+    }
+    text += nvcvMemLayoutGetName(FormatMemLayout(fmt));
+    text += ",";
+    text += nvcvDataKindGetName(FormatDataKind(fmt));
+    text += ",";
+    text += nvcvSwizzleGetName(FormatSwizzle(fmt));
+    text += FormatAlphaType(fmt) == NVCV_ALPHA_ASSOCIATED ? ",ASSOCIATED" : ",UNASSOCIATED";
+    const NVCVExtraChannelInfo ex = FormatExtraChannels(fmt);
+    if (ex.numChannels > 0)
+    {
+        static const char *const types[] = {"U", "D", "POS3D"};
+        text += "," + std::to_string(ex.numChannels) + "," + std::to_string(ex.bitsPerPixel) + ",";
+        text += nvcvDataKindGetName(ex.datakind);
+        text += ",";
+        text += EnumName((int)ex.channelType, types, 3, "NVCVExtraChannel");
+    }
+    for (int p = 0; p < FormatNumPlanes(fmt); ++p)
+    {
+        text += ",";
+        text += nvcvPackingGetName(FormatPlanePacking(fmt, p));
+    }
+    text += ")";
+    // enumerator names appear without their common prefixes
+    for (const char *prefix : {"NVCV_RAW_", "NVCV_COLOR_MODEL_", "NVCV_COLOR_SPEC_", "NVCV_CSS_", "NVCV_MEM_LAYOUT_", "NVCV_DATA_KIND_",
+                               "NVCV_PACKING_", "NVCV_CHROMA_", "NVCV_YCbCr_", "NVCV_COLOR_", "NVCV_ALPHA_", "NVCV_EXTRA_CHANNEL_"})
+    {
+        const size_t n = std::strlen(prefix);
+        for (size_t at = text.find(prefix); at != std::string::npos; at = text.find(prefix, at))
+        {
+            text.erase(at, n);
+        }
+    }
+    return ThreadName("%s", text.c_str());
 }
 }

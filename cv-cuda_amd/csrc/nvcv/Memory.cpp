@@ -602,6 +602,12 @@ NVCVStatus nvcvConfigSetMaxAllocatorCount(int32_t maxCount)
     return Protect([&] { AllocatorPool().setFixedSize(maxCount); });
 }
 
+NVCVStatus nvcvConfigSetMaxArrayCount(int32_t /*maxCount*/)
+{
+    // No array objects exist in this library, so there is no pool to size.
+    return NVCV_SUCCESS;
+}
+
 uint32_t nvcvGetVersion(void)
 {
     return NVCV_VERSION;

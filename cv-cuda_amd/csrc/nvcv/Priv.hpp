@@ -129,11 +129,41 @@ constexpr int32_t kDefaultBaseAlign = 512;
 // Format decoding (Format.cpp)
 struct PackingInfo
 {
-    int     numChannels;  // components stored per pixel in the plane (0 = plane absent)
-    int     bitsPerPixel; // storage bits per pixel
-    int32_t bits[4];      // bits of each component, 0-terminated
-    bool    known;        // false -> packing value not in the table
+    int     numComponents; // values stored per pixel (group) in the plane (0 = plane absent)
+    int     numChannels;   // image channels they carry: the same, except 3 for the 4:2:2 pixel-pair packings
+    int     bitsPerPixel;  // storage bits per pixel
+    int32_t bits[4];       // bits of each component, 0-terminated
+    bool    known;         // false -> packing value not in the table
 };
+
+// One row of PackingTable.inc.
+struct PackingRow
+{
+    NVCVPacking   packing;
+    const char   *name;
+    NVCVByteOrder order;
+    int32_t       alignment;
+    NVCVSwizzle   swizzle;   // positions of the channels among the stored fields; 0000 = fields are the channels
+    int32_t       fields[4]; // widths of the stored fields in memory order, padding included
+    int32_t       bits[4];   // widths of channels X, Y, Z, W
+};
+const PackingRow *FindPacking(NVCVPacking p);  // nullptr when the value is not a known packing
+const PackingRow *PackingTable(int *count);
+
+inline uint64_t FieldGet(uint64_t v, int off, int len)
+{
+    return NVCV_DETAIL_BITS_GET(v, off, len);
+}
+
+inline uint64_t FieldPut(uint64_t v, int off, int len)
+{
+    return NVCV_DETAIL_BITS_PUT(v, off, len);
+}
+
+// printf into one of a few per-thread buffers; the result stays valid for the next three calls of the thread.
+const char *ThreadName(const char *fmt, ...);
+// names[v] for v in [0,count), otherwise "<type>(<v>)".
+const char *EnumName(int v, const char *const *names, int count, const char *type);
 
 PackingInfo           DecodePacking(NVCVPacking p);
 NVCVPacking           FormatPlanePacking(uint64_t fmt, int plane); // plane in [0,4)
@@ -152,7 +182,16 @@ void                  SwizzleChannels(NVCVSwizzle sw, NVCVChannel out[4]);
 int                   SwizzleNumChannels(NVCVSwizzle sw);
 uint64_t              MakeFormatWord(NVCVColorModel model, uint32_t specOrRaw, NVCVChromaSubsampling css,
                                      NVCVMemLayout layout, NVCVDataKind kind, NVCVSwizzle swizzle, NVCVAlphaType alpha,
-                                     NVCVPacking p0, NVCVPacking p1, NVCVPacking p2, NVCVPacking p3);
+                                     NVCVPacking p0, NVCVPacking p1, NVCVPacking p2, NVCVPacking p3,
+                                     const NVCVExtraChannelInfo *ex = nullptr);
+NVCVAlphaType         FormatAlphaType(uint64_t fmt);
+NVCVExtraChannelInfo  FormatExtraChannels(uint64_t fmt);
+int                   FormatRawPattern(uint64_t fmt); // -1 when the colour model is not RAW
+NVCVSwizzle           MakeSwizzle(NVCVChannel x, NVCVChannel y, NVCVChannel z, NVCVChannel w); // UNSUPPORTED if not in the table
+// Validating constructor behind every nvcvMake*ImageFormat entry point and the setters that rebuild a format.
+uint64_t MakeCheckedFormat(NVCVColorModel model, uint32_t specOrRaw, NVCVChromaSubsampling css, NVCVMemLayout layout,
+                           NVCVDataKind kind, NVCVSwizzle swizzle, NVCVPacking p0, NVCVPacking p1, NVCVPacking p2,
+                           NVCVPacking p3, NVCVAlphaType alpha, const NVCVExtraChannelInfo *ex);
 
 inline NVCVPacking DataTypePacking(NVCVDataType t)
 {

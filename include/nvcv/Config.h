@@ -18,6 +18,9 @@ NVCV_PUBLIC NVCVStatus nvcvConfigSetMaxImageCount(int32_t maxCount);
 NVCV_PUBLIC NVCVStatus nvcvConfigSetMaxImageBatchCount(int32_t maxCount);
 NVCV_PUBLIC NVCVStatus nvcvConfigSetMaxTensorCount(int32_t maxCount);
 NVCV_PUBLIC NVCVStatus nvcvConfigSetMaxAllocatorCount(int32_t maxCount);
+/* Accepted for source compatibility with callers of nvcv/Config.hpp; this library has no array objects, so the
+ * limit has nothing to act on. */
+NVCV_PUBLIC NVCVStatus nvcvConfigSetMaxArrayCount(int32_t maxCount);
 
 #ifdef __cplusplus
 }

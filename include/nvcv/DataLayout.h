@@ -195,6 +195,12 @@ NVCV_PUBLIC NVCVStatus nvcvSwizzleGetNumChannels(NVCVSwizzle swizzle, int32_t *o
 NVCV_PUBLIC NVCVStatus nvcvMakeSwizzle(NVCVSwizzle *outSwizzle, NVCVChannel x, NVCVChannel y, NVCVChannel z,
                                        NVCVChannel w);
 
+/* The packing with the given field widths, channel positions and byte order; a word of a single channel matches
+ * either byte order, and `alignment` does not take part in the choice. INVALID_ARGUMENT when no packing fits. nvcvPackingGetParams is the way
+ * back; its `bits` are the widths of the stored fields in memory order, padding included.
+ * (reference: DataLayout.h:498-527) */
+NVCV_PUBLIC NVCVStatus nvcvMakePacking(NVCVPacking *outPacking, const NVCVPackingParams *params);
+NVCV_PUBLIC NVCVStatus nvcvPackingGetParams(NVCVPacking packing, NVCVPackingParams *outParams);
 NVCV_PUBLIC NVCVStatus nvcvPackingGetNumComponents(NVCVPacking packing, int32_t *outNumComponents);
 NVCV_PUBLIC NVCVStatus nvcvPackingGetBitsPerComponent(NVCVPacking packing, int32_t *outBits /* [4] */);
 NVCV_PUBLIC NVCVStatus nvcvPackingGetBitsPerPixel(NVCVPacking packing, int32_t *outBPP);
@@ -203,6 +209,9 @@ NVCV_PUBLIC NVCVStatus nvcvPackingGetAlignment(NVCVPacking packing, int32_t *out
 NVCV_PUBLIC const char *nvcvDataKindGetName(NVCVDataKind kind);
 NVCV_PUBLIC const char *nvcvMemLayoutGetName(NVCVMemLayout memlayout);
 NVCV_PUBLIC const char *nvcvSwizzleGetName(NVCVSwizzle swizzle);
+NVCV_PUBLIC const char *nvcvPackingGetName(NVCVPacking packing);
+NVCV_PUBLIC const char *nvcvChannelGetName(NVCVChannel channel);
+NVCV_PUBLIC const char *nvcvByteOrderGetName(NVCVByteOrder byteOrder);
 
 #ifdef __cplusplus
 }

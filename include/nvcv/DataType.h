@@ -23,6 +23,9 @@ typedef uint64_t NVCVDataType;
                                            packing, 0, 0, 0))
 #define NVCV_DETAIL_DATA_TYPE(kind, packing) NVCV_DETAIL_MAKE_DATA_TYPE(NVCV_DATA_KIND_##kind, NVCV_PACKING_##packing)
 
+/* Compile-time construction of a data type without a named constant (reference: DataType.h:172-190). */
+#define NVCV_MAKE_DATA_TYPE(dataKind, packing) NVCV_DETAIL_MAKE_DATA_TYPE(dataKind, packing)
+
 #define NVCV_DATA_TYPE_NONE ((NVCVDataType)0)
 
 /* <n><kind><bits>: n interleaved components (omitted when 1) of kind U/S/F/C with that many bits each. */

@@ -5,6 +5,7 @@
 
 #include "Fwd.h"
 #include "ImageFormat.h"
+#include "detail/CudaFwd.h"
 
 #include <stdint.h>
 
@@ -32,8 +33,8 @@ typedef struct NVCVImageBufferStridedRec
 /* Layout placeholder for the reference's texture-array variant; never produced or accepted here. */
 typedef struct NVCVImageBufferCudaArrayRec
 {
-    int32_t numPlanes;
-    void   *planes[NVCV_MAX_PLANE_COUNT];
+    int32_t     numPlanes;
+    cudaArray_t planes[NVCV_MAX_PLANE_COUNT];
 } NVCVImageBufferCudaArray;
 
 typedef enum

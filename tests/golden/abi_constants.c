@@ -16,6 +16,7 @@
 
 int main(void)
 {
+#include "abi_constants_all.inc"
     V(NVCV_IMAGE_FORMAT_U8);
     V(NVCV_IMAGE_FORMAT_S8);
     V(NVCV_IMAGE_FORMAT_U16);

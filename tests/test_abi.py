@@ -140,3 +140,118 @@ def test_symbol_versions_match_reference_tags(cv):
     assert "cvcudaResizeCropConvertReformatSubmit@@CVCUDA_0.10" in subprocess.run(
         ["nm", "-D", "--with-symbol-versions", os.path.join(root, "cv-cuda_amd", "lib", "libcvcuda.so")],
         capture_output=True, text=True).stdout
+
+
+# ---- the reference's header-only C++ wrappers, used unchanged -------------------------------------------------
+REF = "/root/reference"
+REF_NVCV_HPP = os.path.join(REF, "src/nvcv/src/include/nvcv")
+REF_CVCUDA_HPP = os.path.join(REF, "src/cvcuda/include/cvcuda")
+needs_reference = pytest.mark.skipif(not os.path.isdir(REF_NVCV_HPP), reason="the reference tree is only present in the build container")
+
+
+def merged_include_tree(dst):
+    """include/ of this repository plus the reference's C++ wrapper headers (*.hpp, *.inc), copied at test time into a
+    scratch directory: the wrappers include their C headers with quotes, so both must sit in one tree. The operator
+    wrappers get the one change a caller makes on this platform: the runtime header and the stream type are HIP's."""
+    import shutil
+    shutil.copytree(INC, dst)
+    for src, sub, patch in ((REF_NVCV_HPP, "nvcv", False), (REF_CVCUDA_HPP, "cvcuda", True)):
+        for dp, _, fs in os.walk(src):
+            for f in fs:
+                if f.endswith((".hpp", ".inc")):
+                    out = os.path.join(dst, sub, os.path.relpath(os.path.join(dp, f), src))
+                    os.makedirs(os.path.dirname(out), exist_ok=True)
+                    text = open(os.path.join(dp, f)).read()
+                    if patch:
+                        text = text.replace("cuda_runtime.h", "hip/hip_runtime.h").replace("cudaStream_t", "hipStream_t")
+                    open(out, "w").write(text)
+    return dst
+
+
+@needs_reference
+def test_reference_cpp_wrappers_compile_unchanged(tmp_path):
+    """nvcv/*.hpp for every object this library has, and cvcuda/Op*.hpp for every operator it has (reference:
+    src/cvcuda/include/cvcuda/OpResizeCropConvertReformat.hpp:63-92 and siblings), in one translation unit."""
+    tree = merged_include_tree(str(tmp_path / "inc"))
+    ops = sorted(f[:-2] for f in os.listdir(os.path.join(INC, "cvcuda")) if f.startswith("Op") and f.endswith(".h") and f != "Operator.h")
+    assert "OpResizeCropConvertReformat" in ops and len(ops) >= 12
+    nvcv = ["Tensor", "TensorData", "TensorDataAccess", "TensorLayout", "TensorShape", "Image", "ImageData", "ImageBatch", "ImageBatchData",
+            "ImageFormat", "DataType", "DataLayout", "ColorSpec", "Size", "Status", "Exception", "Config", "alloc/Allocator", "alloc/Requirements"]
+    tu = tmp_path / "tu.cpp"
+    tu.write_text("".join("#include <nvcv/%s.hpp>\n" % h for h in nvcv) + "".join("#include <cvcuda/%s.hpp>\n" % o for o in ops)
+                  + "void use(hipStream_t s, cvcuda::ResizeCropConvertReformat &op, const nvcv::Tensor &a, const nvcv::Tensor &b,\n"
+                    "         const nvcv::ImageBatchVarShape &batch)\n"
+                    "{\n"
+                    "    op(s, a, b, NVCVSize2D{455, 256}, NVCV_INTERP_LINEAR, int2{115, 16}, NVCV_CHANNEL_NO_OP, 1.f / 255, 0.f, false);\n"
+                    "    op(s, batch, b, NVCVSize2D{455, 256}, NVCV_INTERP_LINEAR, int2{115, 16}, NVCV_CHANNEL_REVERSE, 1.f, 0.f, true);\n"
+                    "}\n")
+    r = subprocess.run(["hipcc", "-std=c++17", "-fsyntax-only", "--cuda-host-only", "--offload-arch=gfx950", "-Wall", "-I" + tree, str(tu)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-4000:]
+
+
+HOST_PROGRAM = r"""
+#include <nvcv/ColorSpec.hpp>
+#include <nvcv/DataType.hpp>
+#include <nvcv/Exception.hpp>
+#include <nvcv/ImageFormat.hpp>
+#include <nvcv/Tensor.hpp>
+#include <nvcv/TensorLayout.hpp>
+#include <cstdio>
+int main()
+{
+    static_assert(nvcv::FMT_NV12.cvalue() == NVCV_IMAGE_FORMAT_NV12, "constexpr formats");
+    constexpr nvcv::ImageFormat made = nvcv::ImageFormat::ConstCreate(nvcv::ColorModel::RGB, nvcv::CSPEC_UNDEFINED, nvcv::MemLayout::PL,
+                                                                     nvcv::DataKind::UNSIGNED, nvcv::Swizzle::S_XYZ1, nvcv::Packing::X8_Y8_Z8);
+    static_assert(made == nvcv::FMT_RGB8, "constexpr construction");
+    nvcv::ImageFormat nv12 = nvcv::FMT_NV12;
+    std::printf("planes %d channels %d\n", nv12.numPlanes(), nv12.numChannels());
+    std::printf("plane1 %s\n", nvcvDataTypeGetName(nv12.planeDataType(1)));
+    nvcv::Size2D half = nv12.planeSize({1920, 1080}, 1);
+    std::printf("plane1 size %dx%d\n", half.w, half.h);
+    std::printf("edited %s\n", nvcvImageFormatGetName(nv12.memLayout(nvcv::MemLayout::BL).colorSpec(nvcv::CSPEC_BT709).cvalue()));
+    std::printf("fourcc %08x\n", nvcv::FMT_YUYV.fourCC());
+    std::printf("from planes %d\n", nvcv::ImageFormat::FromPlanes(nv12.planeFormat(0), nv12.planeFormat(1)) == nv12);
+    nvcv::DataType t = nvcv::TYPE_3F32;
+    std::printf("type %s bpp %d channels %d stride %d\n", nvcvDataTypeGetName(t), t.bitsPerPixel(), t.numChannels(), t.strideBytes());
+    std::printf("layout rank %d C at %d\n", nvcv::TENSOR_NHWC.rank(), nvcv::TENSOR_NHWC.find('C'));
+    nvcv::Tensor::Requirements req = nvcv::Tensor::CalcRequirements(64, nvcv::Size2D{224, 224}, nvcv::FMT_RGBf32p);
+    std::printf("tensor rank %d layout %s strides %lld %lld %lld %lld\n", req.rank, req.layout.data, (long long)req.strides[0],
+                (long long)req.strides[1], (long long)req.strides[2], (long long)req.strides[3]);
+    try
+    {
+        nvcv::Tensor::CalcRequirements(nvcv::TensorShape({-4, 2}, "HW"), nvcv::TYPE_U8);
+        std::printf("no error\n");
+    }
+    catch (nvcv::Exception &e)
+    {
+        std::printf("status %d\n", (int)e.code());
+    }
+    return 0;
+}
+"""
+
+
+@needs_reference
+def test_reference_cpp_wrappers_link_and_run_against_the_core_library(cv, tmp_path):
+    """A host-only program written against the reference's C++ API (formats, data types, layouts, tensor requirements,
+    exceptions) builds with g++ against libnvcv_types.so and prints what the C API's own tests expect."""
+    import cvcuda_amd._capi as capi
+    libdir = os.path.dirname(capi.nvcv._name)
+    tree = merged_include_tree(str(tmp_path / "inc"))
+    src = tmp_path / "host.cpp"
+    src.write_text(HOST_PROGRAM)
+    exe = tmp_path / "host"
+    subprocess.run(["g++", "-std=c++17", "-DCVCUDA_NO_HIP_HEADERS", "-I" + tree, str(src), "-L" + libdir, "-lnvcv_types",
+                    "-Wl,-rpath," + libdir, "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines()
+    assert out == ["planes 2 channels 3",
+                   "plane1 NVCV_DATA_TYPE_2U8",
+                   "plane1 size 960x540",
+                   "edited NVCVImageFormat(YCbCr,BT709,4:2:0,BLOCK2_LINEAR,UNSIGNED,XYZ0,ASSOCIATED,X8,X8_Y8)",
+                   "fourcc %08x" % sum(ord(c) << (8 * i) for i, c in enumerate("YUY2")),
+                   "from planes 1",
+                   "type NVCV_DATA_TYPE_3F32 bpp 96 channels 3 stride 12",
+                   "layout rank 4 C at 3",
+                   "tensor rank 4 layout NCHW strides 602112 200704 896 4",
+                   "status 2"]
