@@ -26,7 +26,7 @@ import time
 
 HBM_PEAK_GBS = 8000.0
 SEED_BASE = 0xC0FFEE00
-NEAREST, LINEAR, CUBIC = 0, 1, 2
+NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
 
 # HBM bytes one launch of a workload's kernel moves, from hardware counters (rocprofv3 --pmc
 # FETCH_SIZE and --pmc WRITE_SIZE in separate runs, each scaled by what the same counter reads for a
@@ -474,7 +474,19 @@ class Streaming:
                                "ResizeLinearPairsU8Kernel<3>", "f32", "Resize LINEAR 1920x1080 -> 1280x720"),
         "resize-linear-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
                                   "ResizeLinearPairsU8Kernel<3>", "f32", "Resize LINEAR 1280x720 -> 1920x1080"),
+        "resize-area-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
+                             "ResizeTensorKernel<unsigned char,3,3>", "f32", "Resize AREA 1920x1080 -> 1280x720"),
+        "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t>>", "f32",
+                             "CvtColor BGR2HSV"),
+        "cvtcolor-bgr2nv12": ("CvtColor", 32, ("uint8", 3), ("uint8", 1, "NHWC", 1620, 1920),
+                              "PixelTensor<Yuv420FromBgr<3,true>>", "int32", "CvtColor BGR2YUV_NV12"),
+        "cvtcolor-yuy2-bgr": ("CvtColor", 32, ("uint8", 1, 1080, 3840), ("uint8", 3, "NHWC", 1080, 1920), "PixelTensor<BgrFromYuv422<3>>", "int32",
+                              "CvtColor YUV2BGR_YUY2"),
     }
+    # what differs from the operator's default call above: colour code by name, interpolation
+    CODES = {"cvtcolor-bgr2rgb": "COLOR_BGR2RGB", "cvtcolor-bgr2gray": "COLOR_BGR2GRAY", "cvtcolor-bgr2hsv": "COLOR_BGR2HSV",
+             "cvtcolor-bgr2nv12": "COLOR_BGR2YUV_NV12", "cvtcolor-yuy2-bgr": "COLOR_YUV2BGR_YUY2"}
+    INTERP = {"resize-area-720p": AREA}
 
     def __init__(self, cv, orc, np, torch, key):
         self.cv, self.orc, self.np, self.torch, self.key = cv, orc, np, torch, key
@@ -507,7 +519,7 @@ class Streaming:
     def submit(self, stream, s):
         K = self.cv.K
         if self.opname == "CvtColor":
-            self.op(stream, s[0], s[1], K.COLOR_BGR2RGB if self.dc == 3 else K.COLOR_BGR2GRAY)
+            self.op(stream, s[0], s[1], getattr(K, self.CODES[self.key]))
         elif self.opname == "Normalize":
             self.op(stream, s[0], self.tbase, self.tscale, s[1], 1.0, 0.0, 0.0, 0)
         elif self.opname == "Reformat":
@@ -517,10 +529,25 @@ class Streaming:
         elif self.opname == "Flip":
             self.op(stream, s[0], s[1], 1)
         else:
-            self.op(stream, s[0], s[1], LINEAR)
+            self.op(stream, s[0], s[1], self.INTERP.get(self.key, LINEAR))
+
+    def _color_oracle(self):
+        if not hasattr(self, "_col"):
+            import importlib.util
+            spec = importlib.util.spec_from_file_location(
+                "color_oracle", os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "color_oracle.py"))
+            self._col = importlib.util.module_from_spec(spec)
+            spec.loader.exec_module(self._col)
+        return self._col
 
     def _reference(self, a, threads=1):
         np, orc = self.np, self.orc
+        if self.key == "cvtcolor-bgr2hsv":
+            return self._color_oracle().hsv_from_bgr(a, True, False)
+        if self.key == "cvtcolor-bgr2nv12":
+            return self._color_oracle().yuv420_from_bgr(a, True, 0, False)
+        if self.key == "cvtcolor-yuy2-bgr":
+            return self._color_oracle().bgr_from_yuv422(a, True, 0, 0, 3)
         if self.opname == "CvtColor":
             if self.dc == 3:
                 return np.ascontiguousarray(a[..., ::-1])
@@ -534,13 +561,16 @@ class Streaming:
             return orc.convert_to(a, np.float32, 1.0 / 255.0, 0.0, 1)
         if self.opname == "Flip":
             return np.ascontiguousarray(a[:, :, ::-1])
-        return orc.resize(a, (self.dh, self.dw), LINEAR, variant=1, threads=threads)
+        return orc.resize(a, (self.dh, self.dw), self.INTERP.get(self.key, LINEAR), variant=1, threads=threads)
 
     def check(self, s):
         got = s[1].torch_view()[:1].cpu().numpy()
         ref = self._reference(self.host1)
         if self.ddt == self.np.float32:
             assert (self.np.abs(got - ref) <= 1e-5 * self.np.maximum(1.0, self.np.abs(ref))).all()
+        elif self.key == "cvtcolor-bgr2hsv":  # float path: products may round apart by one step on a few pixels
+            assert self.np.abs(got.astype(self.np.int16) - ref.astype(self.np.int16)).max() <= 1
+            assert (got != ref).mean() < 1e-3
         else:
             assert (got == ref).all(), "bench output differs from the oracle"
 
