@@ -191,11 +191,36 @@ struct BgrFromYuv
     }
 };
 
+// The two quotients of the integer HSV formula, (hrange << 12) / (6 i) and (255 << 12) / i for i in [0, 256),
+// rounded to nearest: a table in the reference (cvt_color.cu:232-270, filled on the host). Here each block
+// fills its own copy in LDS, one entry of each per thread, so a pixel costs two LDS reads instead of two
+// float divisions (which are a dozen instructions each).
+__device__ __forceinline__ int32_t *HsvDivTable()
+{
+    __shared__ int32_t table[512];
+    return table;
+}
+
 template<class T>
 struct HsvFromBgr
 {
     static constexpr int kItemW = 1, kItemH = 1;
     using Src = Px<T, 3>;
+    static constexpr bool kBlockPrepare = std::is_integral_v<T>;
+
+    // called by every thread of a 256-thread block before any of them returns
+    static __device__ __forceinline__ void Prepare(const PixArgs &a)
+    {
+        if constexpr (kBlockPrepare)
+        {
+            const int hrange = a.full ? 256 : 180;
+            const int i      = threadIdx.x;
+            int32_t  *t      = HsvDivTable();
+            t[i]             = i == 0 ? 0 : SaturateCast<int32_t>((float)(255 << 12) / (float)i);
+            t[256 + i]       = i == 0 ? 0 : SaturateCast<int32_t>((float)(hrange << 12) / (6.f * i));
+            __syncthreads();
+        }
+    }
 
     static __device__ __forceinline__ auto Map(const Src &s, const PixArgs &a)
     {
@@ -208,8 +233,9 @@ struct HsvFromBgr
             const int val  = max(b, max(g, r));
             const int diff = val - vmin;
             const int vr = val == r ? -1 : 0, vg = val == g ? -1 : 0;
-            const int hdiv = diff == 0 ? 0 : SaturateCast<int32_t>((float)(hrange << 12) / (6.f * diff));
-            const int sdiv = val == 0 ? 0 : SaturateCast<int32_t>((float)(255 << 12) / (float)val);
+            const int32_t *table = HsvDivTable();
+            const int      hdiv  = table[256 + diff];
+            const int      sdiv  = table[val];
             const int sat  = (diff * sdiv + (1 << 11)) >> 12;
             int       h    = (vr & (g - b)) + (~vr & ((vg & (b - r + 2 * diff)) + ((~vg) & (r - g + 4 * diff))));
             h              = (h * hdiv + (1 << 11)) >> 12;
@@ -588,9 +614,23 @@ __device__ __forceinline__ void MapRun(const uint8_t *srcRow, uint8_t *dstRow, i
     StoreRowRunNT<TD, P * D::kC>(dstRow + (int64_t)(x0 - lane * P) * sizeof(D), out, lane, lanes);
 }
 
+template<class Op, class = void>
+struct HasBlockPrepare : std::false_type
+{
+};
+
+template<class Op>
+struct HasBlockPrepare<Op, std::enable_if_t<Op::kBlockPrepare>> : std::true_type
+{
+};
+
 template<class Op>
 __global__ __launch_bounds__(256) void MapTensor(const PixArgs a)
 {
+    if constexpr (HasBlockPrepare<Op>::value)
+    {
+        Op::Prepare(a);
+    }
     const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kMapRun<Op>;
     const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= a.W || y >= a.H)
@@ -616,6 +656,10 @@ constexpr int kMapVarRows = kVarShapeRows<MapPieceBytes<Op>()>;
 template<class Op>
 __global__ __launch_bounds__(256) void MapVarShape(const PixArgs a, const VarTiles tiles)
 {
+    if constexpr (HasBlockPrepare<Op>::value)
+    {
+        Op::Prepare(a);
+    }
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
