@@ -51,11 +51,6 @@ int BppFromCode(int code, int sub, int nch)
     }
 }
 
-uint64_t PackSlot(NVCVPacking p, int nsub, int nch, int nbpp)
-{
-    return NVCV_DETAIL_PACKING_SLOT((uint64_t)p, nsub, nch, nbpp);
-}
-
 } // namespace
 
 const PackingRow *FindPacking(NVCVPacking p)
@@ -482,23 +477,6 @@ const char *EnumName(int v, const char *const *names, int count, const char *typ
 }
 
 namespace {
-
-const char *KindLetter(NVCVDataKind k)
-{
-    switch (k)
-    {
-    case NVCV_DATA_KIND_UNSIGNED:
-        return "U";
-    case NVCV_DATA_KIND_SIGNED:
-        return "S";
-    case NVCV_DATA_KIND_FLOAT:
-        return "F";
-    case NVCV_DATA_KIND_COMPLEX:
-        return "C";
-    default:
-        return "?";
-    }
-}
 
 NVCVStatus MakeFormat(NVCVImageFormat *out, NVCVColorModel model, uint32_t spec, NVCVChromaSubsampling css,
                       NVCVMemLayout layout, NVCVDataKind kind, NVCVSwizzle swizzle, NVCVPacking p0, NVCVPacking p1,
@@ -968,37 +946,38 @@ NVCVStatus nvcvDataTypeGetNumChannels(NVCVDataType type, int32_t *outNumChannels
 
 NVCVStatus nvcvDataTypeGetChannelType(NVCVDataType type, int32_t channel, NVCVDataType *outChannelType)
 {
+    // reference: src/nvcv/src/priv/DataType.cpp:51-78. The type of one channel is the one-channel packing of that
+    // many bits (10-, 12-, 14- and 20-bit channels: the form padded to the next word, X10b6 ...); a width no
+    // one-channel packing has is an error, a channel the type does not have is NVCV_DATA_TYPE_NONE.
     return Protect(
         [&]
         {
             NotNull(outChannelType, "Pointer to output");
-            PackingInfo pi = DecodePacking(DataTypePacking(type));
-            if (channel < 0 || channel >= pi.numChannels || !pi.known)
+            if (channel < 0)
             {
-                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Channel %d does not exist in this data type", channel);
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Channel must be >= 0, not %d", channel);
             }
-            NVCVPacking one;
-            switch (pi.bits[channel])
+            const PackingInfo pi   = DecodePacking(DataTypePacking(type));
+            const int         bits = channel < 4 ? pi.bits[channel] : 0;
+            if (bits == 0)
             {
-            case 8:
-                one = NVCV_PACKING_X8;
-                break;
-            case 16:
-                one = NVCV_PACKING_X16;
-                break;
-            case 32:
-                one = NVCV_PACKING_X32;
-                break;
-            case 64:
-                one = NVCV_PACKING_X64;
-                break;
-            case 128:
-                one = NVCV_PACKING_X128;
-                break;
-            default:
-                throw Error(NVCV_ERROR_NOT_IMPLEMENTED, "Channels of %d bits are not supported", pi.bits[channel]);
+                *outChannelType = NVCV_DATA_TYPE_NONE;
+                return;
             }
-            *outChannelType = NVCV_DETAIL_MAKE_DATA_TYPE(FormatDataKind(type), (uint64_t)one);
+            const int pad = (bits == 10 || bits == 12 || bits == 14) ? 16 - bits : bits == 20 ? 12 : 0;
+            int       count;
+            const PackingRow *rows = PackingTable(&count);
+            for (int i = 0; i < count; ++i)
+            {
+                const PackingRow &r = rows[i];
+                if (r.fields[0] == bits && r.fields[1] == pad && r.fields[2] == 0 && r.fields[3] == 0 && r.bits[0] == bits
+                    && r.bits[1] == 0)
+                {
+                    *outChannelType = NVCV_DETAIL_MAKE_DATA_TYPE(FormatDataKind(type), (uint64_t)r.packing);
+                    return;
+                }
+            }
+            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "No data type has one channel of %d bits", bits);
         });
 }
 
@@ -1009,19 +988,32 @@ NVCVStatus nvcvDataTypeGetStrideBytes(NVCVDataType type, int32_t *outStrideBytes
 
 const char *nvcvDataTypeGetName(NVCVDataType type)
 {
-    if (type == NVCV_DATA_TYPE_NONE)
+    // the types the reference names (src/nvcv/src/priv/DataType.cpp:83-160); any other is spelled out
+    static const struct
     {
-        return "NVCV_DATA_TYPE_NONE";
-    }
-    PackingInfo pi = DecodePacking(DataTypePacking(type));
-    if (pi.known && pi.numChannels > 0 && pi.bits[0] * pi.numChannels == pi.bitsPerPixel)
+        NVCVDataType type;
+        const char  *name;
+    } known[] = {
+#define T(x) {NVCV_DATA_TYPE_##x, "NVCV_DATA_TYPE_" #x}
+        T(NONE), T(U8),  T(2U8),  T(3U8),  T(4U8),  T(S8),  T(2S8),  T(3S8),  T(4S8),  T(U16), T(2U16), T(3U16), T(4U16),
+        T(S16),  T(2S16), T(3S16), T(4S16), T(U32), T(2U32), T(3U32), T(4U32), T(S32), T(2S32), T(3S32), T(4S32), T(F16),
+        T(2F16), T(3F16), T(4F16), T(F32), T(2F32), T(3F32), T(4F32), T(U64), T(2U64), T(3U64), T(4U64), T(S64), T(2S64),
+        T(3S64), T(4S64), T(F64), T(2F64), T(3F64), T(4F64), T(C64), T(2C64), T(3C64), T(4C64), T(C128), T(2C128),
+#undef T
+    };
+    for (const auto &k : known)
     {
-        return pi.numChannels == 1
-                 ? ThreadName("NVCV_DATA_TYPE_%s%d", KindLetter(FormatDataKind(type)), pi.bits[0])
-                 : ThreadName("NVCV_DATA_TYPE_%d%s%d", pi.numChannels, KindLetter(FormatDataKind(type)), pi.bits[0]);
+        if (k.type == type)
+        {
+            return k.name;
+        }
     }
-    return ThreadName("NVCVDataType(%s,packing=%d)", nvcvDataKindGetName(FormatDataKind(type)),
-                      (int)DataTypePacking(type));
+    const char *kind = nvcvDataKindGetName(FormatDataKind(type));
+    const char *pack = nvcvPackingGetName(DataTypePacking(type));
+    // enumerator names without their common prefixes
+    kind = std::strncmp(kind, "NVCV_DATA_KIND_", 15) == 0 ? kind + 15 : kind;
+    pack = std::strncmp(pack, "NVCV_PACKING_", 13) == 0 ? pack + 13 : pack;
+    return ThreadName("NVCVDataType(%s,%s)", kind, pack);
 }
 
 // ---- image format ------------------------------------------------------------------------------

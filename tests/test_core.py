@@ -121,7 +121,8 @@ def test_data_type_queries(cv, capi, K):
         assert nv.nvcvDataTypeGetAlignment(dt, C.byref(v)) == 0 and v.value == align
     ch = C.c_uint64()
     assert nv.nvcvDataTypeGetChannelType(K.DATA_TYPE_3F32, 2, C.byref(ch)) == 0 and ch.value == K.DATA_TYPE_F32
-    assert nv.nvcvDataTypeGetChannelType(K.DATA_TYPE_3F32, 3, C.byref(ch)) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvDataTypeGetChannelType(K.DATA_TYPE_3F32, 3, C.byref(ch)) == 0 and ch.value == K.DATA_TYPE_NONE
+    assert nv.nvcvDataTypeGetChannelType(K.DATA_TYPE_3F32, -1, C.byref(ch)) == capi.NVCV_ERROR_INVALID_ARGUMENT
     n = C.c_int32()
     assert nv.nvcvSwizzleGetNumChannels(K.SWIZZLE_XXX1, C.byref(n)) == 0 and n.value == 1
     assert nv.nvcvSwizzleGetNumChannels(K.SWIZZLE_ZYXW, C.byref(n)) == 0 and n.value == 4

@@ -586,3 +586,94 @@ def test_packing_edge_cases(nv, K):
     for align in (0, 1, 8):
         assert nv.nvcvMakePacking(C.byref(out), C.byref(PackingParams(K.ORDER_MSB, align, K.SWIZZLE_XY00, (C.c_int32 * 4)(16, 16, 0, 0)))) == 0
         assert out.value == K.PACKING_X16_Y16
+
+
+# ---- data types: tests/nvcv_types/system/TestDataType.cpp ---------------------------------------------------
+def make_type(nv, K, kind, packing):
+    t = C.c_uint64()
+    assert nv.nvcvMakeDataType(C.byref(t), const(K, "DATA_KIND_" + kind), const(K, "PACKING_" + packing)) == 0
+    return t.value
+
+
+def dtype(nv, K, spec):
+    """'U8' -> the named constant, ('FLOAT', 'X8_Y8_Z8') -> made from kind and packing."""
+    return getattr(K, "DATA_TYPE_" + spec) if isinstance(spec, str) else make_type(nv, K, *spec)
+
+
+DATA_TYPES = [  # TestDataType.cpp:55-74: type, kind, packing, channels, bits per pixel
+    (("FLOAT", "X32_Y32_Z32_W32"), "FLOAT", "X32_Y32_Z32_W32", 4, 128), ("U8", "UNSIGNED", "X8", 1, 8), ("S8", "SIGNED", "X8", 1, 8),
+    ("U16", "UNSIGNED", "X16", 1, 16), ("S16", "SIGNED", "X16", 1, 16), ("2U8", "UNSIGNED", "X8_Y8", 2, 16),
+    ("3U8", "UNSIGNED", "X8_Y8_Z8", 3, 24), ("4U8", "UNSIGNED", "X8_Y8_Z8_W8", 4, 32), ("F32", "FLOAT", "X32", 1, 32),
+    ("F64", "FLOAT", "X64", 1, 64), ("C64", "COMPLEX", "X64", 1, 64), ("4C64", "COMPLEX", "X64_Y64_Z64_W64", 4, 256),
+    ("C128", "COMPLEX", "X128", 1, 128), ("2C128", "COMPLEX", "X128_Y128", 2, 256), (("UNSIGNED", "X10Y11Z11"), "UNSIGNED", "X10Y11Z11", 3, 32),
+    (("UNSIGNED", "X5Y6Z5"), "UNSIGNED", "X5Y6Z5", 3, 16), (("UNSIGNED", "X10b6_Y10b6"), "UNSIGNED", "X10b6_Y10b6", 2, 32),
+    ("2F32", "FLOAT", "X32_Y32", 2, 64)]
+
+
+@pytest.mark.parametrize("spec,kind,packing,channels,bpp", DATA_TYPES, ids=[str(d[0]) for d in DATA_TYPES])
+def test_data_type_properties(nv, K, spec, kind, packing, channels, bpp):
+    t = dtype(nv, K, spec)
+    out = C.c_int(-9)
+    assert nv.nvcvDataTypeGetPacking(C.c_uint64(t), C.byref(out)) == 0 and out.value == const(K, "PACKING_" + packing)
+    assert nv.nvcvDataTypeGetBitsPerPixel(C.c_uint64(t), C.byref(out)) == 0 and out.value == bpp
+    assert nv.nvcvDataTypeGetDataKind(C.c_uint64(t), C.byref(out)) == 0 and out.value == const(K, "DATA_KIND_" + kind)
+    assert nv.nvcvDataTypeGetNumChannels(C.c_uint64(t), C.byref(out)) == 0 and out.value == channels
+    assert make_type(nv, K, kind, packing) == t
+    bits, want = (C.c_int32 * 4)(), (C.c_int32 * 4)()
+    assert nv.nvcvDataTypeGetBitsPerChannel(C.c_uint64(t), bits) == 0
+    assert nv.nvcvPackingGetBitsPerComponent(const(K, "PACKING_" + packing), want) == 0 and list(bits) == list(want)
+
+
+def test_data_types_equal_their_image_formats_and_names(nv, K):
+    # TestDataType.cpp:145-224
+    for n in ("U8", "S8", "U16", "S16", "F32", "2F32", "C64", "2C64", "C128", "2C128"):
+        assert getattr(K, "IMAGE_FORMAT_" + n) == getattr(K, "DATA_TYPE_" + n)
+    assert K.DATA_TYPE_NONE == 0
+    nv.nvcvDataTypeGetName.restype = C.c_char_p
+    nv.nvcvDataTypeGetName.argtypes = [C.c_uint64]
+    names = ["NONE", "U8", "2S8", "3S8", "4S8", "2U16", "3U16", "4U16", "2S16", "3S16", "4S16", "U32", "2U32", "3U32", "4U32", "S32",
+             "2S32", "3S32", "4S32", "F16", "2F16", "3F16", "4F16", "3F32", "U64", "2U64", "3U64", "4U64", "S64", "2S64", "3S64", "4S64",
+             "2F64", "3F64", "4F64", "3C64"]
+    for n in names:
+        assert nv.nvcvDataTypeGetName(getattr(K, "DATA_TYPE_" + n)) == b"NVCV_DATA_TYPE_" + n.encode(), n
+    assert nv.nvcvDataTypeGetName(make_type(nv, K, "FLOAT", "X8_Y8_Z8")) == b"NVCVDataType(FLOAT,X8_Y8_Z8)"
+    out = C.c_int()
+    assert nv.nvcvMakeDataType(None, K.DATA_KIND_FLOAT, K.PACKING_X8_Y8_Z8) == INVALID
+    for f in ("nvcvDataTypeGetPacking", "nvcvDataTypeGetBitsPerPixel", "nvcvDataTypeGetBitsPerChannel", "nvcvDataTypeGetDataKind",
+              "nvcvDataTypeGetNumChannels", "nvcvDataTypeGetStrideBytes", "nvcvDataTypeGetAlignment"):
+        assert getattr(nv, f)(C.c_uint64(K.DATA_TYPE_U8), None) == INVALID, f
+    assert nv.nvcvDataTypeGetChannelType(C.c_uint64(K.DATA_TYPE_U8), 0, None) == INVALID
+
+
+CHANNEL_TYPES = [  # TestDataType.cpp:246-290: type, channel, type of that channel (None = INVALID_ARGUMENT)
+    ("U8", 0, "U8"), ("U8", 4, "NONE"), (("FLOAT", "X32"), 0, ("FLOAT", "X32")), (("FLOAT", "X8_Y8_Z8"), 2, ("FLOAT", "X8")),
+    ("2F32", 0, "F32"), ("2F32", 1, "F32"), ("2C64", 0, "C64"), ("2C64", 1, "C64"), ("2C128", 0, "C128"), ("2C128", 1, "C128"),
+    (("SIGNED", "X64_Y64_Z64_W64"), 3, "S64"), (("UNSIGNED", "X4Y4"), 0, ("UNSIGNED", "X4")), (("UNSIGNED", "b4X4Y4Z4"), 2, ("UNSIGNED", "X4")),
+    (("UNSIGNED", "X3Y3Z2"), 2, ("UNSIGNED", "X2")), (("UNSIGNED", "X1"), 0, ("UNSIGNED", "X1")), (("UNSIGNED", "X2"), 0, ("UNSIGNED", "X2")),
+    ("3S16", 2, "S16"), (("SIGNED", "X24"), 0, ("SIGNED", "X24")), ("2F64", 1, "F64"), (("SIGNED", "X96"), 0, ("SIGNED", "X96")),
+    (("SIGNED", "X128"), 0, ("SIGNED", "X128")), (("SIGNED", "X192"), 0, ("SIGNED", "X192")), (("SIGNED", "X256"), 0, ("SIGNED", "X256")),
+    ("U8", 1, "NONE"), ("2F32", 2, "NONE"), (("UNSIGNED", "b4X4Y4Z4"), 3, "NONE"),
+    ("U8", -1, None), (("UNSIGNED", "X5Y5b1Z5"), 0, None), (("UNSIGNED", "X3Y3Z2"), 1, None)]
+
+
+@pytest.mark.parametrize("spec,channel,want", CHANNEL_TYPES, ids=["%s-%d" % (str(c[0]), c[1]) for c in CHANNEL_TYPES])
+def test_channel_type_of_a_data_type(nv, K, spec, channel, want):
+    out = C.c_uint64(99)
+    st = nv.nvcvDataTypeGetChannelType(C.c_uint64(dtype(nv, K, spec)), channel, C.byref(out))
+    if want is None:
+        assert st == INVALID
+    else:
+        assert st == 0 and out.value == dtype(nv, K, want)
+
+
+def test_data_type_stride_and_alignment(nv, K):
+    # TestDataType.cpp:313-375
+    out = C.c_int32()
+    for spec, stride in (("U8", 1), ("U16", 2), ("3S8", 3), ("2U16", 4), (("SIGNED", "X256"), 32), ("2F32", 8), ("C64", 8), ("4C64", 32),
+                         ("C128", 16), ("2C128", 32), (("FLOAT", "X8_Y8_Z8"), 3)):
+        assert nv.nvcvDataTypeGetStrideBytes(C.c_uint64(dtype(nv, K, spec)), C.byref(out)) == 0 and out.value == stride, spec
+    for spec, align in (("U8", 1), ("U16", 2), ("3S8", 1), ("2U16", 2), (("SIGNED", "X256"), 32), ("2F32", 4), ("C64", 8), ("2C64", 8),
+                        ("C128", 16), ("2C128", 16), (("SIGNED", "X5Y1Z5W5"), 2), (("SIGNED", "X3Y3Z2"), 1), (("SIGNED", "X4b4"), 1),
+                        (("SIGNED", "b4X4"), 1), (("SIGNED", "b4X12"), 2), (("SIGNED", "X10b6"), 2), (("SIGNED", "X4Y4Z4W4"), 2),
+                        (("SIGNED", "X8_Y8__X8_Z8"), 1), (("SIGNED", "X32_Y24b8"), 4)):
+        assert nv.nvcvDataTypeGetAlignment(C.c_uint64(dtype(nv, K, spec)), C.byref(out)) == 0 and out.value == align, spec
