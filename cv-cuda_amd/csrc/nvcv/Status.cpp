@@ -82,7 +82,7 @@ extern "C"
 {
 const char *nvcvStatusGetName(NVCVStatus code)
 {
-    switch (code)
+    switch (EnumValue(code))
     {
 #define NAME(x) \
     case x:     \
@@ -130,7 +130,7 @@ void nvcvSetThreadStatusVarArgList(NVCVStatus status, const char *fmt, va_list v
 {
     if (fmt == nullptr)
     {
-        SetThreadStatus(status, nullptr);
+        SetThreadStatus(status, ""); // no message given: the message is empty, not the status name
         return;
     }
     char buf[NVCV_MAX_STATUS_MESSAGE_LENGTH];

@@ -6,6 +6,7 @@ src/nvcv/src/priv/Tensor.cpp:172-185, validation of TensorWrapDataStrided.cpp:35
 semantics of priv/Status.cpp:31-110 -- with this library's alignment constants (128-byte rows,
 512-byte base)."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -384,3 +385,118 @@ def test_custom_allocator(cv, capi):
     # default allocator (NULL handle) serves host memory too
     assert nv.nvcvAllocatorAllocHostMemory(None, C.byref(p), 256, 128) == 0 and p.value % 128 == 0
     assert nv.nvcvAllocatorFreeHostMemory(None, p, 256, 128) == 0
+
+
+def test_tensor_layout_cases_of_the_reference(cv, tmp_path):
+    """tests/golden/tensor_layout_cases.c restates the cases of the reference's TestTensorLayout.cpp; it exercises the
+    exported functions and the header-inline accessors from plain C."""
+    import subprocess
+    import cvcuda_amd._capi as capi_mod
+    libdir = os.path.dirname(capi_mod.nvcv._name)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = tmp_path / "layout_cases"
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-DCVCUDA_NO_HIP_HEADERS", "-I" + os.path.join(root, "include"),
+                    os.path.join(root, "tests", "golden", "tensor_layout_cases.c"), "-L" + libdir, "-lnvcv_types",
+                    # a sanitizer build of the library leaves its runtime's symbols to the preloaded runtime
+                    "-Wl,--allow-shlib-undefined", "-Wl,-rpath," + libdir, "-o", str(exe)], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.strip() == "0 failures", r.stdout
+
+
+def test_requirements_cases_of_the_reference(cv, capi):
+    # tests/nvcv_types/system/TestRequirements.cpp:57-290
+    nv = capi.nvcv
+    n = len(capi.Requirements().cudaMem.numBlocks)
+    ceil = lambda a, b: -(-a // b)
+    # add_buffer / sub_buffer
+    req = capi.Requirements()
+    assert nv.nvcvRequirementsInit(C.byref(req)) == 0
+    m = req.cudaMem
+    a1, a2 = 256, 16384
+    s1, s2 = 3 * a1 - 5, 6 * a2 - 17
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), s1, a1) == 0
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), s2, a2) == 0
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), a2 // 3, a2) == 0
+    want = [0] * n
+    want[8], want[14] = ceil(s1, a1), ceil(s2 + a2 // 3, a2)
+    assert list(m.numBlocks) == want
+    assert nv.nvcvRequirementsInit(C.byref(req)) == 0
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), s1, a1) == 0 and nv.nvcvMemRequirementsAddBuffer(C.byref(m), -511, a1) == 0
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), s2, a2) == 0 and nv.nvcvMemRequirementsAddBuffer(C.byref(m), -s2 * 5, a2) == 0
+    want = [0] * n
+    want[8] = ceil(s1 - 512, a1)
+    assert list(m.numBlocks) == want
+    # add and total size
+    total, gold, sizes = capi.Requirements(), [[0] * n for _ in range(3)], [0, 0, 0]
+    assert nv.nvcvRequirementsInit(C.byref(total)) == 0
+    for factors in ((3, 5, 7), (17, 21, 37)):
+        part = capi.Requirements()
+        assert nv.nvcvRequirementsInit(C.byref(part)) == 0
+        for i in range(n):
+            align = 1 << i
+            for k, mem in enumerate((part.cudaMem, part.hostMem, part.hostPinnedMem)):
+                size = factors[k] * (i + 1) * align - (k + 1)
+                assert nv.nvcvMemRequirementsAddBuffer(C.byref(mem), size, align) == 0
+                gold[k][i] += ceil(size, align)
+                sizes[k] += ceil(size, align) * align
+        assert nv.nvcvRequirementsAdd(C.byref(total), C.byref(part)) == 0
+        assert [list(total.cudaMem.numBlocks), list(total.hostMem.numBlocks), list(total.hostPinnedMem.numBlocks)] == gold
+    out = C.c_int64()
+    for k, mem in enumerate((total.cudaMem, total.hostMem, total.hostPinnedMem)):
+        assert nv.nvcvMemRequirementsCalcTotalSizeBytes(C.byref(mem), C.byref(out)) == 0 and out.value == sizes[k]
+    assert nv.nvcvRequirementsAdd(C.byref(total), C.byref(total)) == 0
+    assert list(total.cudaMem.numBlocks) == [2 * v for v in gold[0]]
+    # invalid arguments and overflow
+    assert nv.nvcvRequirementsInit(None) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvRequirementsAdd(None, C.byref(req)) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvRequirementsAdd(C.byref(req), None) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvMemRequirementsCalcTotalSizeBytes(None, C.byref(out)) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvMemRequirementsCalcTotalSizeBytes(C.byref(m), None) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvMemRequirementsAddBuffer(None, 256, 256) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), 256, 3) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(m), 256, (1 << 32) + 1) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    big = capi.Requirements()
+    assert nv.nvcvRequirementsInit(C.byref(big)) == 0
+    big.cudaMem.numBlocks[0], big.cudaMem.numBlocks[1] = (1 << 63) - 1, 2
+    assert nv.nvcvMemRequirementsCalcTotalSizeBytes(C.byref(big.cudaMem), C.byref(out)) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    big.cudaMem.numBlocks[1] = (1 << 63) - 1
+    assert nv.nvcvMemRequirementsCalcTotalSizeBytes(C.byref(big.cudaMem), C.byref(out)) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    big.cudaMem.numBlocks[1] = 0
+    assert nv.nvcvMemRequirementsAddBuffer(C.byref(big.cudaMem), 2, 1) == capi.NVCV_ERROR_OVERFLOW
+
+
+def test_status_cases_of_the_reference(cv, capi):
+    # tests/nvcv_types/system/TestStatus.cpp:30-170
+    nv = capi.nvcv
+    nv.nvcvStatusGetName.restype = C.c_char_p
+    names = ["NVCV_SUCCESS", "NVCV_ERROR_NOT_IMPLEMENTED", "NVCV_ERROR_INVALID_ARGUMENT", "NVCV_ERROR_INVALID_IMAGE_FORMAT",
+             "NVCV_ERROR_INVALID_OPERATION", "NVCV_ERROR_DEVICE", "NVCV_ERROR_NOT_READY", "NVCV_ERROR_OUT_OF_MEMORY", "NVCV_ERROR_INTERNAL"]
+    for code, name in enumerate(names):
+        assert nv.nvcvStatusGetName(code) == name.encode()
+    assert nv.nvcvStatusGetName(capi.NVCV_ERROR_OVERFLOW) == b"NVCV_ERROR_OVERFLOW"
+    assert nv.nvcvStatusGetName(capi.NVCV_ERROR_OVERFLOW + 1) == b"NVCV_ERROR_UNDERFLOW"
+    assert nv.nvcvStatusGetName(255) == b"Unknown error"
+    msg = C.create_string_buffer(256)
+    nv.nvcvGetLastError()
+    assert nv.nvcvGetLastError() == 0 and nv.nvcvPeekAtLastError() == 0
+    assert nv.nvcvGetLastErrorMessage(msg, 256) == 0 and msg.value == b"success"
+    nv.nvcvSetThreadStatus(capi.NVCV_ERROR_DEVICE, b"%s", b"")
+    assert nv.nvcvGetLastError() == capi.NVCV_ERROR_DEVICE and nv.nvcvGetLastError() == 0
+    nv.nvcvSetThreadStatus(capi.NVCV_ERROR_DEVICE, b"%s", b"")
+    assert nv.nvcvPeekAtLastError() == capi.NVCV_ERROR_DEVICE and nv.nvcvPeekAtLastError() == capi.NVCV_ERROR_DEVICE
+    nv.nvcvSetThreadStatus(capi.NVCV_ERROR_INTERNAL, b"test message")
+    assert nv.nvcvGetLastErrorMessage(msg, 256) == capi.NVCV_ERROR_INTERNAL and msg.value == b"test message"
+    assert nv.nvcvGetLastErrorMessage(msg, 256) == 0 and msg.value == b"success"
+    assert nv.nvcvPeekAtLastErrorMessage(msg, 256) == 0 and msg.value == b"success"
+    reqs = capi.ImageRequirements()
+    assert nv.nvcvImageCalcRequirements(640, 480, C.c_uint64(cv.K.IMAGE_FORMAT_U8), 0, 0, None) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvImageCalcRequirements(640, 480, C.c_uint64(cv.K.IMAGE_FORMAT_U8), 0, 0, C.byref(reqs)) == 0
+    assert nv.nvcvGetLastError() == capi.NVCV_ERROR_INVALID_ARGUMENT  # the success in between did not reset it
+    nv.nvcvSetThreadStatus(capi.NVCV_ERROR_DEVICE, b"test message")
+    for _ in range(2):
+        msg.value = b""
+        assert nv.nvcvPeekAtLastErrorMessage(msg, 256) == capi.NVCV_ERROR_DEVICE and msg.value == b"test message"
+    nv.nvcvSetThreadStatus(capi.NVCV_ERROR_DEVICE, b"test message %d %c %s", 123, ord("r"), b"lima")
+    assert nv.nvcvGetLastErrorMessage(msg, 256) == capi.NVCV_ERROR_DEVICE and msg.value == b"test message 123 r lima"
+    nv.nvcvSetThreadStatus(capi.NVCV_ERROR_DEVICE, None)
+    assert nv.nvcvGetLastErrorMessage(msg, 256) == capi.NVCV_ERROR_DEVICE and msg.value == b""
