@@ -500,3 +500,23 @@ def test_status_cases_of_the_reference(cv, capi):
     assert nv.nvcvGetLastErrorMessage(msg, 256) == capi.NVCV_ERROR_DEVICE and msg.value == b"test message 123 r lima"
     nv.nvcvSetThreadStatus(capi.NVCV_ERROR_DEVICE, None)
     assert nv.nvcvGetLastErrorMessage(msg, 256) == capi.NVCV_ERROR_DEVICE and msg.value == b""
+
+
+WRAP_CASES = [  # tests/nvcv_types/system/TestTensor.cpp:448-470: shape, layout, strides, dtype, accepted?
+    ([2], "C", [4], np.float32, True), ([1], "W", [1], np.uint8, True), ([10, 5], "HW", [5, 1], np.uint8, True),
+    ([1, 10, 5], "NHW", [1, 5, 1], np.uint8, True), ([3, 1, 5], "NHW", [20, 1, 4], np.float32, True),
+    ([3, 1, 1], "NHW", [20, 1, 1], np.float32, True), ([10, 5, 3], "HWC", [60, 12, 4], np.float32, True),
+    ([2], "C", [3], np.float32, False), ([2], "C", [5], np.float32, False), ([10, 5], "HW", [1, 10], np.uint8, False),
+    ([10, 5, 3], "HWC", [4, 40, 200], np.float32, False), ([1, 10, 5], "NHW", [1, 19, 4], np.float32, False),
+    ([3, 1, 5], "NHW", [19, 1, 4], np.float32, False)]
+
+
+@pytest.mark.parametrize("shape,layout,strides,dt,ok", WRAP_CASES, ids=[str(c[:3]) for c in WRAP_CASES])
+def test_wrap_parameter_cases_of_the_reference(cv, capi, shape, layout, strides, dt, ok):
+    if not ok:
+        with pytest.raises(cv.Error) as e:
+            fake_tensor(cv, shape, strides, dt, layout, 0xDEADBEEF)
+        assert e.value.status == capi.NVCV_ERROR_INVALID_ARGUMENT
+        return
+    t = fake_tensor(cv, shape, strides, dt, layout, 0xDEADBEEF)
+    assert t.shape == shape and t.layout == layout and t.strides == strides
