@@ -6,7 +6,7 @@
 
 #include "Export.h"
 #include "Status.h"
-#include "detail/FormatBits.h"
+#include "detail/FormatUtils.h"
 
 #include <stdint.h>
 

@@ -17,6 +17,7 @@
 int main(void)
 {
 #include "abi_constants_all.inc"
+#include "abi_detail_macros.inc"
     V(NVCV_IMAGE_FORMAT_U8);
     V(NVCV_IMAGE_FORMAT_S8);
     V(NVCV_IMAGE_FORMAT_U16);
