@@ -14,7 +14,7 @@ handle pools, reference counts, stride rules, operator validation - can then be 
 without a GPU:
 
   LD_PRELOAD=$(python cv-cuda_amd/build.py --asan-runtime) ASAN_OPTIONS=detect_leaks=0 \
-  CVCUDA_AMD_LIBDIR=cv-cuda_amd/lib_san python -m pytest tests/test_core.py tests/test_op_validation.py tests/test_format_api.py tests/test_image_format_api.py -q
+  CVCUDA_AMD_LIBDIR=cv-cuda_amd/lib_san python -m pytest -m "not gpu" tests/test_core.py tests/test_op_validation.py tests/test_format_api.py tests/test_image_format_api.py -q
 
 (the interpreter itself is not instrumented, so the sanitizer runtime has to be loaded first; leak detection is
 off because the interpreter's own allocations would drown the report).

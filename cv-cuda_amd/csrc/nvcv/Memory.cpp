@@ -242,6 +242,12 @@ void CheckAllocArgs(int64_t size, int32_t align)
     {
         throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Alignment must be a power of two, not %d", align);
     }
+    // reference: src/nvcv/src/priv/IAllocator.cpp:45-50, a size that is not whole alignment units is rejected
+    if (AlignUp(size, (int64_t)align) != size)
+    {
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Allocation size must be an integral multiple of alignment %d, not %ld",
+                    align, (long)size);
+    }
 }
 
 void *DefaultAllocHost(void *, int64_t size, int32_t align)
@@ -570,7 +576,7 @@ NVCVAMD_ALLOC_PAIR(CudaMemory, allocDevice, freeDevice)
 
 const char *nvcvResourceTypeGetName(NVCVResourceType resource)
 {
-    switch (resource)
+    switch (EnumValue(resource)) // callers may pass any integer
     {
     case NVCV_RESOURCE_MEM_HOST:
         return "NVCV_RESOURCE_MEM_HOST";

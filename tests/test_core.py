@@ -373,11 +373,12 @@ def test_custom_allocator(cv, capi):
     h = C.c_void_p()
     assert nv.nvcvAllocatorConstructCustom(C.byref(ra), 1, C.byref(h)) == 0
     p = C.c_void_p()
-    assert nv.nvcvAllocatorAllocHostMemory(h, C.byref(p), 100, 64) == 0 and p.value and p.value % 64 == 0
-    assert nv.nvcvAllocatorFreeHostMemory(h, p, 100, 64) == 0
-    assert log == [("alloc", 100, 64), ("free", 100, 64)]
+    assert nv.nvcvAllocatorAllocHostMemory(h, C.byref(p), 128, 64) == 0 and p.value and p.value % 64 == 0
+    assert nv.nvcvAllocatorFreeHostMemory(h, p, 128, 64) == 0
+    assert log == [("alloc", 128, 64), ("free", 128, 64)]
     assert nv.nvcvAllocatorAllocHostMemory(h, C.byref(p), 100, 48) == capi.NVCV_ERROR_INVALID_ARGUMENT
     assert nv.nvcvAllocatorAllocHostMemory(h, C.byref(p), -1, 64) == capi.NVCV_ERROR_INVALID_ARGUMENT
+    assert nv.nvcvAllocatorAllocHostMemory(h, C.byref(p), 100, 64) == capi.NVCV_ERROR_INVALID_ARGUMENT  # not whole units
     two = (capi.ResourceAllocator * 2)(ra, ra)
     h2 = C.c_void_p()
     assert nv.nvcvAllocatorConstructCustom(two, 2, C.byref(h2)) == capi.NVCV_ERROR_INVALID_ARGUMENT  # duplicate type
@@ -520,3 +521,30 @@ def test_wrap_parameter_cases_of_the_reference(cv, capi, shape, layout, strides,
         return
     t = fake_tensor(cv, shape, strides, dt, layout, 0xDEADBEEF)
     assert t.shape == shape and t.layout == layout and t.strides == strides
+
+
+def build_c_cases(name, tmp_path):
+    """Compiles tests/golden/<name>.c with gcc against the public headers and the core library."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.environ.get("CVCUDA_AMD_LIBDIR", os.path.join(root, "cv-cuda_amd", "lib"))
+    exe = str(tmp_path / name)
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-D_POSIX_C_SOURCE=200112L", "-DCVCUDA_NO_HIP_HEADERS",
+                    "-I" + os.path.join(root, "include"), os.path.join(root, "tests", "golden", name + ".c"), "-o", exe,
+                    "-L" + libdir, "-lnvcv_types", "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"], check=True)
+    return exe
+
+
+def test_argument_checks_of_the_reference_from_plain_c(cv, tmp_path):
+    import subprocess
+    r = subprocess.run([build_c_cases("core_negative_cases", tmp_path)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.strip().endswith("0 failed"), r.stdout + r.stderr
+
+
+@pytest.mark.gpu
+def test_argument_checks_of_the_reference_from_plain_c_with_image_batches(cv, gpu, tmp_path):
+    import subprocess
+    r = subprocess.run([build_c_cases("core_negative_cases", tmp_path), "device"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0 and r.stdout.strip().endswith("0 failed"), r.stdout + r.stderr
+

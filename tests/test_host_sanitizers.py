@@ -30,7 +30,7 @@ def test_core_and_validation_are_clean_under_asan_and_ubsan():
         env["ASAN_OPTIONS"] = "detect_leaks=0:log_path=" + os.path.join(logs, "asan")
         env["UBSAN_OPTIONS"] = "print_stacktrace=1:log_path=" + os.path.join(logs, "ubsan")
         env["CVCUDA_AMD_LIBDIR"] = os.path.join(PKG, "lib_san")
-        r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-p", "no:cacheprovider",
+        r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "not gpu", "-p", "no:cacheprovider",
                             os.path.join(ROOT, "tests", "test_core.py"), os.path.join(ROOT, "tests", "test_op_validation.py"),
                             os.path.join(ROOT, "tests", "test_format_api.py"), os.path.join(ROOT, "tests", "test_image_format_api.py")],
                            env=env, capture_output=True, text=True, timeout=900)
