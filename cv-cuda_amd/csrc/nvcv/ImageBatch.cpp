@@ -508,6 +508,10 @@ NVCVStatus nvcvImageBatchVarShapeGetMaxSize(NVCVImageBatchHandle handle, int32_t
     return Protect(
         [&]
         {
+            if (maxWidth == nullptr && maxHeight == nullptr)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Both output width and height pointers cannot be NULL");
+            }
             int32_t w, h;
             Batch(handle).maxSize(&w, &h);
             if (maxWidth)
