@@ -1,27 +1,19 @@
 /* Library version as one integer: major*1000000 + minor*10000 + patch*100 + tweak.
- * Replaces: src/nvcv/src/include/nvcv/Version.h:40 and cmake/VersionDef.h.in:47-48. */
+ * Replaces: src/nvcv/src/include/nvcv/Version.h:40; the numbers themselves are in VersionDef.h. */
 #ifndef NVCV_VERSION_H
 #define NVCV_VERSION_H
 
 #include "Export.h"
+#include "VersionDef.h"
 
 #include <stdint.h>
-
-#define NVCV_VERSION_MAJOR 0
-#define NVCV_VERSION_MINOR 15
-#define NVCV_VERSION_PATCH 0
-#define NVCV_VERSION_TWEAK 0
-
-#define NVCV_MAKE_VERSION4(major, minor, patch, tweak) \
-    ((uint32_t)((major)*1000000 + (minor)*10000 + (patch)*100 + (tweak)))
-#define NVCV_VERSION \
-    NVCV_MAKE_VERSION4(NVCV_VERSION_MAJOR, NVCV_VERSION_MINOR, NVCV_VERSION_PATCH, NVCV_VERSION_TWEAK)
 
 #ifdef __cplusplus
 extern "C"
 {
 #endif
 
+/* Version of the loaded library, which may differ from NVCV_VERSION of the headers a program was built with. */
 NVCV_PUBLIC uint32_t nvcvGetVersion(void);
 
 #ifdef __cplusplus

@@ -255,3 +255,63 @@ def test_reference_cpp_wrappers_link_and_run_against_the_core_library(cv, tmp_pa
                    "layout rank 4 C at 3",
                    "tensor rank 4 layout NCHW strides 602112 200704 896 4",
                    "status 2"]
+
+
+VERSION_PROGRAM = r"""
+#include <cvcuda/Version.h>
+#include <nvcv/Version.h>
+#include <stdio.h>
+#include <string.h>
+#define STR_(a) #a
+#define STR(a) STR_(a)
+#define CHECK(x) do { if (!(x)) { printf("line %d: %s\n", __LINE__, #x); ++bad; } } while (0)
+int main(void)
+{
+    int bad = 0;
+    /* the cases of tests/nvcv_types/system/TestVersion.cpp:25-85 */
+    CHECK(NVCV_VERSION == nvcvGetVersion());
+    CHECK(NVCV_VERSION_MAJOR == nvcvGetVersion() / 1000000);
+    CHECK(NVCV_VERSION_MINOR == nvcvGetVersion() / 10000 % 100);
+    CHECK(NVCV_VERSION_PATCH == nvcvGetVersion() / 100 % 100);
+    CHECK(NVCV_VERSION_TWEAK == nvcvGetVersion() % 100);
+    char want[64];
+    snprintf(want, sizeof(want), "%s.%s.%s", STR(NVCV_VERSION_MAJOR), STR(NVCV_VERSION_MINOR), STR(NVCV_VERSION_PATCH));
+#if NVCV_VERSION_TWEAK
+    strcat(want, "." STR(NVCV_VERSION_TWEAK));
+#endif
+    if (NVCV_VERSION_SUFFIX[0]) { strcat(want, "-"); strcat(want, NVCV_VERSION_SUFFIX); }
+    CHECK(strcmp(want, NVCV_VERSION_STRING) == 0);
+    CHECK(1020304 == NVCV_MAKE_VERSION4(1, 2, 3, 4));
+    CHECK(1020300 == NVCV_MAKE_VERSION3(1, 2, 3));
+    CHECK(1020000 == NVCV_MAKE_VERSION2(1, 2));
+    CHECK(1000000 == NVCV_MAKE_VERSION1(1));
+    CHECK(NVCV_MAKE_VERSION4(1, 2, 3, 4) == NVCV_MAKE_VERSION(1, 2, 3, 4));
+    CHECK(NVCV_MAKE_VERSION4(1, 2, 3, 0) == NVCV_MAKE_VERSION(1, 2, 3));
+    CHECK(NVCV_MAKE_VERSION4(1, 2, 0, 0) == NVCV_MAKE_VERSION(1, 2));
+    CHECK(NVCV_MAKE_VERSION4(1, 0, 0, 0) == NVCV_MAKE_VERSION(1));
+    CHECK(NVCV_VERSION_API == NVCV_MAKE_VERSION(NVCV_VERSION_MAJOR, NVCV_VERSION_MINOR));
+    CHECK(NVCV_VERSION_API_IS(NVCV_VERSION_MAJOR, NVCV_VERSION_MINOR));
+    CHECK(NVCV_VERSION_API_AT_LEAST(NVCV_VERSION_MAJOR, 0) && !NVCV_VERSION_API_AT_LEAST(NVCV_VERSION_MAJOR + 1, 0));
+    CHECK(NVCV_VERSION_API_AT_MOST(NVCV_VERSION_MAJOR + 1, 0) && !NVCV_VERSION_API_AT_MOST(NVCV_VERSION_MAJOR, 0));
+    CHECK(NVCV_VERSION_API_IN_RANGE(NVCV_VERSION_MAJOR, 0, NVCV_VERSION_MAJOR, 99));
+    /* the operator library carries the same set under its own prefix */
+    CHECK(CVCUDA_VERSION == cvcudaGetVersion());
+    CHECK(CVCUDA_VERSION == CVCUDA_MAKE_VERSION(CVCUDA_VERSION_MAJOR, CVCUDA_VERSION_MINOR, CVCUDA_VERSION_PATCH));
+    CHECK(1020000 == CVCUDA_MAKE_VERSION(1, 2) && 1020304 == CVCUDA_MAKE_VERSION(1, 2, 3, 4));
+    CHECK(CVCUDA_VERSION_API_IS(CVCUDA_VERSION_MAJOR, CVCUDA_VERSION_MINOR));
+    CHECK(strcmp(CVCUDA_VERSION_STRING, NVCV_VERSION_STRING) == 0);
+    return bad;
+}
+"""
+
+
+def test_version_macros_and_functions(tmp_path):
+    libdir = os.environ.get("CVCUDA_AMD_LIBDIR", os.path.join(ROOT, "cv-cuda_amd", "lib"))
+    src = tmp_path / "version.c"
+    src.write_text(VERSION_PROGRAM)
+    exe = tmp_path / "version"
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-DCVCUDA_NO_HIP_HEADERS", "-I" + INC, str(src), "-o", str(exe),
+                    "-L" + libdir, "-lcvcuda", "-lnvcv_types", "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"],
+                   check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
