@@ -135,8 +135,9 @@ public:
         out.bufferType              = NVCV_IMAGE_BUFFER_STRIDED_CUDA;
         NVCVImageBufferStrided &buf = out.buffer.strided;
         buf.numPlanes               = FormatNumPlanes(m_reqs.format);
-        // Each plane starts at the next multiple of the base alignment, matching how the
-        // requirements were summed (one aligned block run per plane).
+        // Planes follow each other without gaps (reference: src/nvcv/src/priv/Image.cpp:174-187): plane p + 1
+        // starts row pitch x height after plane p, so a planar image is also a dense CHW block. The requirements
+        // sum one aligned block run per plane, which is never less.
         int64_t offset = 0;
         for (int p = 0; p < buf.numPlanes; ++p)
         {
@@ -144,7 +145,7 @@ public:
             FormatPlaneSize(m_reqs.format, p, m_reqs.width, m_reqs.height, &pl.width, &pl.height);
             pl.rowStride = m_reqs.planeRowStride[p];
             pl.basePtr   = static_cast<NVCVByte *>(m_mem) + offset;
-            offset += AlignUp((int64_t)pl.rowStride * pl.height, m_reqs.alignBytes);
+            offset += (int64_t)pl.rowStride * pl.height;
         }
     }
 

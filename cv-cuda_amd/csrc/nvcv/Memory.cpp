@@ -387,8 +387,9 @@ public:
         {
             throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Invalid resource type %d", (int)type);
         }
-        *out         = m_res[type];
-        out->cleanup = nullptr; // ownership of the context stays with this object
+        // The stored descriptor as given (reference: src/nvcv/src/priv/CustomAllocator.cpp:120-124). The context it
+        // names stays owned by this object: the cleanup callback is for the owner to run, once.
+        *out = m_res[type];
     }
 
 private:

@@ -111,36 +111,23 @@ NVCVTensorLayout LayoutForImages(uint64_t fmt, int numImages)
                 nvcvImageFormatGetName(fmt));
 }
 
-// Element type of a tensor holding images of format `fmt`: one component of plane 0.
+// Element type of a tensor holding images of format `fmt`: the first component of plane 0 on its own, when a
+// packing of just that many bits exists (reference: src/nvcv/src/priv/Tensor.cpp:79-91).
 NVCVDataType ChannelDataTypeOf(uint64_t fmt)
 {
-    PackingInfo pi = DecodePacking(FormatPlanePacking(fmt, 0));
-    NVCVPacking one;
-    switch (pi.known ? pi.bits[0] : 0)
+    NVCVPackingParams params;
+    NVCVPacking       one;
+    if (nvcvPackingGetParams(FormatPlanePacking(fmt, 0), &params) != NVCV_SUCCESS)
     {
-    case 8:
-        one = NVCV_PACKING_X8;
-        break;
-    case 16:
-        one = NVCV_PACKING_X16;
-        break;
-    case 32:
-        one = NVCV_PACKING_X32;
-        break;
-    case 64:
-        one = NVCV_PACKING_X64;
-        break;
-    default:
         throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Image format can't be represented in a tensor: %s",
                     nvcvImageFormatGetName(fmt));
     }
-    for (int c = 1; c < pi.numChannels; ++c)
+    params.swizzle = NVCV_SWIZZLE_X000;
+    std::fill(params.bits + 1, params.bits + 4, 0);
+    if (nvcvMakePacking(&one, &params) != NVCV_SUCCESS)
     {
-        if (pi.bits[c] != pi.bits[0])
-        {
-            throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Image format can't be represented in a tensor: %s",
-                        nvcvImageFormatGetName(fmt));
-        }
+        throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Image format can't be represented in a tensor: %s",
+                    nvcvImageFormatGetName(fmt));
     }
     return NVCV_DETAIL_MAKE_DATA_TYPE(FormatDataKind(fmt), (uint64_t)one);
 }
@@ -496,8 +483,13 @@ NVCVStatus nvcvTensorWrapImageConstruct(NVCVImageHandle himg, NVCVTensorHandle *
             {
                 throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Only device-accessible pitch-linear images can be wrapped");
             }
+            // The checks and the layout rule of the reference (src/nvcv/src/priv/TensorData.cpp:50-192).
             uint64_t fmt    = id.format;
             int      planes = id.buffer.strided.numPlanes;
+            if (FormatMemLayout(fmt) != NVCV_MEM_LAYOUT_PL)
+            {
+                throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Image format's memory layout must be pitch-linear");
+            }
             if (FormatCSS(fmt) != NVCV_CSS_444)
             {
                 throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Images with subsampled planes cannot be viewed as a tensor");
@@ -506,10 +498,17 @@ NVCVStatus nvcvTensorWrapImageConstruct(NVCVImageHandle himg, NVCVTensorHandle *
             for (int p = 1; p < planes; ++p)
             {
                 const NVCVImagePlaneStrided &pl = id.buffer.strided.planes[p];
-                if (FormatPlanePacking(fmt, p) != FormatPlanePacking(fmt, 0) || pl.rowStride != p0.rowStride
-                    || pl.width != p0.width || pl.height != p0.height)
+                if (FormatPlaneDataType(fmt, p) != FormatPlaneDataType(fmt, 0))
                 {
-                    throw Error(NVCV_ERROR_INVALID_ARGUMENT, "All image planes must share packing, size and row pitch");
+                    throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Data type of all image planes must be the same");
+                }
+                if (pl.rowStride != p0.rowStride || pl.width != p0.width || pl.height != p0.height)
+                {
+                    throw Error(NVCV_ERROR_INVALID_ARGUMENT, "All image planes must share size and row pitch");
+                }
+                if (pl.basePtr <= p0.basePtr)
+                {
+                    throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Consecutive image planes must have increasing memory addresses");
                 }
                 if (pl.basePtr - id.buffer.strided.planes[p - 1].basePtr
                     != id.buffer.strided.planes[1].basePtr - p0.basePtr)
@@ -519,24 +518,41 @@ NVCVStatus nvcvTensorWrapImageConstruct(NVCVImageHandle himg, NVCVTensorHandle *
             }
             NVCVTensorData td = {};
             td.bufferType     = NVCV_TENSOR_BUFFER_STRIDED_CUDA;
-            td.dtype          = ChannelDataTypeOf(fmt);
-            td.layout         = LayoutForImages(fmt, 1);
             td.rank           = 4;
-            int elem          = DataTypeStrideBytes(td.dtype);
-            int ch            = FormatNumChannels(fmt);
             td.buffer.strided.basePtr = p0.basePtr;
-            if (planes == 1)
+            const int   ch         = FormatNumChannels(fmt);
+            const int   pixelBytes = FormatPlanePixelStrideBytes(fmt, 0);
+            PackingInfo pi         = DecodePacking(FormatPlanePacking(fmt, 0));
+            bool        sameBits   = true;
+            for (int c = 1; c < ch && c < 4; ++c)
             {
+                sameBits = sameBits && pi.bits[c] == pi.bits[0];
+            }
+            if (planes == 1 && ch >= 2 && sameBits)
+            {
+                // equal channels of one interleaved plane become a dimension of their own
+                td.layout = NVCV_TENSOR_NHWC;
+                if (nvcvDataTypeGetChannelType(FormatPlaneDataType(fmt, 0), 0, &td.dtype) != NVCV_SUCCESS)
+                {
+                    throw Error(NVCV_ERROR_INVALID_ARGUMENT, "Image format can't be represented in a tensor: %s",
+                                nvcvImageFormatGetName(fmt));
+                }
                 int64_t shape[4]   = {1, p0.height, p0.width, ch};
-                int64_t strides[4] = {(int64_t)p0.rowStride * p0.height, p0.rowStride, (int64_t)elem * ch, elem};
+                int64_t strides[4] = {(int64_t)p0.rowStride * p0.height, p0.rowStride, pixelBytes, pixelBytes / ch};
                 std::copy_n(shape, 4, td.shape);
                 std::copy_n(strides, 4, td.buffer.strided.strides);
             }
             else
             {
-                int64_t planeStride = id.buffer.strided.planes[1].basePtr - p0.basePtr;
-                int64_t shape[4]    = {1, ch, p0.height, p0.width};
-                int64_t strides[4]  = {planeStride * ch, planeStride, p0.rowStride, elem};
+                // one element per pixel of a plane (a one-channel plane, or a pixel whose fields differ in width).
+                // The plane pitch is the planes' real distance; for planes placed back to back, as image objects
+                // of this library place them, that is row pitch x height.
+                td.layout           = NVCV_TENSOR_NCHW;
+                td.dtype            = FormatPlaneDataType(fmt, 0);
+                int64_t planeStride = planes > 1 ? id.buffer.strided.planes[1].basePtr - p0.basePtr
+                                                 : (int64_t)p0.rowStride * p0.height;
+                int64_t shape[4]    = {1, planes, p0.height, p0.width};
+                int64_t strides[4]  = {planeStride * planes, planeStride, p0.rowStride, pixelBytes};
                 std::copy_n(shape, 4, td.shape);
                 std::copy_n(strides, 4, td.buffer.strided.strides);
             }

@@ -1,7 +1,7 @@
 /* Argument-checking behaviour of the core objects, written in plain C against the public headers. The rows are the
  * cases of the reference's own unit tests (which status each bad call returns):
- *   tests/nvcv_types/system/TestTensor.cpp:529-760, TestImage.cpp:267-515, TestImageBatch.cpp:359-694,
- *   TestAllocatorC.cpp:270-402, TestConfig.cpp:107-131.
+ *   tests/nvcv_types/system/TestTensor.cpp:58-447 (shapes and strides) and 529-760, TestImage.cpp:267-515, TestImageBatch.cpp:359-694,
+ *   TestAllocatorC.cpp:33-135 and 224-402, TestConfig.cpp:107-131.
  * Tensors and images are built on a custom allocator that serves "device" memory from the host heap, so the first
  * part runs without a GPU. `device` as first argument adds the image-batch cases, whose construction needs one.
  * Prints one line per failed check and exits with their count. */
@@ -202,6 +202,163 @@ static NVCVImageHandle MakeImage(NVCVAllocatorHandle alloc, int w, int h, NVCVIm
     EXPECT(OK, nvcvImageCalcRequirements(w, h, fmt, 0, 0, &reqs));
     EXPECT(OK, nvcvImageConstruct(&reqs, alloc, &img));
     return img;
+}
+
+/* What the tensor requirements, a tensor built from them and tensors wrapping data or an image look like. */
+static int32_t g_lastDeviceAlign;
+
+static void *RecordingAlloc(void *ctx, int64_t size, int32_t align)
+{
+    g_lastDeviceAlign = align;
+    return HeapAlloc(ctx, size, align);
+}
+
+static int SameLayout(NVCVTensorLayout a, NVCVTensorLayout b)
+{
+    return a.rank == b.rank && memcmp(a.data, b.data, (size_t)a.rank) == 0;
+}
+
+static void TensorShapeCases(NVCVAllocatorHandle alloc)
+{
+    NVCVTensorRequirements reqs;
+    /* a batch of images as one tensor: planar formats give NCHW, interleaved ones NHWC */
+    EXPECT(OK, nvcvTensorCalcRequirementsForImages(53, 32, 16, NVCV_IMAGE_FORMAT_RGBA8p, 0, 0, &reqs));
+    {
+        const int64_t gold[4] = {53, 4, 16, 32};
+        EXPECT(4, reqs.rank);
+        EXPECT(0, memcmp(reqs.shape, gold, sizeof(gold)));
+        EXPECT(1, SameLayout(reqs.layout, NVCV_TENSOR_NCHW));
+        EXPECT(1, reqs.dtype == NVCV_DATA_TYPE_U8);
+    }
+    EXPECT(OK, nvcvTensorCalcRequirementsForImages(14, 64, 18, NVCV_IMAGE_FORMAT_RGB8, 0, 0, &reqs));
+    {
+        const int64_t gold[4] = {14, 18, 64, 3};
+        EXPECT(4, reqs.rank);
+        EXPECT(0, memcmp(reqs.shape, gold, sizeof(gold)));
+        EXPECT(1, SameLayout(reqs.layout, NVCV_TENSOR_NHWC));
+        EXPECT(1, reqs.dtype == NVCV_DATA_TYPE_U8);
+    }
+
+    /* rows padded to 32 bytes */
+    const struct
+    {
+        NVCVTensorLayout layout;
+        int              rank;
+        int64_t          shape[4], strides[4];
+    } rows[] = {
+        {NVCV_TENSOR_NCHW, 4, {53, 4, 16, 17}, {4 * 16 * 32, 16 * 32, 32, 1}},
+        {NVCV_TENSOR_NHWC, 4, {53, 17, 16, 3},         {17 * 64, 64, 3, 1}},
+        { NVCV_TENSOR_CHW, 3,     {4, 16, 17},            {16 * 32, 32, 1}},
+        { NVCV_TENSOR_HWC, 3,     {17, 16, 3},                  {64, 3, 1}},
+    };
+    for (size_t r = 0; r < sizeof(rows) / sizeof(rows[0]); ++r)
+    {
+        NVCVTensorHandle t = NULL;
+        NVCVTensorData   d;
+        EXPECT(OK, nvcvTensorCalcRequirements(rows[r].rank, rows[r].shape, NVCV_DATA_TYPE_U8, rows[r].layout, 0, 32, &reqs));
+        EXPECT(0, memcmp(reqs.strides, rows[r].strides, rows[r].rank * sizeof(int64_t)));
+        EXPECT(OK, nvcvTensorConstruct(&reqs, alloc, &t));
+        EXPECT(OK, nvcvTensorExportData(t, &d));
+        EXPECT(NVCV_TENSOR_BUFFER_STRIDED_CUDA, d.bufferType);
+        EXPECT(rows[r].rank, d.rank);
+        EXPECT(0, memcmp(d.shape, rows[r].shape, rows[r].rank * sizeof(int64_t)));
+        EXPECT(0, memcmp(d.buffer.strided.strides, rows[r].strides, rows[r].rank * sizeof(int64_t)));
+        EXPECT(1, d.buffer.strided.basePtr != NULL);
+        EXPECT(OK, nvcvTensorDecRef(t, NULL));
+    }
+
+    /* packed rows, 32-byte base: the allocator is asked for exactly that alignment */
+    NVCVResourceAllocator rec = HeapResource(NVCV_RESOURCE_MEM_CUDA);
+    rec.res.mem.fnAlloc       = RecordingAlloc;
+    NVCVAllocatorHandle recording = NULL;
+    NVCVTensorHandle    t = NULL, wrapped = NULL;
+    NVCVTensorData      d, w;
+    EXPECT(OK, nvcvAllocatorConstructCustom(&rec, 1, &recording));
+    EXPECT(OK, nvcvTensorCalcRequirementsForImages(5, 163, 117, NVCV_IMAGE_FORMAT_RGBA8, 32, 1, &reqs));
+    g_lastDeviceAlign = 0;
+    EXPECT(OK, nvcvTensorConstruct(&reqs, recording, &t));
+    EXPECT(32, g_lastDeviceAlign);
+    EXPECT(OK, nvcvTensorExportData(t, &d));
+    EXPECT(1, d.buffer.strided.strides[3]);
+    EXPECT(4, d.buffer.strided.strides[2]);
+    EXPECT(163 * 4, d.buffer.strided.strides[1]);
+    EXPECT(117 * 163 * 4, d.buffer.strided.strides[0]);
+    NVCVAllocatorHandle got = NULL;
+    EXPECT(OK, nvcvTensorGetAllocator(t, &got));
+    EXPECT(1, got == recording);
+    EXPECT(OK, nvcvAllocatorDecRef(got, NULL)); /* the getter hands out a reference */
+    EXPECT(OK, nvcvTensorDecRef(t, NULL));
+    EXPECT(OK, nvcvAllocatorDecRef(recording, NULL));
+
+    /* two half-float planes: NCHW with two channels, and a tensor wrapping the exported data is its twin */
+    NVCVImageFormat twoPlanes = NVCV_DETAIL_MAKE_COLOR_FMT2(RGB, BT601_ER, PL, FLOAT, XY00, ASSOCIATED, X16, X16);
+    EXPECT(OK, nvcvTensorCalcRequirementsForImages(5, 173, 79, twoPlanes, 32, 1, &reqs));
+    EXPECT(OK, nvcvTensorConstruct(&reqs, alloc, &t));
+    EXPECT(OK, nvcvTensorExportData(t, &d));
+    {
+        const int64_t gold[4] = {5, 2, 79, 173};
+        EXPECT(4, d.rank);
+        EXPECT(0, memcmp(d.shape, gold, sizeof(gold)));
+        EXPECT(1, SameLayout(d.layout, NVCV_TENSOR_NCHW));
+        EXPECT(1, d.dtype == NVCV_DATA_TYPE_F16);
+        EXPECT(2, d.buffer.strided.strides[3]);
+        EXPECT(173 * 2, d.buffer.strided.strides[2]);
+    }
+    EXPECT(OK, nvcvTensorWrapDataConstruct(&d, NULL, NULL, &wrapped));
+    EXPECT(OK, nvcvTensorExportData(wrapped, &w));
+    EXPECT(d.rank, w.rank);
+    EXPECT(0, memcmp(d.shape, w.shape, 4 * sizeof(int64_t)));
+    EXPECT(0, memcmp(d.buffer.strided.strides, w.buffer.strided.strides, 4 * sizeof(int64_t)));
+    EXPECT(1, SameLayout(d.layout, w.layout));
+    EXPECT(1, d.dtype == w.dtype);
+    EXPECT(1, d.buffer.strided.basePtr == w.buffer.strided.basePtr);
+    got = alloc;
+    EXPECT(OK, nvcvTensorGetAllocator(wrapped, &got));
+    EXPECT(1, got == NULL); /* foreign memory: no allocator */
+    EXPECT(OK, nvcvTensorDecRef(wrapped, NULL));
+    EXPECT(OK, nvcvTensorDecRef(t, NULL));
+
+    /* one image seen as a tensor */
+    const struct
+    {
+        NVCVImageFormat  fmt;
+        int64_t          shape[4];
+        NVCVTensorLayout layout;
+        NVCVDataType     dtype;
+    } views[] = {
+        {NVCV_IMAGE_FORMAT_RGBA8p, {1, 4, 23, 61}, NVCV_TENSOR_NCHW,  NVCV_DATA_TYPE_U8},
+        { NVCV_IMAGE_FORMAT_RGBA8, {1, 23, 61, 4}, NVCV_TENSOR_NHWC,  NVCV_DATA_TYPE_U8},
+        {  NVCV_IMAGE_FORMAT_RGB8, {1, 23, 61, 3}, NVCV_TENSOR_NHWC,  NVCV_DATA_TYPE_U8},
+        { NVCV_IMAGE_FORMAT_RGB8p, {1, 3, 23, 61}, NVCV_TENSOR_NCHW,  NVCV_DATA_TYPE_U8},
+        {   NVCV_IMAGE_FORMAT_F32, {1, 1, 23, 61}, NVCV_TENSOR_NCHW, NVCV_DATA_TYPE_F32},
+        {  NVCV_IMAGE_FORMAT_2F32, {1, 23, 61, 2}, NVCV_TENSOR_NHWC, NVCV_DATA_TYPE_F32},
+    };
+    for (size_t v = 0; v < sizeof(views) / sizeof(views[0]); ++v)
+    {
+        NVCVImageHandle img = MakeImage(alloc, 61, 23, views[v].fmt);
+        NVCVImageData   id;
+        EXPECT(OK, nvcvImageExportData(img, &id));
+        EXPECT(OK, nvcvTensorWrapImageConstruct(img, &t));
+        EXPECT(OK, nvcvTensorExportData(t, &d));
+        EXPECT(4, d.rank);
+        EXPECT(0, memcmp(d.shape, views[v].shape, 4 * sizeof(int64_t)));
+        EXPECT(1, SameLayout(d.layout, views[v].layout));
+        EXPECT(1, d.dtype == views[v].dtype);
+        EXPECT(1, d.buffer.strided.basePtr == id.buffer.strided.planes[0].basePtr);
+        const int channelFirst = d.layout.data[1] == 'C';
+        const int32_t planes   = id.buffer.strided.numPlanes;
+        EXPECT(channelFirst ? (int)views[v].shape[1] : 1, planes);
+        int32_t pixelBytes = 0;
+        EXPECT(OK, nvcvImageFormatGetPlanePixelStrideBytes(views[v].fmt, 0, &pixelBytes));
+        EXPECT(id.buffer.strided.planes[0].rowStride, d.buffer.strided.strides[channelFirst ? 2 : 1]);
+        EXPECT(pixelBytes, d.buffer.strided.strides[channelFirst ? 3 : 2]);
+        for (int32_t p = 1; p < planes; ++p)
+        {
+            EXPECT(1, id.buffer.strided.planes[p].basePtr == d.buffer.strided.basePtr + p * d.buffer.strided.strides[1]);
+        }
+        EXPECT(OK, nvcvTensorDecRef(t, NULL));
+        EXPECT(OK, nvcvImageDecRef(img, NULL));
+    }
 }
 
 static void TensorFromImageCases(NVCVAllocatorHandle alloc)
@@ -422,6 +579,101 @@ static void AllocatorCases(void)
                nvcvResourceTypeGetName((NVCVResourceType)255));
 }
 
+/* Custom resources count their calls in their context: +1 per allocation, +10 per release; the cleanup callback
+ * sees the final count and the stored descriptor. */
+static void *CountingAlloc(void *ctx, int64_t size, int32_t align)
+{
+    *(int *)ctx += 1;
+    return HeapAlloc(NULL, size, align);
+}
+
+static void CountingFree(void *ctx, void *ptr, int64_t size, int32_t align)
+{
+    *(int *)ctx += 10;
+    HeapFree(NULL, ptr, size, align);
+}
+
+static void CountingCleanup(void *ctx, NVCVResourceAllocator *a)
+{
+    EXPECT(1, ctx == a->ctx);
+    EXPECT(11, *(int *)ctx % 100);
+    *(int *)ctx = -*(int *)ctx;
+}
+
+static void AllocatorUseCases(int device)
+{
+    int                   ctx[2] = {100, 200};
+    NVCVResourceAllocator res[2];
+    for (int i = 0; i < 2; ++i)
+    {
+        memset(&res[i], 0, sizeof(res[i]));
+        res[i].resType         = i == 0 ? NVCV_RESOURCE_MEM_HOST : NVCV_RESOURCE_MEM_CUDA;
+        res[i].ctx             = &ctx[i];
+        res[i].res.mem.fnAlloc = CountingAlloc;
+        res[i].res.mem.fnFree  = CountingFree;
+        res[i].cleanup         = CountingCleanup;
+    }
+    NVCVAllocatorHandle h = NULL;
+    EXPECT(OK, nvcvAllocatorConstructCustom(res, 2, &h));
+    int refs = 0;
+    EXPECT(OK, nvcvAllocatorRefCount(h, &refs));
+    EXPECT(1, refs);
+    for (int i = 0; i < 2; ++i)
+    {
+        NVCVResourceAllocator got;
+        memset(&got, 0, sizeof(got));
+        EXPECT(OK, nvcvAllocatorGet(h, res[i].resType, &got));
+        EXPECT(res[i].resType, got.resType);
+        EXPECT(1, got.ctx == res[i].ctx);
+        EXPECT(1, got.res.mem.fnAlloc == res[i].res.mem.fnAlloc);
+        EXPECT(1, got.res.mem.fnFree == res[i].res.mem.fnFree);
+    }
+    NVCVResourceAllocator pinned;
+    EXPECT(OK, nvcvAllocatorGet(h, NVCV_RESOURCE_MEM_HOST_PINNED, &pinned)); /* the default one fills the gap */
+    EXPECT(NVCV_RESOURCE_MEM_HOST_PINNED, pinned.resType);
+    EXPECT(1, pinned.res.mem.fnAlloc != NULL && pinned.res.mem.fnFree != NULL);
+    EXPECT(BAD_ARG, nvcvAllocatorGet(h, NVCV_RESOURCE_MEM_HOST, NULL));
+
+    void *p = NULL;
+    EXPECT(OK, nvcvAllocatorAllocHostMemory(h, &p, 1 << 20, 256));
+    EXPECT(1, p != NULL);
+    EXPECT(101, ctx[0]);
+    EXPECT(OK, nvcvAllocatorFreeHostMemory(h, p, 1 << 20, 256));
+    EXPECT(111, ctx[0]);
+    EXPECT(OK, nvcvAllocatorAllocCudaMemory(h, &p, 1 << 20, 256));
+    EXPECT(1, p != NULL);
+    EXPECT(201, ctx[1]);
+    EXPECT(OK, nvcvAllocatorFreeCudaMemory(h, p, 1 << 20, 256));
+    EXPECT(211, ctx[1]);
+    if (device)
+    {
+        p = NULL;
+        EXPECT(OK, nvcvAllocatorAllocHostPinnedMemory(h, &p, 1 << 20, 256));
+        EXPECT(1, p != NULL);
+        EXPECT(OK, nvcvAllocatorFreeHostPinnedMemory(h, p, 1 << 20, 256));
+    }
+
+    void *user = (void *)1;
+    EXPECT(OK, nvcvAllocatorGetUserPointer(h, &user));
+    EXPECT(1, user == NULL);
+    EXPECT(OK, nvcvAllocatorSetUserPointer(h, (void *)0x123));
+    EXPECT(OK, nvcvAllocatorGetUserPointer(h, &user));
+    EXPECT(1, user == (void *)0x123);
+    EXPECT(OK, nvcvAllocatorSetUserPointer(h, NULL));
+    EXPECT(OK, nvcvAllocatorGetUserPointer(h, &user));
+    EXPECT(1, user == NULL);
+
+    EXPECT(OK, nvcvAllocatorIncRef(h, &refs));
+    EXPECT(2, refs);
+    EXPECT(OK, nvcvAllocatorDecRef(h, &refs));
+    EXPECT(1, refs);
+    EXPECT(111, ctx[0]); /* not cleaned up while a reference is left */
+    EXPECT(OK, nvcvAllocatorDecRef(h, &refs));
+    EXPECT(0, refs);
+    EXPECT(-111, ctx[0]);
+    EXPECT(-211, ctx[1]);
+}
+
 #define BATCH_CAPACITY 32
 
 static NVCVImageHandle g_pushed[BATCH_CAPACITY + 8];
@@ -518,9 +770,11 @@ int main(int argc, char **argv)
     TensorRequirementCases();
     TensorObjectCases(alloc);
     PermuteCases();
+    TensorShapeCases(alloc);
     TensorFromImageCases(alloc);
     ImageCases(alloc);
     AllocatorCases();
+    AllocatorUseCases(device);
     if (device)
     {
         ImageBatchCases(alloc);
