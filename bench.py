@@ -373,6 +373,164 @@ class WarpC4:
         return 8
 
 
+class FusedVarShape:
+    """Configuration 2's geometry on an image batch: 64 separately allocated u8 RGB images of mixed sizes, each resized
+    to 455x256 (its own scale factors), cropped and written to one f32 NCHW tensor."""
+    key, config_id = "fused-varshape", 2
+    N = 64
+    NEW_W, NEW_H, CROP_X, CROP_Y, OUT_H, OUT_W = Fused.NEW_W, Fused.NEW_H, Fused.CROP_X, Fused.CROP_Y, Fused.OUT_H, Fused.OUT_W
+    SCALE, OFFSET = Fused.SCALE, Fused.OFFSET
+    kernel = "FusedBilinear<float,true,false,false,true>"
+    dtype = "f32"
+    workload = ("fused ResizeCropConvertReformat, image batch: 64 u8 RGB images, W in [1280,1920], H in [720,1080] -> "
+                "bilinear 455x256 -> crop 224x224 @(115,16) -> f32 NCHW tensor, scale/offset")
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        rng = np.random.default_rng(SEED_BASE + 20)
+        self.sizes = [(int(rng.integers(1280, 1921)), int(rng.integers(720, 1081))) for _ in range(self.N)]
+        self.alg_bytes = 0
+        for w, h in self.sizes:
+            rows, _ = span_bytes(self.OUT_H, self.CROP_Y, h, self.NEW_H, LINEAR, 1)
+            _, span = span_bytes(self.OUT_W, self.CROP_X, w, self.NEW_W, LINEAR, 3)
+            self.alg_bytes += rows * span + 3 * self.OUT_H * self.OUT_W * 4
+        self.hosts = [orc.fill_u8((h, w, 3), SEED_BASE + 2000 + i) for i, (w, h) in enumerate(self.sizes)]
+        self.op = cv.ResizeCropConvertReformat()
+
+    def make_set(self):
+        cv = self.cv
+        batch = cv.ImageBatchVarShape(self.N)
+        for a in self.hosts:
+            batch.push_back(cv.Image.from_numpy(a, cv.K.IMAGE_FORMAT_RGB8))
+        return batch, cv.Tensor.alloc([self.N, 3, self.OUT_H, self.OUT_W], self.np.float32, "NCHW")
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], (self.NEW_W, self.NEW_H), LINEAR, (self.CROP_X, self.CROP_Y), 0, self.SCALE,
+                self.OFFSET, False)
+
+    def _oracle(self, a, threads=1):
+        return self.orc.fused_rccr(a[None], (self.OUT_H, self.OUT_W), (self.NEW_W, self.NEW_H), (self.CROP_X, self.CROP_Y),
+                                   LINEAR, self.np.float32, True, 0, self.SCALE, self.OFFSET, False, threads=threads)[0]
+
+    def check(self, s):
+        np = self.np
+        got = s[1].torch_view()[:2].cpu().numpy()
+        for i in range(2):
+            ref = self._oracle(self.hosts[i])
+            assert (np.abs(got[i] - ref) <= 1e-5 * np.maximum(1.0, np.abs(ref))).all(), "bench output differs from oracle"
+
+    def cpu(self, threads):
+        for a in self.hosts[:8]:
+            self._oracle(a, threads)
+        return 8
+
+
+class ResizeVarShape:
+    """Configuration 1's reduction on an image batch: 32 u8 RGB images of mixed sizes, each to its own 224x224 image."""
+    key, config_id = "resize-linear-varshape", 1
+    N, OUT = 32, 224
+    kernel = "ResizePatchVarShapeKernel<uint8_t,3,LINEAR>"
+    dtype = "f32"
+    workload = "Resize LINEAR, image batch: 32 u8 RGB images, W in [1280,1920], H in [720,1080] -> 224x224 each"
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        rng = np.random.default_rng(SEED_BASE + 21)
+        self.sizes = [(int(rng.integers(1280, 1921)), int(rng.integers(720, 1081))) for _ in range(self.N)]
+        self.alg_bytes = 0
+        for w, h in self.sizes:
+            rows, _ = span_bytes(self.OUT, 0, h, self.OUT, LINEAR, 1)
+            _, span = span_bytes(self.OUT, 0, w, self.OUT, LINEAR, 3)
+            self.alg_bytes += rows * span + self.OUT * self.OUT * 3
+        self.hosts = [orc.fill_u8((h, w, 3), SEED_BASE + 3000 + i) for i, (w, h) in enumerate(self.sizes)]
+        self.op = cv.Resize()
+
+    def make_set(self):
+        cv = self.cv
+        bi, bo, outs = cv.ImageBatchVarShape(self.N), cv.ImageBatchVarShape(self.N), []
+        for a in self.hosts:
+            bi.push_back(cv.Image.from_numpy(a, cv.K.IMAGE_FORMAT_RGB8))
+            o = cv.Image.alloc((self.OUT, self.OUT), cv.K.IMAGE_FORMAT_RGB8)
+            outs.append(o)
+            bo.push_back(o)
+        return bi, bo, outs
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], LINEAR)
+
+    def check(self, s):
+        np = self.np
+        for i in range(2):
+            ref = self.orc.resize(self.hosts[i][None], (self.OUT, self.OUT), LINEAR, variant=0)[0]
+            got = s[2][i].plane_view(0, np.uint8, 3).cpu().numpy()
+            assert np.abs(got.astype(np.int16) - ref.astype(np.int16)).max() <= 1
+
+    def cpu(self, threads):
+        for a in self.hosts[:8]:
+            self.orc.resize(a[None], (self.OUT, self.OUT), LINEAR, variant=0, threads=threads)
+        return 8
+
+
+class CropFlipNormalize:
+    """CropFlipNormalizeReformat as the classification pipelines use it: a 224x224 crop of each image of a batch,
+    mirrored or not, (x - mean) / std per channel, written as f32 NCHW."""
+    key, config_id = "crop-flip-normalize-224", 0
+    N, OUT = 64, 224
+    kernel = "CfnrRunsKernel<uint8_t,float,3>"
+    dtype = "f32"
+    workload = ("CropFlipNormalizeReformat: 64 u8 RGB images, W in [256,512], H in [256,384] -> crop 224x224 at a random "
+                "place, random flip code, per-channel (x - base) * scale -> f32 NCHW tensor")
+
+    def __init__(self, cv, orc, np, torch):
+        self.cv, self.orc, self.np, self.torch = cv, orc, np, torch
+        self.images = self.N
+        rng = np.random.default_rng(SEED_BASE + 22)
+        self.sizes = [(int(rng.integers(256, 513)), int(rng.integers(256, 385))) for _ in range(self.N)]
+        self.hosts = [orc.fill_u8((h, w, 3), SEED_BASE + 4000 + i) for i, (w, h) in enumerate(self.sizes)]
+        self.crops = np.zeros((self.N, 1, 1, 4), np.int32)
+        for i, (w, h) in enumerate(self.sizes):
+            self.crops[i, 0, 0] = (rng.integers(0, w - self.OUT + 1), rng.integers(0, h - self.OUT + 1), self.OUT, self.OUT)
+        self.flips = rng.integers(-1, 3, self.N).astype(np.int32)
+        self.base = (np.asarray(Fused.MEAN, np.float32) * 255).reshape(1, 1, 1, 3)
+        self.scale = (1 / (np.asarray(Fused.STD, np.float32) * 255)).astype(np.float32).reshape(1, 1, 1, 3)
+        self.alg_bytes = self.N * self.OUT * self.OUT * 3 * (1 + 4)
+        self.op = cv.CropFlipNormalizeReformat()
+
+    def make_set(self):
+        cv = self.cv
+        batch = cv.ImageBatchVarShape(self.N)
+        for a in self.hosts:
+            batch.push_back(cv.Image.from_numpy(a, cv.K.IMAGE_FORMAT_RGB8))
+        return (batch, cv.Tensor.alloc([self.N, 3, self.OUT, self.OUT], self.np.float32, "NCHW"),
+                cv.Tensor.from_numpy(self.crops, "NHWC"), cv.Tensor.from_numpy(self.flips, "N"),
+                cv.Tensor.from_numpy(self.base, "NHWC"), cv.Tensor.from_numpy(self.scale, "NHWC"))
+
+    def submit(self, stream, s):
+        self.op(stream, s[0], s[1], s[2], 0, 0.0, s[3], s[4], s[5])
+
+    def _oracle(self, i):
+        return self.orc.crop_flip_normalize(self.hosts[i], (self.OUT, self.OUT), self.np.float32, self.crops[i, 0, 0],
+                                            self.flips[i], 0, 0.0, self.base.reshape(-1), self.scale.reshape(-1), 1.0,
+                                            0.0, 0.0, False)
+
+    def check(self, s):
+        np = self.np
+        got = s[1].torch_view()[:2].cpu().numpy().transpose(0, 2, 3, 1)
+        for i in range(2):
+            ref = self._oracle(i)
+            assert np.abs(got[i] - ref).max() <= 1e-5 * max(1.0, np.abs(ref).max()), "bench output differs from oracle"
+
+    def cpu_cores(self, threads):
+        return 1
+
+    def cpu(self, threads):
+        for i in range(self.N):
+            self._oracle(i)
+        return self.N
+
+
 class WarpTensor:
     """WarpAffine on a tensor: 32 u8 RGB images of 1280x780 rotated by 17 degrees about the centre at scale 1.05
     (forward map), constant border 0. Algorithmic bytes: the part of the source the destination's inverse image
@@ -593,6 +751,9 @@ WORKLOADS = {
     "resize-linear": lambda *a: ResizeC1(*a, LINEAR),
     "nv12-to-rgb": Nv12C3,
     "warp-affine-varshape": WarpC4,
+    "fused-varshape": FusedVarShape,
+    "resize-linear-varshape": ResizeVarShape,
+    "crop-flip-normalize-224": CropFlipNormalize,
     "warp-affine-tensor-nearest": lambda *a: WarpTensor(*a, NEAREST),
     "warp-affine-tensor-linear": lambda *a: WarpTensor(*a, LINEAR),
     "warp-affine-tensor-cubic": lambda *a: WarpTensor(*a, CUBIC),
