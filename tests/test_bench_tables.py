@@ -31,3 +31,23 @@ def test_every_workload_named_in_a_profile_exists():
     for f in sorted(os.listdir(os.path.join(ROOT, "profiles"))):
         for wl in re.findall(r"bench\.py --workload (\S+)", open(os.path.join(ROOT, "profiles", f)).read()):
             assert wl in bench.WORKLOADS, (f, wl)
+
+
+def test_byte_conventions_of_the_baseline_configurations():
+    """The three byte counts a launch can be priced with, from the operators' own index maps: the row spans
+    (`roofline.achieved`), whole tensors, referenced pixels only. The expected numbers are closed forms of the
+    configurations' shapes (448 distinct rows and columns for 224 bilinear outputs, 4 taps per output for bicubic)."""
+    b = load_bench()
+    rows, span = b.span_bytes(224, 16, 1080, 256, b.LINEAR, 1)[0], b.span_bytes(224, 115, 1920, 455, b.LINEAR, 3)[1]
+    cols = b.span_bytes(224, 115, 1920, 455, b.LINEAR, 3)[0]
+    out = 3 * 224 * 224 * 4
+    assert (rows, cols, span) == (448, 448, 2829)
+    assert (rows * span + out) * 64 == 119648256            # fused, row spans
+    assert (rows * cols * 3 + out) * 64 == 77070336          # referenced pixels only
+    assert (1080 * 1920 * 3 + out) * 64 == 436666368         # whole tensors
+    rows, cols = b.span_bytes(224, 0, 1080, 224, b.LINEAR, 1)[0], b.span_bytes(224, 0, 1920, 224, b.LINEAR, 3)[0]
+    assert (rows * cols + 224 * 224) * 3 * 8 == 6021120      # Resize LINEAR 1080p -> 224, batch 8
+    rows, cols = b.span_bytes(224, 0, 1080, 224, b.NEAREST, 1)[0], b.span_bytes(224, 0, 1920, 224, b.NEAREST, 3)[0]
+    assert (rows, cols) == (224, 224)
+    rows, cols = b.span_bytes(360, 0, 2160, 360, b.CUBIC, 1)[0], b.span_bytes(640, 0, 3840, 640, b.CUBIC, 16)[0]
+    assert (rows, cols) == (1440, 2560) and (rows * cols + 360 * 640) * 16 * 16 == 1002700800
