@@ -6,6 +6,7 @@
 #include <nvcv/Config.h>
 #include <nvcv/ImageBatch.h>
 #include <nvcv/Tensor.h>
+#include <nvcv/TensorShape.h>
 #include <nvcv/Version.h>
 
 #include <atomic>

@@ -1,4 +1,4 @@
-/* Replaces: src/nvcv/src/include/nvcv/Size.h:31-34 and Rect.h:27-33. */
+/* Width and height of an image in pixels. Replaces: src/nvcv/src/include/nvcv/Size.h:31-34. */
 #ifndef NVCV_SIZE_H
 #define NVCV_SIZE_H
 
@@ -8,10 +8,5 @@ typedef struct
 {
     int32_t w, h;
 } NVCVSize2D;
-
-typedef struct
-{
-    int32_t x, y, width, height;
-} NVCVRectI;
 
 #endif /* NVCV_SIZE_H */

@@ -1,5 +1,5 @@
 /* Tensor layouts: up to 15 one-letter dimension labels, e.g. "NHWC".
- * Replaces: src/nvcv/src/include/nvcv/TensorLayout.h:36-297, TensorLayoutDef.inc, TensorShape.h:45-46.
+ * Replaces: src/nvcv/src/include/nvcv/TensorLayout.h:36-297, TensorLayoutDef.inc.
  * The struct is passed and returned by value across the ABI: 16 chars + int32 rank = 20 bytes. */
 #ifndef NVCV_TENSORLAYOUT_H
 #define NVCV_TENSORLAYOUT_H
@@ -96,10 +96,6 @@ NVCV_PUBLIC NVCVStatus nvcvTensorLayoutMakeFirst(NVCVTensorLayout in, int32_t n,
 NVCV_PUBLIC NVCVStatus nvcvTensorLayoutMakeLast(NVCVTensorLayout in, int32_t n, NVCVTensorLayout *layout);
 NVCV_PUBLIC NVCVStatus nvcvTensorLayoutMakeSubRange(NVCVTensorLayout in, int32_t beg, int32_t end,
                                                     NVCVTensorLayout *layout);
-
-/* dstShape[j] = srcShape[i] where srcLayout[i]==dstLayout[j]; dimensions absent from src become 1. */
-NVCV_PUBLIC NVCVStatus nvcvTensorShapePermute(NVCVTensorLayout srcLayout, const int64_t *srcShape,
-                                              NVCVTensorLayout dstLayout, int64_t *dstShape);
 
 /* Index of the first `label` at or after idxStart (negative idxStart counts from the end), or -1. */
 static inline int32_t nvcvTensorLayoutFindDimIndex(NVCVTensorLayout layout, char label, int idxStart)

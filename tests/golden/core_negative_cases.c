@@ -9,6 +9,7 @@
 #include <nvcv/Image.h>
 #include <nvcv/ImageBatch.h>
 #include <nvcv/Tensor.h>
+#include <nvcv/TensorShape.h>
 #include <nvcv/alloc/Allocator.h>
 #include <stdio.h>
 #include <stdlib.h>
