@@ -195,6 +195,16 @@ struct BgrFromYuv
 // rounded to nearest: a table in the reference (cvt_color.cu:232-270, filled on the host). Here each block
 // fills its own copy in LDS, one entry of each per thread, so a pixel costs two LDS reads instead of two
 // float divisions (which are a dozen instructions each).
+// a * b + c for factors of at most 24 significant bits (sign included) whose product fits 32 bits: one full-rate
+// instruction. The compiler picks it by itself only where it can see the factors' ranges, which it cannot for
+// values read from a table; its 32-bit multiply-add issues at a quarter of the rate.
+__device__ __forceinline__ int MulAdd24(int a, int b, int c)
+{
+    int r;
+    asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 __device__ __forceinline__ int32_t *HsvDivTable()
 {
     __shared__ int32_t table[512];
@@ -236,9 +246,11 @@ struct HsvFromBgr
             const int32_t *table = HsvDivTable();
             const int      hdiv  = table[256 + diff];
             const int      sdiv  = table[val];
-            const int sat  = (diff * sdiv + (1 << 11)) >> 12;
+            // both products have factors of under 24 bits (|h| <= 5 * 255, quotients <= 255 << 12) and fit 32 bits:
+            // the 24-bit multiply is exact here and issues at full rate, the 32-bit one at a quarter of it
+            const int sat  = (MulAdd24(diff, sdiv, 1 << 11)) >> 12;
             int       h    = (vr & (g - b)) + (~vr & ((vg & (b - r + 2 * diff)) + ((~vg) & (r - g + 4 * diff))));
-            h              = (h * hdiv + (1 << 11)) >> 12;
+            h              = (MulAdd24(h, hdiv, 1 << 11)) >> 12;
             h += h < 0 ? hrange : 0;
             o.v[0] = SatInt<T>(h);
             o.v[1] = (T)sat;
