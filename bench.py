@@ -929,7 +929,14 @@ def main():
         done, tcpu = cpu_leg(threads, args.cpu_seconds)
         used = wl.cpu_cores(threads) if hasattr(wl, "cpu_cores") else threads
         done1, tcpu1 = cpu_leg(1, args.cpu_seconds / 2)
+        model = ""
+        try:
+            with open("/proc/cpuinfo") as f:
+                model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
+        except OSError:
+            pass
         cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": used, "kind": "port",
+               "host": {"cpu_model": model, "logical_cpus": os.cpu_count()},
                "sample": "%d images of this workload through the CPU oracle in %.1f s, %d thread%s"
                          % (done, tcpu, used, "" if used == 1 else "s"),
                "single_thread": {"value": round(done1 / tcpu1, 1), "unit": "images/s", "cores": 1,
