@@ -294,15 +294,15 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             }
         };
         auto add = [&](int x, int y, float w) { addRun(x, x + 1, y, w); };
-        // u8x3 at horizontal scales up to 2: the taps of one source row (a partial pixel on the left, up to 2
-        // whole ones, a partial one on the right) lie within 4 pixels, one 12-byte load instead of one 2- and
-        // one 1-byte load per tap (226 -> 151 us per 32 x 1080p -> 720p). Which taps exist differs from lane to
+        // u8 pixels of 1, 3 or 4 channels at horizontal scales up to 2: the taps of one source row (a partial pixel on
+        // the left, up to 2 whole ones, a partial one on the right) lie within 4 pixels, one load of 4 pixels instead
+        // of one per tap (u8x3: a 2- and a 1-byte load per tap before; 226 -> 151 us per 32 x 1080p -> 720p). Which taps exist differs from lane to
         // lane, their order in the sums does not. The kernel is bound by the bytes its lanes ask for, not by
         // latency: with the windows of the 4 rows from ymin - 1 on all loaded before the first sum (4 loads
         // where 2 or 3 are needed) it took 208 us. Rows before the image's last one only: a load may read up
-        // to 9 bytes past its taps.
+        // to 3 pixels past its taps.
         bool windowed = false;
-        if constexpr (std::is_same_v<T, uint8_t> && C == 3)
+        if constexpr (std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4))
         {
             windowed = scaleX <= 2.f && p.srcW >= 4 && ymax < p.srcH - 1;
         }
@@ -310,12 +310,28 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
         const int  winX = xmin - (hasLeft ? 1 : 0), innerN = min(xmax, p.srcW) - xmin, rightI = xmax - winX;
         [[maybe_unused]] auto loadWindow = [&](int y, uint32_t (&px)[4])
         {
-            uint32_t w[3];
-            LoadDwords<3>(p.src + (int64_t)y * p.srcRow + winX * 3, w);
-            px[0] = w[0];
-            px[1] = __builtin_amdgcn_alignbit(w[1], w[0], 24);
-            px[2] = __builtin_amdgcn_alignbit(w[2], w[1], 16);
-            px[3] = w[2] >> 8;
+            // 4 pixels of C bytes, pixel k to px[k] (channel c in byte c; higher bytes are not looked at)
+            uint32_t w[C];
+            LoadDwords<C>(p.src + (int64_t)y * p.srcRow + winX * C, w);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                if constexpr (C == 1)
+                {
+                    px[k] = w[0] >> (8 * k);
+                }
+                else if constexpr (C == 4)
+                {
+                    px[k] = w[k];
+                }
+                else
+                {
+                    px[k] = k == 0 ? w[0]
+                          : k == 1 ? __builtin_amdgcn_alignbit(w[C > 1 ? 1 : 0], w[0], 24)
+                          : k == 2 ? __builtin_amdgcn_alignbit(w[C > 2 ? 2 : 0], w[C > 1 ? 1 : 0], 16)
+                                   : w[C > 2 ? 2 : 0] >> 8;
+                }
+            }
         };
         [[maybe_unused]] auto addPx = [&](uint32_t q, float w)
         {

@@ -199,7 +199,11 @@ AREA_ROWS = [(44, 40, 22, 20, 2, np.uint8, 4), (30, 30, 20, 20, 2, np.uint8, 4),
              # an enlargement, a mixed pair of scales, sources barely wider than the load
              (1920, 1080, 1280, 720, 1, np.uint8, 3), (97, 61, 61, 40, 2, np.uint8, 3), (64, 48, 32, 24, 2, np.uint8, 3),
              (33, 21, 33, 21, 1, np.uint8, 3), (50, 40, 75, 60, 2, np.uint8, 3), (40, 90, 31, 20, 2, np.uint8, 3),
-             (4, 4, 3, 3, 1, np.uint8, 3), (5, 9, 3, 2, 2, np.uint8, 3), (640, 3, 427, 2, 1, np.uint8, 3)]
+             (4, 4, 3, 3, 1, np.uint8, 3), (5, 9, 3, 2, 2, np.uint8, 3), (640, 3, 427, 2, 1, np.uint8, 3),
+             # the same form for 1- and 4-byte pixels
+             (97, 61, 61, 40, 2, np.uint8, 1), (64, 48, 32, 24, 2, np.uint8, 1), (50, 40, 75, 60, 2, np.uint8, 1),
+             (5, 9, 3, 2, 2, np.uint8, 1), (97, 61, 61, 40, 2, np.uint8, 4), (50, 40, 75, 60, 2, np.uint8, 4),
+             (5, 9, 3, 2, 2, np.uint8, 4), (1920, 1080, 1280, 720, 1, np.uint8, 4)]
 
 
 @pytest.mark.parametrize("row", AREA_ROWS, ids=lambda r: "%dx%d-%dx%d-n%d-%s%d" % (r[:5] + (np.dtype(r[5]).name, r[6])))
@@ -239,7 +243,7 @@ def test_area_sources_one_and_two_pixels_wide(cv, orc, gpu):
                 np.testing.assert_array_equal(tout.numpy(), device, err_msg=str((sw, sh, dw, dh, interp)))
 
 
-@pytest.mark.parametrize("dt,c", [(np.uint8, 4), (np.uint8, 3), (np.uint16, 1), (np.int16, 3), (np.float32, 4)])
+@pytest.mark.parametrize("dt,c", [(np.uint8, 4), (np.uint8, 3), (np.uint8, 1), (np.uint16, 1), (np.int16, 3), (np.float32, 4)])
 def test_area_varshape(cv, K, orc, gpu, dt, c):
     # image batches run the reference's separate AREA kernel (reductions: same sums, corners last;
     # enlargements: a bilinear variant). Sizes: the reference's rows (TestOpResize.cpp:67-69) plus
