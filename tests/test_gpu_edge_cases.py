@@ -342,3 +342,42 @@ def test_row_pieces_longer_than_one_store_with_odd_lane_counts(cv, K, orc, gpu):
         cv.ConvertTo()(None, cv.Tensor.from_numpy(a8, "NHWC"), f, 0.5, 1.0)
         torch.cuda.synchronize()
         np.testing.assert_array_equal(f.numpy(), a8.astype(np.float64) * 0.5 + 1.0)
+
+
+@pytest.mark.parametrize("h,w", [(300000, 16), (16, 300000)])
+def test_images_hundreds_of_thousands_of_pixels_tall_or_wide(cv, K, orc, gpu, h, w):
+    # launch grids far beyond 65535 blocks in one dimension; every operator in a form whose result is a closed
+    # form of the input (identity maps, mirrors, transposes)
+    a = orc.fill_u8((1, h, w, 3), 5)
+    tin = cv.Tensor.from_numpy(a, "NHWC")
+
+    def run(op, out_shape, dt, layout, *args):
+        out = cv.Tensor.alloc(out_shape, dt, layout)
+        out.torch_view().fill_(0x5A)
+        op(None, tin, out, *args)
+        torch.cuda.synchronize()
+        return out.numpy()
+
+    same = [1, h, w, 3]
+    np.testing.assert_array_equal(run(cv.CvtColor(), same, np.uint8, "NHWC", K.COLOR_BGR2RGB), a[..., ::-1])
+    np.testing.assert_array_equal(run(cv.Reformat(), [1, 3, h, w], np.uint8, "NCHW"), a.transpose(0, 3, 1, 2))
+    np.testing.assert_array_equal(run(cv.ConvertTo(), same, np.float32, "NHWC", 1.0, 0.0), a.astype(np.float32))
+    np.testing.assert_array_equal(run(cv.Flip(), same, np.uint8, "NHWC", 0), a[:, ::-1])
+    np.testing.assert_array_equal(run(cv.Flip(), same, np.uint8, "NHWC", 1), a[:, :, ::-1])
+    np.testing.assert_array_equal(run(cv.Resize(), same, np.uint8, "NHWC", NEAREST), a)
+    np.testing.assert_array_equal(run(cv.Resize(), same, np.uint8, "NHWC", LINEAR), a)
+    np.testing.assert_array_equal(run(cv.WarpAffine(0), same, np.uint8, "NHWC", [1, 0, 0, 0, 1, 0], LINEAR, 0, (0, 0, 0, 0)), a)
+    np.testing.assert_array_equal(run(cv.CustomCrop(), [1, h - 2, w - 2, 3], np.uint8, "NHWC", (1, 1, w - 2, h - 2)),
+                                  a[:, 1:-1, 1:-1])
+    zero = cv.Tensor.from_numpy(np.zeros((1, 1, 1, 3), np.float32), "NHWC")
+    one = cv.Tensor.from_numpy(np.ones((1, 1, 1, 3), np.float32), "NHWC")
+    out = cv.Tensor.alloc(same, np.uint8, "NHWC")
+    cv.Normalize()(None, tin, zero, one, out)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.numpy(), a)
+    got = run(cv.ResizeCropConvertReformat(), [1, 3, h, w], np.float32, "NCHW", (w, h), LINEAR, (0, 0), 0, 1.0, 0.0, False)
+    np.testing.assert_array_equal(got, a.transpose(0, 3, 1, 2).astype(np.float32))
+    gray = run(cv.CvtColor(), [1, h, w, 1], np.uint8, "NHWC", K.COLOR_BGR2GRAY)
+    want = (a[..., 0].astype(np.int64) * 3735 + a[..., 1].astype(np.int64) * 19235 + a[..., 2].astype(np.int64) * 9798
+            + (1 << 14)) >> 15
+    np.testing.assert_array_equal(gray[..., 0], want.astype(np.uint8))
