@@ -190,3 +190,62 @@ def test_colour_round_trips_on_a_1080p_batch(cv, K, gpu):
     cv.CvtColor()(None, gray, bgr, K.COLOR_GRAY2BGR)
     cv.CvtColor()(None, bgr, g2, K.COLOR_BGR2GRAY)
     assert torch.equal(g2.torch_view(), gray.torch_view())
+
+
+def test_image_batch_forms_on_32_images_of_mixed_sizes(cv, K, gpu):
+    # the sizes of BASELINE configuration 4: W in [640, 1920], H in [480, 1080]
+    rng = np.random.default_rng(4)
+    sizes = [(int(rng.integers(640, 1921)) & ~1, int(rng.integers(480, 1081)) & ~3) for _ in range(32)]
+    srcs = [device_u8(gpu, (h, w, 3), 100 + i) for i, (w, h) in enumerate(sizes)]
+
+    def batch_of(tensors, fmt=None):
+        b, images = cv.ImageBatchVarShape(len(tensors)), []
+        for t in tensors:
+            img = cv.Image.alloc((t.shape[1], t.shape[0]), fmt or K.IMAGE_FORMAT_RGB8)
+            img.plane_view(0, np.uint8, t.shape[2]).copy_(t)
+            images.append(img)
+            b.push_back(img)
+        return b, images
+
+    def empty_like(shapes, fmt=None, c=3):
+        return batch_of([torch.zeros((h, w, c), dtype=torch.uint8, device=gpu) for (w, h) in shapes], fmt)
+
+    bin_, _ = batch_of(srcs)
+
+    def views(images, c=3):
+        return [i.plane_view(0, np.uint8, c) for i in images]
+
+    # Resize to the same size and the identity warp return the images; a mirror twice as well
+    for op, args in ((cv.Resize(), (NEAREST,)), (cv.Resize(), (LINEAR,))):
+        bout, outs = empty_like(sizes)
+        op(None, bin_, bout, *args)
+        assert all(torch.equal(v, s) for v, s in zip(views(outs), srcs))
+    ident = cv.Tensor.from_numpy(np.tile(np.array([1, 0, 0, 0, 1, 0], np.float32), (32, 1)), "NW")
+    bout, outs = empty_like(sizes)
+    cv.WarpAffine(32)(None, bin_, bout, ident, LINEAR, 0, (0, 0, 0, 0))
+    assert all(torch.equal(v, s) for v, s in zip(views(outs), srcs))
+    codes = cv.Tensor.from_numpy(np.full((32,), -1, np.int32), "N")
+    bmid, mids = empty_like(sizes)
+    cv.Flip()(None, bin_, bmid, codes)
+    assert all(torch.equal(v, s.flip((0, 1))) for v, s in zip(views(mids), srcs))
+    bout, outs = empty_like(sizes)
+    cv.Flip()(None, bmid, bout, codes)
+    assert all(torch.equal(v, s) for v, s in zip(views(outs), srcs))
+    # colour: reversal twice; NV12 and back on images of constant 2 x 2 blocks
+    bout, outs = empty_like(sizes)
+    cv.CvtColor()(None, bin_, bmid, K.COLOR_BGR2RGB)
+    cv.CvtColor()(None, bmid, bout, K.COLOR_RGB2BGR)
+    assert all(torch.equal(v, s) for v, s in zip(views(outs), srcs))
+    blocky = [s[::2, ::2].repeat_interleave(2, dim=0).repeat_interleave(2, dim=1).contiguous() for s in srcs]
+    bblock, _ = batch_of(blocky)
+    bnv, nvs = empty_like([(w, h * 3 // 2) for (w, h) in sizes], K.IMAGE_FORMAT_U8, 1)
+    cv.CvtColor()(None, bblock, bnv, K.COLOR_BGR2YUV_NV12)
+    bout, outs = empty_like(sizes)
+    cv.CvtColor()(None, bnv, bout, K.COLOR_YUV2BGR_NV12)
+    for v, s in zip(views(outs), blocky):
+        diff = (v.int() - s.int()).abs()
+        assert float((diff <= 3).float().mean()) > 0.97 and int(diff.max()) < 64
+    # each image of the batch gives what the same image gives alone as a tensor
+    t = cv.Tensor.alloc([1, sizes[31][1] * 3 // 2, sizes[31][0], 1], np.uint8, "NHWC")
+    cv.CvtColor()(None, tensor_from(cv, blocky[31][None], "NHWC"), t, K.COLOR_BGR2YUV_NV12)
+    assert torch.equal(t.torch_view()[0], views(nvs, 1)[31])
