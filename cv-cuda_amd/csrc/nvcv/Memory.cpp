@@ -108,12 +108,13 @@ void HandlePool::addSlab(int count)
 void *HandlePool::create(std::unique_ptr<CoreObject> obj)
 {
     std::lock_guard<std::mutex> lock(m_mtx);
+    // a fixed size caps the live objects also where the pool had grown beyond it before
+    if (m_fixed && m_live.load() >= m_limit)
+    {
+        throw Error(NVCV_ERROR_OUT_OF_MEMORY, "%s handle pool is full (fixed capacity %d)", m_name, m_limit);
+    }
     if (m_free == nullptr)
     {
-        if (m_fixed)
-        {
-            throw Error(NVCV_ERROR_OUT_OF_MEMORY, "%s handle pool is full (fixed capacity %d)", m_name, m_capacity);
-        }
         addSlab(m_capacity == 0 ? 256 : m_capacity);
     }
     HandleSlot *s = m_free;
@@ -203,6 +204,7 @@ void HandlePool::setFixedSize(int32_t maxCount)
         addSlab(maxCount - m_capacity);
     }
     m_fixed = true;
+    m_limit = maxCount;
 }
 
 HandlePool &AllocatorPool()

@@ -270,6 +270,7 @@ private:
     int                      m_slabCount[kMaxSlabs] = {};
     int                      m_capacity             = 0;
     bool                     m_fixed                = false;
+    int                      m_limit                = 0; // live objects allowed while m_fixed
     std::atomic<int>         m_live{0};
 };
 

@@ -523,7 +523,7 @@ def test_wrap_parameter_cases_of_the_reference(cv, capi, shape, layout, strides,
     assert t.shape == shape and t.layout == layout and t.strides == strides
 
 
-def build_c_cases(name, tmp_path):
+def build_c_cases(name, tmp_path, extra=()):
     """Compiles tests/golden/<name>.c with gcc against the public headers and the core library."""
     import subprocess
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -531,7 +531,8 @@ def build_c_cases(name, tmp_path):
     exe = str(tmp_path / name)
     subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-D_POSIX_C_SOURCE=200112L", "-DCVCUDA_NO_HIP_HEADERS",
                     "-I" + os.path.join(root, "include"), os.path.join(root, "tests", "golden", name + ".c"), "-o", exe,
-                    "-L" + libdir, "-lnvcv_types", "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"], check=True)
+                    "-L" + libdir, "-lnvcv_types", "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"]
+                   + list(extra), check=True)
     return exe
 
 
@@ -539,6 +540,15 @@ def test_argument_checks_of_the_reference_from_plain_c(cv, tmp_path):
     import subprocess
     r = subprocess.run([build_c_cases("core_negative_cases", tmp_path)], capture_output=True, text=True)
     assert r.returncode == 0 and r.stdout.strip().endswith("0 failed"), r.stdout + r.stderr
+
+
+def test_handles_created_shared_and_destroyed_by_many_threads(cv, tmp_path):
+    """tests/golden/handle_pool_stress.c: 8 threads create, share by reference count and destroy tensors, images and
+    allocator-backed tensors; every cleanup runs once, nothing stays alive, destroyed handles are refused."""
+    import subprocess
+    r = subprocess.run([build_c_cases("handle_pool_stress", tmp_path, ["-pthread"]), "8", "5000"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().endswith(" 0 failed"), r.stdout + r.stderr
 
 
 @pytest.mark.gpu
