@@ -154,8 +154,8 @@ __device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *base, uint32_t 
     const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(base) & 3u;
     const uint32_t o   = off + mis;
     const W3       w   = *reinterpret_cast<const W3 *>((base - mis) + (o & ~3u));
-    const uint32_t lo  = __builtin_amdgcn_alignbit(w.d[1], w.d[0], o * 8u); // the shift uses bits 4:0
-    const uint32_t hi  = __builtin_amdgcn_alignbit(w.d[2], w.d[1], o * 8u);
+    const uint32_t lo  = __builtin_amdgcn_alignbyte(w.d[1], w.d[0], o); // shifts by the bytes in bits 1:0
+    const uint32_t hi  = __builtin_amdgcn_alignbyte(w.d[2], w.d[1], o);
     return ((uint64_t)hi << 32) | lo;
 }
 

@@ -309,8 +309,9 @@ __device__ __forceinline__ float InsideLimit(int size, bool wide)
 // Same arithmetic as SampleWithBorder for a sample whose taps are all inside the image: no border
 // logic, adjacent taps fetched together, no branches (so the loads of several pixels can be in flight
 // at once). floorf(v) is used directly where the generic path converts floor(v) to int and back.
-template<class T, int C, int INTERP>
-__device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, T (&out)[C])
+// O = T, or float for the unrounded sums (not for NEAREST).
+template<class O, int C, int INTERP, class T = O>
+__device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, O (&out)[C])
 {
     constexpr int PB = C * sizeof(T);
     float         acc[C];
@@ -377,7 +378,45 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
 #pragma unroll
     for (int c = 0; c < C; ++c)
     {
-        out[c] = SaturateCast<T>(acc[c]);
+        if constexpr (std::is_same_v<O, T>)
+        {
+            out[c] = SaturateCast<T>(acc[c]);
+        }
+        else
+        {
+            out[c] = acc[c];
+        }
+    }
+}
+
+// The dwords of the pixel that SampleInside gives. u8 channels are rounded, saturated and placed into
+// their byte by one instruction each (v_cvt_pk_u8_f32 with a byte select and the dword so far), where
+// packing converted bytes takes as many shifts and merges again.
+template<class T, int C, int INTERP>
+__device__ __forceinline__ void SampleInsidePacked(const Img &im, float sx, float sy, uint32_t (&w)[(C * sizeof(T) + 3) / 4])
+{
+    if constexpr (std::is_same_v<T, uint8_t> && INTERP != NVCV_INTERP_NEAREST)
+    {
+        float acc[C];
+        SampleInside<float, C, INTERP, T>(im, sx, sy, acc);
+        uint32_t q = 0;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            q = __builtin_amdgcn_cvt_pk_u8_f32(acc[c], c, q);
+        }
+        w[0] = q;
+    }
+    else
+    {
+        T v[C];
+        SampleInside<T, C, INTERP>(im, sx, sy, v);
+#pragma unroll
+        for (int d = 0; d < (int)((C * sizeof(T) + 3) / 4); ++d)
+        {
+            w[d] = 0;
+        }
+        __builtin_memcpy(w, v, C * sizeof(T));
     }
 }
 
@@ -495,21 +534,19 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     }
     if (allInside)
     {
-        T v[kPxPerLane][C];
+        uint32_t w[kPxPerLane][D];
 #pragma unroll
         for (int k = 0; k < kPxPerLane; ++k)
         {
-            SampleInside<T, C, INTERP>(im, sx[k], sy[k], v[k]);
+            SampleInsidePacked<T, C, INTERP>(im, sx[k], sy[k], w[k]);
         }
 #pragma unroll
         for (int k = 0; k < kPxPerLane; ++k)
         {
-            uint32_t w[D] = {};
-            __builtin_memcpy(w, v[k], PB);
 #pragma unroll
             for (int d = 0; d < D; ++d)
             {
-                q[d][k] = w[d];
+                q[d][k] = w[k][d];
             }
         }
     }
