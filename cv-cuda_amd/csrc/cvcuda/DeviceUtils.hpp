@@ -159,6 +159,20 @@ __device__ __forceinline__ uint64_t LoadU64Window(const uint8_t *base, uint32_t 
     return ((uint64_t)hi << 32) | lo;
 }
 
+// 4 bytes starting at the arbitrary byte address base + off, the same way: 2 aligned dwords and one
+// funnel shift. Reads up to 3 bytes before and up to 4 bytes after the data.
+__device__ __forceinline__ uint32_t LoadU32Window(const uint8_t *base, uint32_t off)
+{
+    struct alignas(4) W2
+    {
+        uint32_t d[2];
+    };
+    const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(base) & 3u;
+    const uint32_t o   = off + mis;
+    const W2       w   = *reinterpret_cast<const W2 *>((base - mis) + (o & ~3u));
+    return __builtin_amdgcn_alignbyte(w.d[1], w.d[0], o);
+}
+
 // The constant a caller gives for pixels outside the image, as an element of type T: truncated toward
 // zero and saturated to T's range (floats pass through).
 template<class T>

@@ -130,20 +130,20 @@ __device__ __forceinline__ int FloorToInt(float v)
 template<class T, int C>
 constexpr bool kWideTapLoads = std::is_same_v<T, uint8_t> && C == 3;
 
-// One pixel at p, known to be inside the image.
+// One pixel at base + off, known to be inside the image.
 template<class T, int C>
-__device__ __forceinline__ void LoadPixelInside(const uint8_t *p, T (&out)[C])
+__device__ __forceinline__ void LoadPixelInside(const uint8_t *base, uint32_t off, T (&out)[C])
 {
     if constexpr (kWideTapLoads<T, C>)
     {
-        const uint32_t q = LoadU32Unaligned(p);
+        const uint32_t q = LoadU32Window(base, off);
         out[0]           = (uint8_t)q;
         out[1]           = (uint8_t)(q >> 8);
         out[2]           = (uint8_t)(q >> 16);
     }
     else
     {
-        const Vec<T, C> v = *reinterpret_cast<const Vec<T, C> *>(p);
+        const Vec<T, C> v = *reinterpret_cast<const Vec<T, C> *>(base + off);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -318,7 +318,7 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
     {
         const int x = (int)floorf(sx + .5f), y = (int)floorf(sy + .5f);
-        LoadPixelInside<T, C>(im.base + PixelOffset<PB>(im, x, y), out);
+        LoadPixelInside<T, C>(im.base, PixelOffset<PB>(im, x, y), out);
         return;
     }
     else if constexpr (INTERP == NVCV_INTERP_LINEAR)
