@@ -5,12 +5,14 @@
  *   - one object is shared by all threads through its reference count;
  *   - threads hand each other tensors through shared slots, each with a reference of its own, so that the last
  *     reference is dropped by whichever thread comes last;
+ *   - every thread sets and reads back its own status message between calls that fail;
  *   - afterwards every wrapped tensor has run its cleanup exactly once, nothing is alive (the pools accept a fixed
  *     size) and a destroyed handle is refused through 15 reuses of its slot.
  * Usage: handle_pool_stress [threads [rounds]]; prints failures, exits with their count. */
 #include <nvcv/alloc/Allocator.h>
 #include <nvcv/Config.h>
 #include <nvcv/Image.h>
+#include <nvcv/Status.h>
 #include <nvcv/Tensor.h>
 #include <pthread.h>
 #include <stdatomic.h>
@@ -132,6 +134,18 @@ static void *Worker(void *arg)
         CHECK(nvcvImageGetSize(img, &w, &h) == NVCV_SUCCESS && w == id_.buffer.strided.planes[0].width && h == 4);
         /* a tensor handle is not an image handle, whichever thread made it */
         CHECK(nvcvImageGetSize((NVCVImageHandle)t, &w, &h) == NVCV_ERROR_INVALID_ARGUMENT);
+        /* the status of the last call belongs to the calling thread (reference: tests/nvcv_types/system/
+         * TestStatus.cpp, the thread-local status) */
+        if (r % 16 == 0)
+        {
+            char want[NVCV_MAX_STATUS_MESSAGE_LENGTH], got[NVCV_MAX_STATUS_MESSAGE_LENGTH];
+            snprintf(want, sizeof(want), "thread %d round %d", id, r);
+            nvcvSetThreadStatus(NVCV_ERROR_INTERNAL, "thread %d round %d", id, r);
+            CHECK(nvcvPeekAtLastErrorMessage(got, (int32_t)sizeof(got)) == NVCV_ERROR_INTERNAL && strcmp(got, want) == 0);
+            CHECK(nvcvImageGetSize((NVCVImageHandle)t, &w, &h) == NVCV_ERROR_INVALID_ARGUMENT);
+            CHECK(nvcvGetLastError() == NVCV_ERROR_INVALID_ARGUMENT); /* the failed call's, and that resets it */
+            CHECK(nvcvGetLastError() == NVCV_SUCCESS);
+        }
         CHECK(nvcvImageDecRef(img, &refs) == NVCV_SUCCESS && refs == 0);
         /* a tensor with memory of its own from the shared allocator, which it holds a reference to */
         if (r % 4 == 0)
