@@ -619,6 +619,51 @@ class EmptyLaunch:
         return 0
 
 
+class StreamMix:
+    """Not an operator: a kernel that only moves bytes (libcvamd_bench.so), dense 16-byte loads and streaming
+    stores in the read : write ratio of one of the configurations and with its byte counts, i.e. what the memory
+    system gives that mix. stream-mix-1-2 has the bytes of nv12-to-rgb, stream-mix-24-1 those of resize-cubic-4k,
+    stream-mix-1-1 is a plain copy of the same size as the first."""
+    config_id, dtype = 0, "none"
+    SPECS = {"stream-mix-1-1": (1, 1, 149299200 // 16), "stream-mix-1-2": (1, 2, 99532800 // 16),
+             "stream-mix-24-1": (24, 1, 58982400 // 16)}
+    images = 0
+
+    def __init__(self, cv, orc, np, torch, key):
+        import ctypes as C
+        self.key, self.cv, self.torch = key, cv, torch
+        self.reads, self.writes, self.lanes = self.SPECS[key]
+        self.kernel = "StreamMix<%d,%d>" % (self.reads, self.writes)
+        self.workload = "plain byte mover: %d x 16 bytes read, %d x 16 written per lane, %d lanes" % (
+            self.reads, self.writes, self.lanes)
+        self.alg_bytes = 16 * self.lanes * (self.reads + self.writes)
+        self.other_bytes = {"whole_tensors": self.alg_bytes, "referenced_pixels_only": self.alg_bytes}
+        lib = C.CDLL(os.path.join(os.path.dirname(os.path.abspath(cv.__file__)), "lib", "libcvamd_bench.so"))
+        self.fn = lib.cvamdBenchStreamMix
+        self.fn.restype = C.c_int
+        self.fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int32]
+
+    def make_set(self):
+        src = self.torch.randint(0, 255, (16 * self.lanes * self.reads,), dtype=self.torch.uint8, device="cuda")
+        return src, self.torch.empty(16 * self.lanes * self.writes, dtype=self.torch.uint8, device="cuda")
+
+    def submit(self, stream, s):
+        assert self.fn(self.cv.stream_ptr(stream), s[0].data_ptr(), s[1].data_ptr(), self.lanes, self.reads, self.writes) == 0
+
+    def check(self, s):
+        # chunk 0 of the output is the XOR of every input chunk of the lane
+        n = min(self.lanes, 4096)
+        src = s[0].view(self.reads, self.lanes, 16)[:, :n].cpu().numpy()
+        want = src[0].copy()
+        for k in range(1, self.reads):
+            want ^= src[k]
+        got = s[1].view(self.writes, self.lanes, 16)[0, :n].cpu().numpy()
+        assert (got == want).all()
+
+    def cpu(self, threads):
+        return 0
+
+
 class Streaming:
     """Operators either side of the five configurations, each on a 1080p batch: algorithmic bytes are
     the input plus the output, the check is the oracle (or the numpy index map) on the first image."""
@@ -772,6 +817,7 @@ WORKLOADS = {
     "resize-cubic-4k": CubicC5,
 }
 WORKLOADS.update({k: (lambda *a, k=k: Streaming(*a, k)) for k in Streaming.SPECS})
+WORKLOADS.update({k: (lambda *a, k=k: StreamMix(*a, k)) for k in StreamMix.SPECS})
 
 
 def main():
