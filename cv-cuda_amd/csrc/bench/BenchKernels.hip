@@ -105,7 +105,7 @@ extern "C" __attribute__((visibility("default"))) int cvamdBenchEmptyLaunch(hipS
 }
 
 // Reads `reads` x 16 bytes and writes `writes` x 16 bytes per lane, for `lanes` lanes: src holds at least
-// reads * lanes * 16 bytes, dst writes * lanes * 16, both 16-byte aligned. Ratios built: 1:1, 1:2, 2:1, 24:1.
+// reads * lanes * 16 bytes, dst writes * lanes * 16, both 16-byte aligned. Ratios built: 1:1, 1:2, 4:2, 24:1.
 extern "C" __attribute__((visibility("default"))) int cvamdBenchStreamMix(hipStream_t stream, const void *src, void *dst,
                                                                           int64_t lanes, int32_t reads, int32_t writes)
 {
@@ -121,9 +121,9 @@ extern "C" __attribute__((visibility("default"))) int cvamdBenchStreamMix(hipStr
     {
         return LaunchStreamMix<1, 2>(stream, src, dst, lanes);
     }
-    if (reads == 2 && writes == 1)
+    if (reads == 4 && writes == 2)
     {
-        return LaunchStreamMix<2, 1>(stream, src, dst, lanes);
+        return LaunchStreamMix<4, 2>(stream, src, dst, lanes);
     }
     if (reads == 24 && writes == 1)
     {
