@@ -340,7 +340,9 @@ ParamView MakeParam(NVCVTensorHandle h, const char *what, int N, int H, int W, i
     }
     if (varshape)
     {
-        if (v.N != 1 || v.H != 1 || v.W != 1 || (v.C != 1 && v.C != C))
+        // one value, or one per channel: of a longer vector the first C are used, as the reference reads it
+        // (legacy/normalize_var_shape.cu:107-140 takes the tensor's first element as a C-vector)
+        if (v.N != 1 || v.H != 1 || v.W != 1 || (v.C != 1 && v.C < C))
         {
             throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "%s tensor must have shape [1,1,1,1] or [1,1,1,%d]", what, C);
         }

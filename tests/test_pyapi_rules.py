@@ -1,0 +1,62 @@
+"""Host-side rules of cvcuda_amd.pyapi that need no GPU: the enumerations (names that share a value resolve to the
+first name of the reference's headers, as its table of output formats does, python/mod_cvcuda/CvtColorUtil.cpp:30-42),
+the output shapes and formats of cvtcolor (CvtColorUtil.cpp:244-330) and the argument checks the reference's bindings
+make themselves."""
+import importlib
+
+import numpy as np
+import pytest
+
+
+@pytest.fixture(scope="module")
+def api(cv):
+    return importlib.import_module("cvcuda_amd.pyapi")
+
+
+def test_enumerations(api, K):
+    assert api.Interp.LINEAR == K.INTERP_LINEAR and api.Interp.WARP_INVERSE_MAP == K.WARP_INVERSE_MAP == 16
+    assert api.Border.REFLECT101 == K.BORDER_REFLECT101 and api.ChannelManip.REVERSE == K.CHANNEL_REVERSE
+    assert api.NormalizeFlags.SCALE_IS_STDDEV == 1
+    assert api.Format.RGB8 == K.IMAGE_FORMAT_RGB8 and api.Type.F32 == K.DATA_TYPE_F32
+    cc = api.ColorConversion
+    assert cc.BGR2RGB == K.COLOR_BGR2RGB and cc.YUV2RGB_NV12 == K.COLOR_YUV2RGB_NV12
+    assert all("SPEC" not in n and "XFER" not in n for n in cc.__members__)
+    # one value, two names: the header's first name is the canonical one
+    assert cc.RGB2RGBA is cc.BGR2BGRA and cc(0).name == "BGR2BGRA"
+    assert cc.BGRA2RGB is cc.RGBA2BGR and cc(3).name == "RGBA2BGR"
+
+
+@pytest.mark.parametrize("code,shape,want", [
+    ("BGR2GRAY", (2, 8, 6, 3), (2, 8, 6, 1)), ("GRAY2BGR", (8, 6, 1), (8, 6, 3)), ("RGB2RGBA", (8, 6, 3), (8, 6, 4)),
+    ("BGRA2RGB", (2, 8, 6, 4), (2, 8, 6, 3)), ("BGR2HSV", (4, 4, 3), (4, 4, 3)), ("BGR2YUV", (8, 6, 3), (8, 6, 3)),
+    ("YUV2RGB_NV12", (2, 12, 6, 1), (2, 8, 6, 3)), ("YUV2BGRA_NV21", (60, 62, 1), (40, 62, 4)),
+    ("BGR2YUV_NV21", (2, 40, 62, 3), (2, 60, 62, 1)), ("RGB2YUV_NV12", (8, 6, 3), (12, 6, 1)),
+    ("YUV2BGR_YUY2", (4, 12, 1), (4, 6, 3)), ("YUV2BGR_YUY2", (4, 6, 2), (4, 6, 3)), ("YUV2GRAY_UYVY", (4, 12, 1), (4, 6, 1)),
+])
+def test_cvtcolor_output_shapes(api, code, shape, want):
+    assert api._cvtcolor_shape(shape, api.ColorConversion[code]) == want
+
+
+def test_cvtcolor_shape_and_format_errors(api):
+    with pytest.raises(RuntimeError):
+        api._cvtcolor_shape((8, 6), api.ColorConversion.BGR2RGB)
+    F, cc = api.Format, api.ColorConversion
+    assert api._cvtcolor_format(F.RGB8, cc.RGB2GRAY) == F.Y8_ER and api._cvtcolor_format(F.Y8, cc.GRAY2BGR) == F.BGR8
+    assert api._cvtcolor_format(F.HSV8, cc.HSV2RGB) == F.RGB8 and api._cvtcolor_format(F.BGRA8, cc.BGRA2RGB) == F.BGR8
+    assert api._cvtcolor_format(F.RGB8, cc.RGB2YUV_NV12) == F.Y8 and api._cvtcolor_format(F.BGRf32, cc.RGB2BGR) == F.RGBf32  # = BGR2RGB
+
+
+def test_small_helpers(api):
+    r = api.RectI(x=1, y=2, width=3, height=4)
+    assert tuple(r) == (1, 2, 3, 4) and tuple(api.RectI(5, 6, 7, 8)) == (5, 6, 7, 8)
+    assert api._border_value([]) == (0.0, 0.0, 0.0, 0.0) and api._border_value(3) == (3.0, 0.0, 0.0, 0.0)
+    assert api._border_value([1, 2, 3, 4]) == (1.0, 2.0, 3.0, 4.0)
+    with pytest.raises(RuntimeError):
+        api._border_value([1, 2, 3, 4, 5])
+    assert api._matrix([[1, 0, 2], [0, 1, 3]], 2) == [1.0, 0.0, 2.0, 0.0, 1.0, 3.0]
+    with pytest.raises(RuntimeError):
+        api._matrix([[1, 0, 2]], 2)
+    assert api._image_axes("NHWC") == (2, 1) and api._image_axes("CHW") == (2, 1) and api._image_axes("NWC") == (1, None)
+    with pytest.raises(ValueError):
+        api._image_axes("NC")
+    assert api._np_dtype(api.Type.F32) == np.float32 and api._np_dtype(np.uint8) == np.uint8
