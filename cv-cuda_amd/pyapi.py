@@ -9,7 +9,9 @@ against the reference's `cvcuda` / `nvcv` modules for these operators runs with
     nvcv = cvcuda
 
 Every function forwards to the C ABI through the operator classes of the package; `stream=None` means the current
-stream (`Stream.current`, or torch's current stream when none was entered). Errors of the C ABI are raised as the
+stream (`Stream.current`: the innermost `with stream:`, else the default stream). Containers keep the bindings'
+ordering across streams: a call on one stream waits for the work of other streams that wrote what it reads or
+still uses what it writes. Errors of the C ABI are raised as the
 package's `Error`; argument errors the reference's bindings raise themselves (`RuntimeError`, `ValueError`) are
 raised as the same types here.
 """
@@ -91,14 +93,26 @@ class RectI:
 # ---- streams -----------------------------------------------------------------------------------------------------
 class _StreamMeta(type):
     @property
+    def default(cls):
+        if cls._default is None:
+            cls._default = cls(torch.cuda.default_stream())
+        return cls._default
+
+    @property
     def current(cls):
+        """The innermost `with stream:` of the calling thread; otherwise the default stream (or torch's current
+        stream, when the caller has entered one of torch's stream contexts)."""
         stack = getattr(cls._tls, "stack", None)
-        return stack[-1] if stack else cls(torch.cuda.current_stream())
+        if stack:
+            return stack[-1]
+        now = torch.cuda.current_stream()
+        return cls.default if now == torch.cuda.default_stream() else cls(now)
 
 
 class Stream(metaclass=_StreamMeta):
     """A HIP stream (python/mod_nvcv/Stream.cpp): `with stream:` makes it the current one of the calling thread."""
     _tls = threading.local()
+    _default = None
 
     def __init__(self, wrapped=None):
         self._s = wrapped if wrapped is not None else torch.cuda.Stream()
@@ -330,6 +344,32 @@ def _op(cls, *args):
         return _ops[key]
 
 
+def _submit(stream, reads, writes, op, *args):
+    """Runs op(stream, *args) with the ordering the reference's bindings give their containers (its ResourceGuard,
+    python/mod_nvcv/ResourceGuard.hpp): work on one stream that reads what another stream wrote, or writes what
+    another stream still reads or writes, waits for that work first. Each container remembers the event of its last
+    write and of the reads since, per stream."""
+    s = _torch_stream(stream)
+    key = s.cuda_stream
+    for obj in reads + writes:
+        wrote = getattr(obj, "_wrote", None)
+        if wrote is not None and wrote[0] != key:
+            s.wait_event(wrote[1])
+    for obj in writes:
+        for other, event in getattr(obj, "_read", {}).items():
+            if other != key:
+                s.wait_event(event)
+    op(s, *args)
+    event = torch.cuda.Event()
+    event.record(s)
+    for obj in reads:
+        if not hasattr(obj, "_read"):
+            obj._read = {}
+        obj._read[key] = event
+    for obj in writes:
+        obj._wrote, obj._read = (key, event), {}
+
+
 def _same_images(src, fmt=None, sizes=None):
     """A new batch with one image per image of `src`: same sizes and formats unless given."""
     out = ImageBatchVarShape(src.capacity)
@@ -346,7 +386,7 @@ def _image_axes(layout):
 
 
 def resize_into(dst, src, interp=Interp.LINEAR, *, stream=None):
-    _op(Resize)(_torch_stream(stream), src, dst, int(interp))
+    _submit(stream, [src], [dst], _op(Resize), src, dst, int(interp))
     return dst
 
 
@@ -416,7 +456,7 @@ def _cvtcolor_format(fmt, code):
 
 
 def cvtcolor_into(dst, src, code, *, stream=None):
-    _op(CvtColor)(_torch_stream(stream), src, dst, int(code))
+    _submit(stream, [src], [dst], _op(CvtColor), src, dst, int(code))
     return dst
 
 
@@ -431,8 +471,8 @@ def cvtcolor(src, code, *, stream=None):
 
 
 def normalize_into(dst, src, base, scale, flags=None, *, globalscale=1.0, globalshift=0.0, epsilon=0.0, stream=None):
-    _op(Normalize)(_torch_stream(stream), src, base, scale, dst, float(globalscale), float(globalshift), float(epsilon),
-                   int(flags or 0))
+    _submit(stream, [src, base, scale], [dst], _op(Normalize), src, base, scale, dst, float(globalscale),
+            float(globalshift), float(epsilon), int(flags or 0))
     return dst
 
 
@@ -443,7 +483,7 @@ def normalize(src, base, scale, flags=None, *, globalscale=1.0, globalshift=0.0,
 
 
 def reformat_into(dst, src, *, stream=None):
-    _op(Reformat)(_torch_stream(stream), src, dst)
+    _submit(stream, [src], [dst], _op(Reformat), src, dst)
     return dst
 
 
@@ -457,7 +497,7 @@ def reformat(src, layout, *, stream=None):
 
 
 def convertto_into(dst, src, scale=1, offset=0, *, stream=None):
-    _op(ConvertTo)(_torch_stream(stream), src, dst, float(scale), float(offset))
+    _submit(stream, [src], [dst], _op(ConvertTo), src, dst, float(scale), float(offset))
     return dst
 
 
@@ -466,7 +506,7 @@ def convertto(src, dtype, scale=1, offset=0, *, stream=None):
 
 
 def customcrop_into(dst, src, rect, *, stream=None):
-    _op(CustomCrop)(_torch_stream(stream), src, dst, tuple(rect))
+    _submit(stream, [src], [dst], _op(CustomCrop), src, dst, tuple(rect))
     return dst
 
 
@@ -483,7 +523,7 @@ def customcrop(src, rect, *, stream=None):
 
 
 def center_crop_into(dst, src, crop_size, *, stream=None):
-    _op(CenterCrop)(_torch_stream(stream), src, dst, (int(crop_size[0]), int(crop_size[1])))
+    _submit(stream, [src], [dst], _op(CenterCrop), src, dst, (int(crop_size[0]), int(crop_size[1])))
     return dst
 
 
@@ -499,9 +539,9 @@ def center_crop(src, crop_size, *, stream=None):
 def flip_into(dst, src, flipCode, *, stream=None):
     """flipCode: an int for tensors; for image batches a tensor with one int32 code per image."""
     if isinstance(src, _ImageBatchVarShape):
-        _op(Flip, src.capacity)(_torch_stream(stream), src, dst, flipCode)
+        _submit(stream, [src, flipCode], [dst], _op(Flip, src.capacity), src, dst, flipCode)
     else:
-        _op(Flip, 0)(_torch_stream(stream), src, dst, int(flipCode))
+        _submit(stream, [src], [dst], _op(Flip, 0), src, dst, int(flipCode))
     return dst
 
 
@@ -529,9 +569,9 @@ def _matrix(xform, rows):
 def _warp_into(cls, rows, dst, src, xform, flags, border_mode, border_value, stream):
     bv = _border_value(border_value)
     if isinstance(src, _ImageBatchVarShape):
-        _op(cls, src.capacity)(_torch_stream(stream), src, dst, xform, int(flags), int(border_mode), bv)
+        _submit(stream, [src, xform], [dst], _op(cls, src.capacity), src, dst, xform, int(flags), int(border_mode), bv)
     else:
-        _op(cls, 0)(_torch_stream(stream), src, dst, _matrix(xform, rows), int(flags), int(border_mode), bv)
+        _submit(stream, [src], [dst], _op(cls, 0), src, dst, _matrix(xform, rows), int(flags), int(border_mode), bv)
     return dst
 
 
@@ -558,9 +598,8 @@ def warp_perspective(src, xform, flags, *, border_mode, border_value, stream=Non
 
 def resize_crop_convert_reformat_into(dst, src, resize_dim, interp, cropPos, *, manip=ChannelManip.NO_OP, scale=1.0,
                                       offset=0.0, srcCast=True, stream=None):
-    _op(ResizeCropConvertReformat)(_torch_stream(stream), src, dst, (int(resize_dim[0]), int(resize_dim[1])),
-                                   int(interp), (int(cropPos[0]), int(cropPos[1])), int(manip), float(scale),
-                                   float(offset), bool(srcCast))
+    _submit(stream, [src], [dst], _op(ResizeCropConvertReformat), src, dst, (int(resize_dim[0]), int(resize_dim[1])),
+            int(interp), (int(cropPos[0]), int(cropPos[1])), int(manip), float(scale), float(offset), bool(srcCast))
     return dst
 
 
@@ -596,8 +635,9 @@ def resize_crop_convert_reformat(src, resize_dim, interp, crop_rect, *, layout="
 
 def crop_flip_normalize_reformat_into(dst, src, rect, flip_code, base, scale, globalscale=1.0, globalshift=0.0,
                                       epsilon=0.0, flags=None, border=Border.CONSTANT, bvalue=0, *, stream=None):
-    _op(CropFlipNormalizeReformat)(_torch_stream(stream), src, dst, rect, int(border), float(bvalue), flip_code, base,
-                                   scale, float(globalscale), float(globalshift), float(epsilon), int(flags or 0))
+    _submit(stream, [src, rect, flip_code, base, scale], [dst], _op(CropFlipNormalizeReformat), src, dst, rect,
+            int(border), float(bvalue), flip_code, base, scale, float(globalscale), float(globalshift), float(epsilon),
+            int(flags or 0))
     return dst
 
 

@@ -587,3 +587,89 @@ def test_op_crop_flip_normalize_reformat(cvcuda, format, num_images, min_size, m
     assert tmp is out_tensor
     stream.sync()
     np.testing.assert_array_equal(host(out_tensor), host(out))
+
+
+# ---- streams (test_multi_stream.py:21-163) ---------------------------------------------------------------------------
+def test_multiple_streams_and_contexts(cvcuda):
+    Stream = cvcuda.cuda.Stream
+    stream1, stream2, stream3 = Stream(), Stream(), Stream()
+    assert stream1 is not stream2 and stream1 is not stream3
+    assert Stream.current is Stream.default
+    assert Stream.current is not stream1 and Stream.current is not stream2 and Stream.current is not stream3
+    with stream1:
+        assert Stream.current is stream1
+        with stream2:
+            assert Stream.current is stream2
+        assert Stream.current is stream1
+    assert Stream.current is Stream.default
+    with pytest.raises(Exception):
+        with stream1:
+            with stream2:
+                assert Stream.current is stream2
+                raise Exception()
+    assert Stream.current is Stream.default
+    with stream2:
+        assert Stream.current is stream2
+    assert Stream.current is Stream.default
+
+
+def test_operator_stream(cvcuda):
+    import torch
+    Stream = cvcuda.cuda.Stream
+    for stream in (Stream(), Stream(), Stream()):
+        with stream:
+            assert Stream.current is stream
+            img = cvcuda.as_tensor(torch.zeros(10, 10, 3, dtype=torch.uint8, device="cuda"), "HWC")
+            gray = cvcuda.cvtcolor(img, cvcuda.ColorConversion.BGR2GRAY)
+            assert gray.shape == (10, 10, 1)
+            assert Stream.current is stream
+    assert Stream.current is Stream.default
+
+
+def test_operator_changing_stream(cvcuda):
+    # the same two tensors handed from stream to stream: each call must see what the call before it wrote
+    import torch
+    N, H, W, C, loop = 10, 1080, 1080, 3, 50
+    streams = [cvcuda.cuda.Stream() for _ in range(4)]
+    input_tensor = torch.randint(0, 256, (N, H, W, C), dtype=torch.uint8).cuda()
+    output_tensor = torch.randint(0, 256, (N, H, W, C), dtype=torch.uint8).cuda()
+    copy = input_tensor.clone()
+    torch.cuda.synchronize()
+    tin, tout = cvcuda.as_tensor(input_tensor.data, "NHWC"), cvcuda.as_tensor(output_tensor.data, "NHWC")
+    for _ in range(loop):
+        for stream in streams:
+            cvcuda.flip_into(tout, tin, -1, stream=stream)
+            cvcuda.flip_into(tin, tout, -1, stream=stream)
+    for stream in streams:
+        stream.sync()
+    assert torch.equal(torch.as_tensor(tin.cuda(), device="cuda").cpu(), copy.cpu())
+
+
+def test_operator_changing_stream_loaded(cvcuda):
+    # one stream is kept busy; the other takes over the tensors it is still writing
+    import torch
+    N, H, W, C, loop = 10, 1080, 1080, 3, 6
+    stream1, stream2 = cvcuda.cuda.Stream(), cvcuda.cuda.Stream()
+    input_tensor = torch.randint(0, 256, (N, H, W, C), dtype=torch.uint8).cuda()
+    tmp_tensor = torch.randint(0, 256, (N, H, W, C), dtype=torch.uint8).cuda()
+    output_tensor = torch.randint(0, 256, (N, H, W, C), dtype=torch.uint8).cuda()
+    copy = input_tensor.clone()
+    torch.cuda.synchronize()
+    tin, ttmp, tout = (cvcuda.as_tensor(t.data, "NHWC") for t in (input_tensor, tmp_tensor, output_tensor))
+    scratch = cvcuda.Tensor((N, H, W, C), np.uint8, "NHWC")
+    for _ in range(loop):
+        for _ in range(loop * 2):
+            cvcuda.flip_into(scratch, ttmp, 0, stream=stream1)
+        cvcuda.flip_into(ttmp, tin, -1, stream=stream1)    # ttmp = both axes flipped, behind the busy work
+        cvcuda.flip_into(tout, ttmp, -1, stream=stream2)   # reads what stream1 is still writing: tout = tin
+        cvcuda.flip_into(tin, tout, 1, stream=stream2)     # tin = columns flipped (stream1 has read tin before)
+        cvcuda.flip_into(tout, tin, 1, stream=stream1)     # tout = the original
+        cvcuda.flip_into(tin, tout, 0, stream=stream1)     # tin = rows flipped
+        cvcuda.flip_into(tout, tin, 0, stream=stream2)     # tout = the original
+        cvcuda.flip_into(tin, tout, -1, stream=stream2)    # tin = both flipped
+        cvcuda.flip_into(tout, tin, -1, stream=stream1)    # tout = the original
+        cvcuda.flip_into(ttmp, tout, 0, stream=stream1)    # ttmp = rows flipped
+        cvcuda.flip_into(tin, ttmp, 0, stream=stream2)     # tin = the original again
+    stream1.sync()
+    stream2.sync()
+    assert torch.equal(torch.as_tensor(tin.cuda(), device="cuda").cpu(), copy.cpu())
