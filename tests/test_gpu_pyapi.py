@@ -673,3 +673,33 @@ def test_operator_changing_stream_loaded(cvcuda):
     stream1.sync()
     stream2.sync()
     assert torch.equal(torch.as_tensor(tin.cuda(), device="cuda").cpu(), copy.cpu())
+
+
+def test_parallel_callers_share_an_input(cvcuda):
+    # after test_multi_threading.py:99-124 (there with an operator outside this path): several threads run an operator
+    # on one shared input, each on a stream of its own; every output equals the lone caller's
+    import threading
+    input, _ = fill(cvcuda, (3, 224, 224, 4), np.uint8, "NHWC", high=256)
+    want = host(cvcuda.resize(input, (3, 100, 120, 4), cvcuda.Interp.LINEAR))
+    outputs, errors = [], []
+
+    def work():
+        try:
+            stream = cvcuda.Stream()
+            for _ in range(20):
+                out = cvcuda.resize(input, (3, 100, 120, 4), cvcuda.Interp.LINEAR, stream=stream)
+            stream.sync()
+            outputs.append(out)
+        except Exception as exc:  # noqa: BLE001 - reported below
+            errors.append(repr(exc))
+
+    threads = [threading.Thread(target=work) for _ in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert len(outputs) == 8
+    for out in outputs:
+        assert out.layout == input.layout and out.dtype == input.dtype
+        np.testing.assert_array_equal(host(out), want)
