@@ -703,3 +703,32 @@ def test_parallel_callers_share_an_input(cvcuda):
     for out in outputs:
         assert out.layout == input.layout and out.dtype == input.dtype
         np.testing.assert_array_equal(host(out), want)
+
+
+def test_classification_sample_preprocessing(cvcuda, orc):
+    # the chain of the reference's classification sample (samples/classification/python/pipelines.py:28-33, 67-90):
+    # resize -> convertto(1/255) -> normalize(mean, stddev) -> reformat(NCHW), and the fused operator beside it
+    import torch
+    frames = torch.randint(0, 256, (4, 360, 640, 3), dtype=torch.uint8).cuda()
+    mean_np = np.array([0.485, 0.456, 0.406], np.float32)
+    std_np = np.array([0.229, 0.224, 0.225], np.float32)
+    mean = cvcuda.as_tensor(torch.from_numpy(mean_np).reshape(1, 1, 1, 3).cuda(), "NHWC")
+    stddev = cvcuda.as_tensor(torch.from_numpy(std_np).reshape(1, 1, 1, 3).cuda(), "NHWC")
+    out_size = (224, 224)
+    frame_nhwc = cvcuda.as_tensor(frames, "NHWC")
+    resized = cvcuda.resize(frame_nhwc, (frame_nhwc.shape[0], out_size[1], out_size[0], frame_nhwc.shape[3]),
+                            cvcuda.Interp.LINEAR)
+    normalized = cvcuda.convertto(resized, np.float32, scale=1 / 255)
+    normalized = cvcuda.normalize(normalized, base=mean, scale=stddev, flags=cvcuda.NormalizeFlags.SCALE_IS_STDDEV)
+    normalized = cvcuda.reformat(normalized, "NCHW")
+    assert normalized.shape == (4, 3, 224, 224) and normalized.dtype == np.float32 and normalized.layout == "NCHW"
+    small = host(resized)
+    want_small = orc.resize(frames.cpu().numpy(), (224, 224), 1, variant=1)
+    assert np.abs(small.astype(np.int32) - want_small.astype(np.int32)).max() <= 1
+    unit = small.astype(np.float32) * np.float32(1 / 255)
+    want = ((unit - mean_np) * (np.float32(1) / np.sqrt(std_np * std_np))).transpose(0, 3, 1, 2)
+    np.testing.assert_allclose(host(normalized), want, rtol=2e-6, atol=2e-6)
+    # one call instead of the first two and the last: within one 8-bit step of the chain's unit-range image
+    fused = cvcuda.resize_crop_convert_reformat(frame_nhwc, out_size, cvcuda.Interp.LINEAR, cvcuda.RectI(0, 0, 224, 224),
+                                                layout="NCHW", data_type=cvcuda.Type.F32, scale=1 / 255)
+    assert np.abs(host(fused) - unit.transpose(0, 3, 1, 2)).max() <= 1 / 255 + 1e-6
