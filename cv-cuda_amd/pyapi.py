@@ -30,7 +30,7 @@ from . import ImageBatchVarShape as _ImageBatchVarShape
 from . import Tensor as _Tensor
 from . import _DT2NP
 
-__all__ = ["Error", "Interp", "Border", "ChannelManip", "NormalizeFlags", "ColorConversion", "Format", "Type", "RectI",
+__all__ = ["Error", "Interp", "Border", "ChannelManip", "NormalizeFlags", "ColorConversion", "Format", "Type", "TensorLayout", "RectI",
            "Stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image"]
 
 
@@ -75,6 +75,13 @@ ColorConversion = enum.IntEnum("ColorConversion", {k: int(v) for k, v in _enum_o
                                                    if re.match(r"^[A-Za-z0-9]+?2[A-Z]", k)})  # not COLOR_SPEC_*, COLOR_XFER_* ...
 Format = _enum_of("Format", "IMAGE_FORMAT_")
 Type = _enum_of("Type", "DATA_TYPE_")
+
+
+class TensorLayout:
+    """The layout names the reference offers as nvcv.TensorLayout members (python/mod_nvcv/TensorLayout.cpp); a layout
+    is passed as its string."""
+    NHWC, NCHW, HWC, CHW, NCHW, NC, NW, NWC, HW, N, C, W = ("NHWC", "NCHW", "HWC", "CHW", "NCHW", "NC", "NW", "NWC", "HW",
+                                                            "N", "C", "W")
 
 
 class RectI:

@@ -732,3 +732,41 @@ def test_classification_sample_preprocessing(cvcuda, orc):
     fused = cvcuda.resize_crop_convert_reformat(frame_nhwc, out_size, cvcuda.Interp.LINEAR, cvcuda.RectI(0, 0, 224, 224),
                                                 layout="NCHW", data_type=cvcuda.Type.F32, scale=1 / 255)
     assert np.abs(host(fused) - unit.transpose(0, 3, 1, 2)).max() <= 1 / 255 + 1e-6
+
+
+def test_decoder_and_encoder_edges_of_the_samples(cvcuda, orc, cv):
+    # samples/common/python/nvcodec_utils.py:125-137 (decoded NV12 frames -> RGB batch) and :295-316 (NCHW RGB batch
+    # -> NHWC -> NV12 for the encoder), with the frames a decoder would hand over replaced by a device buffer
+    import importlib.util
+    import os
+    import torch
+    nvcv = cvcuda
+    spec = importlib.util.spec_from_file_location("color_oracle_for_pyapi", os.path.join(
+        os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "color_oracle.py"))
+    col = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(col)
+    n, height, width = 3, 96, 128
+    surfaces = RNG.integers(16, 236, (n, height * 3 // 2, width, 1)).astype(np.uint8)
+
+    class DecodedFrames:  # what a decoder exposes: device memory through the array interface
+        def __init__(self, t):
+            self.t = t
+            self.__cuda_array_interface__ = t.__cuda_array_interface__
+
+    yuv = nvcv.as_tensor(DecodedFrames(torch.from_numpy(surfaces).cuda()), nvcv.TensorLayout.NHWC)
+    rgb_batch = cvcuda.Tensor((n, height, width, 3), nvcv.Type.U8, nvcv.TensorLayout.NHWC)
+    cvcuda.cvtcolor_into(rgb_batch, yuv, cvcuda.ColorConversion.YUV2RGB_NV12)
+    rgb = host(rgb_batch)
+    np.testing.assert_array_equal(rgb, orc.yuv420_to_rgb(surfaces[..., 0], 3, False, 0, True, variant=0))
+
+    # the encoder side: a torch NCHW batch (what the inference side returns) -> NHWC -> NV12
+    nchw = torch.from_numpy(rgb.transpose(0, 3, 1, 2).copy()).cuda()
+    hwc_batch = cvcuda.Tensor((n, height, width, 3), nvcv.Type.U8, nvcv.TensorLayout.NHWC)
+    yuv_batch = cvcuda.Tensor((n, (height // 2) * 3, width, 1), nvcv.Type.U8, nvcv.TensorLayout.NHWC)
+    cvcuda.reformat_into(hwc_batch, cvcuda.as_tensor(nchw, nvcv.TensorLayout.NCHW))
+    cvcuda.cvtcolor_into(yuv_batch, hwc_batch, cvcuda.ColorConversion.RGB2YUV_NV12)
+    tensor = torch.as_tensor(yuv_batch.cuda(), device="cuda")
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(host(hwc_batch), rgb)
+    np.testing.assert_array_equal(tensor.cpu().numpy().reshape(n, -1, width),
+                                  np.asarray(col.yuv420_from_bgr(rgb, False, 0, False)).reshape(n, -1, width))
