@@ -46,6 +46,7 @@ _NP2DT = {
     np.dtype(np.uint16): K.DATA_TYPE_U16, np.dtype(np.int16): K.DATA_TYPE_S16,
     np.dtype(np.int32): K.DATA_TYPE_S32, np.dtype(np.uint32): K.DATA_TYPE_U32, np.dtype(np.float32): K.DATA_TYPE_F32,
     np.dtype(np.float64): K.DATA_TYPE_F64, np.dtype(np.float16): K.DATA_TYPE_F16,
+    np.dtype(np.complex64): K.DATA_TYPE_C64, np.dtype(np.complex128): K.DATA_TYPE_C128,
 }
 _DT2NP = {v: k for k, v in _NP2DT.items()}
 _NP2TORCH = {
@@ -53,6 +54,7 @@ _NP2TORCH = {
     np.dtype(np.int16): torch.int16, np.dtype(np.int32): torch.int32, np.dtype(np.uint32): torch.uint32,
     np.dtype(np.float32): torch.float32,
     np.dtype(np.float64): torch.float64, np.dtype(np.float16): torch.float16,
+    np.dtype(np.complex64): torch.complex64, np.dtype(np.complex128): torch.complex128,
 }
 
 

@@ -15,6 +15,7 @@ still uses what it writes. Errors of the C ABI are raised as the
 package's `Error`; argument errors the reference's bindings raise themselves (`RuntimeError`, `ValueError`) are
 raised as the same types here.
 """
+import ctypes as C
 import enum
 import re
 import threading
@@ -28,10 +29,11 @@ from . import (CenterCrop, ConvertTo, CropFlipNormalizeReformat, CustomCrop, Cvt
 from . import Image as _Image
 from . import ImageBatchVarShape as _ImageBatchVarShape
 from . import Tensor as _Tensor
-from . import _DT2NP
+from . import _DT2NP, check
+from ._capi import nvcv as _nv
 
 __all__ = ["Error", "Interp", "Border", "ChannelManip", "NormalizeFlags", "ColorConversion", "Format", "Type", "TensorLayout", "RectI",
-           "Stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image"]
+           "Stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image", "as_images"]
 
 
 def _enum_of(name, prefix):
@@ -80,8 +82,8 @@ Type = _enum_of("Type", "DATA_TYPE_")
 class TensorLayout:
     """The layout names the reference offers as nvcv.TensorLayout members (python/mod_nvcv/TensorLayout.cpp); a layout
     is passed as its string."""
-    NHWC, NCHW, HWC, CHW, NCHW, NC, NW, NWC, HW, N, C, W = ("NHWC", "NCHW", "HWC", "CHW", "NCHW", "NC", "NW", "NWC", "HW",
-                                                            "N", "C", "W")
+    NHWC, NCHW, HWC, CHW, NC, NW, NWC, HW, WC, CW, N, C, W = ("NHWC", "NCHW", "HWC", "CHW", "NC", "NW", "NWC", "HW", "WC",
+                                                              "CW", "N", "C", "W")
 
 
 class RectI:
@@ -165,13 +167,20 @@ def _np_dtype(dtype):
 
 
 class _Buffer:
-    """What `.cuda()` returns: device memory through `__cuda_array_interface__` (python/mod_nvcv/ExternalBuffer.cpp)."""
+    """What `.cuda()` returns: device memory through `__cuda_array_interface__` and DLPack
+    (python/mod_nvcv/ExternalBuffer.cpp)."""
 
     def __init__(self, iface, owner):
         self.__cuda_array_interface__ = iface
         self._owner = owner
         self.shape = tuple(iface["shape"])
         self.dtype = np.dtype(iface["typestr"])
+
+    def __dlpack__(self, stream=None):
+        return torch.as_tensor(self, device="cuda").__dlpack__()
+
+    def __dlpack_device__(self):
+        return torch.as_tensor(self, device="cuda").__dlpack_device__()
 
 
 class Tensor:
@@ -223,12 +232,19 @@ class Tensor:
 
 
 def as_tensor(obj, layout=None):
-    """Zero-copy tensor over a torch CUDA tensor or anything with `__cuda_array_interface__`."""
-    if isinstance(obj, Image):
-        raise TypeError("as_tensor of an Image is not part of this interface")
+    """Zero-copy tensor over a torch CUDA tensor, anything with `__cuda_array_interface__` or `__dlpack__`, or an
+    image (one image as a tensor of N = 1, nvcvTensorWrapImageConstruct)."""
+    if isinstance(obj, _Image):
+        handle = C.c_void_p()
+        check(_nv.nvcvTensorWrapImageConstruct(obj.handle, C.byref(handle)))
+        wrapped = _Tensor(handle)
+        wrapped._keep.append(obj)
+        return Tensor(_wrap=wrapped)
     if isinstance(obj, torch.Tensor):
         return Tensor(_wrap=_Tensor.from_torch(obj, layout or ""))
-    return Tensor(_wrap=_Tensor.from_cuda_array_interface(obj, layout or ""))
+    if hasattr(obj, "__cuda_array_interface__"):
+        return Tensor(_wrap=_Tensor.from_cuda_array_interface(obj, layout or ""))
+    return Tensor(_wrap=_Tensor.from_torch(torch.from_dlpack(obj), layout or ""))
 
 
 _PLANE_NP = {int(Format.U8): (np.uint8, 1), int(Format.S8): (np.int8, 1), int(Format.U16): (np.uint16, 1),
@@ -311,6 +327,13 @@ def as_image(buffer, format=None):
     strides = iface.get("strides")
     row = strides[0] if strides else w * c * npdt.itemsize
     return Image.wrap(int(format), [(iface["data"][0], w, h, row)], keep=keep)
+
+
+def as_images(buffers, format=None):
+    """An image batch over a list of (H, W[, C]) device buffers, one image each (capacity = their number)."""
+    batch = ImageBatchVarShape(len(buffers))
+    batch.pushback([as_image(b, format) for b in buffers])
+    return batch
 
 
 class ImageBatchVarShape(_ImageBatchVarShape):

@@ -1,0 +1,152 @@
+"""The reference's Python tests of the containers the path's operators take (tests/nvcv_types/python/test_tensor.py:
+21-260, test_imgbatchvarshape.py:53-218), restated against cvcuda_amd.pyapi."""
+import importlib
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nvcv(cv, gpu):
+    return importlib.import_module("cvcuda_amd.pyapi")
+
+
+@pytest.mark.parametrize("n,size,fmt,gold_layout,gold_shape,gold_dtype", [
+    (5, (32, 16), "RGBA8", "NHWC", (5, 16, 32, 4), np.uint8), (2, (38, 7), "RGB8p", "NCHW", (2, 3, 7, 38), np.uint8),
+])
+def test_tensor_creation_imagebatch_works(nvcv, n, size, fmt, gold_layout, gold_shape, gold_dtype):
+    for tensor in (nvcv.Tensor(n, size, nvcv.Format[fmt]), nvcv.Tensor(nimages=n, imgsize=size, format=nvcv.Format[fmt])):
+        assert tensor.shape == gold_shape and tensor.layout == gold_layout
+        assert tensor.dtype == gold_dtype and tensor.ndim == len(gold_shape)
+
+
+@pytest.mark.parametrize("shape,dtype,layout", [
+    ((5, 16, 32, 4), np.float32, "NHWC"), ((7, 3, 33, 11), np.complex64, "NCHW"), ((3, 11), np.int16, None),
+    ((16, 32, 4), np.float32, "HWC"), ((32, 4), np.float32, "WC"), ((4, 32), np.float32, "CW"), ((32,), np.float32, "W"),
+])
+def test_tensor_creation_shape_works(nvcv, shape, dtype, layout):
+    layout = None if layout is None else getattr(nvcv.TensorLayout, layout)
+    for tensor in (nvcv.Tensor(shape, dtype, layout), nvcv.Tensor(layout=layout, shape=shape, dtype=dtype)):
+        assert tensor.shape == shape and tensor.dtype == dtype and tensor.layout == layout and tensor.ndim == len(shape)
+
+
+WRAP = [((3, 5, 7, 1), np.uint8), ((3, 5, 7, 1), np.int8), ((3, 5, 7, 1), np.int16), ((3, 5, 7, 1), np.float32),
+        ((3, 5, 7, 1), np.float64), ((3, 5, 7, 2), np.float32), ((3, 5, 7, 3), np.uint8), ((3, 5, 7, 4), np.uint8),
+        ((3, 5, 7), np.csingle), ((3, 5, 7), np.cdouble), ((3,), np.int8)]
+
+
+@pytest.mark.parametrize("shape,dtype", WRAP)
+@pytest.mark.parametrize("through", ["torch", "dlpack", "cuda_array_interface"])
+def test_wrap_torch_buffer(nvcv, shape, dtype, through):
+    import torch
+    ttensor = torch.as_tensor(np.zeros(shape, dtype=dtype), device="cuda")
+
+    class Only:
+        pass
+    obj = ttensor
+    if through == "dlpack":
+        obj = Only()
+        obj.__dlpack__, obj.__dlpack_device__ = ttensor.__dlpack__, ttensor.__dlpack_device__
+    elif through == "cuda_array_interface":
+        obj = Only()
+        obj.__cuda_array_interface__ = ttensor.__cuda_array_interface__
+    tensor = nvcv.as_tensor(obj)
+    assert tensor.shape == shape and tensor.dtype == dtype and tensor.layout is None and tensor.ndim == len(shape)
+
+
+@pytest.mark.parametrize("shape,dtype,layout", [
+    ((3, 5, 7, 1), np.uint8, "NHWC"), ((3, 5, 7), np.uint8, "HWC"), ((3, 5, 7, 2), np.int16, "NHWC"),
+    ((3, 5, 7, 2, 4, 2, 5), np.int16, "abcdefg"), ((3, 5), np.uint8, "HW"), ((5,), np.uint8, "W"),
+])
+def test_wrap_torch_buffer_with_layout(nvcv, shape, dtype, layout):
+    import torch
+    tensor = nvcv.as_tensor(torch.as_tensor(np.zeros(shape, dtype=dtype), device="cuda"), layout)
+    assert tensor.shape == shape and tensor.dtype == dtype and tensor.layout == layout and tensor.ndim == len(shape)
+
+
+@pytest.mark.parametrize("size,fmt,gold_layout,gold_shape,gold_dtype", [
+    ((32, 16), "RGBA8", "NHWC", (1, 16, 32, 4), np.uint8), ((38, 7), "RGB8p", "NCHW", (1, 3, 7, 38), np.uint8),
+])
+def test_tensor_wrap_image_works(nvcv, size, fmt, gold_layout, gold_shape, gold_dtype):
+    img = nvcv.Image(size, nvcv.Format[fmt])
+    tensor = nvcv.as_tensor(img)
+    assert tensor.shape == gold_shape and tensor.layout == gold_layout and tensor.dtype == gold_dtype
+
+
+@pytest.mark.parametrize("shape,dtype", [((1, 23, 65, 3), np.uint8), ((5, 23, 65, 3), np.int8), ((65, 3), np.int16),
+                                         ((243, 65, 3), np.int16), ((1, 1), np.int16), ((10,), np.uint8)])
+def test_tensor_export_cuda_buffer(nvcv, shape, dtype):
+    import torch
+    gold = np.random.default_rng(1).integers(0, 128, shape, dtype)
+    tensor = nvcv.as_tensor(torch.as_tensor(gold, device="cuda"))
+    mem = tensor.cuda()
+    assert mem.dtype == dtype and mem.shape == shape
+    assert (gold == torch.as_tensor(mem, device="cuda").cpu().numpy()).all()
+    assert (gold == torch.from_dlpack(mem).cpu().numpy()).all()
+
+
+def test_tensor_hold_reference_of_wrapped_buffer(nvcv):
+    import torch
+    ttensor = torch.as_tensor(np.zeros([10], np.int8), device="cuda")
+    ptr0 = ttensor.data_ptr()
+    cvtensor = nvcv.as_tensor(ttensor)  # noqa: F841 - must keep the first buffer alive
+    del ttensor
+    ttensor = torch.as_tensor(np.zeros([10], np.int8), device="cuda")
+    assert ttensor.data_ptr() != ptr0  # the allocator could not hand the first buffer out again
+
+
+def test_imgbatchvarshape_creation_works(nvcv):
+    batch = nvcv.ImageBatchVarShape(15)
+    assert batch.capacity == 15 and len(batch) == 0 and batch.uniqueformat is None and batch.maxsize == (0, 0)
+    assert sum(1 for _ in batch) == 0
+
+
+def test_imgbatchvarshape_one_image(nvcv):
+    batch = nvcv.ImageBatchVarShape(15)
+    img = nvcv.Image((64, 32), nvcv.Format.RGBA8)
+    batch.pushback(img)
+    assert len(batch) == 1 and batch.uniqueformat == nvcv.Format.RGBA8 and batch.maxsize == (64, 32)
+    assert [b is img for b in batch] == [True]
+    batch.popback()
+    assert len(batch) == 0 and sum(1 for _ in batch) == 0
+
+
+def test_imgbatchvarshape_several_images(nvcv):
+    batch = nvcv.ImageBatchVarShape(15)
+    imgs = [nvcv.Image((m * 2, m), nvcv.Format.RGBA8) for m in range(2, 10, 2)]
+    batch.pushback(imgs)
+    assert len(batch) == 4 and batch.maxsize == (16, 8) and batch.uniqueformat == nvcv.Format.RGBA8
+    assert all(b is i for b, i in zip(batch, imgs)) and sum(1 for _ in batch) == 4
+    batch.popback(2)
+    assert len(batch) == 2 and sum(1 for _ in batch) == 2 and batch.maxsize == (8, 4)
+    batch.pushback(nvcv.Image((58, 26), nvcv.Format.NV12))
+    assert batch.maxsize == (58, 26) and batch.uniqueformat is None
+    batch.clear()
+    assert len(batch) == 0 and sum(1 for _ in batch) == 0 and batch.maxsize == (0, 0)
+
+
+@pytest.mark.parametrize("base_shape,dt,fmt", [
+    ([5, 7, 1], np.uint8, "U8"), ([5, 7], np.uint8, "U8"), ([5, 7, 1], np.float32, "F32"), ([5, 7, 3], np.uint8, "RGB8"),
+    ([5, 7, 4], np.uint8, "RGBA8"),
+])
+def test_wrap_buffer_list(nvcv, base_shape, dt, fmt):
+    import torch
+    shapes = [[base_shape[d] + (i if d < 2 else 0) for d in range(len(base_shape))] for i in range(3)]
+    buffers = [torch.as_tensor(np.zeros(shape, dt), device="cuda") for shape in shapes]
+    batch = nvcv.as_images(buffers)
+    assert batch.capacity == 3 and batch.maxsize == (base_shape[1] + 2, base_shape[0] + 2)
+    assert batch.uniqueformat == nvcv.Format[fmt]
+    for image, sh in zip(batch, shapes):
+        assert image.width == sh[1] and image.height == sh[0] and image.format == nvcv.Format[fmt]
+
+
+def test_imgbatchvarshape_wrapper_nodeletion(nvcv):
+    import torch
+    for i in range(2):
+        np_img = np.random.default_rng(i).random((1 + i, 2 + i)).astype(np.float32)
+        pt_img = torch.from_numpy(np_img).cuda()
+        batch = nvcv.as_images([pt_img])
+        del batch
+        assert (pt_img.cpu().numpy() == np_img).all()
