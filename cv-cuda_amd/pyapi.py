@@ -293,17 +293,94 @@ class Image(_Image):
         except ValueError:
             return value
 
-    def cuda(self):
-        """The single plane as an (H, W, C) buffer."""
-        fmt = int(self.format)
-        if fmt not in _PLANE_NP:
-            raise ValueError("cuda() is offered for single-plane formats with equal channels")
-        npdt, ch = _PLANE_NP[fmt]
-        pl = self.export().buffer.strided.planes[0]
-        es = np.dtype(npdt).itemsize
-        iface = {"shape": (pl.height, pl.width, ch), "typestr": np.dtype(npdt).str, "data": (int(pl.basePtr or 0), False),
-                 "strides": (pl.rowStride, ch * es, es), "version": 3}
-        return _Buffer(iface, self)
+    @classmethod
+    def zeros(cls, size, format, rowalign=0):
+        img = cls(size, format, rowalign)
+        for buf in img._plane_buffers():
+            torch.as_tensor(buf, device="cuda").zero_()
+        return img
+
+    def _plane_buffers(self):
+        """One (H, W, C) buffer per plane."""
+        data = self.export().buffer.strided
+        out = []
+        for p, (npdt, ch) in enumerate(_planes(int(_Image.format.fget(self)))):
+            pl, es = data.planes[p], np.dtype(npdt).itemsize
+            iface = {"shape": (pl.height, pl.width, ch), "typestr": np.dtype(npdt).str,
+                     "data": (int(pl.basePtr or 0), False), "strides": (pl.rowStride, ch * es, es), "version": 3}
+            out.append(_Buffer(iface, self))
+        return out
+
+    def cuda(self, layout=None):
+        """The image's device memory (python/mod_nvcv/Image.cpp, ExternalBuffer.cpp): one buffer for a packed image
+        ((H, W) or (H, W, C)) and for a planar image of equal planes ((C, H, W)), a list of (H, W, C) buffers for
+        planes that differ (NV12 ...). `layout` names the dimensions wanted: H, W and C in any order, any other
+        letter a dimension of 1."""
+        bufs = self._plane_buffers()
+        ifaces = [b.__cuda_array_interface__ for b in bufs]
+        same = all(i["shape"] == ifaces[0]["shape"] and i["typestr"] == ifaces[0]["typestr"] for i in ifaces)
+        if len(bufs) > 1 and not (same and ifaces[0]["shape"][2] == 1):
+            return bufs if layout in (None, "HWC") else [_relayout(b, layout) for b in bufs]
+        first = ifaces[0]
+        h, w, c = first["shape"]
+        if len(bufs) > 1:  # equal one-channel planes: C x H x W with the distance of the planes as the C stride
+            step = ifaces[1]["data"][0] - first["data"][0]
+            merged = dict(first, shape=(len(bufs), h, w), strides=(step, first["strides"][0], first["strides"][2]))
+            planar = _Buffer(merged, self)
+            return planar if layout in (None, "CHW") else _relayout(planar, layout, have="CHW")
+        if layout is None:
+            if c == 1:
+                return _Buffer(dict(first, shape=(h, w), strides=(first["strides"][0], first["strides"][2])), self)
+            return bufs[0]
+        return _relayout(bufs[0], layout)
+
+    def cpu(self, layout=None):
+        got = self.cuda(layout)
+        torch.cuda.synchronize()
+        if isinstance(got, list):
+            return [torch.as_tensor(g, device="cuda").cpu().numpy() for g in got]
+        return torch.as_tensor(got, device="cuda").cpu().numpy()
+
+
+_nv.nvcvImageFormatGetNumPlanes.argtypes = [C.c_uint64, C.POINTER(C.c_int32)]
+_nv.nvcvImageFormatGetPlaneNumChannels.argtypes = [C.c_uint64, C.c_int32, C.POINTER(C.c_int32)]
+_nv.nvcvImageFormatGetPlaneDataType.argtypes = [C.c_uint64, C.c_int32, C.POINTER(C.c_uint64)]
+_nv.nvcvImageFormatGetPlaneBitsPerPixel.argtypes = [C.c_uint64, C.c_int32, C.POINTER(C.c_int32)]
+_nv.nvcvDataTypeGetChannelType.argtypes = [C.c_uint64, C.c_int32, C.POINTER(C.c_uint64)]
+
+
+def _planes(fmt):
+    """(element type, channels) of every plane of an image format."""
+    n = C.c_int32()
+    check(_nv.nvcvImageFormatGetNumPlanes(fmt, C.byref(n)))
+    out = []
+    for p in range(n.value):
+        ch, dt, el = C.c_int32(), C.c_uint64(), C.c_uint64()
+        check(_nv.nvcvImageFormatGetPlaneNumChannels(fmt, p, C.byref(ch)))
+        check(_nv.nvcvImageFormatGetPlaneDataType(fmt, p, C.byref(dt)))
+        check(_nv.nvcvDataTypeGetChannelType(dt.value, 0, C.byref(el)))
+        if el.value not in _DT2NP:
+            raise ValueError("plane %d of format 0x%x has no array element type" % (p, fmt))
+        # elements per pixel as the memory holds them: bits per pixel / element size (4:2:2 formats such as YUYV
+        # name three channels and store two bytes per pixel)
+        bpp = C.c_int32()
+        check(_nv.nvcvImageFormatGetPlaneBitsPerPixel(fmt, p, C.byref(bpp)))
+        out.append((_DT2NP[el.value], max(1, bpp.value // (8 * _DT2NP[el.value].itemsize)) if bpp.value else ch.value))
+    return out
+
+
+def _relayout(buf, layout, have="HWC"):
+    """The buffer with its dimensions in the order of `layout`; letters the buffer does not have are dimensions of 1,
+    and a dimension the layout leaves out must be 1."""
+    iface = buf.__cuda_array_interface__
+    dims = dict(zip(have, zip(iface["shape"], iface["strides"])))
+    for letter, (extent, _) in dims.items():
+        if letter not in layout and extent != 1:
+            raise ValueError("layout %r leaves out dimension %s of extent %d" % (layout, letter, extent))
+    es = np.dtype(iface["typestr"]).itemsize
+    shape = tuple(dims[l][0] if l in dims else 1 for l in layout)
+    strides = tuple(dims[l][1] if l in dims else es for l in layout)
+    return _Buffer(dict(iface, shape=shape, strides=strides), buf._owner)
 
 
 def as_image(buffer, format=None):

@@ -150,3 +150,51 @@ def test_imgbatchvarshape_wrapper_nodeletion(nvcv):
         batch = nvcv.as_images([pt_img])
         del batch
         assert (pt_img.cpu().numpy() == np_img).all()
+
+
+# ---- images (tests/nvcv_types/python/test_image.py:40-60, 327-445) --------------------------------------------------
+def test_image_creation_works(nvcv):
+    for img in (nvcv.Image((7, 5), nvcv.Format.NV12), nvcv.Image(size=(7, 5), format=nvcv.Format.NV12)):
+        assert img.width == 7 and img.height == 5 and img.size == (7, 5) and img.format == nvcv.Format.NV12
+
+
+def test_image_create_packed(nvcv):
+    import torch
+    assert nvcv.Image((37, 11), nvcv.Format.U8, rowalign=1).cuda().__cuda_array_interface__["strides"] == (37, 1)
+    assert nvcv.Image.zeros((37, 11), nvcv.Format.U8, rowalign=1).cuda().__cuda_array_interface__["strides"] == (37, 1)
+    data = nvcv.as_image(torch.zeros((11, 37), dtype=torch.uint8, device="cuda")).cuda()
+    assert data.__cuda_array_interface__["strides"] == (37, 1)
+    assert (nvcv.Image.zeros((67, 34), nvcv.Format.F32).cpu() == np.zeros((34, 67), np.float32)).all()
+
+
+@pytest.mark.parametrize("size,format,layout,out_dtype,out_shape,simple_layout", [
+    ((257, 231), "U8", None, np.uint8, (231, 257), "HWC"), ((257, 231), "U8", "HWC", np.uint8, (231, 257, 1), "HWC"),
+    ((257, 231), "U8", "CHW", np.uint8, (1, 231, 257), "CHW"),
+    ((257, 231), "U8", "xyCrodHlimaWab", np.uint8, (1, 1, 1, 1, 1, 1, 231, 1, 1, 1, 1, 257, 1, 1), "CHW"),
+    ((257, 231), "RGBAf32", None, np.float32, (231, 257, 4), "HWC"), ((257, 231), "RGBA8", "HWC", np.uint8, (231, 257, 4), "HWC"),
+    ((257, 231), "RGBA8p", None, np.uint8, (4, 231, 257), "CHW"), ((257, 231), "RGBAf32p", "CHW", np.float32, (4, 231, 257), "CHW"),
+    ((258, 232), "NV12", None, [np.uint8, np.uint8], [(232, 258, 1), (116, 129, 2)], "HWC"),
+    ((258, 232), "NV12", "HWC", [np.uint8, np.uint8], [(232, 258, 1), (116, 129, 2)], "HWC"),
+    ((258, 232), "YUYV", None, np.uint8, (232, 258, 2), "HWC"), ((258, 232), "YUYV", "HWC", np.uint8, (232, 258, 2), "HWC"),
+])
+def test_image_export_cuda_buffer(nvcv, size, format, layout, out_dtype, out_shape, simple_layout):
+    import torch
+    img = nvcv.Image(size, nvcv.Format[format])
+    mem = img.cuda(layout)
+    if isinstance(mem, list):
+        for m, dt, shp in zip(mem, out_dtype, out_shape):
+            assert m.dtype == dt and m.shape == shp
+    else:
+        assert mem.dtype == out_dtype and mem.shape == out_shape
+    assert img.cuda(layout) is not mem  # a buffer is made per call
+    buffers = img.cuda(simple_layout)
+    buffers = buffers if isinstance(buffers, list) else [buffers]
+    rng = np.random.default_rng(0)
+    gold = []
+    for buf in buffers:  # written on the device side, read back through cpu()
+        gold.append((rng.random(size=buf.shape) * 255).astype(buf.dtype))
+        torch.as_tensor(buf, device="cuda").copy_(torch.as_tensor(gold[-1]))
+    back = img.cpu(simple_layout)
+    back = back if isinstance(back, list) else [back]
+    for b, g in zip(back, gold):
+        np.testing.assert_array_equal(b, g)
