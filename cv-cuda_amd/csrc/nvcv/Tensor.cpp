@@ -292,25 +292,21 @@ bool ViewStrides(int rank, const int64_t *shape, const int64_t *strides, int new
             ++ng;
         }
     }
-    int g = 0;
-    int d = 0;
-    while (d < newRank)
+    if (ng == 0) // nothing but unit dimensions
     {
-        if (newShape[d] == 1)
-        {
-            // unit dimensions take the stride of whatever follows; fixed up below
-            newStrides[d] = 0;
-            ++d;
-            continue;
-        }
-        if (g >= ng)
-        {
-            return false;
-        }
-        // consume output dims until their product equals the group's extent
-        int64_t vol   = 1;
-        int     first = d;
-        while (d < newRank && vol < gshape[g])
+        gshape[0]  = 1;
+        gstride[0] = strides[rank - 1];
+        ng         = 1;
+    }
+    // Every group is split into the next output dimensions whose product is its extent; unit dimensions go with
+    // the group at hand, also when its extent is already reached, and a dimension's stride is the group's stride
+    // times the extents after it inside the group (reference: src/nvcv/src/priv/TensorData.cpp:248-276).
+    int d = 0;
+    for (int g = 0; g < ng && d < newRank; ++g)
+    {
+        int64_t   vol   = 1;
+        const int first = d;
+        while (d < newRank && vol * newShape[d] <= gshape[g])
         {
             vol *= newShape[d];
             ++d;
@@ -325,22 +321,12 @@ bool ViewStrides(int rank, const int64_t *shape, const int64_t *strides, int new
             newStrides[k] = st;
             st *= newShape[k];
         }
-        ++g;
-    }
-    if (g != ng)
-    {
-        return false;
-    }
-    // unit dims: stride = extent*stride of the next dimension (or element stride at the end)
-    for (int k = newRank - 1; k >= 0; --k)
-    {
-        if (newShape[k] == 1)
+        if (g == ng - 1 && d != newRank)
         {
-            newStrides[k] = (k == newRank - 1) ? (ng > 0 ? gstride[ng - 1] : strides[rank - 1])
-                                               : newStrides[k + 1] * newShape[k + 1];
+            return false; // equal volumes make this unreachable; kept as a guard
         }
     }
-    return true;
+    return d == newRank;
 }
 
 } // namespace

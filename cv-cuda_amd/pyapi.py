@@ -33,7 +33,7 @@ from . import _DT2NP, check
 from ._capi import nvcv as _nv
 
 __all__ = ["Error", "Interp", "Border", "ChannelManip", "NormalizeFlags", "ColorConversion", "Format", "Type", "TensorLayout", "RectI",
-           "Stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image", "as_images"]
+           "Stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image", "as_images", "reshape"]
 
 
 def _enum_of(name, prefix):
@@ -176,6 +176,18 @@ class _Buffer:
         self.shape = tuple(iface["shape"])
         self.dtype = np.dtype(iface["typestr"])
 
+    @property
+    def strides(self):
+        """In bytes, as the array interface gives them (dense when it gives none)."""
+        given = self.__cuda_array_interface__.get("strides")
+        if given is not None:
+            return tuple(given)
+        out, acc = [], self.dtype.itemsize
+        for extent in reversed(self.shape):
+            out.insert(0, acc)
+            acc *= extent
+        return tuple(out)
+
     def __dlpack__(self, stream=None):
         return torch.as_tensor(self, device="cuda").__dlpack__()
 
@@ -229,6 +241,11 @@ class Tensor:
     def torch(self):
         """Strided torch view of the tensor's memory (not in the reference: what its tests build by hand)."""
         return self._t.torch_view()
+
+
+def reshape(tensor, shape, layout=None):
+    """A tensor of another shape over the same memory (nvcvTensorReshape); it keeps the memory alive."""
+    return tensor.reshape(shape, layout)
 
 
 def as_tensor(obj, layout=None):

@@ -558,3 +558,16 @@ def test_argument_checks_of_the_reference_from_plain_c_with_image_batches(cv, gp
                        timeout=120)
     assert r.returncode == 0 and r.stdout.strip().endswith("0 failed"), r.stdout + r.stderr
 
+
+
+@pytest.mark.parametrize("shape_arg,layout_arg,expected", [
+    ((1, 10, 10, 3), "XHWC", (320, 32, 3, 1)), ((10, 10, 3, 1), "HWCX", (32, 3, 1, 1)), ((10, 1, 10, 3), "HXWC", (32, 32, 3, 1)),
+    ((10, 2, 5, 3), "HABC", (32, 15, 3, 1)), ((2, 5, 10, 3), "ABWC", (160, 32, 3, 1)),
+])
+def test_reshape_of_padded_rows_gives_the_reference_strides(cv, shape_arg, layout_arg, expected):
+    """tests/nvcv_types/python/test_tensor.py:372-395 on a tensor with the 32-byte row pitch of the reference's device:
+    a unit dimension takes the stride of the group it is split from (src/nvcv/src/priv/TensorData.cpp:248-276)."""
+    t = cv.Tensor.wrap(0x10000, [10, 10, 3], [32, 3, 1], np.uint8, "HWC")
+    assert tuple(t.reshape(list(shape_arg), layout_arg).strides) == expected
+    with pytest.raises(cv.Error):
+        t.reshape([300], "A")  # padded rows cannot become one dense dimension

@@ -198,3 +198,69 @@ def test_image_export_cuda_buffer(nvcv, size, format, layout, out_dtype, out_sha
     back = back if isinstance(back, list) else [back]
     for b, g in zip(back, gold):
         np.testing.assert_array_equal(b, g)
+
+
+# ---- reshape and pitches (test_tensor.py:288-412). Rows are padded to this build's default pitch alignment of 128
+# bytes where the reference's figures show its device's 32 ---------------------------------------------------------------
+PITCH = 128
+
+
+def dense(shape):
+    out, acc = [], 1
+    for extent in reversed(shape):
+        out.insert(0, acc)
+        acc *= extent
+    return tuple(out)
+
+
+def test_tensor_create_packed(nvcv):
+    assert nvcv.Tensor((37, 11, 3), np.uint8, rowalign=1).cuda().strides == (11 * 3, 3, 1)
+    assert nvcv.Tensor(2, (37, 7), nvcv.Format.RGB8, rowalign=1).cuda().strides == (37 * 7 * 3, 37 * 3, 3, 1)
+    assert nvcv.Tensor((10, 10, 3), np.uint8, layout="HWC").cuda().strides == (PITCH, 3, 1)
+
+
+@pytest.mark.parametrize("orig_shape,orig_layout,dtype,shape_arg,layout_arg", [
+    ((1, 23, 65, 3), "NHWC", np.uint8, (23, 65, 3), "HWC"), ((5, 23, 65, 3), None, np.int8, (5, 23 * 65, 3), None),
+    ((5, 23, 65, 3), None, np.int8, (5, 23 * 65, 3), "ABC"), ((1,), "A", np.float32, (1, 1, 1, 1, 1, 1), "ABCDEF"),
+])
+def test_tensor_reshape(nvcv, orig_shape, orig_layout, dtype, shape_arg, layout_arg):
+    tensor = nvcv.Tensor(orig_shape, dtype, layout=orig_layout, rowalign=1)
+    es = np.dtype(dtype).itemsize
+    assert tensor.dtype == dtype and tensor.shape == orig_shape
+    assert tensor.cuda().strides == tuple(s * es for s in dense(orig_shape))
+    for new_tensor in (tensor.reshape(shape_arg, layout=layout_arg), nvcv.reshape(tensor, shape_arg, layout=layout_arg)):
+        assert new_tensor.dtype == dtype and new_tensor.shape == shape_arg
+        assert new_tensor.cuda().strides == tuple(s * es for s in dense(shape_arg))
+
+
+@pytest.mark.parametrize("orig_shape,orig_layout,dtype,shape_arg,layout_arg", [
+    ((1, 23, 65, 3), "NHWC", np.uint8, (23, 65, 3), "ABCD"), ((1, 23, 65, 3), None, np.uint8, (23, 65, 3), "ABCD"),
+    ((5, 23, 65, 3), "NHWC", np.int8, (100, 100), "AB"), ((1,), "A", np.int8, tuple(), ""),
+])
+def test_tensor_reshape_error(nvcv, orig_shape, orig_layout, dtype, shape_arg, layout_arg):
+    tensor = nvcv.Tensor(orig_shape, dtype, layout=orig_layout, rowalign=1)
+    with pytest.raises(RuntimeError):
+        tensor.reshape(shape_arg, layout=layout_arg)
+    with pytest.raises(RuntimeError):
+        nvcv.reshape(tensor, shape_arg, layout=layout_arg)
+
+
+def test_tensor_reshape_lifetime_ref_obj(nvcv):
+    tensor1 = nvcv.Tensor((20, 10, 3), np.uint8, layout="HWC", rowalign=1)
+    tensor2 = tensor1.reshape((200, 3), layout="WC")
+    del tensor1  # the reshaped tensor keeps the memory alive
+    assert tensor2.dtype == np.uint8 and tensor2.shape == (200, 3) and tensor2.cuda().strides == (3, 1)
+
+
+@pytest.mark.parametrize("shape_arg,layout_arg,expected_strides", [
+    ((1, 10, 10, 3), "XHWC", (10 * PITCH, PITCH, 3, 1)), ((10, 10, 3, 1), "HWCX", (PITCH, 3, 1, 1)),
+    ((10, 1, 10, 3), "HXWC", (PITCH, PITCH, 3, 1)), ((10, 2, 5, 3), "HABC", (PITCH, 15, 3, 1)),
+    ((2, 5, 10, 3), "ABWC", (5 * PITCH, PITCH, 3, 1)),
+])
+def test_tensor_reshape_strided(nvcv, shape_arg, layout_arg, expected_strides):
+    tensor = nvcv.Tensor((10, 10, 3), np.uint8, layout="HWC")
+    assert tensor.cuda().strides == (PITCH, 3, 1)  # padded rows
+    for new_tensor in (tensor.reshape(shape_arg, layout=layout_arg), nvcv.reshape(tensor, shape_arg, layout=layout_arg)):
+        assert new_tensor.cuda().strides == expected_strides
+    with pytest.raises(RuntimeError):  # padded rows cannot become one dense dimension
+        tensor.reshape((300,), layout="A")
