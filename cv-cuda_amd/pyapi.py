@@ -75,8 +75,91 @@ class NormalizeFlags(enum.IntEnum):  # cvcuda/OpNormalize.h
 
 ColorConversion = enum.IntEnum("ColorConversion", {k: int(v) for k, v in _enum_of("_", "COLOR_").__members__.items()
                                                    if re.match(r"^[A-Za-z0-9]+?2[A-Z]", k)})  # not COLOR_SPEC_*, COLOR_XFER_* ...
-Format = _enum_of("Format", "IMAGE_FORMAT_")
-Type = _enum_of("Type", "DATA_TYPE_")
+def _members(prefix):
+    """Names of the reference's Python enumerations: the header names without prefix, an underscore in front of
+    those that begin with a digit (_2S16, _3S8 ...)."""
+    out = {}
+    for k, v in vars(K).items():
+        if k.startswith(prefix) and isinstance(v, int):
+            name = k[len(prefix):]
+            out["_" + name if name[0].isdigit() else name] = v
+    return out
+
+
+_nv.nvcvImageFormatGetNumChannels.argtypes = [C.c_uint64, C.POINTER(C.c_int32)]
+_nv.nvcvImageFormatGetNumPlanes.argtypes = [C.c_uint64, C.POINTER(C.c_int32)]
+
+
+class _FormatValue(int):
+    @property
+    def channels(self):
+        n = C.c_int32()
+        check(_nv.nvcvImageFormatGetNumChannels(int(self), C.byref(n)))
+        return n.value
+
+    @property
+    def planes(self):
+        n = C.c_int32()
+        check(_nv.nvcvImageFormatGetNumPlanes(int(self), C.byref(n)))
+        return n.value
+
+
+_SCALAR_NAMES = {"u1": "U8", "i1": "S8", "u2": "U16", "i2": "S16", "u4": "U32", "i4": "S32", "u8": "U64", "i8": "S64",
+                 "f2": "F16", "f4": "F32", "f8": "F64", "c8": "C64", "c16": "C128"}
+
+
+def _type_name_of(dtype):
+    """Member name of Type for a numpy dtype: scalars, and one-dimensional sub-arrays of them ("3i1" -> _3S8)."""
+    try:
+        dt = np.dtype(dtype)
+    except TypeError as exc:
+        raise TypeError("not a data type: %r" % (dtype,)) from exc
+    count = ""
+    if dt.subdtype is not None:
+        dt, shape = dt.subdtype
+        if len(shape) != 1:
+            raise TypeError("only one-dimensional sub-arrays are data types")
+        count = "_%d" % shape[0]
+    key = dt.kind + str(dt.itemsize)
+    if dt.fields is not None or key not in _SCALAR_NAMES:
+        raise TypeError("no data type for %r" % (dtype,))
+    return count + _SCALAR_NAMES[key]
+
+
+class _TypeValue(int):
+    def __eq__(self, other):
+        if isinstance(other, int):
+            return int(self) == int(other)
+        try:
+            return self.name == _type_name_of(other)
+        except TypeError:
+            return NotImplemented
+
+    def __ne__(self, other):
+        result = self.__eq__(other)
+        return result if result is NotImplemented else not result
+
+    __hash__ = int.__hash__
+
+
+Format = enum.Enum("Format", _members("IMAGE_FORMAT_"), type=_FormatValue)
+
+
+class _TypeMeta(enum.EnumMeta):
+    def __call__(cls, value, *args, **kw):
+        if not args and not kw and not isinstance(value, int):
+            name = _type_name_of(value)
+            if name not in cls.__members__:
+                raise TypeError("no data type for %r" % (value,))
+            return cls.__members__[name]
+        return super().__call__(value, *args, **kw)
+
+
+class _TypeBase(_TypeValue, enum.Enum, metaclass=_TypeMeta):
+    """Type(numpy dtype) gives the member; members compare equal to the numpy dtypes they stand for."""
+
+
+Type = _TypeBase("Type", _members("DATA_TYPE_"))
 
 
 class TensorLayout:

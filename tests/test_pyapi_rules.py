@@ -60,3 +60,38 @@ def test_small_helpers(api):
     with pytest.raises(ValueError):
         api._image_axes("NC")
     assert api._np_dtype(api.Type.F32) == np.float32 and api._np_dtype(np.uint8) == np.uint8
+
+
+# ---- tests/nvcv_types/python/test_imgformat.py:20-45, test_datatype.py:21-54, test_rect.py:19-40 ------------------------
+@pytest.mark.parametrize("format,gold_channels,gold_planes", [
+    ("RGBA8", 4, 1), ("RGB8", 3, 1), ("_2S16", 2, 1), ("S8", 1, 1), ("NV12", 3, 2),
+])
+def test_imgformat_numchannels_and_planes(api, format, gold_channels, gold_planes):
+    assert getattr(api.Format, format).channels == gold_channels and getattr(api.Format, format).planes == gold_planes
+
+
+@pytest.mark.parametrize("type,dt", [
+    ("U8", np.uint8), ("U8", np.dtype(np.uint8)), ("S8", np.int8), ("U16", np.uint16), ("S16", np.int16), ("U32", np.uint32),
+    ("S32", np.int32), ("U64", np.uint64), ("S64", np.int64), ("F32", np.float32), ("F64", np.float64), ("C64", np.complex64),
+    ("_2C64", np.dtype("2F")), ("C128", np.complex128), ("_2C128", np.dtype("2D")), ("_3S8", np.dtype("3i1")),
+    ("_4S32", np.dtype("4i")),
+])
+def test_datatype_dtype(api, type, dt):
+    type = getattr(api.Type, type)
+    assert type == dt
+    made = api.Type(dt)
+    assert made == type and made == dt and made is type
+
+
+@pytest.mark.parametrize("dt", [np.dtype([("f1", np.uint64), ("f2", np.int32)]), "invalid"])
+def test_datatype_dtype_conv_error(api, dt):
+    with pytest.raises(TypeError):
+        api.Type(dt)
+
+
+def test_recti(api):
+    r = api.RectI()
+    assert (r.x, r.y, r.width, r.height) == (0, 0, 0, 0)
+    for x, y, w, h in ((0, 0, 0, 0), (10, -12, -45, 14)):
+        for r in (api.RectI(x, y, w, h), api.RectI(y=y, width=w, height=h, x=x)):
+            assert (r.x, r.y, r.width, r.height) == (x, y, w, h)
