@@ -33,7 +33,7 @@ from . import _DT2NP, check
 from ._capi import nvcv as _nv
 
 __all__ = ["Error", "Interp", "Border", "ChannelManip", "NormalizeFlags", "ColorConversion", "Format", "Type", "TensorLayout", "RectI",
-           "Stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image", "as_images", "reshape"]
+           "Stream", "as_stream", "cuda", "Tensor", "Image", "ImageBatchVarShape", "as_tensor", "as_image", "as_images", "reshape"]
 
 
 def _enum_of(name, prefix):
@@ -213,6 +213,9 @@ class Stream(metaclass=_StreamMeta):
     def handle(self):
         return self._s.cuda_stream
 
+    def __int__(self):
+        return self.handle
+
     def sync(self):
         self._s.synchronize()
 
@@ -227,8 +230,23 @@ class Stream(metaclass=_StreamMeta):
         return False
 
 
-class cuda:  # the reference also offers the class as cvcuda.cuda.Stream
+def as_stream(stream):
+    """A Stream over a stream made elsewhere: a torch stream, or a raw hipStream_t given as an int or a
+    ctypes.c_void_p (python/mod_nvcv/Stream.cpp, the external-stream wrappers). The wrapper keeps the object."""
+    if isinstance(stream, Stream):
+        return stream
+    if isinstance(stream, C.c_void_p):
+        stream = stream.value or 0
+    if isinstance(stream, int):
+        return Stream.default if stream == 0 else Stream(torch.cuda.ExternalStream(stream))
+    if hasattr(stream, "cuda_stream"):
+        return Stream(stream)
+    raise TypeError("not a stream: %r" % (stream,))
+
+
+class cuda:  # the reference offers these as cvcuda.cuda.Stream and cvcuda.cuda.as_stream as well
     Stream = Stream
+    as_stream = staticmethod(as_stream)
 
 
 def _torch_stream(stream):

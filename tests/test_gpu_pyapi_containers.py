@@ -264,3 +264,41 @@ def test_tensor_reshape_strided(nvcv, shape_arg, layout_arg, expected_strides):
         assert new_tensor.cuda().strides == expected_strides
     with pytest.raises(RuntimeError):  # padded rows cannot become one dense dimension
         tensor.reshape((300,), layout="A")
+
+
+# ---- streams (tests/nvcv_types/python/test_stream.py:21-112) -----------------------------------------------------------
+def test_current_user_and_nested_streams(nvcv):
+    Stream = nvcv.cuda.Stream
+    assert Stream.current is Stream.default and type(Stream.current) == Stream
+    with Stream():
+        assert Stream.current is not Stream.default
+    stream1, stream2 = Stream(), Stream()
+    with stream1:
+        assert stream1 is Stream.current and stream1 is not Stream.default
+        with stream2:
+            assert stream2 is Stream.current and stream1 is not Stream.current
+        assert stream2 is not Stream.current and stream1 is Stream.current
+    assert stream1 is not Stream.default and stream1 is not Stream.current
+    assert Stream.default.handle == 0
+
+
+def test_wrapped_streams(nvcv):
+    import ctypes
+    import torch
+    stream = torch.cuda.Stream()
+    assert nvcv.cuda.as_stream(ctypes.c_void_p(stream.cuda_stream)).handle == stream.cuda_stream
+    assert nvcv.cuda.as_stream(int(stream.cuda_stream)).handle == int(stream.cuda_stream)
+    own = nvcv.cuda.Stream()
+    assert own.handle == int(own)
+    ext = torch.cuda.Stream()
+    wrapped = nvcv.cuda.as_stream(ext)
+    handle = ext.cuda_stream
+    assert wrapped.handle == handle
+    del ext  # the wrapper keeps the stream alive
+    again = nvcv.cuda.as_stream(torch.cuda.ExternalStream(wrapped.handle))
+    assert again.handle == handle
+    # work submitted on a wrapped stream runs there
+    src = nvcv.as_tensor(torch.arange(24, dtype=torch.uint8, device="cuda").reshape(2, 4, 3), "HWC")
+    out = nvcv.flip(src, 0, stream=wrapped)
+    wrapped.sync()
+    assert torch.equal(out.torch().cpu(), torch.arange(24, dtype=torch.uint8).reshape(2, 4, 3).flip(0))
