@@ -517,16 +517,23 @@ def test_op_resize_crop_convert_reformat(cvcuda, orc, tensor_params, resize_dim,
         assert diff.max() <= abs(scale) * 1.0001 + 1e-4 and (diff > 1e-4 * max(1.0, abs(scale))).mean() < 0.01
 
 
-@pytest.mark.parametrize("num_images,min_size,max_size,resize_dim,interp,crop,out_layout,expected", [
-    (10, (300, 150), (640, 480), (256, 256), "LINEAR", (0, 0, 224, 224), "NCHW", (10, 3, 224, 224)),
-    (5, (60, 40), (100, 90), (128, 64), "NEAREST", (10, 4, 100, 50), "NHWC", (5, 50, 100, 3)),
+@pytest.mark.parametrize("num_images,min_size,max_size,resize_dim,interp,crop,out_layout,out_dtype,manip,expected", [
+    (10, (50, 50), (512, 512), (256, 256), "LINEAR", (0, 0, 224, 224), "NCHW", "F32", "REVERSE", (10, 3, 224, 224)),
+    (1, (500, 300), (800, 700), (400, 200), "LINEAR", (0, 0, 224, 190), "NHWC", "F32", "REVERSE", (1, 190, 224, 3)),
+    (50, (1, 1), (50, 70), (400, 200), "LINEAR", (0, 0, 224, 190), "NHWC", "F32", "NO_OP", (50, 190, 224, 3)),
+    (50, (1, 1), (50, 70), (400, 200), "LINEAR", (0, 0, 224, 190), "NCHW", "U8", "REVERSE", (50, 3, 190, 224)),
+    (50, (1, 1), (50, 70), (400, 200), "LINEAR", (0, 0, 224, 190), "NCHW", "U8", "NO_OP", (50, 3, 190, 224)),
+    (50, (1, 1), (50, 70), (400, 200), "LINEAR", (0, 0, 224, 190), "", 0, "REVERSE", (50, 190, 224, 3)),
 ])
 def test_op_resize_crop_convert_reformat_varshape(cvcuda, orc, num_images, min_size, max_size, resize_dim, interp, crop,
-                                                  out_layout, expected):
-    interp = cvcuda.Interp[interp]
+                                                  out_layout, out_dtype, manip, expected):
+    # test_opresizecropconvertreformat.py:262-520
+    import torch
+    interp, manip = cvcuda.Interp[interp], cvcuda.ChannelManip[manip]
+    out_layout = out_layout if out_layout else "NHWC"
+    out_dtype = cvcuda.Type[out_dtype] if out_dtype else cvcuda.Type.U8
     input = cvcuda.ImageBatchVarShape(num_images)
     data = []
-    import torch
     for i in range(num_images):
         w = min_size[0] + (max_size[0] - min_size[0]) * i // num_images
         h = min_size[1] + (max_size[1] - min_size[1]) * i // num_images
@@ -535,21 +542,19 @@ def test_op_resize_crop_convert_reformat_varshape(cvcuda, orc, num_images, min_s
         img.plane_view(0, np.uint8, 3).copy_(torch.from_numpy(a).cuda())
         input.pushback(img)
         data.append(a)
-    out = cvcuda.resize_crop_convert_reformat(input, resize_dim, interp, cvcuda.RectI(*crop), layout=out_layout,
-                                              data_type=cvcuda.Type.F32, manip=cvcuda.ChannelManip.REVERSE)
-    assert out.shape == expected and out.layout == out_layout and out.dtype == np.float32
-    stream = cvcuda.Stream()
-    out2 = cvcuda.Tensor(expected, np.float32, out_layout)
-    tmp = cvcuda.resize_crop_convert_reformat_into(out2, input, resize_dim, interp, [crop[0], crop[1]],
-                                                  manip=cvcuda.ChannelManip.REVERSE, stream=stream)
+    out1 = cvcuda.resize_crop_convert_reformat(input, resize_dim=resize_dim, interp=interp, crop_rect=cvcuda.RectI(*crop),
+                                               layout=out_layout, data_type=out_dtype, manip=manip, scale=1, offset=0)
+    assert out1.layout == out_layout and out1.shape == expected and out1.dtype == out_dtype
+    out2 = cvcuda.Tensor(expected, out_dtype, out_layout)
+    tmp = cvcuda.resize_crop_convert_reformat_into(out2, input, resize_dim, interp, [crop[1], crop[0]], manip=manip)
     assert tmp is out2
-    stream.sync()
-    got = host(out)
+    assert out2.layout == out_layout and out2.shape == expected and out2.dtype == out_dtype
+    got = host(out1)
     np.testing.assert_array_equal(host(out2), got)
-    for i in (0, num_images - 1):
-        want = orc.fused_rccr(data[i][None], (crop[3], crop[2]), tuple(resize_dim), (crop[0], crop[1]),
-                              int(interp), np.float32, out_layout == "NCHW", 1, 1.0, 0.0, True)
-        diff = np.abs(got[i:i + 1] - want)
+    for i in (0, num_images - 1):  # values: the oracle, within one 8-bit step (the source is cast back to u8 first)
+        want = orc.fused_rccr(data[i][None], (crop[3], crop[2]), tuple(resize_dim), (crop[0], crop[1]), int(interp),
+                              out1.dtype.type, out_layout == "NCHW", int(manip), 1.0, 0.0, True)
+        diff = np.abs(got[i:i + 1].astype(np.float32) - want.astype(np.float32))
         assert diff.max() <= 1.0001 and (diff > 1e-4).mean() < 0.01
 
 
