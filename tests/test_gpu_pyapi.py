@@ -441,7 +441,7 @@ def test_op_warp(cvcuda, perspective, input_args, xform, flags, border_mode, bor
 
 @pytest.mark.parametrize("nimages,format,max_size,max_pixel,max_xval,flags,bmode,border_value", [
     (5, "RGB8", (16, 23), 128, 7, "NEAREST", "CONSTANT", []), (5, "RGB8", (16, 23), 128, 7, "NEAREST", "CONSTANT", [1, 2, 3, 4]),
-    (4, "RGB8", (16, 23), 128, 5, "LINEAR", "WRAP", [0]), (3, "RGB8", (16, 23), 128, 3, "LINEAR", "REPLICATE", [1, 2, 3, 4]),
+    (4, "RGB8", (16, 23), 128, 5, "LINEAR", "WRAP", [0]), (3, "RGB8", (16, 23), 128, 4, "CUBIC", "REPLICATE", [2, 1, 0]),
 ])
 @pytest.mark.parametrize("perspective", [False, True])
 def test_op_warp_varshape(cvcuda, perspective, nimages, format, max_size, max_pixel, max_xval, flags, bmode, border_value):
