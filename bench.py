@@ -125,6 +125,8 @@ class Fused:
     def __init__(self, cv, orc, np, torch, form="fused"):
         self.cv, self.orc, self.np, self.torch, self.form = cv, orc, np, torch, form
         self.key, self.kernel = form, self.KERNELS[form]
+        if form == "fused" and self.N == 64:  # the mover has the bytes of the configuration's own batch
+            self.mover = "stream-mix-4-2"
         self.workload = ("fused ResizeCropConvertReformat: batch %d u8 NHWC 1920x1080 -> bilinear 455x256 -> " % self.N +
                          "crop 224x224 @(115,16) -> f32 NCHW, " + self.TEXT[form])
         self.images = self.N
@@ -251,7 +253,7 @@ class ResizeC1:
 
 
 class CubicC5:
-    key, config_id = "resize-cubic-4k", 5
+    key, config_id, mover = "resize-cubic-4k", 5, "stream-mix-24-1"
     N, SRC_H, SRC_W, OUT_H, OUT_W = 16, 2160, 3840, 360, 640
     kernel = "ResizeCubicStagedKernel<float,4>"
     dtype = "f32"
@@ -289,7 +291,7 @@ class CubicC5:
 
 
 class Nv12C3:
-    key, config_id = "nv12-to-rgb", 3
+    key, config_id, mover = "nv12-to-rgb", 3, "stream-mix-1-2"
     N, H, W = 32, 1080, 1920
     kernel = "Yuv420ToRgbTensor<3,true>"
     dtype = "int32"
@@ -841,6 +843,9 @@ def main():
                     help="independent streams the K steps are dealt to inside the captured graph (default 1: every "
                          "step waits for the one before, as consecutive Submits on one stream do)")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle spot check (kernel experiments only)")
+    ap.add_argument("--no-mover", action="store_true",
+                    help="skip the plain byte mover that the fused, nv12-to-rgb and resize-cubic-4k workloads time beside "
+                         "the operator (roofline.dense_mover)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="after the timed region, also run a plain device copy of this many MiB three times "
                          "(a kernel of known traffic to scale hardware byte counters against)")
@@ -947,6 +952,38 @@ def main():
         eager.append(time.perf_counter() - c0)
     submit_to_sync_ms = sorted(eager)[len(eager) // 2] * 1e3
 
+    # ---- the same bytes through a kernel that only moves them (dense 16-byte loads, streaming stores, no
+    # arithmetic): what the memory system gives a launch of this size, measured in this run beside the operator
+    mover = None
+    mover_key = getattr(wl, "mover", None)
+    if mover_key and not args.no_mover and graph is not None:
+        mw = StreamMix(cv, orc, np, torch, mover_key)
+        msets = [mw.make_set() for _ in range(max(3, int(math.ceil(2 * 268e6 / (16 * mw.lanes * mw.reads)))))]
+        msteps = min(args.steps, 500)
+        for i in range(len(msets)):
+            mw.submit(stream, msets[i])
+        torch.cuda.synchronize()
+        mgraph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(mgraph):
+            mcap = torch.cuda.current_stream()
+            for i in range(msteps):
+                mw.submit(mcap, msets[i % len(msets)])
+        mgraph.replay()
+        torch.cuda.synchronize()
+        mreps = max(1, int(math.ceil(0.1 / max(msteps * mean_kernel_ms * 1e-3, 1e-6))))
+        m0, m1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        m0.record(stream)
+        for _ in range(mreps):
+            mgraph.replay()
+        m1.record(stream)
+        torch.cuda.synchronize()
+        mover_ms = m0.elapsed_time(m1) / (msteps * mreps)
+        mw.check(msets[0])
+        mover = {"workload": mover_key, "kernel": mw.kernel, "bytes_per_launch": mw.alg_bytes,
+                 "ms_per_launch": round(mover_ms, 5), "GB/s": round(mw.alg_bytes / (mover_ms * 1e-3) / 1e9, 1),
+                 "operator_over_mover": round(mean_kernel_ms / mover_ms, 4)}
+        del mgraph, msets
+
     if args.copy_probe > 0:
         a = torch.full((args.copy_probe << 20,), 7, dtype=torch.uint8, device="cuda")
         b = torch.empty_like(a)
@@ -1013,6 +1050,8 @@ def main():
         "cpu_baseline": cpu,
         "submit_to_sync_ms": round(submit_to_sync_ms, 4),
     }
+    if mover is not None:
+        out["roofline"]["dense_mover"] = mover
     if getattr(wl, "other_bytes", None):
         # the same launch time under two other byte conventions: the whole input and output tensors (what the
         # reference's own benchmarks count), and only the pixels an output pixel refers to plus the output

@@ -51,3 +51,22 @@ def test_byte_conventions_of_the_baseline_configurations():
     assert (rows, cols) == (224, 224)
     rows, cols = b.span_bytes(360, 0, 2160, 360, b.CUBIC, 1)[0], b.span_bytes(640, 0, 3840, 640, b.CUBIC, 16)[0]
     assert (rows, cols) == (1440, 2560) and (rows * cols + 360 * 640) * 16 * 16 == 1002700800
+
+
+def test_the_byte_movers_move_at_least_the_bytes_of_the_operators_they_stand_beside():
+    """`roofline.dense_mover` compares an operator with a kernel that only moves bytes: the mover's reads and writes
+    are each at least the operator's (fused: 448 x 2829 bytes of row spans read and 602112 written per image; NV12:
+    1.5 and 3 bytes per pixel; cubic: the row spans and the 640 x 360 x 16-byte output)."""
+    b = load_bench()
+    specs = b.StreamMix.SPECS
+
+    def moved(key):
+        reads, writes, lanes = specs[key]
+        return 16 * lanes * reads, 16 * lanes * writes
+    assert b.Nv12C3.mover in specs and b.CubicC5.mover in specs
+    r, w = moved("stream-mix-4-2")
+    assert r >= 64 * 448 * 2829 and w >= 64 * 602112 and r + w <= 1.02 * 119648256
+    r, w = moved(b.Nv12C3.mover)
+    assert (r, w) == (32 * 1620 * 1920, 32 * 1080 * 1920 * 3)
+    r, w = moved(b.CubicC5.mover)
+    assert w == 16 * 640 * 360 * 16 and r >= 1473822720 - w and r + w <= 1.001 * 1473822720
