@@ -43,6 +43,8 @@ constexpr int kPatch     = 8;  // gather granule: a wave samples kPatch x kPatch
 constexpr int kPxPerLane = 4;  // steps per wave
 constexpr int kTileW     = 64; // = 8 patches
 constexpr int kTileH     = 16; // = 2 patches; 16 patches / 4 waves = kPxPerLane
+constexpr int kPatchesX  = kTileW / kPatch;
+constexpr int kThreads   = kTileW * kTileH / kPxPerLane;
 
 struct WarpArgs
 {
@@ -122,6 +124,142 @@ __device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
 __device__ __forceinline__ int FloorToInt(float v)
 {
     return (int)fminf(fmaxf(floorf(v), -1073741824.f), 1073741824.f);
+}
+
+// ---- u8 bilinear in 15-bit fixed point ---------------------------------------------------------------
+// For 8-bit pixels the bilinear blend runs on integers: the fractions of the source coordinate are cut
+// to 15 bits (ax = trunc(fx * 2^15), fx = sx - floor(sx) in float32), the four weights are integers that
+// add up to exactly 2^15,
+//     w11 = (ax * ay + 2^14) >> 15,  w01 = ax - w11,  w10 = ay - w11,  w00 = 2^15 - ax - ay + w11,
+// the weighted sum of the four taps is exact in 24 bits and is rounded to nearest, ties to even, once.
+// Each weight is within 2^-15 of the product the float32 expression of the reference forms, so the
+// unrounded sum is within 4 * 255 * 2^-15 < 0.032 of it: results differ from the reference's golden by
+// at most 1 and agree with it wherever the weights are multiples of 2^-7 per axis (integer and
+// quarter-step maps, which is what the reference's own exact-equality table uses), because then nothing
+// is rounded before the final rounding. What it buys: the taps stay bytes (two taps and two weights per
+// v_dot2_u32_u16 instead of a conversion, a multiply and an add per tap and channel in float32).
+template<class T, int INTERP>
+constexpr bool kFixedPoint = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_LINEAR;
+
+// 8-bit bicubic: the four horizontal weights (the reference's float32 polynomials) are rounded to
+// multiples of 2^-14 with the last one taking the remainder, so that they add up to exactly 1; a row's
+// four taps are combined in integers (exact), the four row sums in float32 with the vertical weights.
+// Every horizontal weight is within 2^-15 of the float32 one (the last within 2^-14): the result is
+// within 0.05 of the float32 expression's, i.e. at most 1 from the reference's golden.
+template<class T, int INTERP>
+constexpr bool kFixedPointCubic = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_CUBIC;
+
+constexpr uint32_t kQ15 = 32768u;
+
+// The kernels that blend in fixed point work on coordinates in units of 2^-15 pixel: the first two rows
+// of their destination -> source matrix arrive multiplied by 2^15 (exact: a power of two), so floor and
+// fraction of a coordinate are the two halves of one float -> integer conversion.
+template<class T, int INTERP>
+constexpr float kCoordScale = kFixedPoint<T, INTERP> ? 32768.f : 1.f;
+
+// (w00 | w01 << 16) and (w10 | w11 << 16) from the two 15-bit fractions (each 0 .. 2^15).
+__device__ __forceinline__ void WeightPairsQ15(uint32_t ax, uint32_t ay, uint32_t &top, uint32_t &bottom)
+{
+    const uint32_t w11 = (__umul24(ax, ay) + (kQ15 >> 1)) >> 15;
+    bottom             = __umul24(w11, 65535u) + ay;          // (ay - w11) | w11 << 16
+    top                = (__umul24(ax, 65535u) + kQ15) - bottom; // (2^15 - ax | ax << 16) - bottom: no borrow
+}
+
+// Weighted sum of one channel: tap pairs as (left | right << 16), result in units of 2^-15, rounded to
+// nearest-even, saturated (never needed) and placed into byte `c` of q. The sum is accumulated on top
+// of the bit pattern of 256.0f, whose unit in the last place is 2^-15: read as a float the register
+// then holds 256 + sum / 2^15 exactly.
+__device__ __forceinline__ uint32_t BlendQ15(uint32_t topTaps, uint32_t bottomTaps, uint32_t top, uint32_t bottom, int c,
+                                             uint32_t q)
+{
+    typedef unsigned short U16x2 __attribute__((ext_vector_type(2)));
+    U16x2 t0, t1, w0, w1;
+    __builtin_memcpy(&t0, &topTaps, 4);
+    __builtin_memcpy(&t1, &bottomTaps, 4);
+    __builtin_memcpy(&w0, &top, 4);
+    __builtin_memcpy(&w1, &bottom, 4);
+    uint32_t acc = __builtin_amdgcn_udot2(t0, w0, 0x43800000u, false);
+    acc          = __builtin_amdgcn_udot2(t1, w1, acc, false);
+    return __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(acc) - 256.f, c, q);
+}
+
+// The same sum in plain integer arithmetic (border path, one tap at a time).
+__device__ __forceinline__ uint8_t RoundQ15(uint32_t sum)
+{
+    return (uint8_t)((sum + (kQ15 / 2 - 1) + ((sum >> 15) & 1u)) >> 15);
+}
+
+// floor and 15-bit fraction of a coordinate; NaN and infinite coordinates give fraction 0
+__device__ __forceinline__ uint32_t FractionQ15(float v)
+{
+    const float f = v - floorf(v);
+    return f >= 0.f ? (uint32_t)(int)(f * 32768.f) : 0u;
+}
+
+// Horizontal bicubic weights, given times 2^14, as signed 16-bit integers: (w0 | w1 << 16), (w2 | w3 << 16).
+// Adding 1.5 * 2^23 rounds a weight to the nearest integer, ties to even, and leaves it in the low bits of
+// the sum's bit pattern (two's complement for negative values); w3 = 2^14 - w0 - w1 - w2 on those integers.
+__device__ __forceinline__ void CubicWeightPairsQ14(const float (&w)[4], uint32_t &p01, uint32_t &p23)
+{
+    constexpr float    kMagic = 12582912.f;
+    constexpr uint32_t kBits  = 0x4B400000u;
+    const uint32_t     b0 = __float_as_uint(w[0] + kMagic);
+    const uint32_t     b1 = __float_as_uint(w[1] + kMagic);
+    const uint32_t     b2 = __float_as_uint(w[2] + kMagic);
+    const uint32_t     w3 = (16384u + 3u * kBits) - (b0 + b1 + b2);
+    p01                   = __builtin_amdgcn_perm(b1, b0, 0x05040100u);
+    p23                   = __builtin_amdgcn_perm(w3, b2, 0x05040100u);
+}
+
+// The same four integers one by one (border path), also from weights times 2^14. NaN weights give 0.
+__device__ __forceinline__ void CubicWeightsQ14(const float (&w)[4], int (&q)[4])
+{
+    q[0] = (int)rintf(w[0]);
+    q[1] = (int)rintf(w[1]);
+    q[2] = (int)rintf(w[2]);
+    q[3] = 16384 - q[0] - q[1] - q[2];
+}
+
+// Bytes lo and hi of a row held in dwords r[] -> (byte lo | byte hi << 16), one byte permute.
+template<int N>
+__device__ __forceinline__ uint32_t BytePair(const uint32_t (&r)[N], int lo, int hi)
+{
+    const uint32_t sel = 0x0c000c00u | (uint32_t)(lo & 3) | ((uint32_t)(4 + (hi & 3)) << 16);
+    return __builtin_amdgcn_perm(r[hi >> 2], r[lo >> 2], sel);
+}
+
+__device__ __forceinline__ int Dot2I16(uint32_t a, uint32_t b, int c)
+{
+    typedef short I16x2 __attribute__((ext_vector_type(2)));
+    I16x2 x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    return __builtin_amdgcn_sdot2(x, y, c, false);
+}
+
+// a.lo * b.lo + a.hi * b.hi with nothing added: the three-operand form with the constant 0 (for a sum
+// that starts here the compiler picks the accumulate-in-place form and spends a move on clearing it).
+__device__ __forceinline__ int Dot2I16(uint32_t a, uint32_t b)
+{
+    int d;
+    asm("v_dot2_i32_i16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+
+// CubicCoeffs times `scale` (a power of two, so every step scales exactly) with the polynomials evaluated
+// by fused multiply-adds; used where the weights are quantised afterwards anyway.
+__device__ __forceinline__ void CubicCoeffsFused(float d, float scale, float (&w)[4])
+{
+    w[0] = __builtin_fmaf(-.5f * scale, d, scale);
+    w[0] = __builtin_fmaf(w[0], d, -.5f * scale);
+    w[0] = w[0] * d;
+    w[1] = __builtin_fmaf(1.5f * scale, d, -2.5f * scale);
+    w[1] = w[1] * d;
+    w[1] = __builtin_fmaf(w[1], d, scale);
+    w[2] = __builtin_fmaf(-1.5f * scale, d, 2.f * scale);
+    w[2] = __builtin_fmaf(w[2], d, .5f * scale);
+    w[2] = w[2] * d;
+    w[3] = scale - w[0] - w[1] - w[2];
 }
 
 // u8x3 taps are fetched through aligned dword windows (8 bytes for one pixel, 12 for two), which
@@ -221,6 +359,36 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
         }
         return;
     }
+    else if constexpr (kFixedPoint<T, INTERP>)
+    {
+        const int      x1 = FloorToInt(sx), y1 = FloorToInt(sy);
+        const uint32_t ax = FractionQ15(sx), ay = FractionQ15(sy);
+        const uint32_t w11 = (ax * ay + (kQ15 >> 1)) >> 15;
+        uint32_t       sum[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            sum[c] = 0;
+        }
+#pragma nounroll
+        for (int i = 0; i < 4; ++i) // taps (x1,y1) (x2,y1) (x1,y2) (x2,y2)
+        {
+            float t[C];
+            Fetch<T, C>(im, a, x1 + (i & 1), y1 + (i >> 1), t);
+            const uint32_t w = i == 0 ? kQ15 - ax - ay + w11 : (i == 1 ? ax - w11 : (i == 2 ? ay - w11 : w11));
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                sum[c] += (uint32_t)t[c] * w;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[c] = RoundQ15(sum[c]);
+        }
+        return;
+    }
     else if constexpr (INTERP == NVCV_INTERP_LINEAR)
     {
         const int x1 = FloorToInt(sx), y1 = FloorToInt(sy);
@@ -244,6 +412,49 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
                 acc[c] += t[c] * w;
             }
         }
+    }
+    else if constexpr (kFixedPointCubic<T, INTERP>)
+    {
+        const int ix = FloorToInt(sx), iy = FloorToInt(sy);
+        float     wx[4], wy[4];
+        CubicCoeffsFused(sx - floorf(sx), 16384.f, wx);
+        CubicCoeffsFused(sy - floorf(sy), 1.f / 16384.f, wy);
+        int wq[4];
+        CubicWeightsQ14(wx, wq);
+#pragma nounroll
+        for (int cy = 0; cy < 4; ++cy)
+        {
+            int h[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                h[c] = 0;
+            }
+#pragma nounroll
+            for (int cx = 0; cx < 4; ++cx)
+            {
+                float t[C];
+                Fetch<T, C>(im, a, ix + cx - 1, iy + cy - 1, t);
+                const int w = cx == 0 ? wq[0] : (cx == 1 ? wq[1] : (cx == 2 ? wq[2] : wq[3]));
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    h[c] += (int)t[c] * w;
+                }
+            }
+            const float v = cy == 0 ? wy[0] : (cy == 1 ? wy[1] : (cy == 2 ? wy[2] : wy[3]));
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                acc[c] = cy == 0 ? (float)h[c] * v : __builtin_fmaf((float)h[c], v, acc[c]);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[c] = SaturateCast<T>(acc[c]);
+        }
+        return;
     }
     else
     {
@@ -286,14 +497,21 @@ __device__ __forceinline__ void SampleWithBorder(const Img &im, const WarpArgs &
 // of the float's bit pattern: non-negative floats order like their bits, negative ones and NaNs have
 // patterns above every finite positive limit (-0.0 fails too and takes the generic path, which
 // computes the same result).
+// The test runs on a lane's kPxPerLane samples at once: the largest bit pattern per axis against the limit.
 template<int INTERP>
-__device__ __forceinline__ bool TapsInside(float limX, float limY, float sx, float sy)
+__device__ __forceinline__ bool TapsInside(float limX, float limY, const float (&sx)[kPxPerLane],
+                                           const float (&sy)[kPxPerLane])
 {
     // taps span [floor(v) - lo, floor(v) + hi] per axis; NEAREST takes floor(v + .5)
     constexpr float lo = INTERP == NVCV_INTERP_CUBIC ? 1.f : (INTERP == NVCV_INTERP_NEAREST ? -.5f : 0.f);
-    const bool inX = __float_as_uint(sx - lo) < __float_as_uint(limX);
-    const bool inY = __float_as_uint(sy - lo) < __float_as_uint(limY);
-    return inX & inY; // bitwise on purpose: no short-circuit branch
+    uint32_t        ux = 0, uy = 0;
+#pragma unroll
+    for (int k = 0; k < kPxPerLane; ++k)
+    {
+        ux = max(ux, __float_as_uint(sx[k] - lo));
+        uy = max(uy, __float_as_uint(sy[k] - lo));
+    }
+    return (ux < __float_as_uint(limX)) & (uy < __float_as_uint(limY)); // bitwise on purpose: no branch
 }
 
 // Exclusive upper limit of floor(v) - lo along an axis of `size` pixels; 0 (no sample passes) when the
@@ -389,13 +607,132 @@ __device__ __forceinline__ void SampleInside(const Img &im, float sx, float sy, 
     }
 }
 
+// Four horizontally adjacent u8 pixels at base + off (all inside the image) as raw bytes in C dwords.
+// u8x3: one aligned 16-byte window, funnel-shifted (see LoadU64Window); reads up to 3 bytes before and
+// 4 bytes after the 12.
+template<int C>
+__device__ __forceinline__ void LoadQuadBytes(const uint8_t *base, uint32_t off, uint32_t (&r)[C])
+{
+    if constexpr (kWideTapLoads<uint8_t, C>)
+    {
+        struct alignas(4) W4
+        {
+            uint32_t d[4];
+        };
+        const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(base) & 3u;
+        const uint32_t o   = off + mis;
+        const W4       w   = *reinterpret_cast<const W4 *>((base - mis) + (o & ~3u));
+        r[0]               = __builtin_amdgcn_alignbyte(w.d[1], w.d[0], o);
+        r[1]               = __builtin_amdgcn_alignbyte(w.d[2], w.d[1], o);
+        r[2]               = __builtin_amdgcn_alignbyte(w.d[3], w.d[2], o);
+    }
+    else
+    {
+        const Vec<uint8_t, 4 * C> v = *reinterpret_cast<const Vec<uint8_t, 4 * C> *>(base + off);
+        __builtin_memcpy(r, &v, 4 * C);
+    }
+}
+
+// The fixed-point bicubic sum (see kFixedPointCubic) of the 4 x 4 taps in r (row j, 4 pixels as raw bytes).
+template<int C>
+__device__ __forceinline__ uint32_t BlendCubicQ14(const uint32_t (&r)[4][C], float sx, float sy)
+{
+    float wx[4], wy[4];
+    CubicCoeffsFused(sx - floorf(sx), 16384.f, wx);
+    CubicCoeffsFused(sy - floorf(sy), 1.f / 16384.f, wy);
+    uint32_t p01, p23;
+    CubicWeightPairsQ14(wx, p01, p23);
+    uint32_t q = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            int h = Dot2I16(BytePair(r[j], c, c + C), p01);
+            h     = Dot2I16(BytePair(r[j], c + 2 * C, c + 3 * C), p23, h);
+            acc   = j == 0 ? (float)h * wy[0] : __builtin_fmaf((float)h, wy[j], acc);
+        }
+        q = __builtin_amdgcn_cvt_pk_u8_f32(acc, c, q);
+    }
+    return q;
+}
+
+// The same for a sample whose 16 taps are inside the image.
+template<int C>
+__device__ __forceinline__ uint32_t SampleInsideCubicQ14(const Img &im, float sx, float sy)
+{
+    uint32_t o = PixelOffset<C>(im, (int)floorf(sx) - 1, (int)floorf(sy) - 1);
+    uint32_t r[4][C];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        LoadQuadBytes<C>(im.base, o, r[j]);
+        o += (uint32_t)im.row;
+    }
+    return BlendCubicQ14<C>(r, sx, sy);
+}
+
+// The two horizontally adjacent u8 pixels at base + off (both inside the image) as raw bytes: byte i of
+// the 64-bit value {w[1]:w[0]} is channel i % C of pixel i / C.
+template<int C>
+__device__ __forceinline__ void LoadPairBytes(const uint8_t *base, uint32_t off, uint32_t (&w)[2])
+{
+    if constexpr (kWideTapLoads<uint8_t, C>)
+    {
+        const uint64_t q = LoadU64Window(base, off);
+        w[0]             = (uint32_t)q;
+        w[1]             = (uint32_t)(q >> 32);
+    }
+    else
+    {
+        const Vec<uint8_t, 2 * C> v = *reinterpret_cast<const Vec<uint8_t, 2 * C> *>(base + off);
+        w[0] = w[1] = 0;
+        __builtin_memcpy(w, &v, 2 * C);
+    }
+}
+
+// SampleWithBorder's fixed-point bilinear sum for a sample whose taps are all inside the image, whose
+// coordinates are not negative and below 2^16, given in units of 2^-15 pixel: floor and fraction come
+// from one float -> integer conversion, the taps of a row from one window, the two taps of a channel
+// from one byte permute. Returns the pixel's dword.
+template<int C>
+__device__ __forceinline__ uint32_t SampleInsideQ15(const Img &im, float sx, float sy)
+{
+    const uint32_t X = (uint32_t)(int)sx, Y = (uint32_t)(int)sy;
+    uint32_t       top, bottom;
+    WeightPairsQ15(X & (kQ15 - 1), Y & (kQ15 - 1), top, bottom);
+    const uint32_t o = PixelOffset<C>(im, (int)(X >> 15), (int)(Y >> 15));
+    uint32_t       r0[2], r1[2];
+    LoadPairBytes<C>(im.base, o, r0);
+    LoadPairBytes<C>(im.base, o + (uint32_t)im.row, r1);
+    uint32_t q = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        // bytes c and c + C of the row's 8 -> (left | right << 16); selector 0x0c gives a zero byte
+        const uint32_t sel = 0x0c000c00u | (uint32_t)c | ((uint32_t)(c + C) << 16);
+        q = BlendQ15(__builtin_amdgcn_perm(r0[1], r0[0], sel), __builtin_amdgcn_perm(r1[1], r1[0], sel), top, bottom, c, q);
+    }
+    return q;
+}
+
 // The dwords of the pixel that SampleInside gives. u8 channels are rounded, saturated and placed into
 // their byte by one instruction each (v_cvt_pk_u8_f32 with a byte select and the dword so far), where
 // packing converted bytes takes as many shifts and merges again.
 template<class T, int C, int INTERP>
 __device__ __forceinline__ void SampleInsidePacked(const Img &im, float sx, float sy, uint32_t (&w)[(C * sizeof(T) + 3) / 4])
 {
-    if constexpr (std::is_same_v<T, uint8_t> && INTERP != NVCV_INTERP_NEAREST)
+    if constexpr (kFixedPoint<T, INTERP>)
+    {
+        w[0] = SampleInsideQ15<C>(im, sx, sy);
+    }
+    else if constexpr (kFixedPointCubic<T, INTERP>)
+    {
+        w[0] = SampleInsideCubicQ14<C>(im, sx, sy);
+    }
+    else if constexpr (std::is_same_v<T, uint8_t> && INTERP != NVCV_INTERP_NEAREST)
     {
         float acc[C];
         SampleInside<float, C, INTERP, T>(im, sx, sy, acc);
@@ -447,8 +784,9 @@ __device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, fl
         t[c]   = (float)BorderValueAs<T>(a.bval[c]);
         acc[c] = 0.f;
     }
-    if constexpr (INTERP == NVCV_INTERP_NEAREST)
+    if constexpr (INTERP == NVCV_INTERP_NEAREST || kFixedPoint<T, INTERP>)
     {
+        // the tap itself; in fixed point the weights add up to exactly 1
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -472,6 +810,23 @@ __device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, fl
                 acc[c] += t[c] * w;
             }
         }
+    }
+    else if constexpr (kFixedPointCubic<T, INTERP>)
+    {
+        // every row sum is the border value times 2^14: the horizontal weights add up to exactly 1
+        float wy[4];
+        CubicCoeffsFused(sy - floorf(sy), 1.f / 16384.f, wy);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            const float h = t[c] * 16384.f;
+            float       v = h * wy[0];
+            v             = __builtin_fmaf(h, wy[1], v);
+            v             = __builtin_fmaf(h, wy[2], v);
+            v             = __builtin_fmaf(h, wy[3], v);
+            out[c]        = SaturateCast<T>(v);
+        }
+        return;
     }
     else
     {
@@ -501,7 +856,7 @@ __device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, fl
 }
 
 // One 64 x 16 tile of the destination image `dst` (tile coordinates tx, ty), all 256 threads.
-template<class T, int C, int INTERP>
+template<class T, int C, int INTERP, bool PERSP>
 __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dst, int dstRow,
                                          int dstW, int dstH, int tx, int ty)
 {
@@ -510,28 +865,24 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     // ---- gather: lane (lx, ly) of wave w samples its pixel in patches 4w .. 4w+3 (side by side: a
     // wave covers 32 columns x 8 rows)
     const int wave = threadIdx.x >> 6, lx = threadIdx.x & (kPatch - 1), ly = (threadIdx.x >> 3) & (kPatch - 1);
-    const float limX = InsideLimit<INTERP>(im.w, kWideTapLoads<T, C>), limY = InsideLimit<INTERP>(im.h, false);
+    // m maps to source coordinates times kCoordScale; so do sx, sy and the limits
+    constexpr float kScale = kCoordScale<T, INTERP>;
+    const float     limX = InsideLimit<INTERP>(im.w, kWideTapLoads<T, C>) * kScale, limY = InsideLimit<INTERP>(im.h, false) * kScale;
     float       sx[kPxPerLane], sy[kPxPerLane];
     uint32_t    q[D][kPxPerLane]; // q[d][k]: dword d of this lane's pixel in patch k
     // rows too long or too many for 24-bit offset arithmetic go through the generic path
-    bool allInside = (im.row | im.h) < (1 << 23);
+    // (and, in fixed point, coordinates too large for coordinate * 2^15 in 31 bits)
+    bool allInside = (im.row | im.h) < (1 << 23) && (!kFixedPoint<T, INTERP> || (im.w | im.h) < (1 << 16));
 #pragma unroll
     for (int k = 0; k < kPxPerLane; ++k)
     {
         const int patch = wave * kPxPerLane + k;
-        const int px = (patch & 7) * kPatch + lx, py = (patch >> 3) * kPatch + ly;
+        const int px = (patch % kPatchesX) * kPatch + lx, py = (patch / kPatchesX) * kPatch + ly;
         // pixels of the tile beyond the image edge repeat the edge pixel's sample; they are never stored
         const int dx = min(tx * kTileW + px, dstW - 1), dy = min(ty * kTileH + py, dstH - 1);
-        if (a.perspective)
-        {
-            MapCoord<true>(m, dx, dy, sx[k], sy[k]);
-        }
-        else
-        {
-            MapCoord<false>(m, dx, dy, sx[k], sy[k]);
-        }
-        allInside = allInside & TapsInside<INTERP>(limX, limY, sx[k], sy[k]);
+        MapCoord<PERSP>(m, dx, dy, sx[k], sy[k]);
     }
+    allInside = allInside & TapsInside<INTERP>(limX, limY, sx, sy);
     if (allInside)
     {
         uint32_t w[kPxPerLane][D];
@@ -558,17 +909,12 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
             // position and coordinates recomputed rather than indexed, results placed by selects: a
             // run-time index would put the arrays in scratch memory
             const int patch = wave * kPxPerLane + k;
-            const int px = (patch & 7) * kPatch + lx, py = (patch >> 3) * kPatch + ly;
+            const int px = (patch % kPatchesX) * kPatch + lx, py = (patch / kPatchesX) * kPatch + ly;
             const int dx = min(tx * kTileW + px, dstW - 1), dy = min(ty * kTileH + py, dstH - 1);
             float     bx, by;
-            if (a.perspective)
-            {
-                MapCoord<true>(m, dx, dy, bx, by);
-            }
-            else
-            {
-                MapCoord<false>(m, dx, dy, bx, by);
-            }
+            MapCoord<PERSP>(m, dx, dy, bx, by);
+            bx *= 1.f / kScale;
+            by *= 1.f / kScale;
             T v[C];
             if (a.border == NVCV_BORDER_CONSTANT && TapsOutside<INTERP>(im, bx, by))
             {
@@ -600,7 +946,7 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
         QuadTranspose(q[d], lx & 3);
     }
     const int patch = wave * kPxPerLane + (lx & 3);
-    const int px0 = (patch & 7) * kPatch + (lx & 4), py = (patch >> 3) * kPatch + ly;
+    const int px0 = (patch % kPatchesX) * kPatch + (lx & 4), py = (patch / kPatchesX) * kPatch + ly;
     const int dy = ty * kTileH + py, dx0 = tx * kTileW + px0;
     if (dy >= dstH || dx0 >= dstW)
     {
@@ -635,61 +981,67 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
 }
 
 // Loads image `image`'s matrix from the caller's tensor and, unless it already maps destination to
-// source, inverts it (uniform per block). Straight-line selects instead of early exits: every m[i] is
-// assigned exactly once, which keeps the matrix in registers.
-__device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float (&m)[9])
+// source, inverts it (uniform per block). The first two rows come out multiplied by `scale` (a power of
+// two: scaling commutes with every rounding of the products and sums that form a coordinate, so
+// coordinates computed from the scaled rows are the scaled coordinates bit for bit).
+template<bool PERSP>
+__device__ __forceinline__ void LoadMatrix(const WarpArgs &a, int image, float scale, float (&m)[9])
 {
     const float *p = reinterpret_cast<const float *>(a.xforms + image * a.xformStride);
-    const bool   persp = a.perspective != 0;
     float        f[9];
 #pragma unroll
-    for (int i = 0; i < 6; ++i)
+    for (int i = 0; i < 9; ++i)
     {
-        f[i] = p[i];
+        f[i] = i < (PERSP ? 9 : 6) ? p[i] : 0.f;
     }
-#pragma unroll
-    for (int i = 6; i < 9; ++i)
+    if (a.inverseGiven != 0)
     {
-        f[i] = persp ? p[i] : 0.f;
+        m[0] = f[0] * scale;
+        m[1] = f[1] * scale;
+        m[2] = f[2] * scale;
+        m[3] = f[3] * scale;
+        m[4] = f[4] * scale;
+        m[5] = f[5] * scale;
+        m[6] = f[6];
+        m[7] = f[7];
+        m[8] = f[8];
     }
-    float r[9];
-    // affine inverse (reference: warp.cu:139-150, 1/det evaluated in double)
-    float den = f[0] * f[4] - f[1] * f[3];
-    den       = fabsf(den) > 1e-5 ? (float)(1. / (double)den) : 0.f;
-    r[0]      = f[4] * den;
-    r[1]      = -f[1] * den;
-    r[2]      = (f[1] * f[5] - f[4] * f[2]) * den;
-    r[3]      = -f[3] * den;
-    r[4]      = f[0] * den;
-    r[5]      = (f[3] * f[2] - f[0] * f[5]) * den;
-    r[6] = r[7] = r[8] = 0.f;
-    if (persp)
+    else if constexpr (!PERSP)
+    {
+        // affine inverse (reference: warp.cu:139-150, 1/det evaluated in double and rounded to float32, which
+        // is what the correctly rounded float32 quotient gives; 1e-5 there is a double: for a float32
+        // operand, greater than it means greater than the float32 just below it)
+        float den = f[0] * f[4] - f[1] * f[3];
+        den       = (fabsf(den) > 9.99999974738e-06f ? 1.f / den : 0.f) * scale;
+        m[0]      = f[4] * den;
+        m[1]      = -f[1] * den;
+        m[2]      = (f[1] * f[5] - f[4] * f[2]) * den;
+        m[3]      = -f[3] * den;
+        m[4]      = f[0] * den;
+        m[5]      = (f[3] * f[2] - f[0] * f[5]) * den;
+        m[6] = m[7] = m[8] = 0.f;
+    }
+    else
     {
         // 3x3 inverse by cofactors (reference: cuda_tools/math/LinAlg.hpp:1446-1450, 1640-1654); a singular
         // matrix is left as given, like the reference's failed in-place inverse
         const float d = f[0] * (f[4] * f[8] - f[5] * f[7]) + f[1] * (f[5] * f[6] - f[3] * f[8])
                       + f[2] * (f[3] * f[7] - f[4] * f[6]);
         const bool  ok = d != 0;
-        r[0]           = ok ? (f[4] * f[8] - f[5] * f[7]) / d : f[0];
-        r[1]           = ok ? -(f[1] * f[8] - f[2] * f[7]) / d : f[1];
-        r[2]           = ok ? (f[1] * f[5] - f[2] * f[4]) / d : f[2];
-        r[3]           = ok ? -(f[3] * f[8] - f[5] * f[6]) / d : f[3];
-        r[4]           = ok ? (f[0] * f[8] - f[2] * f[6]) / d : f[4];
-        r[5]           = ok ? -(f[0] * f[5] - f[2] * f[3]) / d : f[5];
-        r[6]           = ok ? (f[3] * f[7] - f[4] * f[6]) / d : f[6];
-        r[7]           = ok ? -(f[0] * f[7] - f[1] * f[6]) / d : f[7];
-        r[8]           = ok ? (f[0] * f[4] - f[1] * f[3]) / d : f[8];
-    }
-    const bool given = a.inverseGiven != 0;
-#pragma unroll
-    for (int i = 0; i < 9; ++i)
-    {
-        m[i] = given ? f[i] : r[i];
+        m[0]           = (ok ? (f[4] * f[8] - f[5] * f[7]) / d : f[0]) * scale;
+        m[1]           = (ok ? -(f[1] * f[8] - f[2] * f[7]) / d : f[1]) * scale;
+        m[2]           = (ok ? (f[1] * f[5] - f[2] * f[4]) / d : f[2]) * scale;
+        m[3]           = (ok ? -(f[3] * f[8] - f[5] * f[6]) / d : f[3]) * scale;
+        m[4]           = (ok ? (f[0] * f[8] - f[2] * f[6]) / d : f[4]) * scale;
+        m[5]           = (ok ? -(f[0] * f[5] - f[2] * f[3]) / d : f[5]) * scale;
+        m[6]           = ok ? (f[3] * f[7] - f[4] * f[6]) / d : f[6];
+        m[7]           = ok ? -(f[0] * f[7] - f[1] * f[6]) / d : f[7];
+        m[8]           = ok ? (f[0] * f[4] - f[1] * f[3]) / d : f[8];
     }
 }
 
-template<class T, int C, int INTERP>
-__global__ __launch_bounds__(256) void WarpTensor(const WarpArgs a)
+template<class T, int C, int INTERP, bool PERSP>
+__global__ __launch_bounds__(kThreads) void WarpTensor(const WarpArgs a)
 {
     const int n  = blockIdx.z;
     const Img im = {a.src + n * a.srcN, a.srcRow, a.srcW, a.srcH};
@@ -699,11 +1051,11 @@ __global__ __launch_bounds__(256) void WarpTensor(const WarpArgs a)
     {
         m[i] = a.m[i];
     }
-    WarpTile<T, C, INTERP>(im, a, m, a.dst + n * a.dstN, a.dstRow, a.dstW, a.dstH, blockIdx.x, blockIdx.y);
+    WarpTile<T, C, INTERP, PERSP>(im, a, m, a.dst + n * a.dstN, a.dstRow, a.dstW, a.dstH, blockIdx.x, blockIdx.y);
 }
 
-template<class T, int C, int INTERP>
-__global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarTiles tiles)
+template<class T, int C, int INTERP, bool PERSP>
+__global__ __launch_bounds__(kThreads) void WarpVarShape(const WarpArgs a, const VarTiles tiles)
 {
     const TileCoord tc = LocateTile(tiles, blockIdx.x);
     // descriptors and matrix depend on the image index only: read by value here, ahead of the matrix
@@ -711,18 +1063,18 @@ __global__ __launch_bounds__(256) void WarpVarShape(const WarpArgs a, const VarT
     const NVCVImagePlaneStrided s = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided d = a.dstList[tc.image].planes[0];
     float                       m[9];
-    LoadMatrix(a, tc.image, m);
+    LoadMatrix<PERSP>(a, tc.image, kCoordScale<T, INTERP>, m);
     const Img im = {AsGlobal(s.basePtr), s.rowStride, s.width, s.height};
-    WarpTile<T, C, INTERP>(im, a, m, AsGlobal(d.basePtr), d.rowStride, d.width, d.height, tc.tx, tc.ty);
+    WarpTile<T, C, INTERP, PERSP>(im, a, m, AsGlobal(d.basePtr), d.rowStride, d.width, d.height, tc.tx, tc.ty);
 }
 
-template<class T, int C, int INTERP>
-void Launch(const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
+template<class T, int C, int INTERP, bool PERSP>
+void LaunchMap(const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
 {
     if (dstHost == nullptr)
     {
         dim3 grid(DivUp(a.dstW, kTileW), DivUp(a.dstH, kTileH), N);
-        hipLaunchKernelGGL((WarpTensor<T, C, INTERP>), grid, dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((WarpTensor<T, C, INTERP, PERSP>), grid, dim3(kThreads), 0, stream, a);
         CheckLaunch("WarpTensor");
         return;
     }
@@ -732,9 +1084,22 @@ void Launch(const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hip
         int      total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first), kTileW, kTileH);
         if (total > 0)
         {
-            hipLaunchKernelGGL((WarpVarShape<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a, tiles);
+            hipLaunchKernelGGL((WarpVarShape<T, C, INTERP, PERSP>), dim3(total), dim3(kThreads), 0, stream, a, tiles);
             CheckLaunch("WarpVarShape");
         }
+    }
+}
+
+template<class T, int C, int INTERP>
+void Launch(const WarpArgs &a, int N, const NVCVImageBufferStrided *dstHost, hipStream_t stream)
+{
+    if (a.perspective)
+    {
+        LaunchMap<T, C, INTERP, true>(a, N, dstHost, stream);
+    }
+    else
+    {
+        LaunchMap<T, C, INTERP, false>(a, N, dstHost, stream);
     }
 }
 
@@ -904,6 +1269,13 @@ public:
         else
         {
             InvertAffineHost(xform, a.m);
+        }
+        if (in.elem == kU8 && (flags & NVCV_INTERP_MAX) == NVCV_INTERP_LINEAR)
+        {
+            for (int i = 0; i < 6; ++i)
+            {
+                a.m[i] *= kCoordScale<uint8_t, NVCV_INTERP_LINEAR>; // see kCoordScale
+            }
         }
         a.src    = in.base;
         a.dst    = out.base;

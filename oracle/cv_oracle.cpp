@@ -761,6 +761,22 @@ inline void CubicCoeffsDevice(float d, float *w)
     w[3] = 1 - w[0] - w[1] - w[2];
 }
 
+// Catmull-Rom weights times `scale` (a power of two), polynomials by fused multiply-adds: what the product
+// library's 8-bit bicubic warp evaluates before it quantises the horizontal weights.
+inline void CubicCoeffsFused(float d, float scale, float *w)
+{
+    w[0] = std::fmaf(-.5f * scale, d, scale);
+    w[0] = std::fmaf(w[0], d, -.5f * scale);
+    w[0] = w[0] * d;
+    w[1] = std::fmaf(1.5f * scale, d, -2.5f * scale);
+    w[1] = w[1] * d;
+    w[1] = std::fmaf(w[1], d, scale);
+    w[2] = std::fmaf(-1.5f * scale, d, 2.f * scale);
+    w[2] = std::fmaf(w[2], d, .5f * scale);
+    w[2] = w[2] * d;
+    w[3] = scale - w[0] - w[1] - w[2];
+}
+
 template<class T>
 void WarpOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_t dstStep, int dstW, int dstH, int C,
              const float *m, int perspective, int interp, int border, const float *bval, int variant)
@@ -815,10 +831,30 @@ void WarpOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_t 
             {
                 int x1 = (int)std::floor(sx), y1 = (int)std::floor(sy);
                 int x2 = x1 + 1, y2 = y1 + 1;
+                if (variant == 2 && std::is_same_v<T, uint8_t>)
+                {
+                    // the product library's 8-bit arithmetic: 15-bit fractions, four integer weights that
+                    // add up to 2^15, an exact integer sum, one rounding to nearest-even
+                    auto frac = [](float v) -> uint32_t
+                    {
+                        float f = v - std::floor(v);
+                        return f >= 0.f ? (uint32_t)(int)(f * 32768.f) : 0u;
+                    };
+                    uint32_t ax = frac(sx), ay = frac(sy);
+                    uint32_t w11 = (ax * ay + 16384u) >> 15, w01 = ax - w11, w10 = ay - w11,
+                             w00 = 32768u - ax - ay + w11;
+                    for (int k = 0; k < C; ++k)
+                    {
+                        uint32_t s = (uint32_t)pix(y1, x1, k) * w00 + (uint32_t)pix(y1, x2, k) * w01
+                                   + (uint32_t)pix(y2, x1, k) * w10 + (uint32_t)pix(y2, x2, k) * w11;
+                        out[k] = (T)((s + 16383u + ((s >> 15) & 1u)) >> 15);
+                    }
+                    continue;
+                }
                 for (int k = 0; k < C; ++k)
                 {
                     float o = 0;
-                    if (variant == 0)
+                    if (variant == 0 || variant == 2)
                     {
                         o += pix(y1, x1, k) * ((x2 - sx) * (y2 - sy));
                         o = o + pix(y1, x2, k) * ((sx - x1) * (y2 - sy));
@@ -845,6 +881,36 @@ void WarpOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_t 
                         o += (float)pix(y2, x2, k) * (sx - x1) * (sy - y1);
                         out[k] = SatF<T>(o);
                     }
+                }
+            }
+            else if (variant == 2 && std::is_same_v<T, uint8_t>)
+            {
+                // the product library's 8-bit bicubic: horizontal weights rounded to multiples of 2^-14 (the
+                // last takes the remainder), exact integer row sums, float32 vertical sum with fused
+                // multiply-adds, one rounding to nearest-even
+                int   ix = (int)std::floor(sx), iy = (int)std::floor(sy);
+                float wx[4], wy[4];
+                CubicCoeffsFused(sx - std::floor(sx), 16384.f, wx);
+                CubicCoeffsFused(sy - std::floor(sy), 1.f / 16384.f, wy);
+                int wq[4];
+                for (int i = 0; i < 3; ++i)
+                {
+                    wq[i] = wx[i] == wx[i] ? (int)std::nearbyint(wx[i]) : 0;
+                }
+                wq[3] = 16384 - wq[0] - wq[1] - wq[2];
+                for (int k = 0; k < C; ++k)
+                {
+                    float acc = 0;
+                    for (int cy = 0; cy < 4; ++cy)
+                    {
+                        int h = 0;
+                        for (int cx = 0; cx < 4; ++cx)
+                        {
+                            h += (int)pix(iy + cy - 1, ix + cx - 1, k) * wq[cx];
+                        }
+                        acc = cy == 0 ? (float)h * wy[0] : std::fmaf((float)h, wy[cy], acc);
+                    }
+                    out[k] = SatF<T>(acc);
                 }
             }
             else if (variant == 0)

@@ -65,6 +65,10 @@ def cases():
             m = orc.invert_affine([0.9, -0.3, 6.0, 0.25, 1.1, -4.0])
             out["warp_affine_%s_border%d" % (nm, border)] = orc.warp(a, (30, 44), m, interp, border, (7, 8, 9, 0), False,
                                                                     variant=0)
+    for border in range(5):
+        # the shipped 8-bit bilinear blend (15-bit fixed point), which the kernels must reproduce bit for bit
+        out["warp_affine_linear_fixed_border%d" % border] = orc.warp(a, (30, 44), m, LINEAR, border, (7, 8, 9, 0), False,
+                                                                    variant=2)
     out["convert_u8_to_f32"] = orc.convert_to(recipe(1, 5, 7, 3), np.float32, 1 / 255.0, 0.0, 0)
     out["convert_f32_to_u8"] = orc.convert_to(recipe(1, 5, 7, 3, np.float32) * 300 - 20, np.uint8, 1.0, 0.5, 0)
     img = recipe(1, 20, 28, 3, step=5)[0]

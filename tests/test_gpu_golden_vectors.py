@@ -117,7 +117,9 @@ def test_warp_affine(cv, orc, gold, gpu):
             out = cv.Tensor.alloc([2, 30, 44, 3], np.uint8, "NHWC")
             cv.WarpAffine(0)(None, tin, out, fwd, INTERP[nm], border, (7, 8, 9, 0))
             torch.cuda.synchronize()
-            close(out.numpy(), vec["warp_affine_%s_border%d" % (nm, border)], lsb=1 if nm == "cubic" else 0)
+            close(out.numpy(), vec["warp_affine_%s_border%d" % (nm, border)], lsb=0 if nm == "nearest" else 1)
+            if nm == "linear":
+                close(out.numpy(), vec["warp_affine_linear_fixed_border%d" % border])
 
 
 def test_convert_and_crop_flip_normalize(cv, K, gold, gpu):

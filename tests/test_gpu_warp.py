@@ -1,11 +1,13 @@
 """GPU parity of cvcudaWarpAffine / cvcudaWarpPerspective [VarShape] Submit.
 
-Exact-equality rows: the reference's table on tiny RGBA8 images with small integer matrices, all
-five borders, three interpolations, forward and inverse maps
+Exact-equality rows: the reference's table on tiny RGBA8 images with small integer and quarter-step
+matrices, all five borders, three interpolations, forward and inverse maps
 (tests/cvcuda/system/TestOpWarpAffine.cpp:232-319). Random rotations/scales: <= 1 LSB against the
 reference's golden (oracle variant 0) and bit-exact against the restatement of this build's device
-arithmetic: oracle variant 1 for NEAREST and CUBIC; for LINEAR the kernels evaluate the bilinear sum in
-the golden's own association, so variant 0 IS the device arithmetic and integer results equal the golden. BASELINE configuration 4 at full size."""
+arithmetic: oracle variant 1 for NEAREST and CUBIC; on 8-bit pixels LINEAR is the 15-bit fixed-point blend
+and CUBIC the 14-bit one (oracle variant 2); the bilinear one equals the golden wherever the weights are
+dyadic (every row of the reference's table); LINEAR on the other types evaluates the bilinear sum in the
+golden's own association, so variant 0 IS the device arithmetic there. BASELINE configuration 4 at full size."""
 import itertools
 
 import numpy as np
@@ -17,8 +19,14 @@ NEAREST, LINEAR, CUBIC = 0, 1, 2
 INVERSE_MAP = 16
 
 
-def device_variant(interp):
+def device_variant(interp, dtype=np.uint8):
+    if interp != NEAREST and np.dtype(dtype) == np.uint8:
+        return 2
     return 0 if interp == LINEAR else 1
+
+
+def dyadic(values, bits=7):
+    return all(float(v * (1 << bits)).is_integer() for v in values)
 
 SIZES = [(5, 4, 5, 4), (5, 4, 6, 8), (7, 8, 4, 5)]
 MATS = [(1, 0, 0, 0, 1, 0), (1, 0, 1, 0, 1, 2), (1, 2, 1, 2, 1, 2), (2, 2, 1, 3, 1, 2), (1, 2, 0, 1, 1, 0),
@@ -44,7 +52,8 @@ def test_reference_table_exact(cv, orc, gpu, interp, border):
         dev = orc.warp(src, (dh, dw), minv, interp, border, (1, 2, 3, 4), variant=device_variant(interp))
         np.testing.assert_array_equal(res, dev, err_msg=str((sw, sh, dw, dh, m, inv)))
         gold = orc.warp(src, (dh, dw), minv, interp, border, (1, 2, 3, 4), variant=0)
-        exact = interp != CUBIC and all(float(v).is_integer() for v in minv)
+        # LINEAR weights that are multiples of 2^-7 per axis are exact in the fixed-point blend as in float32
+        exact = interp != CUBIC and dyadic(minv)
         tol = 0 if exact else 1
         assert np.abs(res.astype(np.int16) - gold.astype(np.int16)).max() <= tol, (sw, sh, dw, dh, m, inv)
 
@@ -73,7 +82,7 @@ def test_random_rotations_tensor(cv, orc, gpu, dt, c, interp):
         torch.cuda.synchronize()
         res = tout.numpy()
         minv = orc.invert_affine(m)
-        dev = orc.warp(src, (80, 150), minv, interp, border, (9, 8, 7, 6), variant=device_variant(interp))
+        dev = orc.warp(src, (80, 150), minv, interp, border, (9, 8, 7, 6), variant=device_variant(interp, dt))
         if dt == np.float32:
             assert np.abs(res - dev).max() <= 1e-3
         else:
@@ -112,8 +121,9 @@ def test_config4_varshape_full_size(cv, K, orc, gpu):
         minv = orc.invert_affine(mats[i])
         gold = orc.warp(a[None], a.shape[:2], minv, LINEAR, 0, (0, 0, 0, 0), variant=0, threads=1)[0]
         assert np.abs(res.astype(np.int16) - gold.astype(np.int16)).max() <= 1
+        assert (res != gold).mean() < 0.02  # the fixed-point blend rounds differently on about 1 % of the bytes
         if i < 4:
-            dev = orc.warp(a[None], a.shape[:2], minv, LINEAR, 0, (0, 0, 0, 0), variant=0)[0]
+            dev = orc.warp(a[None], a.shape[:2], minv, LINEAR, 0, (0, 0, 0, 0), variant=2)[0]
             np.testing.assert_array_equal(res, dev)
 
 
@@ -187,7 +197,7 @@ def test_warp_perspective(cv, K, orc, gpu):
     mats = np.asarray([H, H], np.float32)
     op(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), LINEAR | INVERSE_MAP, 1, (0, 0, 0, 0))
     torch.cuda.synchronize()
-    ref = orc.warp(src, (50, 90), H, LINEAR, 1, perspective=True, variant=0)
+    ref = orc.warp(src, (50, 90), H, LINEAR, 1, perspective=True, variant=2)
     for i in range(2):
         np.testing.assert_array_equal(outs[i].plane_view(0, np.uint8, 3).cpu().numpy(), ref[i])
 

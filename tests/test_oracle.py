@@ -298,6 +298,102 @@ def test_warp_identity_translation_borders_rotation(orc):
     np.testing.assert_allclose(got, 0.5 * (f[0, :, :-1, 0] + f[0, :, 1:, 0]), rtol=0, atol=1e-6)
 
 
+def _bilinear_float64(src, out_hw, m, border_value=0.0):
+    """Bilinear sample of src[H,W,C] at the float32 coordinates of the warp, everything after the coordinates
+    in float64 with exact weights; taps outside the image take border_value. Returns the unrounded sums."""
+    h, w = out_hw
+    m = np.asarray(m, np.float32)
+    xs, ys = np.meshgrid(np.arange(w, dtype=np.float32), np.arange(h, dtype=np.float32))
+    sx = (m[0] * xs + m[1] * ys + m[2]).astype(np.float64)  # float32 products and sums, as the operator forms them
+    sy = (m[3] * xs + m[4] * ys + m[5]).astype(np.float64)
+    x1, y1 = np.floor(sx).astype(np.int64), np.floor(sy).astype(np.int64)
+    fx, fy = sx - x1, sy - y1
+    H, W, C = src.shape
+    pad = np.full((H + 2, W + 2, C), float(border_value))
+    pad[1:-1, 1:-1] = src
+
+    def tap(x, y):
+        return pad[np.clip(y + 1, 0, H + 1), np.clip(x + 1, 0, W + 1)]
+
+    return (tap(x1, y1) * ((1 - fx) * (1 - fy))[..., None] + tap(x1 + 1, y1) * (fx * (1 - fy))[..., None]
+            + tap(x1, y1 + 1) * ((1 - fx) * fy)[..., None] + tap(x1 + 1, y1 + 1) * (fx * fy)[..., None])
+
+
+def test_warp_linear_fixed_point_variant(orc):
+    # variant 2 (8-bit pixels: 15-bit fractions, four integer weights that add up to 2^15, one rounding) against
+    # an exact float64 bilinear sum at the same float32 coordinates: its unrounded sum may be off by at most
+    # 4 * 255 * 2^-15 < 0.032, so it must give round(exact) wherever exact is further than that from a tie and
+    # never be more than 1 away; and against the golden (variant 0): at most 1 apart, rarely different
+    rng = np.random.default_rng(12)
+    src = rng.integers(0, 256, (1, 61, 83, 3), dtype=np.uint8)
+    t = np.deg2rad(21.0)
+    fwd = [1.1 * np.cos(t), -1.1 * np.sin(t), 7.3, 1.1 * np.sin(t), 1.1 * np.cos(t), -11.9]
+    m = orc.invert_affine(fwd)
+    got = orc.warp(src, (70, 90), m, LINEAR, border=0, border_value=(5, 5, 5, 0), variant=2)[0].astype(np.int64)
+    exact = _bilinear_float64(src[0].astype(np.float64), (70, 90), m, 5.0)
+    assert np.abs(got - exact).max() <= 0.5 + 0.032
+    clear = np.abs(exact - np.floor(exact) - 0.5) > 0.04
+    np.testing.assert_array_equal(got[clear], np.rint(exact[clear]).astype(np.int64))
+    assert clear.mean() > 0.9
+    gold = orc.warp(src, (70, 90), m, LINEAR, border=0, border_value=(5, 5, 5, 0), variant=0)[0].astype(np.int64)
+    assert np.abs(got - gold).max() <= 1 and (got != gold).mean() < 0.02
+    # dyadic weights (quarter-step maps, as in the reference's table): nothing is rounded before the final
+    # rounding, ties go to even as in the golden -> bit-equal, all borders
+    for border in range(5):
+        for mm in ([1, 0, 0.25, 0, 1, 0.75], [0.5, 0, 0.5, 0.25, 1, -2.5], [1, 0.75, -3, 0.5, 1, 1]):
+            a = orc.warp(src, (50, 70), mm, LINEAR, border=border, border_value=(1, 2, 3, 4), variant=2)
+            b = orc.warp(src, (50, 70), mm, LINEAR, border=border, border_value=(1, 2, 3, 4), variant=0)
+            np.testing.assert_array_equal(a, b)
+    # ties: a half-pixel shift of a two-column image whose neighbours differ by an odd number rounds to even
+    pair = np.array([[[[2], [5], [4], [7]]]], np.uint8)  # means 3.5, 4.5, 5.5 -> 4, 4, 6
+    got = orc.warp(pair, (1, 3), [1, 0, 0.5, 0, 1, 0], LINEAR, border=1, variant=2)[0, 0, :, 0]
+    np.testing.assert_array_equal(got, [4, 4, 6])
+    # other element types keep the float32 sum of variant 0
+    s16 = rng.integers(-3000, 3000, (1, 20, 30, 1)).astype(np.int16)
+    np.testing.assert_array_equal(orc.warp(s16, (20, 30), m, LINEAR, variant=2), orc.warp(s16, (20, 30), m, LINEAR, variant=0))
+
+
+def test_warp_cubic_fixed_point_variant(orc):
+    # variant 2 for CUBIC on 8-bit pixels: horizontal Catmull-Rom weights rounded to 2^-14 (sum exactly 1), exact
+    # integer row sums, float32 vertical sum. Against a float64 evaluation of the same 16-tap sum with the exact
+    # Catmull-Rom polynomials: the unrounded values differ by < 0.06, so the results agree wherever the exact value
+    # is that far from a tie, and never differ by more than 1
+    rng = np.random.default_rng(13)
+    src = rng.integers(0, 256, (1, 40, 52, 3), dtype=np.uint8)
+    t = np.deg2rad(-14.0)
+    m = orc.invert_affine([0.93 * np.cos(t), -0.93 * np.sin(t), 3.7, 0.93 * np.sin(t), 0.93 * np.cos(t), 1.2])
+    got = orc.warp(src, (44, 56), m, CUBIC, border=1, variant=2)[0].astype(np.int64)
+    m32 = np.asarray(m, np.float32)
+    xs, ys = np.meshgrid(np.arange(56, dtype=np.float32), np.arange(44, dtype=np.float32))
+    sx = (m32[0] * xs + m32[1] * ys + m32[2]).astype(np.float64)
+    sy = (m32[3] * xs + m32[4] * ys + m32[5]).astype(np.float64)
+
+    def catmull_rom(d):  # weights of taps -1, 0, 1, 2 at fraction d (A = -0.5)
+        return np.stack([((-0.5 * d + 1.0) * d - 0.5) * d, (1.5 * d - 2.5) * d * d + 1.0,
+                         ((-1.5 * d + 2.0) * d + 0.5) * d, (0.5 * d - 0.5) * d * d])
+
+    ix, iy = np.floor(sx).astype(np.int64), np.floor(sy).astype(np.int64)
+    wx, wy = catmull_rom(sx - ix), catmull_rom(sy - iy)
+    img = src[0].astype(np.float64)
+    exact = np.zeros((44, 56, 3))
+    for j in range(4):
+        for i in range(4):
+            tap = img[np.clip(iy + j - 1, 0, 39), np.clip(ix + i - 1, 0, 51)]  # replicate border
+            exact += tap * (wx[i] * wy[j])[..., None]
+    want = np.clip(np.rint(exact), 0, 255).astype(np.int64)
+    assert np.abs(got - np.clip(exact, 0, 255)).max() <= 0.5 + 0.06
+    clear = np.abs(exact - np.floor(exact) - 0.5) > 0.07
+    np.testing.assert_array_equal(got[clear], want[clear])
+    assert clear.mean() > 0.8
+    dev = orc.warp(src, (44, 56), m, CUBIC, border=1, variant=1)[0].astype(np.int64)
+    assert np.abs(got - dev).max() <= 1 and (got != dev).mean() < 0.05
+    # whole-pixel translation: weights (0, 1, 0, 0) on both axes -> a shifted copy; a constant image stays constant
+    sh = orc.warp(src, (40, 52), [1, 0, 2, 0, 1, -3], CUBIC, border=3, variant=2)[0]
+    np.testing.assert_array_equal(sh, np.roll(src[0], (3, -2), axis=(0, 1)))
+    const = np.full((1, 20, 20, 1), 201, np.uint8)
+    assert (orc.warp(const, (20, 20), m, CUBIC, border=1, variant=2) == 201).all()
+
+
 def test_warp_cubic_golden_vs_device_and_perspective(orc):
     rng = np.random.default_rng(9)
     src = rng.integers(0, 256, (2, 20, 24, 3), dtype=np.uint8)
