@@ -780,7 +780,7 @@ class Streaming:
             return orc.convert_to(a, np.float32, 1.0 / 255.0, 0.0, 1)
         if self.opname == "Flip":
             return np.ascontiguousarray(a[:, :, ::-1])
-        return orc.resize(a, (self.dh, self.dw), self.INTERP.get(self.key, LINEAR), variant=1, threads=threads)
+        return orc.resize_shipped(a, (self.dh, self.dw), self.INTERP.get(self.key, LINEAR), threads=threads)
 
     def check(self, s):
         got = s[1].torch_view()[:1].cpu().numpy()

@@ -25,6 +25,7 @@
 // patches" into "4 consecutive pixels of one row in one patch", which the lane writes as whole dwords;
 // single-byte stores scattered over 8 rows are several times slower.
 #include "DeviceUtils.hpp"
+#include "FixedPointBlend.hpp"
 #include "LaneExchange.hpp"
 #include "OpCommon.hpp"
 #include "VarShapeTiles.hpp"
@@ -126,18 +127,9 @@ __device__ __forceinline__ int FloorToInt(float v)
     return (int)fminf(fmaxf(floorf(v), -1073741824.f), 1073741824.f);
 }
 
-// ---- u8 bilinear in 15-bit fixed point ---------------------------------------------------------------
-// For 8-bit pixels the bilinear blend runs on integers: the fractions of the source coordinate are cut
-// to 15 bits (ax = trunc(fx * 2^15), fx = sx - floor(sx) in float32), the four weights are integers that
-// add up to exactly 2^15,
-//     w11 = (ax * ay + 2^14) >> 15,  w01 = ax - w11,  w10 = ay - w11,  w00 = 2^15 - ax - ay + w11,
-// the weighted sum of the four taps is exact in 24 bits and is rounded to nearest, ties to even, once.
-// Each weight is within 2^-15 of the product the float32 expression of the reference forms, so the
-// unrounded sum is within 4 * 255 * 2^-15 < 0.032 of it: results differ from the reference's golden by
-// at most 1 and agree with it wherever the weights are multiples of 2^-7 per axis (integer and
-// quarter-step maps, which is what the reference's own exact-equality table uses), because then nothing
-// is rounded before the final rounding. What it buys: the taps stay bytes (two taps and two weights per
-// v_dot2_u32_u16 instead of a conversion, a multiply and an add per tap and channel in float32).
+// 8-bit bilinear: the blend of FixedPointBlend.hpp; the fractions are ax = trunc(fx * 2^15) with
+// fx = sx - floor(sx) in float32. Integer and quarter-step maps (the reference's own exact-equality table)
+// give weights that are exact in both arithmetics, hence the same results as the reference's golden.
 template<class T, int INTERP>
 constexpr bool kFixedPoint = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_LINEAR;
 
@@ -149,45 +141,11 @@ constexpr bool kFixedPoint = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP
 template<class T, int INTERP>
 constexpr bool kFixedPointCubic = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_CUBIC;
 
-constexpr uint32_t kQ15 = 32768u;
-
 // The kernels that blend in fixed point work on coordinates in units of 2^-15 pixel: the first two rows
 // of their destination -> source matrix arrive multiplied by 2^15 (exact: a power of two), so floor and
 // fraction of a coordinate are the two halves of one float -> integer conversion.
 template<class T, int INTERP>
 constexpr float kCoordScale = kFixedPoint<T, INTERP> ? 32768.f : 1.f;
-
-// (w00 | w01 << 16) and (w10 | w11 << 16) from the two 15-bit fractions (each 0 .. 2^15).
-__device__ __forceinline__ void WeightPairsQ15(uint32_t ax, uint32_t ay, uint32_t &top, uint32_t &bottom)
-{
-    const uint32_t w11 = (__umul24(ax, ay) + (kQ15 >> 1)) >> 15;
-    bottom             = __umul24(w11, 65535u) + ay;          // (ay - w11) | w11 << 16
-    top                = (__umul24(ax, 65535u) + kQ15) - bottom; // (2^15 - ax | ax << 16) - bottom: no borrow
-}
-
-// Weighted sum of one channel: tap pairs as (left | right << 16), result in units of 2^-15, rounded to
-// nearest-even, saturated (never needed) and placed into byte `c` of q. The sum is accumulated on top
-// of the bit pattern of 256.0f, whose unit in the last place is 2^-15: read as a float the register
-// then holds 256 + sum / 2^15 exactly.
-__device__ __forceinline__ uint32_t BlendQ15(uint32_t topTaps, uint32_t bottomTaps, uint32_t top, uint32_t bottom, int c,
-                                             uint32_t q)
-{
-    typedef unsigned short U16x2 __attribute__((ext_vector_type(2)));
-    U16x2 t0, t1, w0, w1;
-    __builtin_memcpy(&t0, &topTaps, 4);
-    __builtin_memcpy(&t1, &bottomTaps, 4);
-    __builtin_memcpy(&w0, &top, 4);
-    __builtin_memcpy(&w1, &bottom, 4);
-    uint32_t acc = __builtin_amdgcn_udot2(t0, w0, 0x43800000u, false);
-    acc          = __builtin_amdgcn_udot2(t1, w1, acc, false);
-    return __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(acc) - 256.f, c, q);
-}
-
-// The same sum in plain integer arithmetic (border path, one tap at a time).
-__device__ __forceinline__ uint8_t RoundQ15(uint32_t sum)
-{
-    return (uint8_t)((sum + (kQ15 / 2 - 1) + ((sum >> 15) & 1u)) >> 15);
-}
 
 // floor and 15-bit fraction of a coordinate; NaN and infinite coordinates give fraction 0
 __device__ __forceinline__ uint32_t FractionQ15(float v)

@@ -490,7 +490,32 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                     out[c]     = (T)(res < lo ? lo : (res > hi ? hi : res));
                 }
             }
-            else if (interp == 1 && variant == 1)
+            else if (interp == 1 && variant == 4 && std::is_same_v<T, uint8_t>)
+            {
+                // the product library's 8-bit bilinear resize: indices and weights of the device formula, the
+                // weights cut to multiples of 2^-15, four integer weights that add up to 2^15, an exact integer
+                // sum, one rounding to nearest-even
+                float fy = (dy + .5f) * scaleH - .5f;
+                float fx = (dx + .5f) * scaleW - .5f;
+                int   sy = (int)std::floor(fy);
+                int   sx = (int)std::floor(fx);
+                float wyv = (sy < 0) ? 0.f : ((sy > srcH - 2) ? 1.f : fy - sy);
+                float wxv = (sx < 0) ? 0.f : ((sx > srcW - 2) ? 1.f : fx - sx);
+                sy        = std::max(0, std::min(sy, srcH - 2));
+                sx        = std::max(0, std::min(sx, srcW - 2));
+                uint32_t ax = (uint32_t)(wxv * 32768.f), ay = (uint32_t)(wyv * 32768.f);
+                uint32_t w11 = (ax * ay + 16384u) >> 15, w01 = ax - w11, w10 = ay - w11, w00 = 32768u - ax - ay + w11;
+                for (int c = 0; c < C; ++c)
+                {
+                    uint32_t p00 = src[tapY(sy) * srcStep + (int64_t)tapX(sx) * C + c];
+                    uint32_t p01 = src[tapY(sy) * srcStep + (int64_t)tapX(sx + 1) * C + c];
+                    uint32_t p10 = src[tapY(sy + 1) * srcStep + (int64_t)tapX(sx) * C + c];
+                    uint32_t p11 = src[tapY(sy + 1) * srcStep + (int64_t)tapX(sx + 1) * C + c];
+                    uint32_t s   = p00 * w00 + p01 * w01 + p10 * w10 + p11 * w11;
+                    out[c]       = (T)((s + 16383u + ((s >> 15) & 1u)) >> 15);
+                }
+            }
+            else if (interp == 1 && (variant == 1 || variant == 4))
             {
                 float fy = (dy + .5f) * scaleH - .5f;
                 float fx = (dx + .5f) * scaleW - .5f;

@@ -78,6 +78,17 @@ def resize(src, out_hw, interp, variant=0, threads=1):
     return dst
 
 
+def resize_shipped(src, out_hw, interp, varshape=False, threads=1):
+    """The restatement of what the product library's Resize computes for this element type and interpolation:
+    8-bit bilinear is the fixed-point blend (variant 4) for tensors and image batches alike; everything else is
+    the reference's device formula (variant 1; variant 2, its image-batch association, with varshape)."""
+    if int(interp) == 1 and np.dtype(src.dtype) == np.uint8:
+        variant = 4
+    else:
+        variant = 2 if varshape else 1
+    return resize(src, out_hw, interp, variant=variant, threads=threads)
+
+
 def yuv420_to_rgb(src, dcn=3, bgr=False, uidx=0, semi_planar=True, variant=0, threads=1):
     """src: [N, H*3/2, W] u8 (or with a trailing 1); returns [N,H,W,dcn] u8."""
     src = np.ascontiguousarray(src, dtype=np.uint8).reshape(src.shape[0], src.shape[1], src.shape[2])

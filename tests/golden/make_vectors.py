@@ -45,6 +45,9 @@ def cases():
                 # float images take the float32 restatement of the device formula instead
                 variant = 1 if dt == np.float32 and interp != NEAREST else 0
                 out["resize_%s_%s%d_%s" % (nm, np.dtype(dt).name, c, tag)] = orc.resize(a, hw, interp, variant=variant)
+                if interp == LINEAR and dt == np.uint8:
+                    # the shipped 8-bit bilinear blend (15-bit fixed point), to be reproduced bit for bit
+                    out["resize_linear_fixed_uint8%d_%s" % (c, tag)] = orc.resize(a, hw, interp, variant=4)
     y = recipe(2, 12, 16, 1, step=9)[..., 0] // 2 + 60
     uv = recipe(2, 6, 16, 1, step=13)[..., 0] // 2 + 60
     nv = np.concatenate([y, uv], axis=1)

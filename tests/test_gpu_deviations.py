@@ -113,7 +113,7 @@ def test_sources_narrower_than_the_tap_window_read_clamped_taps(cv, orc, gpu, in
         torch.cuda.synchronize()
         res = tout.numpy()
         assert np.abs(res.astype(np.int16) - 77).max() <= (0 if interp == LINEAR else 1), (h, w)
-        np.testing.assert_array_equal(res, orc.resize(src, (5, 6), interp, variant=1))
+        np.testing.assert_array_equal(res, orc.resize_shipped(src, (5, 6), interp))
 
 
 def test_crops_require_equal_batch_sizes_where_the_reference_reads_out_of_bounds(cv, gpu):

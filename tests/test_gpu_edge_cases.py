@@ -40,7 +40,7 @@ def test_one_pixel_and_one_row_images(cv, orc, gpu, dt, c):
             out = cv.Tensor.alloc([2, dh, dw, c], dt, "NHWC")
             cv.Resize()(None, cv.Tensor.from_numpy(src, "NHWC"), out, interp)
             torch.cuda.synchronize()
-            ref = orc.resize(src, (dh, dw), interp, variant=0 if interp == NEAREST else 1)
+            ref = orc.resize_shipped(src, (dh, dw), interp)
             got = out.numpy()
             if dt == np.float32:
                 assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max()), (sh, sw, dh, dw, interp)
@@ -278,7 +278,7 @@ def test_concurrent_submits_on_shared_operator_handles(cv, K, orc, gpu):
             torch.cuda.set_device(0)
             stream = torch.cuda.Stream()
             src = orc.fill_u8((2, 45 + tid, 70 + 3 * tid, 3), 700 + tid)
-            want_small = orc.resize(src, (23, 31), LINEAR, variant=1)
+            want_small = orc.resize_shipped(src, (23, 31), LINEAR)
             want_fused = orc.fused_rccr(src, (16, 16), (32, 24), (5, 3), LINEAR, np.float32, True, 0, 1 / 255.0, 0.0, False)
             start.wait()
             for r in range(rounds):

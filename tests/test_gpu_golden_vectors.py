@@ -61,6 +61,8 @@ def test_resize(cv, gold, gpu, dt, c):
             cv.Resize()(None, tin, out, interp)
             torch.cuda.synchronize()
             got = out.numpy()
+            if interp == LINEAR and dt == np.uint8:
+                close(got, vec["resize_linear_fixed_uint8%d_%s" % (c, tag)])
             if interp == NEAREST:
                 close(got, want)
             elif dt == np.float32:

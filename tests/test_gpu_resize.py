@@ -3,8 +3,8 @@
 Rows are the reference's own table (tests/cvcuda/system/TestOpResize.cpp:49-91)
 with seeded random inputs, plus the two benchmark configurations at full size.
 Bars: NEAREST bit-exact vs the golden; LINEAR/CUBIC on integer types <= 1 LSB vs the golden (the
-reference's own tolerance) and bit-exact vs the float32 device-formula restatement; f32 cubic
-within 1e-4 of that restatement.
+reference's own tolerance) and bit-exact vs the restatement of the shipped arithmetic (the float32 device
+formula; for 8-bit LINEAR the 15-bit fixed-point blend, oracle variant 4); f32 cubic within 1e-4 of it.
 """
 import ctypes as C
 
@@ -25,7 +25,7 @@ def make_input(orc, shape, dtype, seed):
 
 def check(res, src, out_hw, interp, orc, varshape=False):
     golden = orc.resize(src, out_hw, interp, variant=0)
-    device = orc.resize(src, out_hw, interp, variant=2 if varshape else 1)
+    device = orc.resize_shipped(src, out_hw, interp, varshape)
     if interp == NEAREST:
         np.testing.assert_array_equal(res, golden)
     elif res.dtype == np.float32:
@@ -40,7 +40,7 @@ def check(res, src, out_hw, interp, orc, varshape=False):
             # rounding (width * 2^-24 pixels) times the sample range exceeds 1 LSB on wide sources.
             lsb = 1 if res.dtype.itemsize == 1 else 1 + int(np.ceil(max(src.shape[1:3]) * 2.0 ** -24 * 65536 * 2))
             assert np.abs(res.astype(np.int64) - golden.astype(np.int64)).max() <= lsb
-        # no FMA contraction on either side: the device-formula restatement is reproduced exactly
+        # no FMA contraction on either side (integers for 8-bit LINEAR): the restatement is reproduced exactly
         np.testing.assert_array_equal(res, device)
 
 
@@ -239,7 +239,7 @@ def test_area_sources_one_and_two_pixels_wide(cv, orc, gpu):
                 tout = cv.Tensor.alloc([2, dh, dw, 3], np.uint8, "NHWC")
                 cv.Resize()(None, cv.Tensor.from_numpy(src, "NHWC"), tout, interp)
                 torch.cuda.synchronize()
-                device = orc.resize(src, (dh, dw), interp, variant=0 if interp == NEAREST else 1)
+                device = orc.resize_shipped(src, (dh, dw), interp)
                 np.testing.assert_array_equal(tout.numpy(), device, err_msg=str((sw, sh, dw, dh, interp)))
 
 

@@ -319,6 +319,34 @@ def _bilinear_float64(src, out_hw, m, border_value=0.0):
             + tap(x1, y1 + 1) * ((1 - fx) * fy)[..., None] + tap(x1 + 1, y1 + 1) * (fx * fy)[..., None])
 
 
+def test_resize_linear_fixed_point_variant(orc):
+    # variant 4 (8-bit bilinear resize: weights cut to 2^-15, four integer weights that add up to 2^15, one
+    # rounding) against torch's bilinear interpolation in float64 (same half-pixel map and edge clamp): the unrounded
+    # sums differ by < 0.032 + the float32 coordinate error, so the results agree wherever the exact value is clear of
+    # a tie and never differ by more than 1; against the golden (variant 0): at most 1 apart, rarely different
+    rng = np.random.default_rng(14)
+    src = rng.integers(0, 256, (2, 37, 53, 3), dtype=np.uint8)
+    for out_hw in ((23, 31), (61, 90), (37, 53), (5, 200)):
+        got = orc.resize(src, out_hw, LINEAR, variant=4).astype(np.int64)
+        x = torch.from_numpy(src).permute(0, 3, 1, 2).double()
+        exact = F.interpolate(x, size=out_hw, mode="bilinear", align_corners=False, antialias=False)
+        exact = exact.permute(0, 2, 3, 1).numpy()
+        assert np.abs(got - exact).max() <= 0.5 + 0.04
+        clear = np.abs(exact - np.floor(exact) - 0.5) > 0.05
+        np.testing.assert_array_equal(got[clear], np.rint(exact[clear]).astype(np.int64))
+        gold = orc.resize(src, out_hw, LINEAR, variant=0).astype(np.int64)
+        assert np.abs(got - gold).max() <= 1 and (got != gold).mean() < 0.03
+    # same size: identity; 2x reduction: the mean of each 2 x 2 block, ties to even; a constant stays constant
+    np.testing.assert_array_equal(orc.resize(src, (37, 53), LINEAR, variant=4), src)
+    even = src[:, :36, :52].astype(np.int64)
+    blocks = even.reshape(2, 18, 2, 26, 2, 3).sum(axis=(2, 4))
+    np.testing.assert_array_equal(orc.resize(src[:, :36, :52], (18, 26), LINEAR, variant=4), np.rint(blocks / 4.0))
+    assert (orc.resize(np.full((1, 9, 11, 1), 131, np.uint8), (20, 7), LINEAR, variant=4) == 131).all()
+    # other element types keep the float32 sum of variant 1
+    u16 = rng.integers(0, 60000, (1, 20, 30, 1)).astype(np.uint16)
+    np.testing.assert_array_equal(orc.resize(u16, (11, 47), LINEAR, variant=4), orc.resize(u16, (11, 47), LINEAR, variant=1))
+
+
 def test_warp_linear_fixed_point_variant(orc):
     # variant 2 (8-bit pixels: 15-bit fractions, four integer weights that add up to 2^15, one rounding) against
     # an exact float64 bilinear sum at the same float32 coordinates: its unrounded sum may be off by at most
