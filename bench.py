@@ -3,8 +3,10 @@
 
 Default workload (the headline one): a step = one cvcudaResizeCropConvertReformatSubmit over a batch
 of 64 1080p u8 RGB images (bilinear resize to 455x256, centre crop 224x224, scale/offset, f32 NCHW
-output). `--workload` selects the other configurations (plain resize, NV12->RGB, var-shape affine warp,
-4K cubic resize); each is one Submit per step.
+output). With no `--workload` the other BASELINE configurations (plain resize nearest and bilinear, NV12->RGB,
+var-shape affine warp, 4K cubic resize) are timed after it, each the same way on a smaller budget, and reported
+under the extra key `configs` (one entry per configuration, the headline first); `--workload` times one
+workload only. Each is one Submit per step.
 
 Inputs are generated on the host from a fixed seed and uploaded before the timed region. To keep
 the reads coming from HBM rather than from the 256 MB on-die cache, consecutive steps cycle through
@@ -824,28 +826,161 @@ WORKLOADS.update({k: (lambda *a, k=k: Streaming(*a, k)) for k in Streaming.SPECS
 WORKLOADS.update({k: (lambda *a, k=k: StreamMix(*a, k)) for k in StreamMix.SPECS})
 
 
+# What each workload's dominant kernel is bound by, from its hardware counters (profiles/*_sq_counters.txt):
+# "hbm" unless named here. "valu-issue": the vector-ALU instructions of the launch take most of its time at one
+# wave-instruction per CU and cycle; "vmem-issue": the texture addresser is busy for most of the launch (gathers and
+# loads that are not dword aligned cost cache accesses, not bytes); "launch-latency": the launch floor plus one ramp
+# of memory latency is more than half of the time (batch 8).
+BOUNDS = {"warp-affine-varshape": "valu-issue", "warp-affine-tensor-linear": "valu-issue",
+          "warp-affine-tensor-cubic": "valu-issue", "warp-affine-tensor-nearest": "vmem-issue",
+          "resize-area-720p": "valu-issue", "cvtcolor-bgr2hsv": "valu-issue",
+          "resize-linear-720p": "vmem-issue", "resize-linear-upscale": "vmem-issue",
+          "resize-nearest": "launch-latency", "resize-linear": "launch-latency", "empty-launch": "launch-latency"}
+
+# The other BASELINE configurations, timed after the headline when no --workload is given.
+OTHER_CONFIGS = ("resize-nearest", "resize-linear", "nv12-to-rgb", "warp-affine-varshape", "resize-cubic-4k")
+MIN_GRAPH_LAUNCHES = 500
+
+
+def measure(wl, torch, steps, warmup, rotate, use_graph, streams, min_seconds):
+    """Times `wl` on the current device: `warmup` eager Submits, then a HIP graph of max(steps, 500) Submits
+    (so that what is timed does not depend on --steps: a graph of a few dozen launches pays a graph-launch gap
+    every few dozen kernels) replayed until the timed region holds at least `min_seconds` of device work.
+    Returns the buffer sets and the figures."""
+    nsets = rotate if rotate > 0 else max(3, math.ceil(1.5e9 / max(wl.alg_bytes, 1)) if wl.alg_bytes else 1)
+    sets = [wl.make_set() for _ in range(nsets)]
+    stream = torch.cuda.current_stream()
+    torch.cuda.synchronize()
+    for i in range(warmup):
+        wl.submit(stream, sets[i % nsets])
+    torch.cuda.synchronize()
+
+    # Default: the Submits are captured once into a HIP graph (a Submit only validates on the host and launches
+    # one kernel, so it is capturable) and the replay is timed; this keeps the Python call overhead (~10 us per
+    # Submit) out of a ~20 us kernel's way. --no-graph times eager Submits.
+    mode, graph = "eager", None
+    launches = max(steps, MIN_GRAPH_LAUNCHES) if use_graph else steps
+    if use_graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            sides = [torch.cuda.Stream() for _ in range(streams)] if streams > 1 else []
+            with torch.cuda.graph(graph):
+                cap = torch.cuda.current_stream()
+                for sd in sides:
+                    sd.wait_stream(cap)
+                for i in range(launches):
+                    wl.submit(sides[i % len(sides)] if sides else cap, sets[i % nsets])
+                for sd in sides:
+                    cap.wait_stream(sd)
+            graph.replay()  # untimed first replay
+            torch.cuda.synchronize()
+            mode = "hipgraph"
+        except Exception as e:  # capture unsupported -> measure eagerly and say so
+            sys.stderr.write("bench.py: graph capture failed (%s), timing eager submits\n" % e)
+            graph, launches = None, steps
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def run_once():
+        if graph is not None:
+            graph.replay()
+        else:
+            for i in range(launches):
+                wl.submit(stream, sets[i % nsets])
+
+    # One untimed pass sizes the timed region. With a few dozen steps of a ~20 us kernel the clocks would
+    # otherwise mostly see the host's launch and synchronisation latency, and the device would still be
+    # ramping its memory clocks up.
+    torch.cuda.synchronize()
+    e0.record(stream)
+    run_once()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    est_s = max(e0.elapsed_time(e1) * 1e-3, 1e-6)
+    replays = max(1, min(100000, math.ceil(min_seconds / est_s)))
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(replays):
+        run_once()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    timed = launches * replays
+    # mean launch-to-launch duration of a step on the device over the timed region: HIP events on the stream the
+    # kernels are launched on. Consecutive launches overlap the end of one kernel with the start of the next, so
+    # this can be a few tenths of a microsecond below the begin-to-end duration a kernel trace shows per kernel.
+    mean_kernel_ms = e0.elapsed_time(e1) / timed
+    return {"sets": sets, "nsets": nsets, "graph": graph, "mode": mode, "launches": launches, "replays": replays,
+            "timed": timed, "wall": wall, "mean_kernel_ms": mean_kernel_ms, "stream": stream}
+
+
+def cpu_baseline(wl, seconds, single_seconds):
+    """The CPU oracle on a bounded sample of the workload: all host threads (at most 16), then one thread."""
+    if seconds <= 0 or wl.images <= 0:
+        return None
+
+    def leg(threads, budget):
+        reps, done, tcpu = 0, 0, 0.0
+        c0 = time.perf_counter()
+        while reps < 2 or tcpu < budget:
+            done += wl.cpu(threads)
+            reps += 1
+            tcpu = time.perf_counter() - c0
+        return done, tcpu
+
+    threads = min(os.cpu_count() or 1, 16)
+    done, tcpu = leg(threads, seconds)
+    used = wl.cpu_cores(threads) if hasattr(wl, "cpu_cores") else threads
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
+    except OSError:
+        pass
+    cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": used, "kind": "port",
+           "host": {"cpu_model": model, "logical_cpus": os.cpu_count()},
+           "sample": "%d images of this workload through the CPU oracle in %.1f s, %d thread%s"
+                     % (done, tcpu, used, "" if used == 1 else "s")}
+    if single_seconds > 0:
+        done1, tcpu1 = leg(1, single_seconds)
+        cpu["single_thread"] = {"value": round(done1 / tcpu1, 1), "unit": "images/s", "cores": 1,
+                                "sample": "%d images in %.1f s, 1 thread" % (done1, tcpu1)}
+    return cpu
+
+
+def roofline_of(wl, mean_kernel_ms):
+    achieved = wl.alg_bytes / (mean_kernel_ms * 1e-3) / 1e9
+    return {"bound": BOUNDS.get(wl.key, "hbm"), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.key),
+            "kernel": wl.kernel, "kernel_ms_mean": round(mean_kernel_ms, 5),
+            "algorithmic_bytes_per_launch": wl.alg_bytes}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="fused")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
+                    help="one workload only (default: the headline, fused, followed by the other BASELINE "
+                         "configurations under the key `configs`)")
     ap.add_argument("--rotate", type=int, default=0,
                     help="distinct buffer sets cycled through (0 = at least 3 and enough for 1.5 GB of algorithmic bytes, 1 = cache-resident)")
     ap.add_argument("--no-graph", action="store_true", help="time eager Submits instead of a HIP-graph replay")
     ap.add_argument("--min-seconds", type=float, default=0.3,
-                    help="the K steps are repeated until the timed region holds at least this much device work")
+                    help="the captured launches are replayed until the timed region holds at least this much device work")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget of the CPU-oracle leg (0 = skip)")
     ap.add_argument("--batch", type=int, default=0,
                     help="images per step for the fused and resize-nearest / resize-linear workloads (0 = the "
                          "configuration's own batch size); for fits of launch time against batch size")
     ap.add_argument("--streams", type=int, default=1,
-                    help="independent streams the K steps are dealt to inside the captured graph (default 1: every "
+                    help="independent streams the steps are dealt to inside the captured graph (default 1: every "
                          "step waits for the one before, as consecutive Submits on one stream do)")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle spot check (kernel experiments only)")
     ap.add_argument("--no-mover", action="store_true",
                     help="skip the plain byte mover that the fused, nv12-to-rgb and resize-cubic-4k workloads time beside "
                          "the operator (roofline.dense_mover)")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="with no --workload: time the headline only, not the other BASELINE configurations")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="after the timed region, also run a plain device copy of this many MiB three times "
                          "(a kernel of known traffic to scale hardware byte counters against)")
@@ -853,6 +988,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (the path shards by batch with no exchange); "
                  "--gpus %d is not supported" % args.gpus)
+    all_configs = args.workload is None and not args.no_configs and args.batch == 0
+    if args.workload is None:
+        args.workload = "fused"
 
     import numpy as np
     import torch
@@ -875,71 +1013,9 @@ def main():
         else:
             sys.exit("bench.py: --batch applies to the fused and resize-nearest / resize-linear workloads")
     wl = WORKLOADS[args.workload](cv, orc, np, torch)
-    nsets = args.rotate if args.rotate > 0 else max(3, math.ceil(1.5e9 / max(wl.alg_bytes, 1)) if wl.alg_bytes else 1)
-    sets = [wl.make_set() for _ in range(nsets)]
-    stream = torch.cuda.current_stream()
-    torch.cuda.synchronize()
-
-    for i in range(args.warmup):
-        wl.submit(stream, sets[i % nsets])
-    torch.cuda.synchronize()
-
-    # ---- timed region: exactly K steps between two events on the launch stream.
-    # Default: the K Submits are captured once into a HIP graph (a Submit only validates on the host
-    # and launches one kernel, so it is capturable) and the replay is timed; this keeps the Python
-    # call overhead (~10 us per Submit) out of a ~20 us kernel's way. --no-graph times eager Submits.
-    mode = "eager"
-    graph = None
-    if not args.no_graph:
-        try:
-            graph = torch.cuda.CUDAGraph()
-            sides = [torch.cuda.Stream() for _ in range(args.streams)] if args.streams > 1 else []
-            with torch.cuda.graph(graph):
-                cap = torch.cuda.current_stream()
-                for sd in sides:
-                    sd.wait_stream(cap)
-                for i in range(args.steps):
-                    wl.submit(sides[i % len(sides)] if sides else cap, sets[i % nsets])
-                for sd in sides:
-                    cap.wait_stream(sd)
-            graph.replay()  # untimed first replay
-            torch.cuda.synchronize()
-            mode = "hipgraph"
-        except Exception as e:  # capture unsupported -> measure eagerly and say so
-            sys.stderr.write("bench.py: graph capture failed (%s), timing eager submits\n" % e)
-            graph = None
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-
-    def run_steps():
-        if graph is not None:
-            graph.replay()
-        else:
-            for i in range(args.steps):
-                wl.submit(stream, sets[i % nsets])
-
-    # One untimed pass sizes the timed region: the K steps are repeated `replays` times so that the timed
-    # region holds at least --min-seconds of device work whatever K is. With a few dozen steps of a ~20 us
-    # kernel the clocks would otherwise mostly see the host's launch and synchronisation latency, and the
-    # device would still be ramping its memory clocks up.
-    torch.cuda.synchronize()
-    e0.record(stream)
-    run_steps()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    est_s = max(e0.elapsed_time(e1) * 1e-3, 1e-6)
-    replays = max(1, min(100000, math.ceil(args.min_seconds / est_s)))
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for _ in range(replays):
-        run_steps()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall = t1 - t0
-    timed_steps = args.steps * replays
-    # mean launch-to-launch duration of a step on the device over the timed region (includes the gap between
-    # dependent launches, so it is an upper bound of the pure kernel time)
-    mean_kernel_ms = e0.elapsed_time(e1) / timed_steps
+    m = measure(wl, torch, args.steps, args.warmup, args.rotate, not args.no_graph, args.streams, args.min_seconds)
+    sets, nsets, graph, stream = m["sets"], m["nsets"], m["graph"], m["stream"]
+    mean_kernel_ms = m["mean_kernel_ms"]
 
     # One step from Submit to the end of its work, eagerly and one at a time: what a caller that waits for every
     # result sees (the Python call, the descriptor upload of image batches, the launch, the kernel, the wake-up).
@@ -959,7 +1035,7 @@ def main():
     if mover_key and not args.no_mover and graph is not None:
         mw = StreamMix(cv, orc, np, torch, mover_key)
         msets = [mw.make_set() for _ in range(max(3, int(math.ceil(2 * 268e6 / (16 * mw.lanes * mw.reads)))))]
-        msteps = min(args.steps, 500)
+        msteps = MIN_GRAPH_LAUNCHES
         for i in range(len(msets)):
             mw.submit(stream, msets[i])
         torch.cuda.synchronize()
@@ -996,57 +1072,27 @@ def main():
     if not args.no_check:
         wl.check(sets[0])
 
-    achieved = wl.alg_bytes / (mean_kernel_ms * 1e-3) / 1e9
-
     # ---- CPU oracle on the same workload (bounded sample)
-    cpu = None
-    if args.cpu_seconds > 0 and wl.images > 0:
-        def cpu_leg(threads, budget):
-            reps, done, tcpu = 0, 0, 0.0
-            c0 = time.perf_counter()
-            while reps < 2 or tcpu < budget:
-                done += wl.cpu(threads)
-                reps += 1
-                tcpu = time.perf_counter() - c0
-            return done, tcpu
-
-        threads = min(os.cpu_count() or 1, 16)
-        done, tcpu = cpu_leg(threads, args.cpu_seconds)
-        used = wl.cpu_cores(threads) if hasattr(wl, "cpu_cores") else threads
-        done1, tcpu1 = cpu_leg(1, args.cpu_seconds / 2)
-        model = ""
-        try:
-            with open("/proc/cpuinfo") as f:
-                model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
-        except OSError:
-            pass
-        cpu = {"value": round(done / tcpu, 1), "unit": "images/s", "cores": used, "kind": "port",
-               "host": {"cpu_model": model, "logical_cpus": os.cpu_count()},
-               "sample": "%d images of this workload through the CPU oracle in %.1f s, %d thread%s"
-                         % (done, tcpu, used, "" if used == 1 else "s"),
-               "single_thread": {"value": round(done1 / tcpu1, 1), "unit": "images/s", "cores": 1,
-                                 "sample": "%d images in %.1f s, 1 thread" % (done1, tcpu1)}}
+    cpu = cpu_baseline(wl, args.cpu_seconds, args.cpu_seconds / 2)
 
     out = {
         "metric": "images/sec and achieved HBM GB/s (% of roofline), 1 MI355X",
-        "value": round(wl.images * timed_steps / wall, 1),
+        "value": round(wl.images * m["timed"] / m["wall"], 1),
         "unit": "images/s",
         "n_gpus": 1,
         "steps": args.steps,
-        "replays": replays,
+        "launches_per_graph": m["launches"],
+        "replays": m["replays"],
         "warmup": args.warmup,
-        "ms_per_step": round(wall / timed_steps * 1e3, 5),
+        "ms_per_step": round(m["wall"] / m["timed"] * 1e3, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": wl.dtype,
         "data": "synthetic",
-        "config": {"workload": wl.workload, "rotate_buffer_sets": nsets, "launch": mode,
+        "config": {"workload": wl.workload, "rotate_buffer_sets": nsets, "launch": m["mode"],
                    "streams": args.streams if graph is not None else 1},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.key),
-                     "kernel": wl.kernel, "kernel_ms_mean": round(mean_kernel_ms, 5),
-                     "algorithmic_bytes_per_launch": wl.alg_bytes},
+        "roofline": roofline_of(wl, mean_kernel_ms),
         "cpu_baseline": cpu,
         "submit_to_sync_ms": round(submit_to_sync_ms, 4),
     }
@@ -1058,6 +1104,28 @@ def main():
         out["roofline"]["other_conventions"] = {
             k: {"bytes_per_launch": v, "GB/s": round(v / (mean_kernel_ms * 1e-3) / 1e9, 1)}
             for k, v in wl.other_bytes.items()}
+
+    # ---- the other BASELINE configurations, each the same way on a smaller budget: HBM-cold buffer rotation,
+    # at least 0.1 s of device work, an oracle spot check, the CPU oracle for about 2 s
+    if all_configs:
+        configs = [{"workload": wl.key, "description": wl.workload, "images_per_launch": wl.images,
+                    "images_per_s": out["value"], "cpu_baseline": cpu, **out["roofline"]}]
+        del sets, graph, m, wl
+        for key in OTHER_CONFIGS:
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+            w2 = WORKLOADS[key](cv, orc, np, torch)
+            m2 = measure(w2, torch, args.steps, min(args.warmup, 50), args.rotate, not args.no_graph, 1,
+                         min(args.min_seconds, 0.1))
+            if not args.no_check:
+                w2.check(m2["sets"][0])
+            entry2 = {"workload": key, "description": w2.workload, "images_per_launch": w2.images,
+                      "images_per_s": round(w2.images * m2["timed"] / m2["wall"], 1),
+                      "cpu_baseline": cpu_baseline(w2, min(args.cpu_seconds, 1.5), 0.0)}
+            entry2.update(roofline_of(w2, m2["mean_kernel_ms"]))
+            configs.append(entry2)
+            del m2, w2
+        out["configs"] = configs
     print(json.dumps(out))
 
 

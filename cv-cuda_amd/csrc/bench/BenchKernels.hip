@@ -19,9 +19,8 @@ __global__ __launch_bounds__(256) void FusedCopyBound(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
     const int     n    = tp.n;
-    const int     dx   = tp.tx * 64 + (threadIdx.x & 63);
-    const int     wave = threadIdx.x >> 6;
-    const int     dy0  = tp.ty * kRowsPerBlock + wave * kRowsPerWave;
+    const int     dx   = FusedColumnOf(tp.tx);
+    const int     dy0  = FusedFirstRowOf(tp.ty);
     if (dx >= a.dstW)
     {
         return;

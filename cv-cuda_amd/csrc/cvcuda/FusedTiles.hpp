@@ -17,7 +17,24 @@ namespace cvamd {
 // 7 / 6 / 4 of 8 gave 23.7 / 25.9 / 28.8 us).
 constexpr int kRowsPerWave  = 1;
 constexpr int kWavesPerBlk  = 4;
-constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlk;
+// Waves of a workgroup side by side on an output row, the others stacked. One: a workgroup is 64 columns x 4
+// rows. With all four on ONE row (a workgroup then reads two contiguous source spans of 2.8 KB and writes 896
+// contiguous bytes per plane) the same launch took 22.46 us against 22.57 us: within the noise of the memory
+// system, not shipped.
+constexpr int kWavesAcross = 1;
+constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlk / kWavesAcross;
+constexpr int kColsPerBlock = 64 * kWavesAcross;
+
+// Output column of this lane and first output row of its wave within tile (tx, ty).
+__device__ __forceinline__ int FusedColumnOf(int tx)
+{
+    return tx * kColsPerBlock + (int)(threadIdx.x & (kColsPerBlock - 1));
+}
+
+__device__ __forceinline__ int FusedFirstRowOf(int ty)
+{
+    return ty * kRowsPerBlock + (int)(threadIdx.x / kColsPerBlock) * kRowsPerWave;
+}
 
 struct FusedArgs
 {
@@ -82,7 +99,7 @@ constexpr int kFusedImagesPerLaunch = 65535;
 // images (at most kFusedImagesPerLaunch) starting at a.firstImage.
 inline dim3 SetFusedGrid(FusedArgs &a, int images)
 {
-    a.tilesX = (uint32_t)((a.dstW + 63) / 64);
+    a.tilesX = (uint32_t)((a.dstW + kColsPerBlock - 1) / kColsPerBlock);
     a.tilesY = (uint32_t)((a.dstH + kRowsPerBlock - 1) / kRowsPerBlock);
     return dim3(a.tilesX * kXcdCount, (a.tilesY + kXcdCount - 1) / kXcdCount, (uint32_t)images);
 }
