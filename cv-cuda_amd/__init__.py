@@ -243,7 +243,11 @@ class Tensor(_Handle):
         h = C.c_void_p()
         shp = (C.c_int64 * len(shape))(*shape)
         check(_nv.nvcvTensorReshape(self.handle, len(shape), shp, capi.TensorLayout.make(layout), C.byref(h)))
-        return Tensor(h)
+        t = Tensor(h)
+        # the new handle holds a reference on this one, but the owner of externally wrapped memory (a torch tensor,
+        # an object with __cuda_array_interface__) is only held by this wrapper: it must live as long as the view
+        t._keep.append(self)
+        return t
 
 
 def _as_dtype(dtype):

@@ -81,16 +81,16 @@ def asan_runtime():
 
 
 def build(force=False, jobs=8, verbose=True, sanitize=False):
-    global LIBDIR, OBJDIR
+    libdir, objdir = LIBDIR, OBJDIR
     host_extra, hip_extra, link_extra = [], [], []
     if sanitize:
-        LIBDIR, OBJDIR = os.path.join(HERE, "lib_san"), os.path.join(HERE, "build_san")
+        libdir, objdir = os.path.join(HERE, "lib_san"), os.path.join(HERE, "build_san")
         # on a hipcc line every -fsanitize= goes directly after -Xarch_host: the device pass must not see it
         hip_extra = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-fno-omit-frame-pointer", "-g"]
         host_extra = hip_extra # hipcc compiles the plain .cpp sources as HIP too
         link_extra = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-shared-libsan"]
-    os.makedirs(LIBDIR, exist_ok=True)
-    os.makedirs(OBJDIR, exist_ok=True)
+    os.makedirs(libdir, exist_ok=True)
+    os.makedirs(objdir, exist_ok=True)
     newest_header = max(os.path.getmtime(h) for h in _headers())
     core = [(s, host_extra) for s in _sources("nvcv", (".cpp",))]
     ops = [(s, DEVICE + hip_extra if s.endswith(".hip") else host_extra) for s in _sources("cvcuda", (".cpp", ".hip"))]
@@ -99,7 +99,7 @@ def build(force=False, jobs=8, verbose=True, sanitize=False):
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
         for group, items in (("nvcv", core), ("cvcuda", ops), ("bench", bench)):
             for src, extra in items:
-                obj = os.path.join(OBJDIR, group + "_" + os.path.basename(src) + ".o")
+                obj = os.path.join(objdir, group + "_" + os.path.basename(src) + ".o")
                 tasks.append((group, obj, ex.submit(_compile, src, obj, extra, force, newest_header)))
         for group, obj, fut in tasks:
             msgs = fut.result()
@@ -107,19 +107,34 @@ def build(force=False, jobs=8, verbose=True, sanitize=False):
                 print(msgs)
     core_objs = [o for g, o, _ in tasks if g == "nvcv"]
     ops_objs = [o for g, o, _ in tasks if g == "cvcuda"]
-    nvcv_so = os.path.join(LIBDIR, "libnvcv_types.so")
-    cvcuda_so = os.path.join(LIBDIR, "libcvcuda.so")
+    nvcv_so = os.path.join(libdir, "libnvcv_types.so")
+    cvcuda_so = os.path.join(libdir, "libcvcuda.so")
+    # (the sanitized libraries leave the sanitizer runtime's symbols to the preloaded runtime, so they cannot be
+    # linked with --no-undefined)
     link = ["hipcc", "-shared", "-fPIC", "--offload-arch=" + ARCH] + (link_extra if sanitize else ["-Wl,--no-undefined"])
     # ELF symbol versions of the reference's ABI (FUNC@@NVCV_x.y / FUNC@@CVCUDA_x.y), see csrc/abi
     maps = os.path.join(CSRC, "abi")
     subprocess.run(link + core_objs + ["-o", nvcv_so, "-Wl,-soname,libnvcv_types.so",
                                        "-Wl,--version-script=" + os.path.join(maps, "nvcv_types.map")], check=True)
-    subprocess.run(link + ops_objs + ["-o", cvcuda_so, "-Wl,-soname,libcvcuda.so", "-L" + LIBDIR, "-lnvcv_types",
+    subprocess.run(link + ops_objs + ["-o", cvcuda_so, "-Wl,-soname,libcvcuda.so", "-L" + libdir, "-lnvcv_types",
                                       "-Wl,-rpath,$ORIGIN",
                                       "-Wl,--version-script=" + os.path.join(maps, "cvcuda.map")], check=True)
-    bench_so = os.path.join(LIBDIR, "libcvamd_bench.so")
+    bench_so = os.path.join(libdir, "libcvamd_bench.so")
     subprocess.run(link + [o for g, o, _ in tasks if g == "bench"] + ["-o", bench_so], check=True)
+    if not sanitize:
+        build_c_caller(libdir)
     return nvcv_so, cvcuda_so, bench_so
+
+
+def build_c_caller(libdir=LIBDIR):
+    """tests/golden/abi_gpu_calls.c -> lib/abi_gpu_calls: a plain C11 program (gcc, the public headers, the HIP
+    runtime's C API) that runs three operators through the C ABI; a GPU test runs it and compares what it wrote."""
+    src = os.path.join(ROOT, "tests", "golden", "abi_gpu_calls.c")
+    exe = os.path.join(libdir, "abi_gpu_calls")
+    subprocess.run(["gcc", "-std=c11", "-O1", "-Wall", "-Wextra", "-Werror", "-D__HIP_PLATFORM_AMD__", "-I" + INCLUDE,
+                    "-I/opt/rocm/include", src, "-o", exe, "-L" + libdir, "-lcvcuda", "-lnvcv_types", "-L/opt/rocm/lib",
+                    "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    return exe
 
 
 if __name__ == "__main__":

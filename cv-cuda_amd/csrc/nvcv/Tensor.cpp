@@ -267,7 +267,10 @@ private:
 
 // Computes strides of `newShape` viewing memory described by (shape, strides), numpy-style: runs of
 // input dimensions that are contiguous with each other are merged, and every merged run must be
-// covered exactly by consecutive output dimensions.
+// covered exactly by consecutive output dimensions. Unit dimensions of the input take no part in the
+// merge whatever their stride says (an element of such a dimension is never stepped over), which is more
+// lenient than the reference: its merge (src/nvcv/src/priv/TensorData.cpp:196-246) lets a unit dimension
+// with a stride that does not continue its neighbours split a run, and then refuses the reshape.
 bool ViewStrides(int rank, const int64_t *shape, const int64_t *strides, int newRank, const int64_t *newShape,
                  int64_t *newStrides)
 {

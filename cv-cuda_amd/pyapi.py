@@ -576,23 +576,35 @@ def _submit(stream, reads, writes, op, *args):
     write and of the reads since, per stream."""
     s = _torch_stream(stream)
     key = s.cuda_stream
-    for obj in reads + writes:
-        wrote = getattr(obj, "_wrote", None)
-        if wrote is not None and wrote[0] != key:
-            s.wait_event(wrote[1])
-    for obj in writes:
-        for other, event in getattr(obj, "_read", {}).items():
-            if other != key:
-                s.wait_event(event)
+    # the containers' event records are shared by every thread that submits work on them: they are read and
+    # updated under one lock (the Submit itself runs outside it)
+    with _events_lock:
+        waits = []
+        for obj in reads + writes:
+            wrote = getattr(obj, "_wrote", None)
+            if wrote is not None and wrote[0] != key:
+                waits.append(wrote[1])
+        for obj in writes:
+            for other, event in list(getattr(obj, "_read", {}).items()):
+                if other != key:
+                    waits.append(event)
+    for event in waits:
+        s.wait_event(event)
     op(s, *args)
-    event = torch.cuda.Event()
+    event = _new_event()
     event.record(s)
-    for obj in reads:
-        if not hasattr(obj, "_read"):
-            obj._read = {}
-        obj._read[key] = event
-    for obj in writes:
-        obj._wrote, obj._read = (key, event), {}
+    with _events_lock:
+        for obj in reads:
+            obj.__dict__.setdefault("_read", {})[key] = event
+        for obj in writes:
+            obj._wrote, obj._read = (key, event), {}
+
+
+_events_lock = threading.Lock()
+
+
+def _new_event():
+    return torch.cuda.Event()
 
 
 def _same_images(src, fmt=None, sizes=None):

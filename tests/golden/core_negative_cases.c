@@ -165,6 +165,35 @@ static void TensorObjectCases(NVCVAllocatorHandle alloc)
     /* the same call with everything in place is a view of the one NHWC sample as 4 planes */
     EXPECT(OK, nvcvTensorReshape(handle, 3, chw, NVCV_TENSOR_CHW, &other));
     EXPECT(OK, nvcvTensorDecRef(other, NULL));
+    {
+        /* a unit dimension whose stride does not continue its neighbours: this build steps over it (no element of it
+         * is ever addressed) and gives the 12 dense elements as one dimension; the reference's merge of contiguous
+         * dimensions lets it split the run and refuses (src/nvcv/src/priv/TensorData.cpp:196-246) */
+        NVCVTensorData odd;
+        memset(&odd, 0, sizeof(odd));
+        odd.bufferType = NVCV_TENSOR_BUFFER_STRIDED_CUDA;
+        odd.rank       = 3;
+        odd.dtype      = NVCV_DATA_TYPE_U8;
+        EXPECT(OK, nvcvTensorLayoutMake("HWC", &odd.layout));
+        const int64_t oshape[3] = {4, 1, 3}, ostrides[3] = {3, 999, 1};
+        for (int i = 0; i < 3; ++i)
+        {
+            odd.shape[i]                  = oshape[i];
+            odd.buffer.strided.strides[i] = ostrides[i];
+        }
+        odd.buffer.strided.basePtr = (NVCVByte *)0x2000;
+        NVCVTensorHandle wrapped = NULL, flat = NULL;
+        EXPECT(OK, nvcvTensorWrapDataConstruct(&odd, NULL, NULL, &wrapped));
+        const int64_t    twelve[1] = {12};
+        NVCVTensorLayout w;
+        EXPECT(OK, nvcvTensorLayoutMake("W", &w));
+        EXPECT(OK, nvcvTensorReshape(wrapped, 1, twelve, w, &flat));
+        NVCVTensorData seen;
+        EXPECT(OK, nvcvTensorExportData(flat, &seen));
+        EXPECT(1, (int)seen.buffer.strided.strides[0]);
+        EXPECT(OK, nvcvTensorDecRef(flat, NULL));
+        EXPECT(OK, nvcvTensorDecRef(wrapped, NULL));
+    }
 
     int newRef = -1;
     EXPECT(OK, nvcvTensorDecRef(handle, &newRef));

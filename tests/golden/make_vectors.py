@@ -72,6 +72,9 @@ def cases():
         # the shipped 8-bit bilinear blend (15-bit fixed point), which the kernels must reproduce bit for bit
         out["warp_affine_linear_fixed_border%d" % border] = orc.warp(a, (30, 44), m, LINEAR, border, (7, 8, 9, 0), False,
                                                                     variant=2)
+    # the call of tests/golden/abi_gpu_calls.c: RGBA8, a border colour of four different values
+    out["abi_warp_affine_rgba8_linear"] = orc.warp(recipe(1, 30, 44, 4, step=5), (30, 44), m, LINEAR, 0, (7, 80, 159, 250),
+                                                   False, variant=2)
     out["convert_u8_to_f32"] = orc.convert_to(recipe(1, 5, 7, 3), np.float32, 1 / 255.0, 0.0, 0)
     out["convert_f32_to_u8"] = orc.convert_to(recipe(1, 5, 7, 3, np.float32) * 300 - 20, np.uint8, 1.0, 0.5, 0)
     img = recipe(1, 20, 28, 3, step=5)[0]

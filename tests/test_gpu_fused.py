@@ -88,6 +88,98 @@ def test_tensor_rows(cv, orc, gpu, row, data):
     compare(ref1, ref, interp, odt)
 
 
+# The reference's own table, all 63 rows (tests/cvcuda/system/TestOpResizeCropConvertReformat.cpp:232-329):
+# source (w, h, n), resize (w, h), interpolation, destination (w, h), crop (x, y), scale, offset, source format,
+# destination format, srcCast. The formats give the channel manipulation (order differs -> REVERSE), the layout
+# (a trailing p -> planar) and the output type.
+REFERENCE_ROWS = [
+    (8, 8, 1, 8, 8, LINEAR, 6, 6, 1, 1, 1, 0, "RGB8", "BGRf32p", False),
+    (8, 8, 1, 16, 16, LINEAR, 12, 12, 2, 2, 1, 0, "RGB8", "BGRf32p", False),
+    (42, 48, 1, 23, 24, LINEAR, 15, 13, 0, 0, 1, 0, "RGB8", "BGRf32p", False),
+    (42, 40, 3, 21, 20, LINEAR, 17, 13, 1, 1, 1, 0, "RGB8", "BGRf32p", False),
+    (21, 21, 5, 42, 42, LINEAR, 32, 32, 10, 10, 1, 0, "RGB8", "BGRf32p", False),
+    (113, 12, 7, 12, 36, LINEAR, 7, 13, 3, 11, 1, 0, "RGB8", "BGRf32p", False),
+    (17, 151, 7, 48, 16, LINEAR, 32, 16, 4, 0, 1, 0, "RGB8", "BGRf32p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "BGRf32p", False),
+    (1080, 1920, 13, 800, 600, LINEAR, 640, 480, 101, 64, 1, 0, "RGB8", "BGRf32p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "BGRf32p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "BGR8p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "BGR8p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "RGBf32p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "RGBf32p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "RGB8p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "RGB8p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "BGR8", "RGBf32p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "BGR8", "RGBf32p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "BGR8", "RGB8p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "BGR8", "RGB8p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "BGR8", "BGRf32p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "BGR8", "BGRf32p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "BGR8", "BGR8p", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "BGR8", "BGR8p", False),
+    (8, 8, 1, 8, 8, LINEAR, 6, 6, 1, 1, 1, 0, "RGB8", "BGRf32", False),
+    (8, 8, 1, 16, 16, LINEAR, 12, 12, 2, 2, 1, 0, "RGB8", "BGRf32", False),
+    (113, 12, 7, 12, 36, LINEAR, 7, 13, 3, 11, 1, 0, "RGB8", "BGRf32", False),
+    (17, 151, 7, 48, 16, LINEAR, 32, 16, 4, 0, 1, 0, "RGB8", "BGRf32", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "BGRf32", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "BGRf32", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "BGR8", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "BGR8", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "RGBf32", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "RGBf32", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "RGB8", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "RGB8", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "RGBf32", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "RGBf32", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "RGB8", "RGB8", False),
+    (1280, 960, 3, 300, 225, LINEAR, 250, 200, 15, 16, 1, 0, "RGB8", "RGB8", False),
+    (8, 8, 1, 8, 8, NEAREST, 6, 6, 1, 1, 1, 0, "RGB8", "BGRf32p", False),
+    (8, 8, 5, 16, 16, NEAREST, 12, 12, 2, 2, 1, 0, "RGB8", "BGRf32p", False),
+    (42, 48, 1, 23, 24, NEAREST, 15, 13, 0, 0, 1, 0, "RGB8", "BGRf32p", False),
+    (313, 212, 4, 412, 336, NEAREST, 412, 336, 0, 0, 1, 0, "RGB8", "BGRf32p", False),
+    (1080, 1920, 13, 800, 600, NEAREST, 640, 480, 101, 64, 1, 0, "RGB8", "BGRf32p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 1, 0, "RGB8", "BGRf32p", False),
+    (313, 212, 4, 412, 336, NEAREST, 412, 336, 0, 0, 1, 0, "RGB8", "BGR8p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 1, 0, "RGB8", "BGR8p", False),
+    (313, 212, 4, 412, 336, NEAREST, 412, 336, 0, 0, 1, 0, "BGR8", "RGBf32p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 1, 0, "BGR8", "RGBf32p", False),
+    (313, 212, 4, 412, 336, NEAREST, 412, 336, 0, 0, 1, 0, "BGR8", "RGB8p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 1, 0, "BGR8", "RGB8p", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1/127.5, -1, "BGR8", "RGBf32p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 2, -255, "BGR8", "RGBf32p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, -1, 255, "BGR8", "RGB8", False),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 0.5, 0, "BGR8", "RGB8p", False),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 2, 0, "BGR8", "RGB8p", False),
+    (353, 450, 3, 256, 256, LINEAR, 224, 224, 16, 16, 1, 0, "BGR8", "RGBf32p", True),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1/127.5, -1, "BGR8", "RGBf32p", True),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 2, -255, "BGR8", "RGBf32p", True),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, -1, 255, "BGR8", "RGB8", True),
+    (313, 212, 4, 412, 336, LINEAR, 412, 336, 0, 0, 1, 0, "BGR8", "RGB8p", True),
+    (1280, 960, 3, 300, 225, NEAREST, 250, 200, 15, 16, 1, 0, "BGR8", "RGB8p", True),
+]
+
+
+@pytest.mark.parametrize("index", range(len(REFERENCE_ROWS)))
+def test_reference_table_rows(cv, orc, gpu, index):
+    sw, sh, n, nw, nh, interp, ow, oh, cx, cy, scale, offset, sfmt, dfmt, cast = REFERENCE_ROWS[index]
+    odt = np.float32 if "f32" in dfmt else np.uint8
+    planar, manip = dfmt.endswith("p"), int(sfmt[:3] != dfmt[:3])
+    src = ramp(n, sh, sw)  # the reference test's input recipe
+    ref = orc.fused_rccr(src, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast, order=0)
+    res = run_tensor(cv, src, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast)
+    if cast and interp == LINEAR and odt == np.float32:
+        # srcCast rounds the bilinear value to 8 bits before scale and offset: where that value is a tie within
+        # float32 rounding, the golden's order of summation and the kernel's round to neighbouring integers, one
+        # unit of `scale` apart (the reference's own tolerance is 1 in output units, its line 437). The kernel's
+        # order (oracle order 1) is reproduced to the float bar, the golden's to one unit on a handful of pixels.
+        compare(res, orc.fused_rccr(src, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast,
+                                    order=1), interp, odt)
+        d = np.abs(res - ref)
+        assert d.max() <= abs(scale) * (1 + 1e-5) and (d > 1e-5 * np.maximum(1.0, np.abs(ref))).mean() < 1e-4
+    else:
+        compare(res, ref, interp, odt)
+
+
 def test_single_image_layouts(cv, orc, gpu):
     src = orc.fill_u8((1, 37, 53, 3), 11)
     for planar in (True, False):

@@ -176,6 +176,33 @@ def test_resize_cubic_edge_quirk(orc):
     assert np.all(out[:, 0] == 1.0)
 
 
+def test_resize_cubic_hand_weights_interior_and_border_row(orc):
+    # 6 x 6 -> 4 x 4 (scale 1.5): output index 1 maps to source 1.75 (centre 1, fraction 0.75, interior), output
+    # index 0 to 0.25 (centre 0, fraction 0.25, in the border band). Keys kernel with A = -0.75, written out by hand:
+    #   W(x) = 1.25|x|^3 - 2.25|x|^2 + 1 (|x| <= 1),  -0.75|x|^3 + 3.75|x|^2 - 6|x| + 3 (1 < |x| < 2)
+    #   fraction 0.75: taps at distances 1.75, 0.75, 0.25, 1.25
+    w75 = np.array([-0.03515625, 0.26171875, 0.87890625, -0.10546875])
+    w25 = w75[::-1]  # fraction 0.25: distances 1.25, 0.25, 0.75, 1.75
+    assert w75.sum() == 1.0
+    rng = np.random.default_rng(21)
+    img = (rng.random((1, 6, 6, 1)) * 4 + 1).astype(np.float32)
+    a = img[0, :, :, 0].astype(np.float64)
+    for variant in (1, 2):
+        out = orc.resize(img, (4, 4), CUBIC, variant)[0, :, :, 0]
+        # interior in both axes: centre (1, 1), taps rows 0..3 x columns 0..3
+        assert abs(out[1, 1] - w75 @ a[0:4, 0:4] @ w75) < 1e-5
+        # border band along y only (output row 0): the centre is clamped to row 1 but the fraction 0.25 is KEPT
+        # (src/cvcuda/priv/OpResize.cu:357-366 zeroes the horizontal fraction only), taps rows 0..3
+        assert abs(out[0, 1] - w25 @ a[0:4, 0:4] @ w75) < 1e-5
+        # border band along x only (output column 0): centre clamped to column 1 AND fraction forced to 0 -> column 1
+        assert abs(out[1, 0] - w75 @ a[0:4, 1]) < 1e-5
+        # both: column 1 with the vertical weights of fraction 0.25
+        assert abs(out[0, 0] - w25 @ a[0:4, 1]) < 1e-5
+        # the far side: output index 3 maps to 4.75 (centre 4 >= 6 - 3: band), centre clamped to 3, taps 2..5
+        assert abs(out[3, 1] - w75 @ a[2:6, 0:4] @ w75) < 1e-5   # vertical fraction kept
+        assert abs(out[1, 3] - w75 @ a[0:4, 3]) < 1e-5           # horizontal fraction zeroed: column 3
+
+
 # ------------------------------------------------------------------------------------------ NV12
 def _all_triples_nv12():
     W = H = 4096
@@ -420,6 +447,26 @@ def test_warp_cubic_fixed_point_variant(orc):
     np.testing.assert_array_equal(sh, np.roll(src[0], (3, -2), axis=(0, 1)))
     const = np.full((1, 20, 20, 1), 201, np.uint8)
     assert (orc.warp(const, (20, 20), m, CUBIC, border=1, variant=2) == 201).all()
+
+
+def test_warp_cubic_reproduces_quadratics(orc):
+    # Catmull-Rom (A = -0.5) interpolation reproduces polynomials up to degree 2: a CUBIC warp of a quadratic image by a
+    # fractional translation equals the quadratic at the shifted coordinates, both for the golden (variant 0, which
+    # normalises by the weight sum) and the device formula (variant 1). With any other A (the resize's -0.75, say) the
+    # second-order term is off by (A + 0.5) * f'' * t(1 - t) per axis: ~1e-3 here.
+    h, w = 24, 28
+    ys, xs = np.meshgrid(np.arange(h, dtype=np.float64), np.arange(w, dtype=np.float64), indexing="ij")
+
+    def quad(x, y):
+        return 0.011 * x * x - 0.007 * x * y + 0.013 * y * y + 0.05 * x - 0.03 * y + 2.0
+
+    img = quad(xs, ys).astype(np.float32).reshape(1, h, w, 1)
+    tx, ty = 0.3125, 0.6875
+    for variant in (0, 1):
+        out = orc.warp(img, (h, w), [1, 0, tx, 0, 1, ty], CUBIC, border=1, variant=variant)[0, :, :, 0]
+        want = quad(xs + tx, ys + ty)
+        inner = (slice(2, h - 3), slice(2, w - 3))
+        assert np.abs(out[inner] - want[inner]).max() < 2e-5, variant
 
 
 def test_warp_cubic_golden_vs_device_and_perspective(orc):

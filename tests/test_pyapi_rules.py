@@ -95,3 +95,75 @@ def test_recti(api):
     for x, y, w, h in ((0, 0, 0, 0), (10, -12, -45, 14)):
         for r in (api.RectI(x, y, w, h), api.RectI(y=y, width=w, height=h, x=x)):
             assert (r.x, r.y, r.width, r.height) == (x, y, w, h)
+
+
+def test_reshape_of_wrapped_memory_keeps_its_owner_alive(api):
+    # nvcvTensorReshape takes a reference on the source handle, but the owner of externally wrapped memory is held by the
+    # Python wrapper of the source only: the reshaped tensor must hold it too (no GPU: the pointer is never followed)
+    import gc
+    import weakref
+
+    class Owner:
+        def __init__(self):
+            self.__cuda_array_interface__ = {"shape": (8, 3, 3), "typestr": "|u1", "data": (0x7F0000001000, False),
+                                             "version": 3, "strides": None}
+
+    owner = Owner()
+    alive = weakref.ref(owner)
+    source = api.as_tensor(owner, "HWC")
+    for view in (source.reshape((24, 3), "WC"), api.reshape(source, (72,), "W")):
+        del source, owner
+        gc.collect()
+        assert alive() is not None, "the owner of the wrapped memory was collected while a reshaped tensor refers to it"
+        assert view.cuda().__cuda_array_interface__["data"][0] == 0x7F0000001000
+        owner = alive()
+        source = api.as_tensor(owner, "HWC")
+        del view
+    del source, owner
+    gc.collect()
+    assert alive() is None
+
+
+def test_submit_bookkeeping_under_parallel_readers(api, monkeypatch):
+    # several threads record reads of one shared input on their own streams while another thread keeps writing it:
+    # no read event may be lost (a later writer waits for every stream that read) and no iteration may trip over a
+    # concurrent update. No GPU: streams and events are stand-ins that only record what was asked of them.
+    import threading
+
+    class FakeStream:
+        def __init__(self, key):
+            self.cuda_stream, self.waited = key, []
+
+        def wait_event(self, event):
+            self.waited.append(event)
+
+    class FakeEvent:
+        def record(self, stream):
+            self.stream = stream.cuda_stream
+
+    class Box:
+        pass
+
+    monkeypatch.setattr(api, "_torch_stream", lambda s: s)
+    monkeypatch.setattr(api, "_new_event", FakeEvent)
+    shared, errors = Box(), []
+
+    def reader(key):
+        try:
+            out = Box()
+            for _ in range(300):
+                api._submit(FakeStream(key), [shared], [out], lambda s: None)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=reader, args=(100 + i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert sorted(shared._read) == [100 + i for i in range(8)]
+    writer = FakeStream(7)
+    api._submit(writer, [], [shared], lambda s: None)
+    assert sorted(e.stream for e in writer.waited) == [100 + i for i in range(8)]
+    assert shared._read == {} and shared._wrote[0] == 7
