@@ -1054,6 +1054,36 @@ __device__ __forceinline__ uint32_t WindowPixel(const TapWindow<C> &t, int k)
     }
 }
 
+// The 4 pixels of source row y that start at column xs (rows before the image's last one only: the load may read
+// past the row).
+template<int C>
+__device__ __forceinline__ TapWindow<C> LoadTapWindow(const Plane &p, int y, int xs)
+{
+    // u8x3: the aligned 16 bytes that hold the window's 12, funnel-shifted into place. The texture path takes a
+    // 12-byte load that is not dword aligned apart into about three times as many cache accesses (counters:
+    // 63 against 20 per wave-load), and this kernel waits for that unit: 1080p -> 720p 61.5 -> 59.9 us,
+    // 720p -> 1080p 117 -> 101 us. Reads at most 3 bytes before and 4 after the window.
+    const uint8_t *at  = p.src + (int64_t)y * p.srcRow + xs * C;
+    const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(at) & 3u;
+    struct alignas(4) W4
+    {
+        uint32_t d[4];
+    };
+    TapWindow<C> t;
+    if constexpr (C == 3)
+    {
+        const W4 w = *reinterpret_cast<const W4 *>(at - mis);
+        t.w[0]     = __builtin_amdgcn_alignbyte(w.d[1], w.d[0], mis);
+        t.w[1]     = __builtin_amdgcn_alignbyte(w.d[2], w.d[1], mis);
+        t.w[2]     = __builtin_amdgcn_alignbyte(w.d[3], w.d[2], mis);
+    }
+    else
+    {
+        t = *reinterpret_cast<const TapWindow<C> *>(at);
+    }
+    return t;
+}
+
 // One pixel from its four taps (a dword each, channel c in byte c) and the float32 weights of the second taps.
 template<int C>
 __device__ __forceinline__ uint32_t BilinearU8(uint32_t p00, uint32_t p01, uint32_t p10, uint32_t p11, float wx, float wy)
@@ -1099,32 +1129,7 @@ __device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int 
             t[3] |= (uint32_t)b[1][c] << (8 * c);
         }
     };
-    auto window = [&](int y)
-    {
-        // u8x3: the aligned 16 bytes that hold the window's 12, funnel-shifted into place. The texture path takes a
-        // 12-byte load that is not dword aligned apart into about three times as many cache accesses (counters:
-        // 63 against 20 per wave-load), and this kernel waits for that unit: 1080p -> 720p 61.5 -> 59.9 us,
-        // 720p -> 1080p 117 -> 101 us. Reads at most 3 bytes before and 4 after the window.
-        const uint8_t *at  = p.src + (int64_t)y * p.srcRow + colA.s * C;
-        const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(at) & 3u;
-        struct alignas(4) W4
-        {
-            uint32_t d[4];
-        };
-        const W4     w = *reinterpret_cast<const W4 *>(at - mis);
-        TapWindow<C> t;
-        if constexpr (C == 3)
-        {
-            t.w[0] = __builtin_amdgcn_alignbyte(w.d[1], w.d[0], mis);
-            t.w[1] = __builtin_amdgcn_alignbyte(w.d[2], w.d[1], mis);
-            t.w[2] = __builtin_amdgcn_alignbyte(w.d[3], w.d[2], mis);
-        }
-        else
-        {
-            t = *reinterpret_cast<const TapWindow<C> *>(at);
-        }
-        return t;
-    };
+    auto window = [&](int y) { return LoadTapWindow<C>(p, y, colA.s); };
     auto unpack = [&](const TapWindow<C> &win, uint32_t (&t)[4])
     {
         const uint32_t k0 = WindowPixel<C>(win, 0), k1 = WindowPixel<C>(win, 1), k2 = WindowPixel<C>(win, 2),
@@ -1221,6 +1226,125 @@ __device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int 
     }
 }
 
+// Enlargements by 1.5 or more (3 * srcW <= 2 * dstW): the taps of FOUR neighbouring output columns lie within 4
+// source pixels, so a lane owns 4 columns x 2 rows on the same window loads as the two-column form: half the loads,
+// column-independent work (row terms, addresses, funnel shifts) spread over twice the pixels, and a lane's 4 pixels
+// of a row are consecutive, so nothing changes lanes before the store. A wave covers 256 columns x 2 rows. The
+// distance between the first and the last of a lane's four source columns is at most 2 by the scale; should
+// float32 rounding ever make it 3, or the image's last row be involved, the wave takes the two-column form.
+template<int C>
+__device__ __forceinline__ void ResizeLinearQuadsU8(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    const int            lane = threadIdx.x & 63;
+    const int            dx0  = x0 + 4 * lane;
+    AxisTerms<1>         col[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        col[j] = Axis<NVCV_INTERP_LINEAR>(p.scaleX, min(dx0 + j, p.dstW - 1), p.srcW);
+    }
+    const auto rows = Axis<NVCV_INTERP_LINEAR>(p.scaleY, min(y0 + (lane & 1), p.dstH - 1), p.srcH);
+    const auto row0 = FromLane(rows, 0), row1 = FromLane(rows, 1);
+    const int  ya0 = row0.s, yb0 = min(row0.s + 1, p.srcH - 1), ya1 = row1.s, yb1 = min(row1.s + 1, p.srcH - 1);
+    const bool narrow = col[3].s - col[0].s <= 2;
+    if (max(yb0, yb1) >= p.srcH - 1 || __builtin_amdgcn_ballot_w64(!narrow) != 0) // wave-uniform
+    {
+        ResizeLinearPairsU8<C, false>(p, x0, y0);
+        ResizeLinearPairsU8<C, false>(p, x0 + 128, y0);
+        return;
+    }
+    // pixels (s, s + 1) of column j out of the window's four
+    auto taps = [&](const TapWindow<C> &win, uint32_t (&first)[4], uint32_t (&second)[4])
+    {
+        const uint32_t k0 = WindowPixel<C>(win, 0), k1 = WindowPixel<C>(win, 1), k2 = WindowPixel<C>(win, 2),
+                       k3 = WindowPixel<C>(win, 3);
+        first[0]  = k0;
+        second[0] = k1;
+#pragma unroll
+        for (int j = 1; j < 4; ++j)
+        {
+            const int d = col[j].s - col[0].s;
+            first[j]    = d == 0 ? k0 : (d == 1 ? k1 : k2);
+            second[j]   = d == 0 ? k1 : (d == 1 ? k2 : k3);
+        }
+    };
+    uint32_t topA[2][4], topB[2][4], botA[2][4], botB[2][4]; // [output row][column]: first and second tap, upper and lower source row
+    taps(LoadTapWindow<C>(p, ya0, col[0].s), topA[0], topB[0]);
+    taps(LoadTapWindow<C>(p, yb0, col[0].s), botA[0], botB[0]);
+    if (ya1 == ya0)
+    {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            topA[1][j] = topA[0][j];
+            topB[1][j] = topB[0][j];
+            botA[1][j] = botA[0][j];
+            botB[1][j] = botB[0][j];
+        }
+    }
+    else if (ya1 == yb0)
+    {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            topA[1][j] = botA[0][j];
+            topB[1][j] = botB[0][j];
+        }
+        taps(LoadTapWindow<C>(p, yb1, col[0].s), botA[1], botB[1]);
+    }
+    else
+    {
+        taps(LoadTapWindow<C>(p, ya1, col[0].s), topA[1], topB[1]);
+        taps(LoadTapWindow<C>(p, yb1, col[0].s), botA[1], botB[1]);
+    }
+    if (dx0 >= p.dstW)
+    {
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+    {
+        const int dy = y0 + r;
+        if (dy >= p.dstH)
+        {
+            break;
+        }
+        const float    wy = r == 0 ? row0.w[0] : row1.w[0];
+        uint32_t       q[1][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            q[0][j] = BilinearU8<C>(topA[r][j], topB[r][j], botA[r][j], botB[r][j], col[j].w[0], wy);
+        }
+        uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * C;
+        if (dx0 + 4 <= p.dstW)
+        {
+            uint32_t w[C];
+            PackQuad<C>(q, w);
+            StoreDwordsNT<C>(to, w);
+        }
+        else
+        {
+#pragma unroll
+            for (int k = 0; k < 3; ++k)
+            {
+                if (dx0 + k < p.dstW)
+                {
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                    {
+                        to[C * k + c] = (uint8_t)(q[0][k] >> (8 * c));
+                    }
+                }
+            }
+        }
+    }
+}
+
 // Which (type, channels, interpolation) take the two-columns-per-lane form. The code is written for 1, 3
 // and 4 channels; with 1 and 4 it measured slower than the wave patches (u8x1 43 -> 58 us, u8x4 91 -> 104 us
 // on 1080p -> 720p: the column terms of two columns are amortised over 2 rows only), so 3 it is.
@@ -1234,6 +1358,15 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArg
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
     ResizeLinearPairsU8<C, false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+}
+
+constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x 2 rows, stacked
+
+template<int C>
+__global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArgs a)
+{
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizeLinearQuadsU8<C>(p, blockIdx.x * kQuadsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
 }
 
 // Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
@@ -1413,6 +1546,13 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     }
     if constexpr (kPairsForm<T, C, INTERP>)
     {
+        if (a.srcW >= 4 && 3 * (int64_t)a.srcW <= 2 * (int64_t)a.dstW)
+        {
+            dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, kPairsTileH), N);
+            hipLaunchKernelGGL((ResizeLinearQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeLinearQuadsU8Kernel");
+            return;
+        }
         if (a.srcW >= 4 && a.srcW <= 2 * a.dstW)
         {
             dim3 pgrid(DivUp(a.dstW, kPairsTileW), DivUp(a.dstH, kPairsTileH), N);

@@ -89,7 +89,12 @@ PAIRS = [(sw, sh, dw, dh, LINEAR, n, np.uint8, c)
          for c in (3, 1, 4)
          for (sw, sh, dw, dh, n) in [(131, 37, 66, 19, 2), (100, 40, 50, 20, 1), (64, 48, 97, 71, 2), (640, 360, 431, 243, 1),
                                      (33, 9, 130, 30, 1), (5, 4, 7, 3, 3), (4, 4, 2, 2, 1), (257, 33, 129, 17, 1),
-                                     (1280, 720, 1920, 1080, 1), (1920, 1080, 1280, 720, 1)]]
+                                     (1280, 720, 1920, 1080, 1), (1920, 1080, 1280, 720, 1),
+                                     # enlargements by 1.5 or more: four columns per lane; ragged widths, odd heights,
+                                     # the limit itself (3 * src == 2 * dst), one wave's worth and less
+                                     (100, 40, 151, 61, 2), (257, 33, 771, 99, 1), (40, 30, 61, 46, 1), (4, 4, 7, 9, 2),
+                                     (640, 360, 1921, 1079, 1), (86, 20, 129, 30, 1), (171, 7, 257, 11, 1),
+                                     (6, 5, 9, 8, 1), (341, 50, 1023, 75, 1)]]
 
 
 @pytest.mark.parametrize("row", PAIRS, ids=lambda r: "%dx%d-%dx%d-i%d-n%d-%s%d" % (r[:6] + (np.dtype(r[6]).name, r[7])))
