@@ -36,8 +36,8 @@ NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
 # kernel and the workload, not of a run, so it is recorded here rather than re-measured; read and
 # write parts are in the summary files named below. The counters sit between the L2s and the fabric:
 # a batch that fits the memory-side cache (warp-affine-varshape) has part of those reads served there.
-MEASURED_TRAFFIC_BYTES = {"fused": 122961076, "resize-cubic-4k": 1474461132, "resize-nearest": 12234391,
-                          "resize-linear": 23284857, "nv12-to-rgb": 298659913, "warp-affine-varshape": 301970150}
+MEASURED_TRAFFIC_BYTES = {"fused": 122963923, "resize-cubic-4k": 1474458644, "resize-nearest": 12249763,
+                          "resize-linear": 23286608, "nv12-to-rgb": 298655003, "warp-affine-varshape": 299660530}
 # The rocprofv3 counter summary each figure above is the "total" line of (a CPU test compares them).
 TRAFFIC_PROFILES = {"fused": "FusedBilinear_batch64_1080p_to_224",
                     "resize-cubic-4k": "ResizeCubicStagedKernel_f32x4_batch16_4k_to_640x360",
@@ -223,6 +223,7 @@ class ResizeC1:
         name = "NEAREST" if interp == NEAREST else "LINEAR"
         self.key = "resize-" + name.lower()
         self.kernel = "ResizePatchTensorKernel<uint8_t,3,%s>" % name
+        self.dtype = "f32" if interp == NEAREST else "i32"  # index map in float32; bilinear blend in fixed point
         self.workload = "Resize %s: batch %d u8 NHWC 1920x1080 -> 224x224" % (name, self.N)
         self.images = self.N
         rows, _ = span_bytes(self.OUT_H, 0, self.SRC_H, self.OUT_H, interp, 1)
@@ -332,7 +333,7 @@ class WarpC4:
     key, config_id = "warp-affine-varshape", 4
     N = 32
     kernel = "WarpVarShape<uint8_t,3,LINEAR>"
-    dtype = "f32"
+    dtype = "i32"  # coordinates in float32, the 8-bit blend in 15-bit fixed point
     workload = ("WarpAffine var-shape LINEAR: 32 u8 RGB images, W in [640,1920], H in [480,1080], rotation +-30 deg "
                 "x scale 0.8-1.2 about the centre, constant border 0")
 
@@ -447,7 +448,7 @@ class ResizeVarShape:
     key, config_id = "resize-linear-varshape", 1
     N, OUT = 32, 224
     kernel = "ResizePatchVarShapeKernel<uint8_t,3,LINEAR>"
-    dtype = "f32"
+    dtype = "i32"  # coordinates in float32, the 8-bit blend in 15-bit fixed point
     workload = "Resize LINEAR, image batch: 32 u8 RGB images, W in [1280,1920], H in [720,1080] -> 224x224 each"
 
     def __init__(self, cv, orc, np, torch):
@@ -560,10 +561,11 @@ class WarpTensor:
         name = {NEAREST: "NEAREST", LINEAR: "LINEAR", CUBIC: "CUBIC"}[interp]
         self.key = "warp-affine-tensor-" + name.lower()
         self.kernel = "WarpTensor<uint8_t,3,%s>" % name
+        self.dtype = "f32" if interp == NEAREST else "i32"  # coordinates in float32; 8-bit blends in fixed point
         self.workload = "WarpAffine %s: batch 32 u8 NHWC 1280x780x3, rotation 17 deg x scale 1.05, constant border 0" % name
         self.images = self.N
         w, h = self.W, self.H
-        t, sc = math.radians(17.0), 1.05
+        t, sc = math.radians(float(os.environ.get("CVAMD_BENCH_WARP_DEGREES", "17"))), 1.05
         c, sn, cx, cy = sc * math.cos(t), sc * math.sin(t), (w - 1) / 2.0, (h - 1) / 2.0
         self.m = [c, -sn, cx - c * cx + sn * cy, sn, c, cy - sn * cx - c * cy]
         inv = orc.invert_affine(self.m).astype(np.float64)
@@ -692,9 +694,9 @@ class Streaming:
         "flip-horizontal": ("Flip", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "PixelMapTensor<uint8_t,3>", "u8",
                             "Flip (columns mirrored)"),
         "resize-linear-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
-                               "ResizeLinearPairsU8Kernel<3>", "f32", "Resize LINEAR 1920x1080 -> 1280x720"),
+                               "ResizeLinearPairsU8Kernel<3>", "i32", "Resize LINEAR 1920x1080 -> 1280x720"),
         "resize-linear-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
-                                  "ResizeLinearQuadsU8Kernel<3>", "f32", "Resize LINEAR 1280x720 -> 1920x1080"),
+                                  "ResizeLinearQuadsU8Kernel<3>", "i32", "Resize LINEAR 1280x720 -> 1920x1080"),
         "resize-area-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
                              "ResizeTensorKernel<unsigned char,3,3>", "f32", "Resize AREA 1920x1080 -> 1280x720"),
         "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t>>", "f32",
@@ -834,7 +836,7 @@ WORKLOADS.update({k: (lambda *a, k=k: StreamMix(*a, k)) for k in StreamMix.SPECS
 BOUNDS = {"warp-affine-varshape": "valu-issue", "warp-affine-tensor-linear": "valu-issue",
           "warp-affine-tensor-cubic": "valu-issue", "warp-affine-tensor-nearest": "vmem-issue",
           "resize-area-720p": "valu-issue", "cvtcolor-bgr2hsv": "valu-issue",
-          "resize-linear-720p": "vmem-issue", "resize-linear-upscale": "vmem-issue",
+          "resize-linear-720p": "vmem-issue", "resize-linear-upscale": "valu-issue",
           "resize-nearest": "launch-latency", "resize-linear": "launch-latency", "empty-launch": "launch-latency"}
 
 # The other BASELINE configurations, timed after the headline when no --workload is given.
