@@ -1,4 +1,4 @@
-// Resize with nearest / bilinear / bicubic sampling, tensors and var-shape batches.
+// Resize with nearest / bilinear / bicubic / area sampling, tensors and var-shape batches.
 //
 // Index maps and weights follow the reference kernels expression for expression in float32
 // (src/cvcuda/priv/OpResize.cu:142-164 nearest, 177-330 bilinear, 334-388 bicubic;
@@ -7,13 +7,15 @@
 // reference's CPU golden (tests/cvcuda/system/ResizeUtils.cpp:206-221) for every pixel, so results
 // are bit-exact against it also where the coordinate lands on an integer.
 //
-// Four kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
+// Five kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
 //  * u8x3 bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows and fetches each source
 //    row once for both columns, lane pairs swap a pixel pair each;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
-//  * everything else (12/16-byte pixels, AREA): one lane per output pixel, a 256-thread block covers
+//  * AREA of 8-bit pixels at reductions of up to 3: fixed-point row sums, a wave owns 64 columns x 16 rows and
+//    produces vertically adjacent rows in pairs from the source rows they share;
+//  * everything else (12/16-byte pixels, other AREA): one lane per output pixel, a 256-thread block covers
 //    64 columns x 4 rows, pixels moved as whole C-channel vectors.
 #include "DeviceUtils.hpp"
 #include "FixedPointBlend.hpp"
@@ -926,6 +928,52 @@ __device__ __forceinline__ AxisTerms<kWeights<INTERP>> FinishedAxis(float scale,
     return a;
 }
 
+// Stores a wave's 64-column x 4-row patch at (x0, y0): q[d][k] is dword d of the pixel (x0 + lane, y0 + k). After
+// the 4x4 transposes lane l owns row y0 + (l & 3), columns x0 + 4 * (l >> 2) .. + 3, written as whole dwords.
+template<class T, int C>
+__device__ __forceinline__ void StoreWavePatch(const Plane &p, int x0, int y0, int lane,
+                                               uint32_t (&q)[(sizeof(Pixel<T, C>) + 3) / 4][4])
+{
+    constexpr int PB = sizeof(Pixel<T, C>), D = (PB + 3) / 4;
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+    {
+        QuadTranspose(q[d], lane & 3);
+    }
+    const int dy = y0 + (lane & 3), dx0 = x0 + 4 * (lane >> 2);
+    if (dy >= p.dstH || dx0 >= p.dstW)
+    {
+        return;
+    }
+    uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * PB;
+
+    if (dx0 + 4 <= p.dstW)
+    {
+        uint32_t w[PB];
+        PackQuad<PB>(q, w);
+        StoreDwordsNT<PB>(to, w);
+    }
+    else
+    {
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+        {
+            if (dx0 + k < p.dstW)
+            {
+                uint32_t w[D];
+#pragma unroll
+                for (int d = 0; d < D; ++d)
+                {
+                    w[d] = q[d][k];
+                }
+                Pixel<T, C> px;
+                __builtin_memcpy(&px, w, PB);
+                reinterpret_cast<Pixel<T, C> *>(to)[k] = px;
+            }
+        }
+    }
+}
+
 // One wave resizes a 64-column x 4-row patch of the output whose top left pixel is (x0, y0), both
 // wave-uniform. Sampling: lane l owns column x0 + l and computes its 4 rows (the column terms are
 // shared; neighbouring lanes read neighbouring source pixels whatever the scale). Storing: after
@@ -981,42 +1029,7 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
             }
         }
     }
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-    {
-        QuadTranspose(q[d], lane & 3);
-    }
-    const int dy = y0 + (lane & 3), dx0 = x0 + 4 * (lane >> 2);
-    if (dy >= p.dstH || dx0 >= p.dstW)
-    {
-        return;
-    }
-    uint8_t *to = p.dst + (int64_t)dy * p.dstRow + (int64_t)dx0 * PB;
-    if (dx0 + 4 <= p.dstW)
-    {
-        uint32_t w[PB];
-        PackQuad<PB>(q, w);
-        StoreDwordsNT<PB>(to, w);
-    }
-    else
-    {
-#pragma unroll
-        for (int k = 0; k < 3; ++k)
-        {
-            if (dx0 + k < p.dstW)
-            {
-                uint32_t w[D];
-#pragma unroll
-                for (int d = 0; d < D; ++d)
-                {
-                    w[d] = q[d][k];
-                }
-                Pixel<T, C> px;
-                __builtin_memcpy(&px, w, PB);
-                reinterpret_cast<Pixel<T, C> *>(to)[k] = px;
-            }
-        }
-    }
+    StoreWavePatch<T, C>(p, x0, y0, lane, q);
 }
 
 // 8-bit bilinear at horizontal scales up to 2. The cost of the wave-patch form there is the number
@@ -1406,6 +1419,346 @@ __global__ __launch_bounds__(256) void ResizePatchVarShapeKernel(const ResizeArg
     ResizeWavePatch<T, C, INTERP, true>(p, tc.tx * kPatchTileW, tc.ty * kPatchTileH + (threadIdx.x >> 6) * 4);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Box filter (AREA) of 8-bit pixels at reductions of up to 3 along both axes, in fixed point.
+//
+// The weight of a source pixel is the length of its overlap with the box the output pixel covers,
+// [d * scale, d * scale + scale): for scales of 1 and more exactly the reference's left-partial, whole and
+// right-partial weights (cuda_tools/InterpolationWrap.hpp:668-760; each is one float32 subtraction of the
+// same operands), pixels outside the image weigh nothing, and the sum is divided by the length of the box
+// inside the image along each axis. A box of up to 3 touches at most 4 pixels per axis; the window of 4
+// starts at the box's first pixel or, at the image's far edge, 4 before its end (pixels in front of the box
+// then get the weight 0 from the same expression), so a window never leaves its row. Per source row the 4
+// pixels are one load of the dwords that hold them; the horizontal weights, already divided, are rounded to
+// 15 bits and a row's sum is two v_dot2_u32_u16 per channel on bytes (exact, below 2^24); the rows' sums are
+// added in float32 with the rows' weights (wave-uniform), and the result is rounded once.
+//
+// One wave produces 64 columns x 16 rows: lane l owns column l (its terms are computed once), the 16 rows'
+// terms are computed side by side in lanes 0-15 and read back as wave-uniform values, and every 4 rows leave
+// through the 4x4 lane transposes as whole dwords.
+template<class T, int C, int INTERP>
+constexpr bool kAreaFixed = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_AREA && (C == 1 || C == 3 || C == 4);
+
+constexpr int kAreaRowsPerWave = 16;
+constexpr int kAreaTileW = 64, kAreaTileH = 4 * kAreaRowsPerWave; // block = 4 waves stacked vertically
+
+// Per image: both scales within 1 .. 3 and a source of at least 4 rows of at least 32 bytes.
+__host__ __device__ __forceinline__ bool AreaFixedDomain(float scaleX, float scaleY, int srcRowBytes, int srcH)
+{
+    return scaleX >= 1.f && scaleX <= 3.f && scaleY >= 1.f && scaleY <= 3.f && srcRowBytes >= 32 && srcH >= 4;
+}
+
+// Weights of the 4 source indices from `start` on (a whole number) for output index d: each one's overlap with
+// the box, divided by the box's length inside the image, times `unit`. The overlap of index x is written
+// clamp(f2 - x, 0, 1) - clamp(f1 - x, 0, 1) (a clamp is one v_med3_f32): for an index the box
+// covers partly, wholly or not at all that is f2 - x or (x + 1) - f1 (both exact), 1, or 0. With `bounded`,
+// indices behind the image weigh nothing (callers that pass a start of at most srcSize - 4 need no test).
+__device__ __forceinline__ void AreaWeights(float scale, int d, int srcSize, float unit, float start, bool bounded, float (&w)[4])
+{
+    const float f1 = d * scale, end = f1 + scale;
+    const float f2 = bounded ? fminf(end, (float)srcSize) : end;
+    const float norm = (1.f / fminf(scale, srcSize - f1)) * unit;
+    float       x = start;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        w[k] = (__builtin_amdgcn_fmed3f(f2 - x, 0.f, 1.f) - __builtin_amdgcn_fmed3f(f1 - x, 0.f, 1.f)) * norm;
+        x += 1.f;
+    }
+}
+
+// The window's bytes: D dwords that hold the 4 pixels at byte offset `at` + `shift` of the row (shift 0 .. 3;
+// 4 channels: none), brought to the front: pixel k, channel c in byte k * C + c.
+template<int C, bool GUARDED>
+__device__ __forceinline__ void LoadAreaWindow(const uint8_t *row, uint32_t at, uint32_t shift, bool lastRow, uint32_t rowBytes,
+                                               uint32_t (&r)[C])
+{
+    constexpr int D = C == 4 ? 4 : C + 1;
+    struct __attribute__((packed, aligned(1))) Window
+    {
+        uint32_t d[D];
+    };
+    if constexpr (C == 4)
+    {
+        const Window w = *reinterpret_cast<const Window *>(row + at);
+        __builtin_memcpy(r, &w, 16);
+    }
+    else
+    {
+        // the load runs up to 4 bytes past the window, harmless except behind the image's last row, where it is
+        // moved back to end with the row (GUARDED: the rows passed may include that one)
+        bool whole = false;
+        if (GUARDED && lastRow)
+        {
+            const uint32_t back = min(at, rowBytes - 4 * D);
+            shift += at - back; // up to 4
+            at    = back;
+            whole = shift == 4;
+            shift = whole ? 0 : shift;
+        }
+        const Window w = *reinterpret_cast<const Window *>(row + at);
+#pragma unroll
+        for (int i = 0; i < C; ++i)
+        {
+            r[i] = __builtin_amdgcn_alignbyte(w.d[i + 1], w.d[i], shift);
+            if constexpr (GUARDED)
+            {
+                r[i] = whole ? w.d[i + 1] : r[i];
+            }
+        }
+    }
+}
+
+// Channel c of pixels ka and ka + 1 of such a window as (first | second << 16).
+template<int C>
+__device__ __forceinline__ uint32_t AreaTapPair(const uint32_t (&r)[C], int ka, int c)
+{
+    const int      b0 = ka * C + c, b1 = b0 + C, j = b0 / 4;
+    const uint32_t sel = 0x0c000c00u | (uint32_t)(b0 - 4 * j) | ((uint32_t)(b1 - 4 * j) << 16);
+    return __builtin_amdgcn_perm(r[j + 1 < C ? j + 1 : C - 1], r[j], sel);
+}
+
+__device__ __forceinline__ uint32_t Dot2U16(uint32_t taps, uint32_t weights, uint32_t acc)
+{
+    typedef unsigned short U16x2 __attribute__((ext_vector_type(2)));
+    U16x2 t, w;
+    __builtin_memcpy(&t, &taps, 4);
+    __builtin_memcpy(&w, &weights, 4);
+    return __builtin_amdgcn_udot2(t, w, acc, false);
+}
+
+// A source row's sums per channel from its window and the packed horizontal weights.
+template<int C>
+__device__ __forceinline__ void AreaRowSums(const uint32_t (&r)[C], uint32_t w01, uint32_t w23, float (&s)[C])
+{
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        s[c] = (float)Dot2U16(AreaTapPair<C>(r, 2, c), w23, Dot2U16(AreaTapPair<C>(r, 0, c), w01, 0u));
+    }
+}
+
+// K output pixels per lane (vertically adjacent) from N source rows, the first at `row`; wy[k][j] is the weight of
+// source row j in output pixel k. All N windows are requested before the first sum; every row's sums are formed once.
+// Rows are added in ascending order, the first as a product, the others with fused multiply-adds: a row of weight 0
+// changes nothing, so the result does not depend on which rows are passed beside those of the pixel's box.
+template<int C, int N, int K, bool GUARDED>
+__device__ __forceinline__ void AreaFixedPixels(const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
+                                                uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
+                                                uint32_t (&out)[K])
+{
+    uint32_t r[N][C];
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+    {
+        LoadAreaWindow<C, GUARDED>(row + (int64_t)j * srcRow, at, shift, j == lastRowIn, rowBytes, r[j]);
+    }
+    float acc[K][C];
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+    {
+        float s[C];
+        AreaRowSums<C>(r[j], w01, w23, s);
+#pragma unroll
+        for (int k = 0; k < K; ++k)
+        {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                acc[k][c] = j == 0 ? s[c] * wy[k][0] : fmaf(s[c], wy[k][j], acc[k][c]);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+    {
+        out[k] = 0;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            out[k] = __builtin_amdgcn_cvt_pk_u8_f32(acc[k][c], c, out[k]);
+        }
+    }
+}
+
+template<int C, int K, bool GUARDED>
+__device__ __forceinline__ void AreaFixedRowsOf(int n, const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
+                                                uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
+                                                uint32_t (&out)[K])
+{
+    // (wave-uniform)
+    if (n == 3)
+    {
+        AreaFixedPixels<C, 3, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+    }
+    else if (n == 2)
+    {
+        AreaFixedPixels<C, 2, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+    }
+    else if (n == 4)
+    {
+        AreaFixedPixels<C, 4, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+    }
+    else
+    {
+        AreaFixedPixels<C, 1, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+    }
+}
+
+// n source rows from `row` on; lastRowIn: which of them is the image's last row (n or more: none).
+template<int C, int K>
+__device__ __forceinline__ void AreaFixedRows(int n, const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
+                                              uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
+                                              uint32_t (&out)[K])
+{
+    if (C != 4 && lastRowIn < n) // wave-uniform, once per image and column tile
+    {
+        AreaFixedRowsOf<C, K, true>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+    }
+    else
+    {
+        AreaFixedRowsOf<C, K, false>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+    }
+}
+
+__device__ __forceinline__ float ReadLane(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// The tile of 64 columns x 16 rows whose top left pixel is (x0, y0), both wave-uniform (y0 even).
+template<int C>
+__device__ __forceinline__ void ResizeAreaFixedWaveTile(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    const int lane = threadIdx.x & 63;
+    // columns and rows past the output compute a duplicate of the last one: every lane takes part in the transposes
+    const int   dx = min(x0 + lane, p.dstW - 1);
+    const float colStart = fminf(floorf(dx * p.scaleX), (float)(p.srcW - 4)); // the window never leaves its row
+    float       cw[4];
+    AreaWeights(p.scaleX, dx, p.srcW, 32768.f, colStart, false, cw);
+    // rounding to an integer by adding 1.5 * 2^23: the low 16 bits of the sum's pattern are the integer
+    uint32_t wq[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        wq[k] = __float_as_uint(cw[k] + 12582912.f);
+    }
+    const uint32_t w01 = __builtin_amdgcn_perm(wq[1], wq[0], 0x05040100u), w23 = __builtin_amdgcn_perm(wq[3], wq[2], 0x05040100u);
+    const uint32_t off = (uint32_t)(int)colStart * C, at = C == 4 ? off : off & ~3u, shift = off & 3u;
+    const uint32_t rowBytes = (uint32_t)p.srcW * C;
+
+    // Row terms, lane l: output row y0 + (l & 15). Two vertically adjacent output rows (2i, 2i + 1) share the source
+    // row between their boxes wherever the scale is not a whole number, so they are produced together from the
+    // source rows first(2i) .. first(2i) + n - 1 when those are at most 4 (`pairRows`, else 0): `pw` are this row's
+    // weights counted from first(2i). Otherwise each row on its own from its box's first row: `ow`, `ownRows`.
+    const int   dy = min(y0 + (lane & (kAreaRowsPerWave - 1)), p.dstH - 1);
+    const float ownStart = floorf(dy * p.scaleY), pairStart = floorf((dy & ~1) * p.scaleY);
+    float       ow[4], pw[4];
+    AreaWeights(p.scaleY, dy, p.srcH, 1.f / 32768.f, ownStart, true, ow);
+    AreaWeights(p.scaleY, dy, p.srcH, 1.f / 32768.f, pairStart, true, pw);
+    const int  ownRows = 1 + (ow[1] != 0.f) + (ow[2] != 0.f) + (ow[3] != 0.f);
+    const bool fits    = fminf(dy * p.scaleY + p.scaleY, (float)p.srcH) <= pairStart + 4.f;
+    const int  pairRows = !fits ? 0 : pw[3] != 0.f ? 4 : pw[2] != 0.f ? 3 : pw[1] != 0.f ? 2 : 1;
+    const int  ownFirst = (int)ownStart, pairFirst = (int)pairStart;
+
+    const int rowsHere = min(kAreaRowsPerWave, p.dstH - y0);
+    uint32_t  q[1][4] = {};
+#pragma unroll 1
+    for (int i = 0; i < rowsHere; i += 2)
+    {
+        const int n = __builtin_amdgcn_readlane(pairRows, i + 1);
+        uint32_t  out[2];
+        if (n != 0)
+        {
+            const int first = __builtin_amdgcn_readlane(pairFirst, i);
+            float     wy[2][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                wy[0][j] = ReadLane(pw[j], i);
+                wy[1][j] = ReadLane(pw[j], i + 1);
+            }
+            AreaFixedRows<C, 2>(n, p.src + (int64_t)first * p.srcRow, p.srcRow, p.srcH - 1 - first, at, shift, rowBytes, w01,
+                                w23, wy, out);
+        }
+        else
+        {
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+            {
+                const int first = __builtin_amdgcn_readlane(ownFirst, i + k);
+                float     wy[1][4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    wy[0][j] = ReadLane(ow[j], i + k);
+                }
+                uint32_t one[1];
+                AreaFixedRows<C, 1>(__builtin_amdgcn_readlane(ownRows, i + k), p.src + (int64_t)first * p.srcRow, p.srcRow,
+                                    p.srcH - 1 - first, at, shift, rowBytes, w01, w23, wy, one);
+                out[k] = one[0];
+            }
+        }
+        const bool upper = (i & 2) == 0; // rows 0, 1 or 2, 3 of the group of 4 that is stored together
+        q[0][0]          = upper ? out[0] : q[0][0];
+        q[0][1]          = upper ? out[1] : q[0][1];
+        q[0][2]          = upper ? q[0][2] : out[0];
+        q[0][3]          = upper ? q[0][3] : out[1];
+        if (!upper)
+        {
+            StoreWavePatch<uint8_t, C>(p, x0, y0 + (i & ~3), lane, q);
+        }
+    }
+    // an odd pair of rows at the lower edge of the output: rows 2, 3 of the group duplicate what is not stored
+    if ((((rowsHere + 1) >> 1) & 1) != 0)
+    {
+        StoreWavePatch<uint8_t, C>(p, x0, y0 + ((rowsHere - 1) & ~3), lane, q);
+    }
+}
+
+// The same tile outside the fixed-point form's scales (image batches decide per image): one pixel at a time.
+template<int C, bool VARSHAPE>
+__device__ __forceinline__ void ResizeAreaPlainWaveTile(const Plane &p, int x0, int y0)
+{
+    const int dx = x0 + (int)(threadIdx.x & 63);
+    if (dx >= p.dstW)
+    {
+        return;
+    }
+#pragma unroll 1
+    for (int dy = y0; dy < min(y0 + kAreaRowsPerWave, p.dstH); ++dy)
+    {
+        ResizePixel<uint8_t, C, NVCV_INTERP_AREA, VARSHAPE>(p, dx, dy);
+    }
+}
+
+template<int C>
+__global__ __launch_bounds__(256) void ResizeAreaFixedTensorKernel(const ResizeArgs a)
+{
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizeAreaFixedWaveTile<C>(p, blockIdx.x * kAreaTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kAreaRowsPerWave);
+}
+
+template<int C>
+__global__ __launch_bounds__(256) void ResizeAreaVarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc = LocateTile(tiles, blockIdx.x);
+    const Plane     p  = GetPlanes<true>(a, tc.image);
+    const int       x0 = tc.tx * kAreaTileW, y0 = tc.ty * kAreaTileH + (threadIdx.x >> 6) * kAreaRowsPerWave;
+    if (AreaFixedDomain(p.scaleX, p.scaleY, p.srcW * C, p.srcH))
+    {
+        ResizeAreaFixedWaveTile<C>(p, x0, y0);
+    }
+    else
+    {
+        ResizeAreaPlainWaveTile<C, true>(p, x0, y0);
+    }
+}
+
 // Bicubic for strong horizontal reductions. With one lane per output pixel the four taps of
 // neighbouring lanes lie scale*pixel bytes apart, so each of a wave's tap loads touches 64 separate
 // cache lines. Here the same 256 taps of a wave's row are fetched tap-major instead: lane l loads
@@ -1561,6 +1914,16 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             return;
         }
     }
+    if constexpr (kAreaFixed<T, C, INTERP>)
+    {
+        if (AreaFixedDomain(a.scaleX, a.scaleY, a.srcW * C, a.srcH))
+        {
+            dim3 agrid(DivUp(a.dstW, kAreaTileW), DivUp(a.dstH, kAreaTileH), N);
+            hipLaunchKernelGGL((ResizeAreaFixedTensorKernel<C>), agrid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeAreaFixedTensorKernel");
+            return;
+        }
+    }
     if constexpr (kPatchForm<T, C, INTERP>)
     {
         // a launch of under 8 four-wave blocks per CU is spread as single-wave blocks: it is latency-bound
@@ -1590,6 +1953,16 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, 
             {
                 hipLaunchKernelGGL((ResizeLinearPairsU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
                 CheckLaunch("ResizeLinearPairsU8VarShapeKernel");
+            }
+            continue;
+        }
+        if constexpr (kAreaFixed<T, C, INTERP>)
+        {
+            int total = BuildVarTiles(tiles, dstHost, first, count, kAreaTileW, kAreaTileH);
+            if (total > 0)
+            {
+                hipLaunchKernelGGL((ResizeAreaVarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeAreaVarShapeKernel");
             }
             continue;
         }

@@ -343,6 +343,72 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
         return;
     }
     const float scaleX = static_cast<float>(srcW) / dstW, scaleY = static_cast<float>(srcH) / dstH;
+    if (variant == 5 || variant == 6)
+    {
+        // the product library's 8-bit box filter at reductions of up to 3 (sources of 4 rows of 32 bytes or more):
+        // a source pixel's weight along an axis is its overlap with the box [d * scale, d * scale + scale) - for
+        // scales of 1 and more the same float32 differences as in variants 1 and 2 -, nothing outside the image,
+        // divided by the length of the box inside the image. Horizontal weights rounded to multiples of 2^-15 (to nearest,
+        // ties to even), a row's sum exact in integers; the rows' sums added in ascending order with fused
+        // multiply-adds (the first is a product); one rounding to nearest-even. Outside those scales:
+        // variant 1 (5) or 2 (6).
+        if (std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4) && scaleX >= 1.f && scaleX <= 3.f && scaleY >= 1.f
+            && scaleY <= 3.f && srcW * C >= 32 && srcH >= 4)
+        {
+            struct Axis
+            {
+                int   first;
+                float w[4];
+            };
+            auto box = [](float scale, int d, int size, float unit, bool window)
+            {
+                Axis        a;
+                auto        clamp01 = [](float v) { return std::fmin(std::fmax(v, 0.f), 1.f); };
+                const float f1 = d * scale, end = f1 + scale;
+                const float f2 = window ? end : std::fmin(end, (float)size); // rows: nothing behind the image
+                const float ff = window ? std::fmin(std::floor(f1), (float)(size - 4)) : std::floor(f1);
+                const float norm = (1.f / std::fmin(scale, size - f1)) * unit;
+                a.first = (int)ff;
+                for (int k = 0; k < 4; ++k)
+                {
+                    // the overlap of pixel x with the box: f2 - x or (x + 1) - f1 for a partly covered one (both
+                    // exact), 1 or 0
+                    const float x = ff + (float)k;
+                    a.w[k]        = (clamp01(f2 - x) - clamp01(f1 - x)) * norm;
+                }
+                return a;
+            };
+            // columns: the 4 pixels from the box's first one on, or the image's last 4 where that is earlier;
+            // rows: from the box's first one on, none behind the image
+            const Axis col = box(scaleX, dx, srcW, 32768.f, true), row = box(scaleY, dy, srcH, 1.f / 32768.f, false);
+            uint32_t   wq[4];
+            for (int k = 0; k < 4; ++k)
+            {
+                wq[k] = (uint32_t)std::nearbyint(col.w[k]);
+            }
+            for (int c = 0; c < C; ++c)
+            {
+                float acc = 0.f;
+                for (int j = 0; j < 4; ++j)
+                {
+                    if (j > 0 && row.w[j] == 0.f)
+                    {
+                        continue;
+                    }
+                    uint32_t sum = 0;
+                    for (int k = 0; k < 4; ++k)
+                    {
+                        sum += (uint32_t)src[(row.first + j) * srcStep + (int64_t)(col.first + k) * C + c] * wq[k];
+                    }
+                    acc = j == 0 ? (float)sum * row.w[j] : std::fmaf((float)sum, row.w[j], acc);
+                }
+                const float v = std::nearbyint(acc);
+                out[c]        = (T)(v < 0.f ? 0.f : (v > 255.f ? 255.f : v));
+            }
+            return;
+        }
+        variant = variant == 5 ? 1 : 2;
+    }
     const float fsx1 = dx * scaleX, fsy1 = dy * scaleY, fsx2 = fsx1 + scaleX, fsy2 = fsy1 + scaleY;
     const int   xmin = (int)std::ceil(fsx1), xmax = (int)std::floor(fsx2);
     const int   ymin = (int)std::ceil(fsy1), ymax = (int)std::floor(fsy2);

@@ -48,6 +48,9 @@ def cases():
                 if interp == LINEAR and dt == np.uint8:
                     # the shipped 8-bit bilinear blend (15-bit fixed point), to be reproduced bit for bit
                     out["resize_linear_fixed_uint8%d_%s" % (c, tag)] = orc.resize(a, hw, interp, variant=4)
+                if interp == AREA and dt == np.uint8 and tag == "down":
+                    # the shipped 8-bit box filter at reductions of up to 3 (fixed-point rows), bit for bit
+                    out["resize_area_fixed_uint8%d_down" % c] = orc.resize(a, hw, interp, variant=5)
     y = recipe(2, 12, 16, 1, step=9)[..., 0] // 2 + 60
     uv = recipe(2, 6, 16, 1, step=13)[..., 0] // 2 + 60
     nv = np.concatenate([y, uv], axis=1)

@@ -8,7 +8,7 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-NEAREST, LINEAR, CUBIC = 0, 1, 2
+NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
 
 
 def device_u8(gpu, shape, seed):
@@ -99,6 +99,21 @@ def test_resize_and_warp_identities_on_a_1080p_batch(cv, K, gpu):
     mean = (blocks[:, :, 0, :, 0] * 0.25 + blocks[:, :, 0, :, 1] * 0.25 + blocks[:, :, 1, :, 0] * 0.25
             + blocks[:, :, 1, :, 1] * 0.25)
     assert torch.equal(half.torch_view(), torch.round(mean).to(torch.uint8))
+    # the box filter of an exact 2x reduction is the same block mean (weights 2^-1 per axis, nothing rounded before
+    # the last step), and at equal sizes it is a copy
+    cv.Resize()(None, tin, half, AREA)
+    assert torch.equal(half.torch_view(), torch.round(mean).to(torch.uint8))
+    out.torch_view().zero_()
+    cv.Resize()(None, tin, out, AREA)
+    assert torch.equal(out.torch_view(), src)
+    # 1080p -> 720p (scale 1.5): output pixel (2i, 2j) covers source pixel (3i, 3j) and half of the next along each
+    # axis, so with weights 4/9, 2/9, 2/9, 1/9 it is within rounding of that sum everywhere
+    small = cv.Tensor.alloc([n, 720, 1280, 3], np.uint8, "NHWC")
+    cv.Resize()(None, tin, small, AREA)
+    f = src.double()
+    want = (4 * f[:, 0::3, 0::3] + 2 * f[:, 0::3, 1::3] + 2 * f[:, 1::3, 0::3] + f[:, 1::3, 1::3]) / 9
+    got = small.torch_view()[:, 0::2, 0::2].double()
+    assert float((got - want).abs().max()) <= 0.5 + 1e-2
     # warps: the identity map, and a whole-pixel shift with a constant border
     warp = cv.WarpAffine(0)
     for interp in (NEAREST, LINEAR, CUBIC):

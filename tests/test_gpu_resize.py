@@ -214,8 +214,9 @@ AREA_ROWS = [(44, 40, 22, 20, 2, np.uint8, 4), (30, 30, 20, 20, 2, np.uint8, 4),
 @pytest.mark.parametrize("row", AREA_ROWS, ids=lambda r: "%dx%d-%dx%d-n%d-%s%d" % (r[:5] + (np.dtype(r[5]).name, r[6])))
 def test_area_tensor(cv, orc, gpu, row):
     # box-filter resize, tensors (reference rows TestOpResize.cpp:67-78 plus other types and the
-    # 1080p -> 224 case): <= 1 LSB against the float64 golden, and against the float32 device-order
-    # restatement within float rounding of the long sums
+    # 1080p -> 224 case): <= 1 LSB against the float64 golden, and against the restatement of the shipped
+    # arithmetic (8-bit pixels at reductions of up to 3: the fixed-point form; otherwise the reference's device
+    # order in float32) exactly for integers, within float rounding of the long sums for float32
     sw, sh, dw, dh, n, dt, c = row
     src = make_input(orc, (n, sh, sw, c), dt, 0xA0EA + sw + dh)
     tout = cv.Tensor.alloc([n, dh, dw, c], dt, "NHWC")
@@ -223,7 +224,7 @@ def test_area_tensor(cv, orc, gpu, row):
     torch.cuda.synchronize()
     res = tout.numpy()
     golden = orc.resize(src, (dh, dw), AREA, variant=0, threads=8)
-    device = orc.resize(src, (dh, dw), AREA, variant=1, threads=8)
+    device = orc.resize_shipped(src, (dh, dw), AREA, threads=8)
     if dt == np.float32:
         assert np.abs(res - device).max() <= 1e-5 and np.abs(res - golden).max() <= 1e-4
     else:
@@ -270,7 +271,7 @@ def test_area_varshape(cv, K, orc, gpu, dt, c):
     for a, o, (sw, sh, dw, dh) in zip(hosts, outs, sizes):
         res = o.plane_view(0, dt, c).cpu().numpy()[None]
         golden = orc.resize(a[None], (dh, dw), AREA, variant=3)
-        device = orc.resize(a[None], (dh, dw), AREA, variant=2)
+        device = orc.resize_shipped(a[None], (dh, dw), AREA, varshape=True)
         if dt == np.float32:
             assert np.abs(res - device).max() <= 1e-5 and np.abs(res - golden).max() <= 1e-4
         else:

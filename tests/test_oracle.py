@@ -9,7 +9,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-NEAREST, LINEAR, CUBIC = 0, 1, 2
+NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
 
 
 # ------------------------------------------------------------------------------------------ saturate
@@ -174,6 +174,53 @@ def test_resize_cubic_edge_quirk(orc):
     img = np.tile(np.arange(w, dtype=np.float32), (12, 1)).reshape(1, 12, w, 1)
     out = orc.resize(img, (12, 20), CUBIC, 1)[0, :, :, 0]
     assert np.all(out[:, 0] == 1.0)
+
+
+
+def _box_filter_float64(src, dh, dw):
+    """Area resize straight from its definition, in float64: output pixel (i, j) is the mean of the source over the
+    rectangle [j * sw / dw, (j + 1) * sw / dw) x [i * sh / dh, (i + 1) * sh / dh), pixels as unit squares."""
+    n, sh, sw, c = src.shape
+
+    def overlaps(s, d):
+        edges = np.arange(d + 1, dtype=np.float64) * (s / d)
+        lo, hi = edges[:-1, None], edges[1:, None]
+        x = np.arange(s, dtype=np.float64)[None, :]
+        w = np.clip(np.minimum(x + 1, hi) - np.maximum(x, lo), 0, None)
+        return w / w.sum(axis=1, keepdims=True)
+
+    return np.einsum("iy,nyxc,jx->nijc", overlaps(sh, dh), src.astype(np.float64), overlaps(sw, dw))
+
+
+def test_resize_area_fixed_point_variant(orc):
+    # Variants 5 and 6 (the product library's 8-bit box filter at reductions of up to 3) against the definition of
+    # the box filter in float64: never more than 1 apart, equal wherever the exact value is further than 0.03 from a
+    # rounding boundary (the horizontal weights are rounded to 2^-15: 4 * 255 * 2^-16 < 0.02), and equal to the
+    # exact mean for the 2x reduction (weights 2^-1, nothing rounded before the end) and for equal sizes (a copy).
+    # A dropped or misplaced partial pixel, a wrong normalisation at the image's far edge or a weight table shifted
+    # by one fails the first two.
+    rng = np.random.default_rng(55)
+    for (sw, sh, dw, dh, c) in [(97, 61, 61, 40, 3), (90, 70, 31, 24, 4), (97, 61, 61, 40, 1), (50, 40, 17, 14, 3),
+                                (120, 90, 47, 31, 3), (48, 27, 20, 13, 3), (64, 36, 43, 24, 3), (11, 4, 4, 2, 3)]:
+        src = rng.integers(0, 256, (2, sh, sw, c), dtype=np.uint8)
+        exact = _box_filter_float64(src, dh, dw)
+        for variant in (5, 6):
+            got = orc.resize(src, (dh, dw), AREA, variant=variant)
+            assert np.abs(got - exact).max() <= 0.5 + 0.03, (sw, sh, dw, dh, c, variant)
+            clear = np.abs(exact - np.floor(exact) - 0.5) > 0.03
+            np.testing.assert_array_equal(got[clear], np.rint(exact)[clear].astype(np.uint8))
+    src = rng.integers(0, 256, (1, 40, 64, 3), dtype=np.uint8)
+    blocks = src.astype(np.float64).reshape(1, 20, 2, 32, 2, 3)
+    np.testing.assert_array_equal(orc.resize(src, (20, 32), AREA, variant=5), np.rint(blocks.mean(axis=(2, 4))).astype(np.uint8))
+    np.testing.assert_array_equal(orc.resize(src, (40, 64), AREA, variant=5), src)
+    const = np.full((1, 33, 70, 3), 201, np.uint8)
+    assert np.unique(orc.resize(const, (14, 37), AREA, variant=5)).tolist() == [201]
+    # outside the form's scales (an enlargement, a reduction beyond 3, a source of under 32 bytes per row) the
+    # variants are the device formulas
+    for (sw, sh, dw, dh) in [(30, 30, 60, 60), (97, 61, 13, 9), (9, 40, 5, 20)]:
+        src = rng.integers(0, 256, (1, sh, sw, 3), dtype=np.uint8)
+        np.testing.assert_array_equal(orc.resize(src, (dh, dw), AREA, variant=5), orc.resize(src, (dh, dw), AREA, variant=1))
+        np.testing.assert_array_equal(orc.resize(src, (dh, dw), AREA, variant=6), orc.resize(src, (dh, dw), AREA, variant=2))
 
 
 def test_resize_cubic_hand_weights_interior_and_border_row(orc):
