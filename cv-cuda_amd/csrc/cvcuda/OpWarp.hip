@@ -676,6 +676,38 @@ __device__ __forceinline__ uint32_t SampleInsideQ15(const Img &im, float sx, flo
     return q;
 }
 
+// SampleWithBorder's fixed-point bilinear sum for the two border modes that need no division - a constant
+// colour (`constant`: borderPx, channel c in byte c) or the nearest pixel of the image -, straight-line: the
+// four taps are fetched at coordinates clamped into the image and, for the constant border, replaced where the
+// unclamped coordinate is outside. sx, sy in units of 2^-15 pixel, below 2^30 in magnitude. Same weights, same
+// exact sum and the same single rounding as the generic path, so which path a sample takes does not show.
+template<int C>
+__device__ __forceinline__ uint32_t SampleNearBorderQ15(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
+{
+    const int X = __float2int_rd(sx), Y = __float2int_rd(sy);
+    const int x0 = X >> 15, y0 = Y >> 15;
+    const int cx0 = min(max(x0, 0), im.w - 1), cx1 = min(max(x0 + 1, 0), im.w - 1);
+    const int cy0 = min(max(y0, 0), im.h - 1), cy1 = min(max(y0 + 1, 0), im.h - 1);
+    // a pixel is fetched with one 4-byte load, moved back where it would run past the image's last byte
+    const uint32_t lastLoad = (uint32_t)__mul24(im.h - 1, im.row) + (uint32_t)im.w * C - 4;
+    auto pixel = [&](int x, int y) -> uint32_t
+    {
+        const uint32_t at = PixelOffset<C>(im, x, y), from = min(at, lastLoad);
+        return LoadU32Unaligned(im.base + from) >> (8 * (at - from));
+    };
+    uint32_t p00 = pixel(cx0, cy0), p01 = pixel(cx1, cy0), p10 = pixel(cx0, cy1), p11 = pixel(cx1, cy1);
+    if (constant) // uniform
+    {
+        const bool inX0 = (uint32_t)x0 < (uint32_t)im.w, inX1 = (uint32_t)(x0 + 1) < (uint32_t)im.w;
+        const bool inY0 = (uint32_t)y0 < (uint32_t)im.h, inY1 = (uint32_t)(y0 + 1) < (uint32_t)im.h;
+        p00             = inX0 && inY0 ? p00 : borderPx;
+        p01             = inX1 && inY0 ? p01 : borderPx;
+        p10             = inX0 && inY1 ? p10 : borderPx;
+        p11             = inX1 && inY1 ? p11 : borderPx;
+    }
+    return BilinearQ15<C>(p00, p01, p10, p11, (uint32_t)X & (kQ15 - 1), (uint32_t)Y & (kQ15 - 1));
+}
+
 // The dwords of the pixel that SampleInside gives. u8 channels are rounded, saturated and placed into
 // their byte by one instruction each (v_cvt_pk_u8_f32 with a byte select and the dword so far), where
 // packing converted bytes takes as many shifts and merges again.
@@ -813,6 +845,29 @@ __device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, fl
     }
 }
 
+// Whether a lane's samples can take SampleNearBorderQ15: 8-bit bilinear, one of its two border modes, rows and
+// columns within its 24-bit offsets and 16-bit coordinates (the caller's test), an image of 4 bytes or more, and
+// every coordinate (times 2^15) below 2^30 in magnitude.
+template<class T, int C, int INTERP>
+__device__ __forceinline__ bool NearBorderForm(const Img &im, const WarpArgs &a, const float (&sx)[kPxPerLane],
+                                               const float (&sy)[kPxPerLane])
+{
+    if constexpr (!kFixedPoint<T, INTERP>)
+    {
+        return false;
+    }
+    else
+    {
+        uint32_t u = 0;
+#pragma unroll
+        for (int k = 0; k < kPxPerLane; ++k)
+        {
+            u = max(u, max(__float_as_uint(sx[k]) & 0x7fffffffu, __float_as_uint(sy[k]) & 0x7fffffffu));
+        }
+        return a.border <= NVCV_BORDER_REPLICATE && u < 0x4e800000u /* the pattern of 2^30 */ && (im.h > 1 || im.w * C >= 4);
+    }
+}
+
 // One 64 x 16 tile of the destination image `dst` (tile coordinates tx, ty), all 256 threads.
 template<class T, int C, int INTERP, bool PERSP>
 __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const float (&m)[9], uint8_t *dst, int dstRow,
@@ -830,7 +885,8 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     uint32_t    q[D][kPxPerLane]; // q[d][k]: dword d of this lane's pixel in patch k
     // rows too long or too many for 24-bit offset arithmetic go through the generic path
     // (and, in fixed point, coordinates too large for coordinate * 2^15 in 31 bits)
-    bool allInside = (im.row | im.h) < (1 << 23) && (!kFixedPoint<T, INTERP> || (im.w | im.h) < (1 << 16));
+    const bool fits = (im.row | im.h) < (1 << 23) && (!kFixedPoint<T, INTERP> || (im.w | im.h) < (1 << 16));
+    bool       allInside = fits;
 #pragma unroll
     for (int k = 0; k < kPxPerLane; ++k)
     {
@@ -856,6 +912,45 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
             for (int d = 0; d < D; ++d)
             {
                 q[d][k] = w[k][d];
+            }
+        }
+    }
+    else if (fits && NearBorderForm<T, C, INTERP>(im, a, sx, sy))
+    {
+        // 8-bit bilinear under a constant or replicating border: the border logic as selects, all four samples
+        // in flight (the generic loop below costs a wave that straddles the image's edge about 4 times as much)
+        if constexpr (kFixedPoint<T, INTERP>)
+        {
+            uint32_t borderPx = 0;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                borderPx |= (uint32_t)BorderValueAs<T>(a.bval[c]) << (8 * c);
+            }
+            // under a constant border a lane whose samples lie outside with all their taps takes the colour itself
+            // (the weights add up to exactly 1): whole waves in the corners a rotation leaves empty
+            const bool constant = a.border == NVCV_BORDER_CONSTANT;
+            bool       outside  = constant;
+#pragma unroll
+            for (int k = 0; k < kPxPerLane; ++k)
+            {
+                outside &= TapsOutside<INTERP>(im, sx[k] * (1.f / kScale), sy[k] * (1.f / kScale));
+            }
+            if (outside)
+            {
+#pragma unroll
+                for (int k = 0; k < kPxPerLane; ++k)
+                {
+                    q[0][k] = borderPx;
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int k = 0; k < kPxPerLane; ++k)
+                {
+                    q[0][k] = SampleNearBorderQ15<C>(im, constant, borderPx, sx[k], sy[k]);
+                }
             }
         }
     }
