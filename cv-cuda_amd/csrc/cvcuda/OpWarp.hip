@@ -681,21 +681,25 @@ __device__ __forceinline__ uint32_t SampleInsideQ15(const Img &im, float sx, flo
 // four taps are fetched at coordinates clamped into the image and, for the constant border, replaced where the
 // unclamped coordinate is outside. sx, sy in units of 2^-15 pixel, below 2^30 in magnitude. Same weights, same
 // exact sum and the same single rounding as the generic path, so which path a sample takes does not show.
+// Pixel (x, y) of an 8-bit image, inside it, as a dword (channel c in byte c, the rest is not looked at): one
+// 4-byte load, moved back where it would run past the image's last byte.
+template<int C>
+__device__ __forceinline__ uint32_t LoadPixelGuarded(const Img &im, uint32_t rowOffset, int x)
+{
+    const uint32_t lastLoad = (uint32_t)__mul24(im.h - 1, im.row) + (uint32_t)im.w * C - 4;
+    const uint32_t at = rowOffset + (uint32_t)x * C, from = min(at, lastLoad);
+    return LoadU32Unaligned(im.base + from) >> (8 * (at - from));
+}
+
 template<int C>
 __device__ __forceinline__ uint32_t SampleNearBorderQ15(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
 {
     const int X = __float2int_rd(sx), Y = __float2int_rd(sy);
     const int x0 = X >> 15, y0 = Y >> 15;
     const int cx0 = min(max(x0, 0), im.w - 1), cx1 = min(max(x0 + 1, 0), im.w - 1);
-    const int cy0 = min(max(y0, 0), im.h - 1), cy1 = min(max(y0 + 1, 0), im.h - 1);
-    // a pixel is fetched with one 4-byte load, moved back where it would run past the image's last byte
-    const uint32_t lastLoad = (uint32_t)__mul24(im.h - 1, im.row) + (uint32_t)im.w * C - 4;
-    auto pixel = [&](int x, int y) -> uint32_t
-    {
-        const uint32_t at = PixelOffset<C>(im, x, y), from = min(at, lastLoad);
-        return LoadU32Unaligned(im.base + from) >> (8 * (at - from));
-    };
-    uint32_t p00 = pixel(cx0, cy0), p01 = pixel(cx1, cy0), p10 = pixel(cx0, cy1), p11 = pixel(cx1, cy1);
+    const uint32_t r0 = (uint32_t)__mul24(min(max(y0, 0), im.h - 1), im.row), r1 = (uint32_t)__mul24(min(max(y0 + 1, 0), im.h - 1), im.row);
+    uint32_t p00 = LoadPixelGuarded<C>(im, r0, cx0), p01 = LoadPixelGuarded<C>(im, r0, cx1);
+    uint32_t p10 = LoadPixelGuarded<C>(im, r1, cx0), p11 = LoadPixelGuarded<C>(im, r1, cx1);
     if (constant) // uniform
     {
         const bool inX0 = (uint32_t)x0 < (uint32_t)im.w, inX1 = (uint32_t)(x0 + 1) < (uint32_t)im.w;
@@ -706,6 +710,69 @@ __device__ __forceinline__ uint32_t SampleNearBorderQ15(const Img &im, bool cons
         p11             = inX1 && inY1 ? p11 : borderPx;
     }
     return BilinearQ15<C>(p00, p01, p10, p11, (uint32_t)X & (kQ15 - 1), (uint32_t)Y & (kQ15 - 1));
+}
+
+// The same for the fixed-point bicubic sum: the 4 x 4 taps fetched at clamped coordinates (replaced by the colour
+// where the unclamped one is outside), put together as the rows BlendCubicQ14 takes. |sx|, |sy| below 2^24.
+template<int C>
+__device__ __forceinline__ uint32_t SampleNearBorderCubicQ14(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
+{
+    const int ix = (int)floorf(sx) - 1, iy = (int)floorf(sy) - 1;
+    int       cx[4];
+    bool      inX[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        cx[i]  = min(max(ix + i, 0), im.w - 1);
+        inX[i] = (uint32_t)(ix + i) < (uint32_t)im.w;
+    }
+    uint32_t r[4][C];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const uint32_t rowOffset = (uint32_t)__mul24(min(max(iy + j, 0), im.h - 1), im.row);
+        const bool     inY       = (uint32_t)(iy + j) < (uint32_t)im.h;
+        uint32_t       p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            p[i] = LoadPixelGuarded<C>(im, rowOffset, cx[i]);
+            if (constant) // uniform
+            {
+                p[i] = inX[i] && inY ? p[i] : borderPx;
+            }
+        }
+        if constexpr (C == 3)
+        {
+            r[j][0] = __builtin_amdgcn_perm(p[1], p[0], 0x04020100u);
+            r[j][1] = __builtin_amdgcn_perm(p[2], p[1], 0x05040201u);
+            r[j][2] = __builtin_amdgcn_perm(p[3], p[2], 0x06050402u);
+        }
+        else if constexpr (C == 4)
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                r[j][i] = p[i];
+            }
+        }
+        else
+        {
+            r[j][0] = __builtin_amdgcn_perm(__builtin_amdgcn_perm(p[3], p[2], 0x04000c0cu), __builtin_amdgcn_perm(p[1], p[0], 0x0c0c0400u),
+                                            0x07060100u);
+        }
+    }
+    return BlendCubicQ14<C>(r, sx, sy);
+}
+
+// And for the nearest pixel.
+template<int C>
+__device__ __forceinline__ uint32_t SampleNearBorderNearest(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
+{
+    const int      x = FloorToInt(sx + .5f), y = FloorToInt(sy + .5f);
+    const uint32_t p = LoadPixelGuarded<C>(im, (uint32_t)__mul24(min(max(y, 0), im.h - 1), im.row), min(max(x, 0), im.w - 1));
+    // (the bytes above the pixel's must be 0: the stores merge neighbouring pixels' dwords)
+    return constant && !((uint32_t)x < (uint32_t)im.w && (uint32_t)y < (uint32_t)im.h) ? borderPx : p & (0xffffffffu >> (32 - 8 * C));
 }
 
 // The dwords of the pixel that SampleInside gives. u8 channels are rounded, saturated and placed into
@@ -845,14 +912,18 @@ __device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, fl
     }
 }
 
-// Whether a lane's samples can take SampleNearBorderQ15: 8-bit bilinear, one of its two border modes, rows and
-// columns within its 24-bit offsets and 16-bit coordinates (the caller's test), an image of 4 bytes or more, and
-// every coordinate (times 2^15) below 2^30 in magnitude.
+// 8-bit pixels of 1, 3 or 4 channels have straight-line samplers for samples next to the image's edge.
+template<class T, int C>
+constexpr bool kNearBorderForms = std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4);
+
+// Whether a lane's samples can take them: one of the two border modes that need no division, an image of 4 bytes or
+// more within the 24-bit offsets (the caller's test), and every coordinate small enough for the sampler's integer
+// conversion (bilinear: times 2^15 below 2^30; bicubic: below 2^24; nearest: any).
 template<class T, int C, int INTERP>
 __device__ __forceinline__ bool NearBorderForm(const Img &im, const WarpArgs &a, const float (&sx)[kPxPerLane],
                                                const float (&sy)[kPxPerLane])
 {
-    if constexpr (!kFixedPoint<T, INTERP>)
+    if constexpr (!kNearBorderForms<T, C>)
     {
         return false;
     }
@@ -864,7 +935,8 @@ __device__ __forceinline__ bool NearBorderForm(const Img &im, const WarpArgs &a,
         {
             u = max(u, max(__float_as_uint(sx[k]) & 0x7fffffffu, __float_as_uint(sy[k]) & 0x7fffffffu));
         }
-        return a.border <= NVCV_BORDER_REPLICATE && u < 0x4e800000u /* the pattern of 2^30 */ && (im.h > 1 || im.w * C >= 4);
+        const uint32_t limit = INTERP == NVCV_INTERP_LINEAR ? 0x4e800000u : (INTERP == NVCV_INTERP_CUBIC ? 0x4b800000u : 0x7f800000u);
+        return a.border <= NVCV_BORDER_REPLICATE && u < limit && (im.h > 1 || im.w * C >= 4);
     }
 }
 
@@ -917,9 +989,9 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
     }
     else if (fits && NearBorderForm<T, C, INTERP>(im, a, sx, sy))
     {
-        // 8-bit bilinear under a constant or replicating border: the border logic as selects, all four samples
-        // in flight (the generic loop below costs a wave that straddles the image's edge about 4 times as much)
-        if constexpr (kFixedPoint<T, INTERP>)
+        // 8-bit pixels under a constant or replicating border: the border logic as selects, all four samples in
+        // flight (the generic loop below costs a wave that straddles the image's edge about 4 times as much)
+        if constexpr (kNearBorderForms<T, C>)
         {
             uint32_t borderPx = 0;
 #pragma unroll
@@ -927,8 +999,8 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
             {
                 borderPx |= (uint32_t)BorderValueAs<T>(a.bval[c]) << (8 * c);
             }
-            // under a constant border a lane whose samples lie outside with all their taps takes the colour itself
-            // (the weights add up to exactly 1): whole waves in the corners a rotation leaves empty
+            // under a constant border a lane whose samples lie outside with all their taps needs no pixel: whole
+            // waves in the corners a rotation leaves empty
             const bool constant = a.border == NVCV_BORDER_CONSTANT;
             bool       outside  = constant;
 #pragma unroll
@@ -941,7 +1013,17 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
 #pragma unroll
                 for (int k = 0; k < kPxPerLane; ++k)
                 {
-                    q[0][k] = borderPx;
+                    if constexpr (INTERP == NVCV_INTERP_CUBIC)
+                    {
+                        T v[C];
+                        SampleAllOutside<T, C, INTERP>(a, sx[k], sy[k], v);
+                        q[0][k] = 0;
+                        __builtin_memcpy(&q[0][k], v, C);
+                    }
+                    else
+                    {
+                        q[0][k] = borderPx; // the tap itself, or taps whose weights add up to exactly 1
+                    }
                 }
             }
             else
@@ -949,7 +1031,18 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
 #pragma unroll
                 for (int k = 0; k < kPxPerLane; ++k)
                 {
-                    q[0][k] = SampleNearBorderQ15<C>(im, constant, borderPx, sx[k], sy[k]);
+                    if constexpr (INTERP == NVCV_INTERP_LINEAR)
+                    {
+                        q[0][k] = SampleNearBorderQ15<C>(im, constant, borderPx, sx[k], sy[k]);
+                    }
+                    else if constexpr (INTERP == NVCV_INTERP_CUBIC)
+                    {
+                        q[0][k] = SampleNearBorderCubicQ14<C>(im, constant, borderPx, sx[k], sy[k]);
+                    }
+                    else
+                    {
+                        q[0][k] = SampleNearBorderNearest<C>(im, constant, borderPx, sx[k], sy[k]);
+                    }
                 }
             }
         }
