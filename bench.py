@@ -699,7 +699,7 @@ class Streaming:
                                   "ResizeLinearQuadsU8Kernel<3>", "i32", "Resize LINEAR 1280x720 -> 1920x1080"),
         "resize-area-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
                              "ResizeAreaFixedTensorKernel<3>", "i32", "Resize AREA 1920x1080 -> 1280x720"),
-        "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t>>", "f32",
+        "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t,false>>", "f32",
                              "CvtColor BGR2HSV"),
         "cvtcolor-bgr2nv12": ("CvtColor", 32, ("uint8", 3), ("uint8", 1, "NHWC", 1620, 1920),
                               "PixelTensor<Yuv420FromBgr<3,true>>", "int32", "CvtColor BGR2YUV_NV12"),

@@ -211,7 +211,9 @@ __device__ __forceinline__ int32_t *HsvDivTable()
     return table;
 }
 
-template<class T>
+// RED_FIRST: the source pixel is R, G, B (the order is a template parameter: chosen per pixel it cost two selects
+// and two masks of the 42 instructions an 8-bit pixel takes).
+template<class T, bool RED_FIRST = false>
 struct HsvFromBgr
 {
     static constexpr int kItemW = 1, kItemH = 1;
@@ -238,7 +240,7 @@ struct HsvFromBgr
         if constexpr (std::is_integral_v<T>)
         {
             const int hrange = a.full ? 256 : 180;
-            const int b = a.bidx ? s.v[2] : s.v[0], g = s.v[1], r = a.bidx ? s.v[0] : s.v[2];
+            const int b = RED_FIRST ? s.v[2] : s.v[0], g = s.v[1], r = RED_FIRST ? s.v[0] : s.v[2];
             const int vmin = min(b, min(g, r));
             const int val  = max(b, max(g, r));
             const int diff = val - vmin;
@@ -258,7 +260,7 @@ struct HsvFromBgr
         }
         else
         {
-            const float b = a.bidx ? s.v[2] : s.v[0], g = s.v[1], r = a.bidx ? s.v[0] : s.v[2];
+            const float b = RED_FIRST ? s.v[2] : s.v[0], g = s.v[1], r = RED_FIRST ? s.v[0] : s.v[2];
             const float vmin = fminf(r, fminf(g, b));
             const float val  = fmaxf(r, fmaxf(g, b));
             float       diff = val - vmin;
@@ -1015,10 +1017,10 @@ bool RunPixelColorFamily(ColorCode code, const ColorIO &io, hipStream_t stream)
         switch (io.srcElem)
         {
         case kU8:
-            Launch<HsvFromBgr<uint8_t>>(io, a, stream);
+            a.bidx ? Launch<HsvFromBgr<uint8_t, true>>(io, a, stream) : Launch<HsvFromBgr<uint8_t, false>>(io, a, stream);
             break;
         case kF32:
-            Launch<HsvFromBgr<float>>(io, a, stream);
+            a.bidx ? Launch<HsvFromBgr<float, true>>(io, a, stream) : Launch<HsvFromBgr<float, false>>(io, a, stream);
             break;
         default:
             Bad("Unsupported DataType");
