@@ -1527,14 +1527,17 @@ __device__ __forceinline__ uint32_t Dot2U16(uint32_t taps, uint32_t weights, uin
     return __builtin_amdgcn_udot2(t, w, acc, false);
 }
 
-// A source row's sums per channel from its window and the packed horizontal weights.
+// A source row's sums per channel from its window and the packed horizontal weights, each plus 2^23: the integer sum
+// (below 2^23) is accumulated on the bit pattern of 8388608.0f, whose unit in the last place is 1, so the register
+// read as a float IS 2^23 + sum and no conversion is needed. The caller's accumulator starts at minus 2^23 times
+// the sum of the rows' weights.
 template<int C>
 __device__ __forceinline__ void AreaRowSums(const uint32_t (&r)[C], uint32_t w01, uint32_t w23, float (&s)[C])
 {
 #pragma unroll
     for (int c = 0; c < C; ++c)
     {
-        s[c] = (float)Dot2U16(AreaTapPair<C>(r, 2, c), w23, Dot2U16(AreaTapPair<C>(r, 0, c), w01, 0u));
+        s[c] = __uint_as_float(Dot2U16(AreaTapPair<C>(r, 2, c), w23, Dot2U16(AreaTapPair<C>(r, 0, c), w01, 0x4b000000u)));
     }
 }
 
@@ -1542,17 +1545,10 @@ __device__ __forceinline__ void AreaRowSums(const uint32_t (&r)[C], uint32_t w01
 // source row j in output pixel k. All N windows are requested before the first sum; every row's sums are formed once.
 // Rows are added in ascending order, the first as a product, the others with fused multiply-adds: a row of weight 0
 // changes nothing, so the result does not depend on which rows are passed beside those of the pixel's box.
-template<int C, int N, int K, bool GUARDED>
-__device__ __forceinline__ void AreaFixedPixels(const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
-                                                uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
-                                                uint32_t (&out)[K])
+template<int C, int N, int K>
+__device__ __forceinline__ void AreaSumRows(const uint32_t (&r)[N][C], uint32_t w01, uint32_t w23, const float (&wy)[K][4],
+                                            const float (&start)[K], uint32_t *out)
 {
-    uint32_t r[N][C];
-#pragma unroll
-    for (int j = 0; j < N; ++j)
-    {
-        LoadAreaWindow<C, GUARDED>(row + (int64_t)j * srcRow, at, shift, j == lastRowIn, rowBytes, r[j]);
-    }
     float acc[K][C];
 #pragma unroll
     for (int j = 0; j < N; ++j)
@@ -1565,7 +1561,7 @@ __device__ __forceinline__ void AreaFixedPixels(const uint8_t *row, int srcRow, 
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
-                acc[k][c] = j == 0 ? s[c] * wy[k][0] : fmaf(s[c], wy[k][j], acc[k][c]);
+                acc[k][c] = fmaf(s[c], wy[k][j], j == 0 ? start[k] : acc[k][c]);
             }
         }
     }
@@ -1581,27 +1577,64 @@ __device__ __forceinline__ void AreaFixedPixels(const uint8_t *row, int srcRow, 
     }
 }
 
+template<int C, int N, int K, bool GUARDED>
+__device__ __forceinline__ void AreaFixedPixels(const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
+                                                uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
+                                                const float (&start)[K], uint32_t (&out)[K])
+{
+    uint32_t r[N][C];
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+    {
+        LoadAreaWindow<C, GUARDED>(row + (int64_t)j * srcRow, at, shift, j == lastRowIn, rowBytes, r[j]);
+    }
+    AreaSumRows<C, N, K>(r, w01, w23, wy, start, out);
+}
+
+// Two such pairs of output pixels (4 vertically adjacent ones) from 3 source rows each, none of them the image's last:
+// the six windows are requested together. A pair that needs only 2 rows passes a third of weight 0.
+template<int C>
+__device__ __forceinline__ void AreaFixedTwoPairs(const uint8_t *rowA, const uint8_t *rowB, int srcRow, uint32_t at, uint32_t shift,
+                                                  uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wyA)[2][4],
+                                                  const float (&wyB)[2][4], const float (&startA)[2], const float (&startB)[2],
+                                                  uint32_t (&out)[4])
+{
+    uint32_t ra[3][C], rb[3][C];
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+    {
+        LoadAreaWindow<C, false>(rowA + (int64_t)j * srcRow, at, shift, false, rowBytes, ra[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+    {
+        LoadAreaWindow<C, false>(rowB + (int64_t)j * srcRow, at, shift, false, rowBytes, rb[j]);
+    }
+    AreaSumRows<C, 3, 2>(ra, w01, w23, wyA, startA, &out[0]);
+    AreaSumRows<C, 3, 2>(rb, w01, w23, wyB, startB, &out[2]);
+}
+
 template<int C, int K, bool GUARDED>
 __device__ __forceinline__ void AreaFixedRowsOf(int n, const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
                                                 uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
-                                                uint32_t (&out)[K])
+                                                const float (&start)[K], uint32_t (&out)[K])
 {
     // (wave-uniform)
     if (n == 3)
     {
-        AreaFixedPixels<C, 3, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+        AreaFixedPixels<C, 3, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
     else if (n == 2)
     {
-        AreaFixedPixels<C, 2, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+        AreaFixedPixels<C, 2, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
     else if (n == 4)
     {
-        AreaFixedPixels<C, 4, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+        AreaFixedPixels<C, 4, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
     else
     {
-        AreaFixedPixels<C, 1, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+        AreaFixedPixels<C, 1, K, GUARDED>(row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
 }
 
@@ -1609,15 +1642,15 @@ __device__ __forceinline__ void AreaFixedRowsOf(int n, const uint8_t *row, int s
 template<int C, int K>
 __device__ __forceinline__ void AreaFixedRows(int n, const uint8_t *row, int srcRow, int lastRowIn, uint32_t at, uint32_t shift,
                                               uint32_t rowBytes, uint32_t w01, uint32_t w23, const float (&wy)[K][4],
-                                              uint32_t (&out)[K])
+                                              const float (&start)[K], uint32_t (&out)[K])
 {
     if (C != 4 && lastRowIn < n) // wave-uniform, once per image and column tile
     {
-        AreaFixedRowsOf<C, K, true>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+        AreaFixedRowsOf<C, K, true>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
     else
     {
-        AreaFixedRowsOf<C, K, false>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, out);
+        AreaFixedRowsOf<C, K, false>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
 }
 
@@ -1664,26 +1697,31 @@ __device__ __forceinline__ void ResizeAreaFixedWaveTile(const Plane &p, int x0, 
     const bool fits    = fminf(dy * p.scaleY + p.scaleY, (float)p.srcH) <= pairStart + 4.f;
     const int  pairRows = !fits ? 0 : pw[3] != 0.f ? 4 : pw[2] != 0.f ? 3 : pw[1] != 0.f ? 2 : 1;
     const int  ownFirst = (int)ownStart, pairFirst = (int)pairStart;
+    // the accumulator's start: minus 2^23 times the sum of the row's weights (see AreaRowSums), added in ascending order;
+    // weights of 0 in front or behind change nothing, so the pair form and the single form start alike
+    const float rowStart = -8388608.f * (((ow[0] + ow[1]) + ow[2]) + ow[3]);
 
     const int rowsHere = min(kAreaRowsPerWave, p.dstH - y0);
-    uint32_t  q[1][4] = {};
-#pragma unroll 1
-    for (int i = 0; i < rowsHere; i += 2)
+    // output rows i, i + 1 -> out[0], out[1]
+    auto rowPair = [&](int i, uint32_t *out)
     {
         const int n = __builtin_amdgcn_readlane(pairRows, i + 1);
-        uint32_t  out[2];
         if (n != 0)
         {
             const int first = __builtin_amdgcn_readlane(pairFirst, i);
             float     wy[2][4];
+            uint32_t  two[2];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
                 wy[0][j] = ReadLane(pw[j], i);
                 wy[1][j] = ReadLane(pw[j], i + 1);
             }
+            const float start[2] = {ReadLane(rowStart, i), ReadLane(rowStart, i + 1)};
             AreaFixedRows<C, 2>(n, p.src + (int64_t)first * p.srcRow, p.srcRow, p.srcH - 1 - first, at, shift, rowBytes, w01,
-                                w23, wy, out);
+                                w23, wy, start, two);
+            out[0] = two[0];
+            out[1] = two[1];
         }
         else
         {
@@ -1697,26 +1735,45 @@ __device__ __forceinline__ void ResizeAreaFixedWaveTile(const Plane &p, int x0, 
                 {
                     wy[0][j] = ReadLane(ow[j], i + k);
                 }
-                uint32_t one[1];
+                uint32_t    one[1];
+                const float start[1] = {ReadLane(rowStart, i + k)};
                 AreaFixedRows<C, 1>(__builtin_amdgcn_readlane(ownRows, i + k), p.src + (int64_t)first * p.srcRow, p.srcRow,
-                                    p.srcH - 1 - first, at, shift, rowBytes, w01, w23, wy, one);
+                                    p.srcH - 1 - first, at, shift, rowBytes, w01, w23, wy, start, one);
                 out[k] = one[0];
             }
         }
-        const bool upper = (i & 2) == 0; // rows 0, 1 or 2, 3 of the group of 4 that is stored together
-        q[0][0]          = upper ? out[0] : q[0][0];
-        q[0][1]          = upper ? out[1] : q[0][1];
-        q[0][2]          = upper ? q[0][2] : out[0];
-        q[0][3]          = upper ? q[0][3] : out[1];
-        if (!upper)
-        {
-            StoreWavePatch<uint8_t, C>(p, x0, y0 + (i & ~3), lane, q);
-        }
-    }
-    // an odd pair of rows at the lower edge of the output: rows 2, 3 of the group duplicate what is not stored
-    if ((((rowsHere + 1) >> 1) & 1) != 0)
+    };
+    // 4 output rows per step (rows past the output are duplicates of its last one and are not stored)
+#pragma unroll 1
+    for (int i = 0; i < rowsHere; i += 4)
     {
-        StoreWavePatch<uint8_t, C>(p, x0, y0 + ((rowsHere - 1) & ~3), lane, q);
+        uint32_t  q[1][4];
+        const int nA = __builtin_amdgcn_readlane(pairRows, i + 1), nB = __builtin_amdgcn_readlane(pairRows, i + 3);
+        const int firstA = __builtin_amdgcn_readlane(pairFirst, i), firstB = __builtin_amdgcn_readlane(pairFirst, i + 2);
+        // the usual case at scales up to 1.5: both pairs from at most 3 rows each, clear of the image's last row
+        // (wave-uniform)
+        if (nA != 0 && nB != 0 && max(nA, nB) <= 3 && max(firstA, firstB) + 2 < p.srcH - 1)
+        {
+            float wyA[2][4], wyB[2][4];
+#pragma unroll
+            for (int j = 0; j < 3; ++j)
+            {
+                wyA[0][j] = ReadLane(pw[j], i);
+                wyA[1][j] = ReadLane(pw[j], i + 1);
+                wyB[0][j] = ReadLane(pw[j], i + 2);
+                wyB[1][j] = ReadLane(pw[j], i + 3);
+            }
+            const float startA[2] = {ReadLane(rowStart, i), ReadLane(rowStart, i + 1)};
+            const float startB[2] = {ReadLane(rowStart, i + 2), ReadLane(rowStart, i + 3)};
+            AreaFixedTwoPairs<C>(p.src + (int64_t)firstA * p.srcRow, p.src + (int64_t)firstB * p.srcRow, p.srcRow, at, shift,
+                                 rowBytes, w01, w23, wyA, wyB, startA, startB, q[0]);
+        }
+        else
+        {
+            rowPair(i, &q[0][0]);
+            rowPair(i + 2, &q[0][2]);
+        }
+        StoreWavePatch<uint8_t, C>(p, x0, y0 + i, lane, q);
     }
 }
 

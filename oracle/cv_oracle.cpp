@@ -350,7 +350,7 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
         // scales of 1 and more the same float32 differences as in variants 1 and 2 -, nothing outside the image,
         // divided by the length of the box inside the image. Horizontal weights rounded to multiples of 2^-15 (to nearest,
         // ties to even), a row's sum exact in integers; the rows' sums added in ascending order with fused
-        // multiply-adds (the first is a product); one rounding to nearest-even. Outside those scales:
+        // multiply-adds; one rounding to nearest-even. Outside those scales:
         // variant 1 (5) or 2 (6).
         if (std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4) && scaleX >= 1.f && scaleX <= 3.f && scaleY >= 1.f
             && scaleY <= 3.f && srcW * C >= 32 && srcH >= 4)
@@ -386,12 +386,15 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
             {
                 wq[k] = (uint32_t)std::nearbyint(col.w[k]);
             }
+            // a row's integer sum (below 2^23) enters as the float 2^23 + sum, which the kernel gets for free by
+            // summing on that float's bit pattern; the accumulator starts at minus 2^23 times the sum of the weights
+            const float start = -8388608.f * (((row.w[0] + row.w[1]) + row.w[2]) + row.w[3]);
             for (int c = 0; c < C; ++c)
             {
-                float acc = 0.f;
+                float acc = start;
                 for (int j = 0; j < 4; ++j)
                 {
-                    if (j > 0 && row.w[j] == 0.f)
+                    if (row.w[j] == 0.f)
                     {
                         continue;
                     }
@@ -400,7 +403,7 @@ void AreaPixel(const T *src, int64_t srcStep, int srcW, int srcH, T *out, int C,
                     {
                         sum += (uint32_t)src[(row.first + j) * srcStep + (int64_t)(col.first + k) * C + c] * wq[k];
                     }
-                    acc = j == 0 ? (float)sum * row.w[j] : std::fmaf((float)sum, row.w[j], acc);
+                    acc = std::fmaf(8388608.f + (float)sum, row.w[j], acc);
                 }
                 const float v = std::nearbyint(acc);
                 out[c]        = (T)(v < 0.f ? 0.f : (v > 255.f ? 255.f : v));
