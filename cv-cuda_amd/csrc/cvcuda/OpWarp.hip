@@ -936,7 +936,7 @@ __device__ __forceinline__ bool NearBorderForm(const Img &im, const WarpArgs &a,
             u = max(u, max(__float_as_uint(sx[k]) & 0x7fffffffu, __float_as_uint(sy[k]) & 0x7fffffffu));
         }
         const uint32_t limit = INTERP == NVCV_INTERP_LINEAR ? 0x4e800000u : (INTERP == NVCV_INTERP_CUBIC ? 0x4b800000u : 0x7f800000u);
-        return a.border <= NVCV_BORDER_REPLICATE && u < limit && (im.h > 1 || im.w * C >= 4);
+        return a.border <= NVCV_BORDER_REPLICATE && u < limit && __mul24(im.h - 1, im.row) + im.w * C >= 4;
     }
 }
 

@@ -58,6 +58,24 @@ def test_reference_table_exact(cv, orc, gpu, interp, border):
         assert np.abs(res.astype(np.int16) - gold.astype(np.int16)).max() <= tol, (sw, sh, dw, dh, m, inv)
 
 
+
+@pytest.mark.parametrize("c", [1, 3, 4])
+def test_tiny_sources_at_the_border_forms_limits(cv, orc, gpu, c):
+    # 8-bit samples next to the image's edge take straight-line forms that fetch a pixel with one 4-byte load, moved
+    # back where it would pass the image's last byte; images of under 4 bytes keep the generic loop. Sources of 1 to
+    # 5 pixels, every interpolation, both border modes of those forms and one other: exact against the restatement.
+    op = cv.WarpAffine(0)
+    m = [0.8, 0.3, -0.4, -0.2, 0.9, 0.6]
+    for (sw, sh) in [(1, 1), (2, 1), (1, 2), (3, 1), (1, 4), (2, 2), (5, 1), (1, 5)]:
+        src = orc.fill_u8((2, sh, sw, c), 40 + sw * 7 + sh)
+        for interp, border in itertools.product((NEAREST, LINEAR, CUBIC), (0, 1, 4)):
+            tout = cv.Tensor.alloc([2, 6, 9, c], np.uint8, "NHWC")
+            op(None, cv.Tensor.from_numpy(src, "NHWC"), tout, m, interp | INVERSE_MAP, border, (9, 200, 31, 77))
+            torch.cuda.synchronize()
+            dev = orc.warp(src, (6, 9), np.asarray(m, np.float32), interp, border, (9, 200, 31, 77), variant=device_variant(interp))
+            np.testing.assert_array_equal(tout.numpy(), dev, err_msg=str((sw, sh, c, interp, border)))
+
+
 def rotation(w, h, deg, s):
     t = np.deg2rad(deg)
     c, sn = s * np.cos(t), s * np.sin(t)
