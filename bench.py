@@ -697,6 +697,8 @@ class Streaming:
                                "ResizeLinearPairsU8Kernel<3>", "i32", "Resize LINEAR 1920x1080 -> 1280x720"),
         "resize-linear-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
                                   "ResizeLinearQuadsU8Kernel<3>", "i32", "Resize LINEAR 1280x720 -> 1920x1080"),
+        "resize-cubic-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
+                              "ResizePatchTensorKernel<unsigned char,3,2>", "i32", "Resize CUBIC 1920x1080 -> 1280x720"),
         "resize-area-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
                              "ResizeAreaFixedTensorKernel<3>", "i32", "Resize AREA 1920x1080 -> 1280x720"),
         "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t,false>>", "f32",
@@ -709,7 +711,7 @@ class Streaming:
     # what differs from the operator's default call above: colour code by name, interpolation
     CODES = {"cvtcolor-bgr2rgb": "COLOR_BGR2RGB", "cvtcolor-bgr2gray": "COLOR_BGR2GRAY", "cvtcolor-bgr2hsv": "COLOR_BGR2HSV",
              "cvtcolor-bgr2nv12": "COLOR_BGR2YUV_NV12", "cvtcolor-yuy2-bgr": "COLOR_YUV2BGR_YUY2"}
-    INTERP = {"resize-area-720p": AREA}
+    INTERP = {"resize-area-720p": AREA, "resize-cubic-720p": CUBIC}
 
     def __init__(self, cv, orc, np, torch, key):
         self.cv, self.orc, self.np, self.torch, self.key = cv, orc, np, torch, key
@@ -835,7 +837,7 @@ WORKLOADS.update({k: (lambda *a, k=k: StreamMix(*a, k)) for k in StreamMix.SPECS
 # of memory latency is more than half of the time (batch 8).
 BOUNDS = {"warp-affine-varshape": "valu-issue", "warp-affine-tensor-linear": "valu-issue",
           "warp-affine-tensor-cubic": "valu-issue", "warp-affine-tensor-nearest": "vmem-issue",
-          "resize-area-720p": "valu-issue", "cvtcolor-bgr2hsv": "valu-issue",
+          "resize-area-720p": "valu-issue", "resize-cubic-720p": "valu-issue", "cvtcolor-bgr2hsv": "valu-issue",
           "resize-linear-720p": "vmem-issue", "resize-linear-upscale": "valu-issue",
           "resize-nearest": "launch-latency", "resize-linear": "launch-latency", "empty-launch": "launch-latency"}
 

@@ -221,6 +221,58 @@ __device__ __forceinline__ void LoadTapPairBytes(const uint8_t *row, int xoff, b
     }
 }
 
+// Four horizontally adjacent 8-bit pixels as raw bytes (the box filter's and the bicubic blend's row window): the
+// D dwords that hold the 4 pixels at byte offset `at` + `shift` of the row (shift 0 .. 3; 4 channels: none),
+// brought to the front: pixel k, channel c in byte k * C + c.
+template<int C, bool GUARDED>
+__device__ __forceinline__ void LoadQuadWindow(const uint8_t *row, uint32_t at, uint32_t shift, bool lastRow, uint32_t rowBytes,
+                                               uint32_t (&r)[C])
+{
+    constexpr int D = C == 4 ? 4 : C + 1;
+    struct __attribute__((packed, aligned(1))) Window
+    {
+        uint32_t d[D];
+    };
+    if constexpr (C == 4)
+    {
+        const Window w = *reinterpret_cast<const Window *>(row + at);
+        __builtin_memcpy(r, &w, 16);
+    }
+    else
+    {
+        // the load runs up to 4 bytes past the window, harmless except behind the image's last row, where it is
+        // moved back to end with the row (GUARDED: the rows passed may include that one)
+        bool whole = false;
+        if (GUARDED && lastRow)
+        {
+            const uint32_t back = min(at, rowBytes - 4 * D);
+            shift += at - back; // up to 4
+            at    = back;
+            whole = shift == 4;
+            shift = whole ? 0 : shift;
+        }
+        const Window w = *reinterpret_cast<const Window *>(row + at);
+#pragma unroll
+        for (int i = 0; i < C; ++i)
+        {
+            r[i] = __builtin_amdgcn_alignbyte(w.d[i + 1], w.d[i], shift);
+            if constexpr (GUARDED)
+            {
+                r[i] = whole ? w.d[i + 1] : r[i];
+            }
+        }
+    }
+}
+
+// Channel c of pixels ka and ka + 1 of such a window as (first | second << 16).
+template<int C>
+__device__ __forceinline__ uint32_t QuadTapPair(const uint32_t (&r)[C], int ka, int c)
+{
+    const int      b0 = ka * C + c, b1 = b0 + C, j = b0 / 4;
+    const uint32_t sel = 0x0c000c00u | (uint32_t)(b0 - 4 * j) | ((uint32_t)(b1 - 4 * j) << 16);
+    return __builtin_amdgcn_perm(r[j + 1 < C ? j + 1 : C - 1], r[j], sel);
+}
+
 __device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
 {
     constexpr float A = -0.75f;
@@ -235,6 +287,14 @@ __device__ __forceinline__ void CubicCoeffs(float d, float (&w)[4])
 // the reference's float32 expression) is cut to a multiple of 2^-15.
 template<class T>
 constexpr bool kFixedLinear = std::is_same_v<T, uint8_t>;
+
+// 8-bit pixels are blended bicubically with the four horizontal weights (the reference's float32 polynomials)
+// rounded to multiples of 2^-14, the last one taking the remainder so that they add up to exactly 1; a row's four
+// taps are combined in integers (exact), the four row sums in float32 with the vertical weights, ascending, by
+// fused multiply-adds; the magnitude is rounded once. Tensors and image batches alike, whichever kernel form a
+// shape takes. Within 0.05 of the float32 expression, i.e. at most 1 from the reference's golden.
+template<class T>
+constexpr bool kFixedCubic = std::is_same_v<T, uint8_t>;
 
 __device__ __forceinline__ uint32_t FractionQ15(float w)
 {
@@ -682,6 +742,17 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
         {
             sum[c] = 0.f;
         }
+        [[maybe_unused]] int wq[4];
+        if constexpr (kFixedCubic<T>)
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                wx[i] *= 16384.f;
+                wy[i] *= 1.f / 16384.f;
+            }
+            CubicWeightsQ14(wx, wq);
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
         {
@@ -693,6 +764,16 @@ __device__ __forceinline__ Pixel<T, C> ResizeValue(const Plane &p, int dx, int d
             for (int i = 0; i < 4; ++i)
             {
                 t[i] = LoadPx<T, C>(row, max(0, min(sx - 1 + i, p.srcW - 1)));
+            }
+            if constexpr (kFixedCubic<T>)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    const int h = (int)t[0].v[c] * wq[0] + (int)t[1].v[c] * wq[1] + (int)t[2].v[c] * wq[2] + (int)t[3].v[c] * wq[3];
+                    sum[c]      = j == 0 ? (float)h * wy[0] : fmaf((float)h, wy[j], sum[c]);
+                }
+                continue;
             }
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -815,6 +896,43 @@ __device__ __forceinline__ AxisTerms<W> FromLane(const AxisTerms<W> &a, int from
     return r;
 }
 
+// The 8-bit bicubic sum of one output pixel per lane: rows y0 .. y0 + 3 (clamped into the image), their windows of 4
+// pixels at `at` + `shift`, the packed horizontal weights and the vertical ones times 2^-14 (wave-uniform). All four
+// windows are requested before the first sum.
+template<int C, bool GUARDED>
+__device__ __forceinline__ uint32_t CubicRowsQ14(const Plane &p, int y0, uint32_t at, uint32_t shift, uint32_t rowBytes,
+                                                 uint32_t w01, uint32_t w23, const float (&wy)[4])
+{
+    uint32_t       r[4][C];
+    const uint8_t *first = p.src + (int64_t)y0 * p.srcRow;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const int      yy   = GUARDED ? max(0, min(y0 + j, p.srcH - 1)) : y0 + j;
+        const uint8_t *line = GUARDED ? p.src + (int64_t)yy * p.srcRow : first + (int64_t)j * p.srcRow;
+        LoadQuadWindow<C, GUARDED>(line, at, shift, yy == p.srcH - 1, rowBytes, r[j]);
+    }
+    float acc[C];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const float w = wy[j];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            const int h = Dot2I16(QuadTapPair<C>(r[j], 2, c), w23, Dot2I16(QuadTapPair<C>(r[j], 0, c), w01));
+            acc[c]      = j == 0 ? (float)h * w : fmaf((float)h, w, acc[c]);
+        }
+    }
+    uint32_t q = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        q = __builtin_amdgcn_cvt_pk_u8_f32(fabsf(acc[c]), c, q);
+    }
+    return q;
+}
+
 // One output pixel from its column terms (per lane) and row terms (wave-uniform).
 template<class T, int C, int INTERP, bool VARSHAPE>
 __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerms<kWeights<INTERP>> &col,
@@ -871,6 +989,32 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
             }
             out.v[c] = SaturateCast<T>(v);
         }
+    }
+    else if constexpr (kFixedCubic<T>)
+    {
+        // (the column's part of this does not depend on the row and is computed once per lane)
+        float wx[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            wx[i] = col.w[i] * 16384.f;
+        }
+        uint32_t w01, w23;
+        CubicWeightPairsQ14(wx, w01, w23);
+        const uint32_t off = (uint32_t)(col.s - 1) * C, at = C == 4 ? off : off & ~3u, shift = off & 3u;
+        const int      y0 = row.s - 1; // rows y0 .. y0 + 3, inside the image for sources of 4 rows and more
+        uint32_t       q;
+        // the four windows are requested together; the form that guards the image's last row only where it is among them
+        // (wave-uniform)
+        if (y0 + 3 >= p.srcH - 1 || y0 < 0)
+        {
+            q = CubicRowsQ14<C, true>(p, y0, at, shift, (uint32_t)rowBytes, w01, w23, row.w);
+        }
+        else
+        {
+            q = CubicRowsQ14<C, false>(p, y0, at, shift, (uint32_t)rowBytes, w01, w23, row.w);
+        }
+        __builtin_memcpy(&out, &q, PB);
     }
     else
     {
@@ -988,7 +1132,9 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
     }
     const int   lane   = threadIdx.x & 63;
     const float scaleX = p.scaleX, scaleY = p.scaleY;
-    const bool  wide   = p.srcW >= 4; // uniform per image
+    // uniform per image (the 8-bit bicubic form loads whole dwords around 4 pixels: rows of 16 bytes or more, 8 for
+    // one channel)
+    const bool wide = p.srcW >= 4 && (INTERP != NVCV_INTERP_CUBIC || !kFixedCubic<T> || p.srcW * C >= (C == 1 ? 8 : 16));
     // columns and rows past the output compute a duplicate of the last one: every lane takes part in
     // the transposes
     const int dx = min(x0 + lane, p.dstW - 1);
@@ -997,7 +1143,16 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
     {
         const auto col = FinishedAxis<INTERP>(scaleX, dx, p.srcW, true);
         // the 4 rows' terms are computed side by side (lane l: row l & 3) and then read as uniform values
-        const auto rows = FinishedAxis<INTERP>(scaleY, min(y0 + (lane & 3), p.dstH - 1), p.srcH, false);
+        auto rows = FinishedAxis<INTERP>(scaleY, min(y0 + (lane & 3), p.dstH - 1), p.srcH, false);
+        if constexpr (INTERP == NVCV_INTERP_CUBIC && kFixedCubic<T>)
+        {
+            // the vertical weights go with row sums in units of 2^-14
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                rows.w[i] *= 1.f / 16384.f;
+            }
+        }
 #pragma unroll
         for (int k = 0; k < 4; ++k)
         {
@@ -1467,57 +1622,6 @@ __device__ __forceinline__ void AreaWeights(float scale, int d, int srcSize, flo
     }
 }
 
-// The window's bytes: D dwords that hold the 4 pixels at byte offset `at` + `shift` of the row (shift 0 .. 3;
-// 4 channels: none), brought to the front: pixel k, channel c in byte k * C + c.
-template<int C, bool GUARDED>
-__device__ __forceinline__ void LoadAreaWindow(const uint8_t *row, uint32_t at, uint32_t shift, bool lastRow, uint32_t rowBytes,
-                                               uint32_t (&r)[C])
-{
-    constexpr int D = C == 4 ? 4 : C + 1;
-    struct __attribute__((packed, aligned(1))) Window
-    {
-        uint32_t d[D];
-    };
-    if constexpr (C == 4)
-    {
-        const Window w = *reinterpret_cast<const Window *>(row + at);
-        __builtin_memcpy(r, &w, 16);
-    }
-    else
-    {
-        // the load runs up to 4 bytes past the window, harmless except behind the image's last row, where it is
-        // moved back to end with the row (GUARDED: the rows passed may include that one)
-        bool whole = false;
-        if (GUARDED && lastRow)
-        {
-            const uint32_t back = min(at, rowBytes - 4 * D);
-            shift += at - back; // up to 4
-            at    = back;
-            whole = shift == 4;
-            shift = whole ? 0 : shift;
-        }
-        const Window w = *reinterpret_cast<const Window *>(row + at);
-#pragma unroll
-        for (int i = 0; i < C; ++i)
-        {
-            r[i] = __builtin_amdgcn_alignbyte(w.d[i + 1], w.d[i], shift);
-            if constexpr (GUARDED)
-            {
-                r[i] = whole ? w.d[i + 1] : r[i];
-            }
-        }
-    }
-}
-
-// Channel c of pixels ka and ka + 1 of such a window as (first | second << 16).
-template<int C>
-__device__ __forceinline__ uint32_t AreaTapPair(const uint32_t (&r)[C], int ka, int c)
-{
-    const int      b0 = ka * C + c, b1 = b0 + C, j = b0 / 4;
-    const uint32_t sel = 0x0c000c00u | (uint32_t)(b0 - 4 * j) | ((uint32_t)(b1 - 4 * j) << 16);
-    return __builtin_amdgcn_perm(r[j + 1 < C ? j + 1 : C - 1], r[j], sel);
-}
-
 __device__ __forceinline__ uint32_t Dot2U16(uint32_t taps, uint32_t weights, uint32_t acc)
 {
     typedef unsigned short U16x2 __attribute__((ext_vector_type(2)));
@@ -1537,7 +1641,7 @@ __device__ __forceinline__ void AreaRowSums(const uint32_t (&r)[C], uint32_t w01
 #pragma unroll
     for (int c = 0; c < C; ++c)
     {
-        s[c] = __uint_as_float(Dot2U16(AreaTapPair<C>(r, 2, c), w23, Dot2U16(AreaTapPair<C>(r, 0, c), w01, 0x4b000000u)));
+        s[c] = __uint_as_float(Dot2U16(QuadTapPair<C>(r, 2, c), w23, Dot2U16(QuadTapPair<C>(r, 0, c), w01, 0x4b000000u)));
     }
 }
 
@@ -1586,7 +1690,7 @@ __device__ __forceinline__ void AreaFixedPixels(const uint8_t *row, int srcRow, 
 #pragma unroll
     for (int j = 0; j < N; ++j)
     {
-        LoadAreaWindow<C, GUARDED>(row + (int64_t)j * srcRow, at, shift, j == lastRowIn, rowBytes, r[j]);
+        LoadQuadWindow<C, GUARDED>(row + (int64_t)j * srcRow, at, shift, j == lastRowIn, rowBytes, r[j]);
     }
     AreaSumRows<C, N, K>(r, w01, w23, wy, start, out);
 }
@@ -1603,12 +1707,12 @@ __device__ __forceinline__ void AreaFixedTwoPairs(const uint8_t *rowA, const uin
 #pragma unroll
     for (int j = 0; j < 3; ++j)
     {
-        LoadAreaWindow<C, false>(rowA + (int64_t)j * srcRow, at, shift, false, rowBytes, ra[j]);
+        LoadQuadWindow<C, false>(rowA + (int64_t)j * srcRow, at, shift, false, rowBytes, ra[j]);
     }
 #pragma unroll
     for (int j = 0; j < 3; ++j)
     {
-        LoadAreaWindow<C, false>(rowB + (int64_t)j * srcRow, at, shift, false, rowBytes, rb[j]);
+        LoadQuadWindow<C, false>(rowB + (int64_t)j * srcRow, at, shift, false, rowBytes, rb[j]);
     }
     AreaSumRows<C, 3, 2>(ra, w01, w23, wyA, startA, &out[0]);
     AreaSumRows<C, 3, 2>(rb, w01, w23, wyB, startB, &out[2]);

@@ -154,56 +154,6 @@ __device__ __forceinline__ uint32_t FractionQ15(float v)
     return f >= 0.f ? (uint32_t)(int)(f * 32768.f) : 0u;
 }
 
-// Horizontal bicubic weights, given times 2^14, as signed 16-bit integers: (w0 | w1 << 16), (w2 | w3 << 16).
-// Adding 1.5 * 2^23 rounds a weight to the nearest integer, ties to even, and leaves it in the low bits of
-// the sum's bit pattern (two's complement for negative values); w3 = 2^14 - w0 - w1 - w2 on those integers.
-__device__ __forceinline__ void CubicWeightPairsQ14(const float (&w)[4], uint32_t &p01, uint32_t &p23)
-{
-    constexpr float    kMagic = 12582912.f;
-    constexpr uint32_t kBits  = 0x4B400000u;
-    const uint32_t     b0 = __float_as_uint(w[0] + kMagic);
-    const uint32_t     b1 = __float_as_uint(w[1] + kMagic);
-    const uint32_t     b2 = __float_as_uint(w[2] + kMagic);
-    const uint32_t     w3 = (16384u + 3u * kBits) - (b0 + b1 + b2);
-    p01                   = __builtin_amdgcn_perm(b1, b0, 0x05040100u);
-    p23                   = __builtin_amdgcn_perm(w3, b2, 0x05040100u);
-}
-
-// The same four integers one by one (border path), also from weights times 2^14. NaN weights give 0.
-__device__ __forceinline__ void CubicWeightsQ14(const float (&w)[4], int (&q)[4])
-{
-    q[0] = (int)rintf(w[0]);
-    q[1] = (int)rintf(w[1]);
-    q[2] = (int)rintf(w[2]);
-    q[3] = 16384 - q[0] - q[1] - q[2];
-}
-
-// Bytes lo and hi of a row held in dwords r[] -> (byte lo | byte hi << 16), one byte permute.
-template<int N>
-__device__ __forceinline__ uint32_t BytePair(const uint32_t (&r)[N], int lo, int hi)
-{
-    const uint32_t sel = 0x0c000c00u | (uint32_t)(lo & 3) | ((uint32_t)(4 + (hi & 3)) << 16);
-    return __builtin_amdgcn_perm(r[hi >> 2], r[lo >> 2], sel);
-}
-
-__device__ __forceinline__ int Dot2I16(uint32_t a, uint32_t b, int c)
-{
-    typedef short I16x2 __attribute__((ext_vector_type(2)));
-    I16x2 x, y;
-    __builtin_memcpy(&x, &a, 4);
-    __builtin_memcpy(&y, &b, 4);
-    return __builtin_amdgcn_sdot2(x, y, c, false);
-}
-
-// a.lo * b.lo + a.hi * b.hi with nothing added: the three-operand form with the constant 0 (for a sum
-// that starts here the compiler picks the accumulate-in-place form and spends a move on clearing it).
-__device__ __forceinline__ int Dot2I16(uint32_t a, uint32_t b)
-{
-    int d;
-    asm("v_dot2_i32_i16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
-    return d;
-}
-
 // CubicCoeffs times `scale` (a power of two, so every step scales exactly) with the polynomials evaluated
 // by fused multiply-adds; used where the weights are quantised afterwards anyway.
 __device__ __forceinline__ void CubicCoeffsFused(float d, float scale, float (&w)[4])

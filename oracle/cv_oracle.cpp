@@ -682,10 +682,40 @@ void ResizeOne(const T *src, int64_t srcStep, int srcW, int srcH, T *dst, int64_
                 };
                 coeffs(fx, wx);
                 coeffs(fy, wy);
+                if (variant == 7 && std::is_same_v<T, uint8_t>)
+                {
+                    // the product library's 8-bit bicubic resize: indices and weights of the device formula, the
+                    // horizontal weights rounded to multiples of 2^-14 (to nearest, ties to even) with the last one
+                    // taking the remainder, a row's sum exact in integers, the four row sums added in float32,
+                    // ascending, the first as a product and the others by fused multiply-adds, the magnitude
+                    // rounded to nearest-even
+                    int wq[4];
+                    for (int i = 0; i < 3; ++i)
+                    {
+                        wq[i] = (int)std::nearbyint(wx[i] * 16384.f);
+                    }
+                    wq[3] = 16384 - wq[0] - wq[1] - wq[2];
+                    for (int c = 0; c < C; ++c)
+                    {
+                        float acc = 0.f;
+                        for (int row = 0; row < 4; ++row)
+                        {
+                            int h = 0;
+                            for (int i = 0; i < 4; ++i)
+                            {
+                                h += (int)src[tapY(sy + row - 1) * srcStep + (int64_t)tapX(sx + i - 1) * C + c] * wq[i];
+                            }
+                            const float w = wy[row] * (1.f / 16384.f);
+                            acc           = row == 0 ? (float)h * w : std::fmaf((float)h, w, acc);
+                        }
+                        out[c] = SatF<T>(std::abs(acc));
+                    }
+                    continue;
+                }
                 for (int c = 0; c < C; ++c)
                 {
                     float sum = 0.f;
-                    if (variant == 1) // tensor kernel: sum += p * (wx*wy), y outer, x inner
+                    if (variant == 1 || variant == 7) // tensor kernel: sum += p * (wx*wy), y outer, x inner
                     {
                         for (int cy = -1; cy <= 2; ++cy)
                         {

@@ -80,12 +80,15 @@ def resize(src, out_hw, interp, variant=0, threads=1):
 
 def resize_shipped(src, out_hw, interp, varshape=False, threads=1):
     """The restatement of what the product library's Resize computes for this element type and interpolation:
-    8-bit bilinear is the fixed-point blend (variant 4) for tensors and image batches alike; the 8-bit box filter
+    8-bit bilinear and bicubic are the fixed-point blends (variants 4 and 7) for tensors and image batches alike; the
+    8-bit box filter
     is the fixed-point form at reductions of up to 3 and the device formula elsewhere (variants 5 and, for image
     batches, 6); everything else is the reference's device formula (variant 1; variant 2, its image-batch
     association, with varshape)."""
     if int(interp) == 1 and np.dtype(src.dtype) == np.uint8:
         variant = 4
+    elif int(interp) == 2 and np.dtype(src.dtype) == np.uint8:
+        variant = 7
     elif int(interp) == 3 and np.dtype(src.dtype) == np.uint8:
         variant = 6 if varshape else 5
     else:

@@ -48,6 +48,9 @@ def cases():
                 if interp == LINEAR and dt == np.uint8:
                     # the shipped 8-bit bilinear blend (15-bit fixed point), to be reproduced bit for bit
                     out["resize_linear_fixed_uint8%d_%s" % (c, tag)] = orc.resize(a, hw, interp, variant=4)
+                if interp == CUBIC and dt == np.uint8:
+                    # the shipped 8-bit bicubic blend (14-bit horizontal weights, integer row sums), bit for bit
+                    out["resize_cubic_fixed_uint8%d_%s" % (c, tag)] = orc.resize(a, hw, interp, variant=7)
                 if interp == AREA and dt == np.uint8 and tag == "down":
                     # the shipped 8-bit box filter at reductions of up to 3 (fixed-point rows), bit for bit
                     out["resize_area_fixed_uint8%d_down" % c] = orc.resize(a, hw, interp, variant=5)

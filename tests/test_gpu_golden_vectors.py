@@ -63,6 +63,8 @@ def test_resize(cv, gold, gpu, dt, c):
             got = out.numpy()
             if interp == LINEAR and dt == np.uint8:
                 close(got, vec["resize_linear_fixed_uint8%d_%s" % (c, tag)])
+            if interp == CUBIC and dt == np.uint8:
+                close(got, vec["resize_cubic_fixed_uint8%d_%s" % (c, tag)])
             if interp == AREA and dt == np.uint8 and tag == "down":
                 close(got, vec["resize_area_fixed_uint8%d_down" % c])
             if interp == NEAREST:

@@ -223,6 +223,38 @@ def test_resize_area_fixed_point_variant(orc):
         np.testing.assert_array_equal(orc.resize(src, (dh, dw), AREA, variant=6), orc.resize(src, (dh, dw), AREA, variant=2))
 
 
+
+def test_resize_cubic_fixed_point_variant(orc):
+    # Variant 7 (the product library's 8-bit bicubic resize) against the float64 golden: never more than 1 apart,
+    # under 1 % of the outputs differ (the horizontal weights are rounded to 2^-14 and add up to exactly 1); constant
+    # images stay constant, equal sizes copy the interior (fractions 0: weights 0, 1, 0, 0), and the hand-computed pixels of
+    # test_resize_cubic_hand_weights_interior_and_border_row hold for it as for the float32 variants. Other element
+    # types take the float32 device formula.
+    rng = np.random.default_rng(77)
+    for (sw, sh, dw, dh, c) in [(97, 61, 61, 40, 3), (64, 48, 100, 77, 3), (50, 40, 17, 14, 4), (30, 20, 45, 33, 1), (5, 4, 9, 7, 3)]:
+        src = rng.integers(0, 256, (2, sh, sw, c), dtype=np.uint8)
+        got = orc.resize(src, (dh, dw), CUBIC, variant=7).astype(np.int32)
+        gold = orc.resize(src, (dh, dw), CUBIC, variant=0).astype(np.int32)
+        assert np.abs(got - gold).max() <= 1 and (got != gold).mean() < 0.01, (sw, sh, dw, dh, c)
+    src = rng.integers(0, 256, (1, 23, 31, 3), dtype=np.uint8)
+    # (the reference's border band, 1 pixel in front and 3 behind, moves the centre: equal sizes copy the interior)
+    np.testing.assert_array_equal(orc.resize(src, (23, 31), CUBIC, variant=7)[:, 1:-3, 1:-3], src[:, 1:-3, 1:-3])
+    const = np.full((1, 19, 27, 3), 143, np.uint8)
+    assert np.unique(orc.resize(const, (31, 11), CUBIC, variant=7)).tolist() == [143]
+    f = rng.random((1, 12, 14, 2)).astype(np.float32)
+    np.testing.assert_array_equal(orc.resize(f, (7, 9), CUBIC, variant=7), orc.resize(f, (7, 9), CUBIC, variant=1))
+    # 6 x 6 -> 4 x 4: the weights of fractions 0.75 and 0.25 are multiples of 2^-8, exact in 14 bits, so every pixel is
+    # the hand-computed sum rounded once (interior, the row band that keeps its fraction, the column band that drops it)
+    w75 = np.array([-0.03515625, 0.26171875, 0.87890625, -0.10546875])
+    w25 = w75[::-1]
+    img = rng.integers(0, 256, (1, 6, 6, 1), dtype=np.uint8)
+    a = img[0, :, :, 0].astype(np.float64)
+    out = orc.resize(img, (4, 4), CUBIC, variant=7)[0, :, :, 0].astype(np.float64)
+    for got, want in [(out[1, 1], w75 @ a[0:4, 0:4] @ w75), (out[0, 1], w25 @ a[0:4, 0:4] @ w75), (out[1, 0], w75 @ a[0:4, 1]),
+                      (out[0, 0], w25 @ a[0:4, 1]), (out[3, 1], w75 @ a[2:6, 0:4] @ w75), (out[1, 3], w75 @ a[0:4, 3])]:
+        assert abs(got - min(abs(want), 255.0)) <= 0.5 + 1e-3, (got, want)
+
+
 def test_resize_cubic_hand_weights_interior_and_border_row(orc):
     # 6 x 6 -> 4 x 4 (scale 1.5): output index 1 maps to source 1.75 (centre 1, fraction 0.75, interior), output
     # index 0 to 0.25 (centre 0, fraction 0.25, in the border band). Keys kernel with A = -0.75, written out by hand:
