@@ -5,7 +5,9 @@
 // src/cvcuda/priv/legacy/resize_var_shape.cu:92-231 for the var-shape association of the sums).
 // The nearest-neighbour source index uses the single-multiply form floor((d+.5f)*scale) of the
 // reference's CPU golden (tests/cvcuda/system/ResizeUtils.cpp:206-221) for every pixel, so results
-// are bit-exact against it also where the coordinate lands on an integer.
+// are bit-exact against it also where the coordinate lands on an integer. 8-bit pixels are blended in fixed
+// point on those indices and weights (bilinear: FixedPointBlend.hpp; bicubic: kFixedCubic; box filter:
+// kAreaFixed), at most 1 from the reference's goldens.
 //
 // Five kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
@@ -933,8 +935,11 @@ __device__ __forceinline__ uint32_t CubicRowsQ14(const Plane &p, int y0, uint32_
     return q;
 }
 
-// One output pixel from its column terms (per lane) and row terms (wave-uniform).
-template<class T, int C, int INTERP, bool VARSHAPE>
+// One output pixel from its column terms (per lane) and row terms (wave-uniform). GUARDED: the image's last row may
+// be among the rows read, so every tap load tests for it (its loads must not run past the image's end); the caller
+// settles that once per wave patch, because a wave-uniform test in front of a load keeps the compiler from requesting
+// the next load before this one has returned.
+template<class T, int C, int INTERP, bool VARSHAPE, bool GUARDED>
 __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerms<kWeights<INTERP>> &col,
                                                   const AxisTerms<kWeights<INTERP>> &row)
 {
@@ -944,7 +949,7 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
     if constexpr (INTERP == NVCV_INTERP_NEAREST)
     {
         float t[1][C];
-        LoadTaps<T, C, 1>(p.src + (int64_t)row.s * p.srcRow, col.s * PB, row.s == p.srcH - 1, rowBytes, t);
+        LoadTaps<T, C, 1>(p.src + (int64_t)row.s * p.srcRow, col.s * PB, GUARDED && row.s == p.srcH - 1, rowBytes, t);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -958,8 +963,8 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
         if constexpr (kFixedLinear<T>)
         {
             uint32_t r0[2], r1[2], top, bottom, q = 0;
-            LoadTapPairBytes<C>(p.src + (int64_t)y0 * p.srcRow, col.s * PB, y0 == p.srcH - 1, rowBytes, r0);
-            LoadTapPairBytes<C>(p.src + (int64_t)y1 * p.srcRow, col.s * PB, y1 == p.srcH - 1, rowBytes, r1);
+            LoadTapPairBytes<C>(p.src + (int64_t)y0 * p.srcRow, col.s * PB, GUARDED && y0 == p.srcH - 1, rowBytes, r0);
+            LoadTapPairBytes<C>(p.src + (int64_t)y1 * p.srcRow, col.s * PB, GUARDED && y1 == p.srcH - 1, rowBytes, r1);
             WeightPairsQ15(FractionQ15(wx), FractionQ15(wy), top, bottom);
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -971,8 +976,8 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
             return out;
         }
         float       t0[2][C], t1[2][C];
-        LoadTaps<T, C, 2>(p.src + (int64_t)y0 * p.srcRow, col.s * PB, y0 == p.srcH - 1, rowBytes, t0);
-        LoadTaps<T, C, 2>(p.src + (int64_t)y1 * p.srcRow, col.s * PB, y1 == p.srcH - 1, rowBytes, t1);
+        LoadTaps<T, C, 2>(p.src + (int64_t)y0 * p.srcRow, col.s * PB, GUARDED && y0 == p.srcH - 1, rowBytes, t0);
+        LoadTaps<T, C, 2>(p.src + (int64_t)y1 * p.srcRow, col.s * PB, GUARDED && y1 == p.srcH - 1, rowBytes, t1);
 #pragma unroll
         for (int c = 0; c < C; ++c)
         {
@@ -1004,16 +1009,7 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
         const uint32_t off = (uint32_t)(col.s - 1) * C, at = C == 4 ? off : off & ~3u, shift = off & 3u;
         const int      y0 = row.s - 1; // rows y0 .. y0 + 3, inside the image for sources of 4 rows and more
         uint32_t       q;
-        // the four windows are requested together; the form that guards the image's last row only where it is among them
-        // (wave-uniform)
-        if (y0 + 3 >= p.srcH - 1 || y0 < 0)
-        {
-            q = CubicRowsQ14<C, true>(p, y0, at, shift, (uint32_t)rowBytes, w01, w23, row.w);
-        }
-        else
-        {
-            q = CubicRowsQ14<C, false>(p, y0, at, shift, (uint32_t)rowBytes, w01, w23, row.w);
-        }
+        q = CubicRowsQ14<C, GUARDED>(p, y0, at, shift, (uint32_t)rowBytes, w01, w23, row.w); // four windows together
         __builtin_memcpy(&out, &q, PB);
     }
     else
@@ -1029,7 +1025,7 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
         {
             const int yy = max(0, min(row.s - 1 + j, p.srcH - 1));
             float     t[4][C];
-            LoadTaps<T, C, 4>(p.src + (int64_t)yy * p.srcRow, (col.s - 1) * PB, yy == p.srcH - 1, rowBytes, t);
+            LoadTaps<T, C, 4>(p.src + (int64_t)yy * p.srcRow, (col.s - 1) * PB, GUARDED && yy == p.srcH - 1, rowBytes, t);
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
@@ -1153,17 +1149,31 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
                 rows.w[i] *= 1.f / 16384.f;
             }
         }
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
+        // the last source row the patch reads (row indices ascend with the output row; bilinear reads one more, bicubic
+        // two): only a patch that reaches the image's last row needs the guarded loads (wave-uniform)
+        constexpr int reach = INTERP == NVCV_INTERP_NEAREST ? 0 : (INTERP == NVCV_INTERP_LINEAR ? 1 : 2);
+        auto          sample = [&](auto guarded)
         {
-            const Pixel<T, C> out  = SampleWide<T, C, INTERP, VARSHAPE>(p, col, FromLane(rows, k));
-            uint32_t          w[D] = {};
-            __builtin_memcpy(w, &out, PB);
 #pragma unroll
-            for (int d = 0; d < D; ++d)
+            for (int k = 0; k < 4; ++k)
             {
-                q[d][k] = w[d];
+                const Pixel<T, C> out  = SampleWide<T, C, INTERP, VARSHAPE, decltype(guarded)::value>(p, col, FromLane(rows, k));
+                uint32_t          w[D] = {};
+                __builtin_memcpy(w, &out, PB);
+#pragma unroll
+                for (int d = 0; d < D; ++d)
+                {
+                    q[d][k] = w[d];
+                }
             }
+        };
+        if (__builtin_amdgcn_readlane(rows.s, 3) + reach >= p.srcH - 1)
+        {
+            sample(std::true_type{});
+        }
+        else
+        {
+            sample(std::false_type{});
         }
     }
     else
