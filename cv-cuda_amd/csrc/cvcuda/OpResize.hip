@@ -935,6 +935,111 @@ __device__ __forceinline__ uint32_t CubicRowsQ14(const Plane &p, int y0, uint32_
     return q;
 }
 
+// The same for TWO vertically adjacent output pixels per lane whose 4-row windows start `N - 4` rows apart (0 .. 2) and
+// lie inside the image, clear of its last row: the N source rows from y0 on are loaded once, each row's sums are
+// formed once, and each pixel adds its own four in ascending order - the sums and their order are those of
+// CubicRowsQ14, so the result is the same bit for bit. At scale 1.5 that is 5 or 6 row sums where two pixels took 8.
+template<int C, int N>
+__device__ __forceinline__ void CubicRowPairQ14(const Plane &p, int y0, uint32_t at, uint32_t shift, uint32_t rowBytes,
+                                                uint32_t w01, uint32_t w23, const float (&wyA)[4], const float (&wyB)[4],
+                                                uint32_t (&out)[2])
+{
+    uint32_t       r[N][C];
+    const uint8_t *first = p.src + (int64_t)y0 * p.srcRow;
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+    {
+        LoadQuadWindow<C, false>(first + (int64_t)j * p.srcRow, at, shift, false, rowBytes, r[j]);
+    }
+    float accA[C], accB[C];
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            const float h = (float)Dot2I16(QuadTapPair<C>(r[j], 2, c), w23, Dot2I16(QuadTapPair<C>(r[j], 0, c), w01));
+            if (j < 4)
+            {
+                accA[c] = j == 0 ? h * wyA[0] : fmaf(h, wyA[j], accA[c]);
+            }
+            if (j >= N - 4)
+            {
+                accB[c] = j == N - 4 ? h * wyB[0] : fmaf(h, wyB[j - (N - 4)], accB[c]);
+            }
+        }
+    }
+    out[0] = out[1] = 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        out[0] = __builtin_amdgcn_cvt_pk_u8_f32(fabsf(accA[c]), c, out[0]);
+        out[1] = __builtin_amdgcn_cvt_pk_u8_f32(fabsf(accB[c]), c, out[1]);
+    }
+}
+
+// The part of the 8-bit bicubic sum that depends on the output column only.
+struct CubicColumnQ14
+{
+    uint32_t w01, w23;  // horizontal weights in units of 2^-14, packed in pairs
+    uint32_t at, shift; // the window load's byte offset in a row and the window's position in it
+};
+
+template<int C>
+__device__ __forceinline__ CubicColumnQ14 CubicColumn(const AxisTerms<4> &col)
+{
+    CubicColumnQ14 q;
+    float          wx[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        wx[i] = col.w[i] * 16384.f;
+    }
+    CubicWeightPairsQ14(wx, q.w01, q.w23);
+    const uint32_t off = (uint32_t)(col.s - 1) * C;
+    q.at               = C == 4 ? off : off & ~3u;
+    q.shift            = off & 3u;
+    return q;
+}
+
+// A lane's 4 output pixels (rows k = 0 .. 3 of a wave patch, row terms in lanes 0 .. 3 of `rows`, vertical weights
+// already in units of 2^-14) of the 8-bit bicubic form, clear of the image's last row: output rows in pairs that
+// share the source rows between their windows (wave-uniform choice by how far the windows are apart; farther than
+// 2: one by one).
+template<int C>
+__device__ __forceinline__ void CubicPatchPairsQ14(const Plane &p, const AxisTerms<4> &col, const AxisTerms<4> &rows,
+                                                   uint32_t (&q)[4])
+{
+    const CubicColumnQ14 cq = CubicColumn<C>(col);
+    const uint32_t       rb = (uint32_t)p.srcW * C;
+#pragma unroll
+    for (int k = 0; k < 4; k += 2)
+    {
+        const auto rowA = FromLane(rows, k), rowB = FromLane(rows, k + 1);
+        const int  apart = rowB.s - rowA.s;
+        uint32_t   two[2];
+        if (apart == 1)
+        {
+            CubicRowPairQ14<C, 5>(p, rowA.s - 1, cq.at, cq.shift, rb, cq.w01, cq.w23, rowA.w, rowB.w, two);
+        }
+        else if (apart == 2)
+        {
+            CubicRowPairQ14<C, 6>(p, rowA.s - 1, cq.at, cq.shift, rb, cq.w01, cq.w23, rowA.w, rowB.w, two);
+        }
+        else if (apart == 0)
+        {
+            CubicRowPairQ14<C, 4>(p, rowA.s - 1, cq.at, cq.shift, rb, cq.w01, cq.w23, rowA.w, rowB.w, two);
+        }
+        else
+        {
+            two[0] = CubicRowsQ14<C, false>(p, rowA.s - 1, cq.at, cq.shift, rb, cq.w01, cq.w23, rowA.w);
+            two[1] = CubicRowsQ14<C, false>(p, rowB.s - 1, cq.at, cq.shift, rb, cq.w01, cq.w23, rowB.w);
+        }
+        q[k]     = two[0];
+        q[k + 1] = two[1];
+    }
+}
+
 // One output pixel from its column terms (per lane) and row terms (wave-uniform). GUARDED: the image's last row may
 // be among the rows read, so every tap load tests for it (its loads must not run past the image's end); the caller
 // settles that once per wave patch, because a wave-uniform test in front of a load keeps the compiler from requesting
@@ -998,18 +1103,9 @@ __device__ __forceinline__ Pixel<T, C> SampleWide(const Plane &p, const AxisTerm
     else if constexpr (kFixedCubic<T>)
     {
         // (the column's part of this does not depend on the row and is computed once per lane)
-        float wx[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-        {
-            wx[i] = col.w[i] * 16384.f;
-        }
-        uint32_t w01, w23;
-        CubicWeightPairsQ14(wx, w01, w23);
-        const uint32_t off = (uint32_t)(col.s - 1) * C, at = C == 4 ? off : off & ~3u, shift = off & 3u;
-        const int      y0 = row.s - 1; // rows y0 .. y0 + 3, inside the image for sources of 4 rows and more
-        uint32_t       q;
-        q = CubicRowsQ14<C, GUARDED>(p, y0, at, shift, (uint32_t)rowBytes, w01, w23, row.w); // four windows together
+        const CubicColumnQ14 cq = CubicColumn<C>(col);
+        // rows row.s - 1 .. row.s + 2, inside the image for sources of 4 rows and more; four windows together
+        const uint32_t q = CubicRowsQ14<C, GUARDED>(p, row.s - 1, cq.at, cq.shift, (uint32_t)rowBytes, cq.w01, cq.w23, row.w);
         __builtin_memcpy(&out, &q, PB);
     }
     else
@@ -1170,6 +1266,10 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
         if (__builtin_amdgcn_readlane(rows.s, 3) + reach >= p.srcH - 1)
         {
             sample(std::true_type{});
+        }
+        else if constexpr (INTERP == NVCV_INTERP_CUBIC && kFixedCubic<T>)
+        {
+            CubicPatchPairsQ14<C>(p, col, rows, q[0]);
         }
         else
         {
