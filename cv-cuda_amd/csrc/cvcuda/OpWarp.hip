@@ -631,6 +631,42 @@ __device__ __forceinline__ uint32_t SampleInsideQ15(const Img &im, float sx, flo
 // four taps are fetched at coordinates clamped into the image and, for the constant border, replaced where the
 // unclamped coordinate is outside. sx, sy in units of 2^-15 pixel, below 2^30 in magnitude. Same weights, same
 // exact sum and the same single rounding as the generic path, so which path a sample takes does not show.
+// The border modes' index maps for coordinates no farther than one image size outside the image (-(s - 1) .. 2s - 2
+// for an axis of s pixels), where each is a single fold: index = c inside, k * c + lo in front, k * c + hi behind,
+// with wave-uniform k, lo, hi per mode (DeviceUtils.hpp:BorderIndex for any coordinate, with its divisions):
+//   constant, replicate  0 * c + 0      | 0 * c + s - 1     (the nearest pixel; the constant colour replaces it later)
+//   reflect             -1 * c - 1      | -1 * c + 2s - 1
+//   wrap                 1 * c + s      |  1 * c - s
+//   reflect101          -1 * c          | -1 * c + 2s - 2
+struct BorderFold
+{
+    int k, lo, hi, size;
+};
+
+__device__ __forceinline__ BorderFold MakeBorderFold(int border, int s)
+{
+    BorderFold f = {0, 0, s - 1, s};
+    if (border == NVCV_BORDER_REFLECT)
+    {
+        f = {-1, -1, 2 * s - 1, s};
+    }
+    else if (border == NVCV_BORDER_WRAP)
+    {
+        f = {1, s, -s, s};
+    }
+    else if (border == NVCV_BORDER_REFLECT101)
+    {
+        f = {-1, 0, 2 * s - 2, s};
+    }
+    return f;
+}
+
+__device__ __forceinline__ int Fold(const BorderFold &f, int c)
+{
+    const int kc = f.k * c;
+    return c < 0 ? kc + f.lo : (c >= f.size ? kc + f.hi : c);
+}
+
 // Pixel (x, y) of an 8-bit image, inside it, as a dword (channel c in byte c, the rest is not looked at): one
 // 4-byte load, moved back where it would run past the image's last byte.
 template<int C>
@@ -642,12 +678,13 @@ __device__ __forceinline__ uint32_t LoadPixelGuarded(const Img &im, uint32_t row
 }
 
 template<int C>
-__device__ __forceinline__ uint32_t SampleNearBorderQ15(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
+__device__ __forceinline__ uint32_t SampleNearBorderQ15(const Img &im, const BorderFold &fx, const BorderFold &fy, bool constant,
+                                                        uint32_t borderPx, float sx, float sy)
 {
     const int X = __float2int_rd(sx), Y = __float2int_rd(sy);
     const int x0 = X >> 15, y0 = Y >> 15;
-    const int cx0 = min(max(x0, 0), im.w - 1), cx1 = min(max(x0 + 1, 0), im.w - 1);
-    const uint32_t r0 = (uint32_t)__mul24(min(max(y0, 0), im.h - 1), im.row), r1 = (uint32_t)__mul24(min(max(y0 + 1, 0), im.h - 1), im.row);
+    const int cx0 = Fold(fx, x0), cx1 = Fold(fx, x0 + 1);
+    const uint32_t r0 = (uint32_t)__mul24(Fold(fy, y0), im.row), r1 = (uint32_t)__mul24(Fold(fy, y0 + 1), im.row);
     uint32_t p00 = LoadPixelGuarded<C>(im, r0, cx0), p01 = LoadPixelGuarded<C>(im, r0, cx1);
     uint32_t p10 = LoadPixelGuarded<C>(im, r1, cx0), p11 = LoadPixelGuarded<C>(im, r1, cx1);
     if (constant) // uniform
@@ -665,7 +702,8 @@ __device__ __forceinline__ uint32_t SampleNearBorderQ15(const Img &im, bool cons
 // The same for the fixed-point bicubic sum: the 4 x 4 taps fetched at clamped coordinates (replaced by the colour
 // where the unclamped one is outside), put together as the rows BlendCubicQ14 takes. |sx|, |sy| below 2^24.
 template<int C>
-__device__ __forceinline__ uint32_t SampleNearBorderCubicQ14(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
+__device__ __forceinline__ uint32_t SampleNearBorderCubicQ14(const Img &im, const BorderFold &fx, const BorderFold &fy,
+                                                             bool constant, uint32_t borderPx, float sx, float sy)
 {
     const int ix = (int)floorf(sx) - 1, iy = (int)floorf(sy) - 1;
     int       cx[4];
@@ -673,14 +711,14 @@ __device__ __forceinline__ uint32_t SampleNearBorderCubicQ14(const Img &im, bool
 #pragma unroll
     for (int i = 0; i < 4; ++i)
     {
-        cx[i]  = min(max(ix + i, 0), im.w - 1);
+        cx[i]  = Fold(fx, ix + i);
         inX[i] = (uint32_t)(ix + i) < (uint32_t)im.w;
     }
     uint32_t r[4][C];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
     {
-        const uint32_t rowOffset = (uint32_t)__mul24(min(max(iy + j, 0), im.h - 1), im.row);
+        const uint32_t rowOffset = (uint32_t)__mul24(Fold(fy, iy + j), im.row);
         const bool     inY       = (uint32_t)(iy + j) < (uint32_t)im.h;
         uint32_t       p[4];
 #pragma unroll
@@ -717,10 +755,11 @@ __device__ __forceinline__ uint32_t SampleNearBorderCubicQ14(const Img &im, bool
 
 // And for the nearest pixel.
 template<int C>
-__device__ __forceinline__ uint32_t SampleNearBorderNearest(const Img &im, bool constant, uint32_t borderPx, float sx, float sy)
+__device__ __forceinline__ uint32_t SampleNearBorderNearest(const Img &im, const BorderFold &fx, const BorderFold &fy,
+                                                            bool constant, uint32_t borderPx, float sx, float sy)
 {
     const int      x = FloorToInt(sx + .5f), y = FloorToInt(sy + .5f);
-    const uint32_t p = LoadPixelGuarded<C>(im, (uint32_t)__mul24(min(max(y, 0), im.h - 1), im.row), min(max(x, 0), im.w - 1));
+    const uint32_t p = LoadPixelGuarded<C>(im, (uint32_t)__mul24(Fold(fy, y), im.row), Fold(fx, x));
     // (the bytes above the pixel's must be 0: the stores merge neighbouring pixels' dwords)
     return constant && !((uint32_t)x < (uint32_t)im.w && (uint32_t)y < (uint32_t)im.h) ? borderPx : p & (0xffffffffu >> (32 - 8 * C));
 }
@@ -866,9 +905,10 @@ __device__ __forceinline__ void SampleAllOutside(const WarpArgs &a, float sx, fl
 template<class T, int C>
 constexpr bool kNearBorderForms = std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4);
 
-// Whether a lane's samples can take them: one of the two border modes that need no division, an image of 4 bytes or
-// more within the 24-bit offsets (the caller's test), and every coordinate small enough for the sampler's integer
-// conversion (bilinear: times 2^15 below 2^30; bicubic: below 2^24; nearest: any).
+// Whether a lane's samples can take them: an image of 4 bytes or more within the 24-bit offsets (the caller's test),
+// every coordinate small enough for the sampler's integer conversion (bilinear: times 2^15 below 2^30; bicubic:
+// below 2^24; nearest: any) and, for the three modes that mirror or repeat the image, every tap no farther than one
+// image size outside it (BorderFold; with a margin of two pixels for the widest tap window).
 template<class T, int C, int INTERP>
 __device__ __forceinline__ bool NearBorderForm(const Img &im, const WarpArgs &a, const float (&sx)[kPxPerLane],
                                                const float (&sy)[kPxPerLane])
@@ -879,14 +919,27 @@ __device__ __forceinline__ bool NearBorderForm(const Img &im, const WarpArgs &a,
     }
     else
     {
-        uint32_t u = 0;
+        constexpr float kScale = kCoordScale<T, INTERP>;
+        uint32_t        u = 0;
+        float           minX = sx[0], maxX = sx[0], minY = sy[0], maxY = sy[0];
 #pragma unroll
         for (int k = 0; k < kPxPerLane; ++k)
         {
-            u = max(u, max(__float_as_uint(sx[k]) & 0x7fffffffu, __float_as_uint(sy[k]) & 0x7fffffffu));
+            u    = max(u, max(__float_as_uint(sx[k]) & 0x7fffffffu, __float_as_uint(sy[k]) & 0x7fffffffu));
+            minX = fminf(minX, sx[k]);
+            maxX = fmaxf(maxX, sx[k]);
+            minY = fminf(minY, sy[k]);
+            maxY = fmaxf(maxY, sy[k]);
         }
         const uint32_t limit = INTERP == NVCV_INTERP_LINEAR ? 0x4e800000u : (INTERP == NVCV_INTERP_CUBIC ? 0x4b800000u : 0x7f800000u);
-        return a.border <= NVCV_BORDER_REPLICATE && u < limit && __mul24(im.h - 1, im.row) + im.w * C >= 4;
+        bool           ok = u < limit && __mul24(im.h - 1, im.row) + im.w * C >= 4;
+        if (a.border > NVCV_BORDER_REPLICATE) // wave-uniform
+        {
+            // taps reach from floor(v) - 1 to floor(v) + 2 at most: all of them within -(s - 1) .. 2s - 2
+            ok = ok && minX >= (float)(2 - im.w) * kScale && maxX < (float)(2 * im.w - 4) * kScale
+              && minY >= (float)(2 - im.h) * kScale && maxY < (float)(2 * im.h - 4) * kScale;
+        }
+        return ok;
     }
 }
 
@@ -951,8 +1004,9 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
             }
             // under a constant border a lane whose samples lie outside with all their taps needs no pixel: whole
             // waves in the corners a rotation leaves empty
-            const bool constant = a.border == NVCV_BORDER_CONSTANT;
-            bool       outside  = constant;
+            const bool       constant = a.border == NVCV_BORDER_CONSTANT;
+            const BorderFold foldX = MakeBorderFold(a.border, im.w), foldY = MakeBorderFold(a.border, im.h);
+            bool             outside = constant;
 #pragma unroll
             for (int k = 0; k < kPxPerLane; ++k)
             {
@@ -983,15 +1037,15 @@ __device__ __forceinline__ void WarpTile(const Img &im, const WarpArgs &a, const
                 {
                     if constexpr (INTERP == NVCV_INTERP_LINEAR)
                     {
-                        q[0][k] = SampleNearBorderQ15<C>(im, constant, borderPx, sx[k], sy[k]);
+                        q[0][k] = SampleNearBorderQ15<C>(im, foldX, foldY, constant, borderPx, sx[k], sy[k]);
                     }
                     else if constexpr (INTERP == NVCV_INTERP_CUBIC)
                     {
-                        q[0][k] = SampleNearBorderCubicQ14<C>(im, constant, borderPx, sx[k], sy[k]);
+                        q[0][k] = SampleNearBorderCubicQ14<C>(im, foldX, foldY, constant, borderPx, sx[k], sy[k]);
                     }
                     else
                     {
-                        q[0][k] = SampleNearBorderNearest<C>(im, constant, borderPx, sx[k], sy[k]);
+                        q[0][k] = SampleNearBorderNearest<C>(im, foldX, foldY, constant, borderPx, sx[k], sy[k]);
                     }
                 }
             }

@@ -63,17 +63,36 @@ def test_reference_table_exact(cv, orc, gpu, interp, border):
 def test_tiny_sources_at_the_border_forms_limits(cv, orc, gpu, c):
     # 8-bit samples next to the image's edge take straight-line forms that fetch a pixel with one 4-byte load, moved
     # back where it would pass the image's last byte; images of under 4 bytes keep the generic loop. Sources of 1 to
-    # 5 pixels, every interpolation, both border modes of those forms and one other: exact against the restatement.
+    # 5 pixels (the mirroring and repeating borders' single folds do not reach that far: generic loop), every
+    # interpolation and border mode: exact against the restatement.
     op = cv.WarpAffine(0)
     m = [0.8, 0.3, -0.4, -0.2, 0.9, 0.6]
     for (sw, sh) in [(1, 1), (2, 1), (1, 2), (3, 1), (1, 4), (2, 2), (5, 1), (1, 5)]:
         src = orc.fill_u8((2, sh, sw, c), 40 + sw * 7 + sh)
-        for interp, border in itertools.product((NEAREST, LINEAR, CUBIC), (0, 1, 4)):
+        for interp, border in itertools.product((NEAREST, LINEAR, CUBIC), (0, 1, 2, 3, 4)):
             tout = cv.Tensor.alloc([2, 6, 9, c], np.uint8, "NHWC")
             op(None, cv.Tensor.from_numpy(src, "NHWC"), tout, m, interp | INVERSE_MAP, border, (9, 200, 31, 77))
             torch.cuda.synchronize()
             dev = orc.warp(src, (6, 9), np.asarray(m, np.float32), interp, border, (9, 200, 31, 77), variant=device_variant(interp))
             np.testing.assert_array_equal(tout.numpy(), dev, err_msg=str((sw, sh, c, interp, border)))
+
+
+
+@pytest.mark.parametrize("c", [1, 3, 4])
+def test_mirroring_and_repeating_borders_near_and_far(cv, orc, gpu, c):
+    # Under REFLECT, WRAP and REFLECT101 samples whose taps lie within one image size of the image take straight-line
+    # forms with a single fold of the index; farther out the generic loop with its modulo. A destination 5 times the
+    # source's size around it, shifted and slightly rotated, has both kinds in every interpolation: exact.
+    op = cv.WarpAffine(0)
+    sw, sh = 23, 17
+    src = orc.fill_u8((2, sh, sw, c), 77 + c)
+    m = [0.93, 0.11, -2.3 * sw, -0.07, 1.04, -1.9 * sh]  # destination (0, 0) maps about two image sizes in front
+    for interp, border in itertools.product((NEAREST, LINEAR, CUBIC), (2, 3, 4)):
+        tout = cv.Tensor.alloc([2, 5 * sh, 5 * sw, c], np.uint8, "NHWC")
+        op(None, cv.Tensor.from_numpy(src, "NHWC"), tout, m, interp | INVERSE_MAP, border, (0, 0, 0, 0))
+        torch.cuda.synchronize()
+        dev = orc.warp(src, (5 * sh, 5 * sw), np.asarray(m, np.float32), interp, border, (0, 0, 0, 0), variant=device_variant(interp))
+        np.testing.assert_array_equal(tout.numpy(), dev, err_msg=str((c, interp, border)))
 
 
 def rotation(w, h, deg, s):
