@@ -143,6 +143,25 @@ __global__ __launch_bounds__(256) void ReformatRunsKernel(const ReformatArgs a)
 template<class T, int C>
 void LaunchC(const ReformatArgs &a, int N, bool srcIl, bool dstIl, hipStream_t stream)
 {
+    // Rows that are one dense run on both sides in the same order (packed interleaved to packed interleaved, or a
+    // single channel) are copied 16 bytes per lane whatever the pixel: as rows of 4-byte pixels in runs of 4.
+    {
+        const int64_t rowBytes = (int64_t)a.W * C * (int64_t)sizeof(T);
+        const bool    packed   = C == 1 ? (a.sW == (int64_t)sizeof(T) && a.dW == (int64_t)sizeof(T))
+                                        : (srcIl && dstIl && a.sW == (int64_t)(C * sizeof(T)) && a.dW == (int64_t)(C * sizeof(T)));
+        if (packed && rowBytes % 4 == 0 && (sizeof(T) < 4 || C == 1))
+        {
+            ReformatArgs b = a;
+            b.W            = (int32_t)(rowBytes / 4);
+            b.C            = 4;
+            b.sW = b.dW = 4;
+            b.sC = b.dC = 1;
+            dim3 grid(DivUp(b.W, kRunTileW), DivUp(b.H, kRunTileH), N), block(256);
+            hipLaunchKernelGGL((ReformatRunsKernel<uint8_t, 4, true, true>), grid, block, 0, stream, b);
+            CheckLaunch("ReformatRunsKernel");
+            return;
+        }
+    }
     if constexpr (sizeof(T) <= 2)
     {
         const bool srcPlanar = a.sW == (int64_t)sizeof(T), dstPlanar = a.dW == (int64_t)sizeof(T);
