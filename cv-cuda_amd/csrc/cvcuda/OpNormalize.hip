@@ -102,11 +102,17 @@ __global__ __launch_bounds__(256) void NormVarShape(const NormArgs a, const VarT
     NormPixel<TI, TO, C>(a, AsGlobal(s.basePtr) + (int64_t)y * s.rowStride, AsGlobal(d.basePtr) + (int64_t)y * d.rowStride, 0, 0, x);
 }
 
+// Pixels per lane of the run kernels: kRunPixelsFor, and for single-channel images as many as make 16 bytes on the
+// wider side (a lane that moves 4 bytes per instruction left the kernel at 3.3 of the 6.5 TB/s the 3-channel form
+// reaches on cached inputs).
+template<class TI, class TO, int C>
+constexpr int kNormRunPixels = C == 1 ? 16 / (int)(sizeof(TI) > sizeof(TO) ? sizeof(TI) : sizeof(TO)) : kRunPixelsFor<TI, TO>;
+
 // Per-channel base/scale: runs of P pixels per lane, one row per wave.
 template<class TI, class TO, int C>
 __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow, uint8_t *dstRow, int W, int x0)
 {
-    constexpr int P = kRunPixelsFor<TI, TO>;
+    constexpr int P = kNormRunPixels<TI, TO, C>;
     // every uniform value is loaded before the first use, so the loads share one round trip
     float b[C], m[C];
 #pragma unroll
@@ -166,7 +172,7 @@ __device__ __forceinline__ void NormRun(const NormArgs &a, const uint8_t *srcRow
 template<class TI, class TO, int C>
 __global__ __launch_bounds__(256) void NormRunsTensor(const NormArgs a)
 {
-    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kRunPixelsFor<TI, TO>;
+    const int x0 = (blockIdx.x * 64 + (threadIdx.x & 63)) * kNormRunPixels<TI, TO, C>;
     const int y  = blockIdx.y * kRunTileH + (threadIdx.x >> 6);
     if (x0 >= a.W || y >= a.H)
     {
@@ -178,7 +184,7 @@ __global__ __launch_bounds__(256) void NormRunsTensor(const NormArgs a)
 }
 
 template<class TI, class TO, int C>
-constexpr int kVarRows = kVarShapeRows<kRunPixelsFor<TI, TO> * C * (int)sizeof(TO)>;
+constexpr int kVarRows = kVarShapeRows<kNormRunPixels<TI, TO, C> * C * (int)sizeof(TO)>;
 
 template<class TI, class TO, int C>
 __global__ __launch_bounds__(256) void NormRunsVarShape(const NormArgs a, const VarTiles tiles)
@@ -186,7 +192,7 @@ __global__ __launch_bounds__(256) void NormRunsVarShape(const NormArgs a, const 
     const TileCoord              tc = LocateTile(tiles, blockIdx.x);
     const NVCVImagePlaneStrided &s  = a.srcList[tc.image].planes[0];
     const NVCVImagePlaneStrided &d  = a.dstList[tc.image].planes[0];
-    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kRunPixelsFor<TI, TO>;
+    const int                    x0 = (tc.tx * 64 + (threadIdx.x & 63)) * kNormRunPixels<TI, TO, C>;
     const uint8_t *src = AsGlobal(s.basePtr);
     uint8_t       *dst = AsGlobal(d.basePtr);
     const int      W = d.width, H = d.height, srcRow = s.rowStride, dstRow = d.rowStride;
@@ -218,7 +224,7 @@ void Launch(const NormArgs &a, int N, const NVCVImageBufferStrided *dstHost, hip
     {
         if (dstHost == nullptr)
         {
-            dim3 grid(DivUp(a.W, 64 * kRunPixelsFor<TI, TO>), DivUp(a.H, kRunTileH), N);
+            dim3 grid(DivUp(a.W, 64 * kNormRunPixels<TI, TO, C>), DivUp(a.H, kRunTileH), N);
             hipLaunchKernelGGL((NormRunsTensor<TI, TO, C>), grid, dim3(256), 0, stream, a);
             CheckLaunch("NormRunsTensor");
             return;
@@ -227,7 +233,7 @@ void Launch(const NormArgs &a, int N, const NVCVImageBufferStrided *dstHost, hip
         {
             VarTiles tiles;
             int total = BuildVarTiles(tiles, dstHost, first, std::min(kMaxTileImages, N - first),
-                                      64 * kRunPixelsFor<TI, TO>, kRunTileH * kVarRows<TI, TO, C>);
+                                      64 * kNormRunPixels<TI, TO, C>, kRunTileH * kVarRows<TI, TO, C>);
             if (total > 0)
             {
                 hipLaunchKernelGGL((NormRunsVarShape<TI, TO, C>), dim3(total), dim3(256), 0, stream, a, tiles);
