@@ -53,11 +53,49 @@ __device__ __forceinline__ void NormPixel(const NormArgs &a, const uint8_t *srcR
     const float     *pb = a.base.ptr + n * a.base.sN + y * a.base.sH + x * a.base.sW;
     const float     *ps = a.scale.ptr + n * a.scale.sN + y * a.scale.sH + x * a.scale.sW;
     Vec<TO, C>      *o  = reinterpret_cast<Vec<TO, C> *>(dstRow) + x;
+    // parameters whose channels are adjacent come as one load per pixel (wave-uniform choice), and a pixel of whole
+    // dwords leaves as one store: per channel, both were a third of the rate on 3-channel float images
+    float bv[C], sv[C];
+    if (a.base.sC == 1)
+    {
+        const Vec<float, C> t = *reinterpret_cast<const Vec<float, C> *>(pb);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            bv[c] = t.v[c];
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            bv[c] = pb[c * a.base.sC];
+        }
+    }
+    if (a.scale.sC == 1)
+    {
+        const Vec<float, C> t = *reinterpret_cast<const Vec<float, C> *>(ps);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            sv[c] = t.v[c];
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            sv[c] = ps[c * a.scale.sC];
+        }
+    }
+    Vec<TO, C> out;
 #pragma unroll
     for (int c = 0; c < C; ++c)
     {
-        const float b = pb[c * a.base.sC];
-        const float s = ps[c * a.scale.sC];
+        const float b = bv[c];
+        const float s = sv[c];
         float       mul;
         if (a.stddev)
         {
@@ -69,7 +107,21 @@ __device__ __forceinline__ void NormPixel(const NormArgs &a, const uint8_t *srcR
             mul = s;
         }
         const float v = ((float)in.v[c] - b) * mul * a.gscale + a.shift;
-        __builtin_nontemporal_store(SaturateCast<TO>(v), &o->v[c]);
+        out.v[c]      = SaturateCast<TO>(v);
+    }
+    if constexpr (sizeof(Vec<TO, C>) % 4 == 0)
+    {
+        uint32_t w[sizeof(Vec<TO, C>) / 4];
+        __builtin_memcpy(w, &out, sizeof(w));
+        StoreDwordsNT<sizeof(Vec<TO, C>) / 4>(reinterpret_cast<uint8_t *>(o), w);
+    }
+    else
+    {
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            __builtin_nontemporal_store(out.v[c], &o->v[c]);
+        }
     }
 }
 
