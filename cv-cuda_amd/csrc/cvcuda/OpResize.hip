@@ -12,8 +12,8 @@
 // Five kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
-//  * u8x3 bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows and fetches each source
-//    row once for both columns, lane pairs swap a pixel pair each;
+//  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows (4 x 2 when enlarging by 1.5 or
+//    more) and fetches each source row once for all its columns, lane pairs swap a pixel pair each;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
 //  * AREA of 8-bit pixels at reductions of up to 3: fixed-point row sums, a wave owns 64 columns x 16 rows and
 //    produces vertically adjacent rows in pairs from the source rows they share;
@@ -1627,7 +1627,15 @@ __device__ __forceinline__ void ResizeLinearQuadsU8(const Plane &p, int x0, int 
 // and 4 channels; with 1 and 4 it measured slower than the wave patches (u8x1 43 -> 58 us, u8x4 91 -> 104 us
 // on 1080p -> 720p: the column terms of two columns are amortised over 2 rows only), so 3 it is.
 template<class T, int C, int INTERP>
-constexpr bool kPairsForm = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_LINEAR && C == 3;
+constexpr bool kPairsForm = std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_LINEAR && (C == 1 || C == 3 || C == 4);
+
+// The scales at which the two-column form is the faster one (per image): horizontal scales up to 2; 4-byte pixels
+// only when not reducing (16 x 1080p -> 720p: 34.4 us against the wave patches' 29.9; 720p -> 900p: 37.9 against 42.0).
+template<int C>
+__host__ __device__ __forceinline__ bool PairsFormScale(int srcW, int dstW)
+{
+    return srcW >= 4 && srcW <= 2 * dstW && (C != 4 || srcW <= dstW);
+}
 
 constexpr int kPairsTileW = 128, kPairsTileH = 8; // block = 4 waves of 128 columns x 2 rows, stacked
 
@@ -1655,7 +1663,7 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8VarShapeKernel(const R
     const TileCoord tc   = LocateTile(tiles, blockIdx.x);
     const Plane     p    = GetPlanes<true>(a, tc.image);
     const int       wave = threadIdx.x >> 6;
-    if (p.srcW >= 4 && p.srcW <= 2 * p.dstW)
+    if (PairsFormScale<C>(p.srcW, p.dstW))
     {
         ResizeLinearPairsU8<C, true>(p, tc.tx * kPairsTileW, tc.ty * kPairsTileH + wave * 2);
     }
@@ -2177,7 +2185,7 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             CheckLaunch("ResizeLinearQuadsU8Kernel");
             return;
         }
-        if (a.srcW >= 4 && a.srcW <= 2 * a.dstW)
+        if (PairsFormScale<C>(a.srcW, a.dstW))
         {
             dim3 pgrid(DivUp(a.dstW, kPairsTileW), DivUp(a.dstH, kPairsTileH), N);
             hipLaunchKernelGGL((ResizeLinearPairsU8Kernel<C>), pgrid, dim3(256), 0, stream, a);
