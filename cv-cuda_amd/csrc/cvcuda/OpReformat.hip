@@ -122,7 +122,10 @@ __global__ __launch_bounds__(256) void ReformatRunsKernel(const ReformatArgs a)
     }
     if constexpr (DST_IL)
     {
-        StoreRunNT<T, kRunPixels * C>(d, px);
+        // a wave's lanes 0 .. lanes-1 hold consecutive pieces of the row (pieces of 24 or 32 bytes are regrouped
+        // into dense 16-byte stores there)
+        const int lane = threadIdx.x & 63, lanes = min(64, (a.W - (x0 - lane * kRunPixels)) / kRunPixels);
+        StoreRowRunNT<T, kRunPixels * C>(d - (int64_t)lane * kRunPixels * a.dW, px, lane, lanes);
     }
     else
     {

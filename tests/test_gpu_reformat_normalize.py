@@ -15,7 +15,8 @@ def rand(orc, shape, dt, seed):
 
 
 @pytest.mark.parametrize("dt", [np.uint8, np.int8, np.uint16, np.int16, np.int32, np.float32, np.float64])
-@pytest.mark.parametrize("shape", [(2, 37, 53, 3), (1, 224, 224, 3), (3, 16, 20, 4), (2, 9, 11, 1), (1, 8, 9, 6)])
+@pytest.mark.parametrize("shape", [(2, 37, 53, 3), (1, 224, 224, 3), (3, 16, 20, 4), (2, 9, 11, 1), (1, 8, 9, 6),
+                                   (1, 5, 531, 3), (2, 3, 300, 4)])
 def test_reformat_nhwc_nchw_roundtrip(cv, orc, gpu, dt, shape):
     n, h, w, c = shape
     if dt == np.float64:
