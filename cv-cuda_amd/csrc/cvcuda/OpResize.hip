@@ -1332,34 +1332,81 @@ __device__ __forceinline__ uint32_t WindowPixel(const TapWindow<C> &t, int k)
     }
 }
 
-// The 4 pixels of source row y that start at column xs (rows before the image's last one only: the load may read
-// past the row).
+// The 4 pixels that start at `at` (rows before the image's last one only: the load may read past the row), in two
+// steps so that a caller can request several windows before it touches the first.
+// u8x3: the aligned 16 bytes that hold the window's 12, funnel-shifted into place. The texture path takes a
+// 12-byte load that is not dword aligned apart into about three times as many cache accesses (counters:
+// 63 against 20 per wave-load), and these kernels wait for that unit: 1080p -> 720p 61.5 -> 59.9 us,
+// 720p -> 1080p 117 -> 101 us. Reads at most 3 bytes before and 4 after the window.
 template<int C>
-__device__ __forceinline__ TapWindow<C> LoadTapWindow(const Plane &p, int y, int xs)
+struct RawTapWindow
 {
-    // u8x3: the aligned 16 bytes that hold the window's 12, funnel-shifted into place. The texture path takes a
-    // 12-byte load that is not dword aligned apart into about three times as many cache accesses (counters:
-    // 63 against 20 per wave-load), and this kernel waits for that unit: 1080p -> 720p 61.5 -> 59.9 us,
-    // 720p -> 1080p 117 -> 101 us. Reads at most 3 bytes before and 4 after the window.
-    const uint8_t *at  = p.src + (int64_t)y * p.srcRow + xs * C;
-    const uint32_t mis = (uint32_t)reinterpret_cast<uintptr_t>(at) & 3u;
-    struct alignas(4) W4
-    {
-        uint32_t d[4];
-    };
-    TapWindow<C> t;
+    uint32_t d[C == 3 ? 4 : C];
+    uint32_t mis;
+};
+
+template<int C>
+__device__ __forceinline__ RawTapWindow<C> RequestTapWindow(const uint8_t *at)
+{
+    RawTapWindow<C> r;
     if constexpr (C == 3)
     {
-        const W4 w = *reinterpret_cast<const W4 *>(at - mis);
-        t.w[0]     = __builtin_amdgcn_alignbyte(w.d[1], w.d[0], mis);
-        t.w[1]     = __builtin_amdgcn_alignbyte(w.d[2], w.d[1], mis);
-        t.w[2]     = __builtin_amdgcn_alignbyte(w.d[3], w.d[2], mis);
+        struct alignas(4) W4
+        {
+            uint32_t d[4];
+        };
+        r.mis      = (uint32_t)reinterpret_cast<uintptr_t>(at) & 3u;
+        const W4 w = *reinterpret_cast<const W4 *>(at - r.mis);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            r.d[i] = w.d[i];
+        }
     }
     else
     {
-        t = *reinterpret_cast<const TapWindow<C> *>(at);
+        r.mis                = 0;
+        const TapWindow<C> t = *reinterpret_cast<const TapWindow<C> *>(at);
+#pragma unroll
+        for (int i = 0; i < C; ++i)
+        {
+            r.d[i] = t.w[i];
+        }
+    }
+    return r;
+}
+
+template<int C>
+__device__ __forceinline__ TapWindow<C> FinishTapWindow(const RawTapWindow<C> &r)
+{
+    TapWindow<C> t;
+    if constexpr (C == 3)
+    {
+        t.w[0] = __builtin_amdgcn_alignbyte(r.d[1], r.d[0], r.mis);
+        t.w[1] = __builtin_amdgcn_alignbyte(r.d[2], r.d[1], r.mis);
+        t.w[2] = __builtin_amdgcn_alignbyte(r.d[3], r.d[2], r.mis);
+    }
+    else
+    {
+#pragma unroll
+        for (int i = 0; i < C; ++i)
+        {
+            t.w[i] = r.d[i];
+        }
     }
     return t;
+}
+
+template<int C>
+__device__ __forceinline__ TapWindow<C> LoadTapWindowAt(const uint8_t *at)
+{
+    return FinishTapWindow<C>(RequestTapWindow<C>(at));
+}
+
+template<int C>
+__device__ __forceinline__ TapWindow<C> LoadTapWindow(const Plane &p, int y, int xs)
+{
+    return LoadTapWindowAt<C>(p.src + (int64_t)y * p.srcRow + xs * C);
 }
 
 // One pixel from its four taps (a dword each, channel c in byte c) and the float32 weights of the second taps.
@@ -1421,8 +1468,17 @@ __device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int 
     uint32_t  top[2][4], bot[2][4];
     if (max(yb0, yb1) < p.srcH - 1) // wave-uniform; the usual case: all four window loads go out together
     {
-        // the two output rows often share source rows (always when enlarging): those are fetched once
-        const TapWindow<C> w0 = window(ya0), w1 = window(yb0);
+        // All four windows are requested before anything else (a load behind one of the tests below would wait for
+        // the loads before it); the two output rows often share source rows (always when enlarging), whose taps
+        // are taken apart once.
+        auto request = [&](int y) { return RequestTapWindow<C>(p.src + (int64_t)y * p.srcRow + colA.s * C); };
+        const RawTapWindow<C> r0 = request(ya0), r1 = request(yb0), r2 = request(ya1), r3 = request(yb1);
+        // a use the compiler cannot move (without it the last two loads sink into the branches that need them) behind
+        // a line the instruction scheduler does not cross (or it starts on the first window between the loads)
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::"v"(r0.d[0]), "v"(r1.d[0]), "v"(r2.d[0]), "v"(r3.d[0]));
+        const TapWindow<C> w0 = FinishTapWindow<C>(r0), w1 = FinishTapWindow<C>(r1), w2 = FinishTapWindow<C>(r2),
+                           w3 = FinishTapWindow<C>(r3);
         unpack(w0, top[0]);
         unpack(w1, bot[0]);
         if (ya1 == ya0)
@@ -1434,19 +1490,20 @@ __device__ __forceinline__ void ResizeLinearPairsU8(const Plane &p, int x0, int 
                 bot[1][i] = bot[0][i];
             }
         }
-        else if (ya1 == yb0)
-        {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-            {
-                top[1][i] = bot[0][i];
-            }
-            unpack(window(yb1), bot[1]);
-        }
         else
         {
-            const TapWindow<C> w2 = window(ya1), w3 = window(yb1);
-            unpack(w2, top[1]);
+            if (ya1 == yb0)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    top[1][i] = bot[0][i];
+                }
+            }
+            else
+            {
+                unpack(w2, top[1]);
+            }
             unpack(w3, bot[1]);
         }
     }
@@ -1623,6 +1680,134 @@ __device__ __forceinline__ void ResizeLinearQuadsU8(const Plane &p, int x0, int 
     }
 }
 
+// The four-column form over a strip of kStripRows output rows per wave. When not reducing vertically those rows
+// lie between at most kStripRows + 1 consecutive source rows. All their windows are requested up front (rows past
+// the last one needed repeat it), a source row's tap pairs are formed once for every output row that uses it as
+// its upper or its lower row, and the column terms are paid once per 8 rows instead of once per 2. The blend per
+// output pixel is BilinearQ15 as everywhere. A wave that reaches the image's last source row, reduces vertically
+// (more source rows than fit) or has a lane whose columns do not fit its window runs as four two-row steps.
+constexpr int kStripRows = 8, kStripWindows = kStripRows + 1;
+
+template<int C>
+__device__ __forceinline__ void ResizeLinearQuadStripU8(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    const int    lane = threadIdx.x & 63;
+    const int    dx0  = x0 + 4 * lane;
+    AxisTerms<1> col[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        col[j] = Axis<NVCV_INTERP_LINEAR>(p.scaleX, min(dx0 + j, p.dstW - 1), p.srcW);
+    }
+    // lane r holds the terms of output row y0 + r
+    const auto     rows   = Axis<NVCV_INTERP_LINEAR>(p.scaleY, min(y0 + (lane & (kStripRows - 1)), p.dstH - 1), p.srcH);
+    const uint32_t ayLane = FractionQ15(rows.w[0]);
+    const int      yFirst = __builtin_amdgcn_readlane(rows.s, 0), yLast = __builtin_amdgcn_readlane(rows.s, kStripRows - 1) + 1;
+    const bool     narrow = col[3].s - col[0].s <= 2;
+    if (yLast >= p.srcH - 1 || yLast - yFirst >= kStripWindows || __builtin_amdgcn_ballot_w64(!narrow) != 0) // wave-uniform
+    {
+#pragma unroll 1
+        for (int k = 0; k < kStripRows; k += 2)
+        {
+            ResizeLinearQuadsU8<C>(p, x0, y0 + k);
+        }
+        return;
+    }
+    TapWindow<C>   win[kStripWindows];
+    const uint8_t *at = p.src + (int64_t)yFirst * p.srcRow + col[0].s * C;
+#pragma unroll
+    for (int k = 0; k < kStripWindows; ++k)
+    {
+        win[k] = LoadTapWindowAt<C>(at + (int64_t)min(k, yLast - yFirst) * p.srcRow);
+    }
+    // lanes past the last column stay (the row terms are read from lanes 0 .. 7 below); they store nothing
+    uint32_t ax[4];
+    int      d[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        ax[j] = FractionQ15(col[j].w[0]);
+        d[j]  = col[j].s - col[0].s;
+    }
+    // (first tap | second tap << 16) of every column and channel of a source row
+    auto pairs = [&](const TapWindow<C> &w, uint32_t (&t)[4][C])
+    {
+        const uint32_t k0 = WindowPixel<C>(w, 0), k1 = WindowPixel<C>(w, 1), k2 = WindowPixel<C>(w, 2), k3 = WindowPixel<C>(w, 3);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const uint32_t first  = j == 0 ? k0 : (d[j] == 0 ? k0 : (d[j] == 1 ? k1 : k2));
+            const uint32_t second = j == 0 ? k1 : (d[j] == 0 ? k1 : (d[j] == 1 ? k2 : k3));
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                t[j][c] = ChannelPair(first, second, c);
+            }
+        }
+    };
+    const int nRows = min(kStripRows, p.dstH - y0);
+    int       r     = 0;
+    uint8_t  *to    = p.dst + (int64_t)y0 * p.dstRow + (int64_t)dx0 * C;
+    uint32_t  top[4][C], bot[4][C];
+    pairs(win[0], bot);
+#pragma unroll
+    for (int k = 0; k + 1 < kStripWindows; ++k)
+    {
+        if (r < nRows) // wave-uniform
+        {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    top[j][c] = bot[j][c];
+                }
+            }
+            pairs(win[k + 1], bot);
+            // the output rows between source rows yFirst + k and the next one
+            while (r < nRows && __builtin_amdgcn_readlane(rows.s, r) == yFirst + k)
+            {
+                const uint32_t ay = __builtin_amdgcn_readlane(ayLane, r);
+                uint32_t       w[C] = {}; // the row's 4 pixels as stored: every channel is rounded into its byte
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uint32_t wt, wb;
+                    WeightPairsQ15(ax[j], ay, wt, wb);
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                    {
+                        const int at     = j * C + c;
+                        w[at >> 2] = BlendQ15(top[j][c], bot[j][c], wt, wb, at & 3, w[at >> 2]);
+                    }
+                }
+                if (dx0 + 4 <= p.dstW)
+                {
+                    StoreDwordsNT<C>(to, w);
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < 3 * C; ++i)
+                    {
+                        if (dx0 + i / C < p.dstW)
+                        {
+                            to[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+                        }
+                    }
+                }
+                to += p.dstRow;
+                ++r;
+            }
+        }
+    }
+}
+
 // Which (type, channels, interpolation) take the two-columns-per-lane form. The code is written for 1, 3
 // and 4 channels; with 1 and 4 it measured slower than the wave patches (u8x1 43 -> 58 us, u8x4 91 -> 104 us
 // on 1080p -> 720p: the column terms of two columns are amortised over 2 rows only), so 3 it is.
@@ -1646,13 +1831,13 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArg
     ResizeLinearPairsU8<C, false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
 }
 
-constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x 2 rows, stacked
+constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x kStripRows rows, stacked
 
 template<int C>
 __global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeLinearQuadsU8<C>(p, blockIdx.x * kQuadsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+    ResizeLinearQuadStripU8<C>(p, blockIdx.x * kQuadsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * kStripRows);
 }
 
 // Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
@@ -2180,7 +2365,7 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     {
         if (a.srcW >= 4 && 3 * (int64_t)a.srcW <= 2 * (int64_t)a.dstW)
         {
-            dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, kPairsTileH), N);
+            dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, 4 * kStripRows), N);
             hipLaunchKernelGGL((ResizeLinearQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
             CheckLaunch("ResizeLinearQuadsU8Kernel");
             return;
