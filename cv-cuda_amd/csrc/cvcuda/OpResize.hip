@@ -9,11 +9,13 @@
 // point on those indices and weights (bilinear: FixedPointBlend.hpp; bicubic: kFixedCubic; box filter:
 // kAreaFixed), at most 1 from the reference's goldens.
 //
-// Five kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
+// Six kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
-//  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows (4 x 2 when enlarging by 1.5 or
+//  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows (4 x 8 when enlarging by 1.5 or
 //    more) and fetches each source row once for all its columns, lane pairs swap a pixel pair each;
+//  * 8-bit bicubic tensors at vertical scales up to 2, large launches: a wave owns 64 columns x 16 rows and forms
+//    every source row's sums once, adding them to the output rows in flight;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
 //  * AREA of 8-bit pixels at reductions of up to 3: fixed-point row sums, a wave owns 64 columns x 16 rows and
 //    produces vertically adjacent rows in pairs from the source rows they share;
@@ -898,6 +900,11 @@ __device__ __forceinline__ AxisTerms<W> FromLane(const AxisTerms<W> &a, int from
     return r;
 }
 
+__device__ __forceinline__ float ReadLane(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
 // The 8-bit bicubic sum of one output pixel per lane: rows y0 .. y0 + 3 (clamped into the image), their windows of 4
 // pixels at `at` + `shift`, the packed horizontal weights and the vertical ones times 2^-14 (wave-uniform). All four
 // windows are requested before the first sum.
@@ -1295,6 +1302,197 @@ __device__ __forceinline__ void ResizeWavePatch(const Plane &p, int x0, int y0)
         }
     }
     StoreWavePatch<T, C>(p, x0, y0, lane, q);
+}
+
+// ---- the 8-bit bicubic form over strips of 16 output rows per wave
+
+constexpr int kCubicStripRows = 16;
+
+// A row window as LoadQuadWindow reads it, in two steps: a strip requests the rows of its next output row before it
+// works on the current one.
+template<int C>
+struct RawQuadWindow
+{
+    uint32_t d[C == 4 ? 4 : C + 1];
+};
+
+// (row: wave-uniform; at: the lane's byte offset in it - the load then takes the row as its scalar base and the
+// lane needs no address arithmetic)
+template<int C>
+__device__ __forceinline__ RawQuadWindow<C> RequestQuadWindow(const uint8_t *row, uint32_t at)
+{
+    struct __attribute__((packed, aligned(1))) Window
+    {
+        uint32_t d[C == 4 ? 4 : C + 1];
+    };
+    const Window     w = *reinterpret_cast<const Window *>(row + at);
+    RawQuadWindow<C> r;
+    __builtin_memcpy(&r, &w, sizeof(r));
+    return r;
+}
+
+// The row's sums of 4 taps times the horizontal weights (units of 2^-14), as CubicRowsQ14 forms them.
+template<int C>
+__device__ __forceinline__ void CubicRowSumsQ14(const RawQuadWindow<C> &w, uint32_t shift, uint32_t w01, uint32_t w23,
+                                                float (&h)[C])
+{
+    uint32_t r[C];
+#pragma unroll
+    for (int i = 0; i < C; ++i)
+    {
+        if constexpr (C == 4)
+        {
+            r[i] = w.d[i];
+        }
+        else
+        {
+            r[i] = __builtin_amdgcn_alignbyte(w.d[i + 1], w.d[i], shift);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+    {
+        h[c] = (float)Dot2I16(QuadTapPair<C>(r, 2, c), w23, Dot2I16(QuadTapPair<C>(r, 0, c), w01));
+    }
+}
+
+// One wave resizes 64 columns x 16 rows whose top left pixel is (x0, y0), both wave-uniform; lane l owns column
+// x0 + l. The windows of consecutive output rows overlap (at scale 1.5 they advance by 1 or 2 source rows), so the
+// strip walks down the source rows once: a row's sums are formed once and added, times the row's weight in each,
+// to the output pixels whose windows hold it - the current output row and the three after it, which is all of them
+// while windows advance by at least one row. The four running pixels live in fixed registers (output row r in slot
+// r mod 4, four steps unrolled); a row outside a pixel's window is added with weight 0, which changes nothing, so
+// the instruction stream does not depend on the scale. An output row is finished when the last row of its window
+// has been added, its slot then starts the pixel four rows down. Every pixel adds its four row sums in ascending
+// order (the first to a zero, which gives the product), as CubicRowsQ14 does: the same result bit for bit. Per
+// output pixel 1.5 row sums at scale 1.5 where the patch form takes 2.75, and the column terms once per 16 rows.
+// The one or two rows a step adds are requested a step ahead, both always (no test in front of a load).
+// A strip takes this form when its windows advance by 1 or 2 rows from each output row to the next and stay clear
+// of the image's last row; others (the image's top and bottom, other scales) go one output row at a time with
+// guarded loads. The launch requires sources wide enough for the window loads (16 bytes a row, 8 for one channel).
+template<int C>
+__device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    constexpr int R    = kCubicStripRows;
+    const int     lane = threadIdx.x & 63;
+    const int     dx   = min(x0 + lane, p.dstW - 1); // columns past the output compute a duplicate of the last one
+    const auto    col  = FinishedAxis<NVCV_INTERP_CUBIC>(p.scaleX, dx, p.srcW, true);
+    // lane 4 r + t holds the second tap's row of output row y0 + r and its weight for tap t, in units of 2^-14
+    // (the row sums' unit)
+    const auto  rows  = FinishedAxis<NVCV_INTERP_CUBIC>(p.scaleY, min(y0 + (lane >> 2), p.dstH - 1), p.srcH, false);
+    const int   t     = lane & 3;
+    const float wLane = (t == 0 ? rows.w[0] : t == 1 ? rows.w[1] : t == 2 ? rows.w[2] : rows.w[3]) * (1.f / 16384.f);
+    const int   apartLane = __shfl_down(rows.s, 4) - rows.s;
+    const bool  regular   = lane >= 4 * (R - 1) || (apartLane >= 1 && apartLane <= 2);
+    const CubicColumnQ14 cq = CubicColumn<C>(col);
+    auto second = [&](int r) { return __builtin_amdgcn_readlane(rows.s, 4 * min(r, R - 1)); }; // the row of output row r's second tap
+    if (y0 + R > p.dstH || __builtin_amdgcn_ballot_w64(!regular) != 0 || second(R - 1) + 2 >= p.srcH - 1) // wave-uniform
+    {
+        // one output row at a time, every window load guarded against the image's last row
+#pragma unroll 1
+        for (int g = 0; g < R && y0 + g < p.dstH; g += 4)
+        {
+            uint32_t q[1][4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                const int   r     = g + k;
+                const float wy[4] = {ReadLane(wLane, 4 * r), ReadLane(wLane, 4 * r + 1), ReadLane(wLane, 4 * r + 2),
+                                     ReadLane(wLane, 4 * r + 3)};
+                q[0][k] = CubicRowsQ14<C, true>(p, second(r) - 1, cq.at, cq.shift, (uint32_t)p.srcW * C, cq.w01, cq.w23, wy);
+            }
+            StoreWavePatch<uint8_t, C>(p, x0, y0 + g, lane, q);
+        }
+        return;
+    }
+    auto request = [&](int row) { return RequestQuadWindow<C>(p.src + (int64_t)row * p.srcRow, cq.at); };
+
+    float acc[4][C] = {};
+    // The weight of source row j in output row r, whose second tap is row sr: tap j - (sr - 1) where that is 0 .. 3,
+    // else 0. Output rows past the strip (r >= 16, terms of row 15) collect sums that are never stored. The lane is
+    // read either way (no branch; the instruction takes the lane number modulo 64) and the choice is written as scalar
+    // instructions, which the compiler otherwise turns into a move and a select on the vector unit per weight.
+    // always: the tap is known to be one of the four (windows advance by 1 or 2 rows), nothing to choose.
+    auto weight = [&](int j, int sr, int r, bool always)
+    {
+        const int tap = j - sr + 1;
+        const int w   = __builtin_amdgcn_readlane(__float_as_int(wLane), 4 * r + tap);
+        if (always)
+        {
+            return __int_as_float(w);
+        }
+        int chosen;
+        asm("s_cmp_lt_u32 %1, 4\n\ts_cselect_b32 %0, %2, 0" : "=s"(chosen) : "s"(tap), "s"(w) : "scc");
+        return __int_as_float(chosen);
+    };
+    // Source row j, whose window is w, into the output rows r .. r + outputs - 1 (slots K .. ; K is a constant once
+    // unrolled), whose second taps are rows sr[0 .. 3]; the first `sure` of them hold the row for certain.
+    auto add = [&](int K, const RawQuadWindow<C> &w, int j, int r, const int (&sr)[4], int outputs, int sure)
+    {
+        float h[C];
+        CubicRowSumsQ14<C>(w, cq.shift, cq.w01, cq.w23, h);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            if (i >= outputs)
+            {
+                break;
+            }
+            const float wi = weight(j, sr[i], r + i, i < sure);
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                acc[(K + i) & 3][c] = fmaf(h[c], wi, acc[(K + i) & 3][c]);
+            }
+        }
+    };
+    int sr[4] = {second(0), second(1), second(2), second(3)};
+    // output row 0's window but for its last row
+    {
+        const RawQuadWindow<C> w0 = request(sr[0] - 1), w1 = request(sr[0]), w2 = request(sr[0] + 1);
+        add(0, w0, sr[0] - 1, 0, sr, 4, 1);
+        add(0, w1, sr[0], 0, sr, 4, 1);
+        add(0, w2, sr[0] + 1, 0, sr, 4, 1);
+    }
+    // the step to output row r adds rows sr + 1 (if the window advanced by 2) and sr + 2; they are requested two
+    // steps ahead (even steps use one pair of registers, odd steps the other)
+    RawQuadWindow<C> ahead[2][2] = {{request(sr[0] + 1), request(sr[0] + 2)}, {request(sr[1] + 1), request(sr[1] + 2)}};
+    int              apart       = 1; // row sr[0] + 1 is in already
+#pragma unroll 1
+    for (int g = 0; g < R; g += 4)
+    {
+        uint32_t q[1][4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+        {
+            const int              r  = g + k;
+            const RawQuadWindow<C> c0 = ahead[k & 1][0], c1 = ahead[k & 1][1];
+            ahead[k & 1][0] = request(sr[2] + 1);
+            ahead[k & 1][1] = request(sr[2] + 2);
+            if (apart == 2)
+            {
+                add(k, c0, sr[0] + 1, r, sr, 3, 2); // the row above the window's last is in none of output row r + 3's
+            }
+            add(k, c1, sr[0] + 2, r, sr, 4, 2);
+            apart = sr[1] - sr[0];
+            sr[0] = sr[1];
+            sr[1] = sr[2];
+            sr[2] = sr[3];
+            sr[3] = second(r + 4);
+            q[0][k] = 0;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+            {
+                q[0][k]   = __builtin_amdgcn_cvt_pk_u8_f32(fabsf(acc[k][c]), c, q[0][k]);
+                acc[k][c] = 0.f;
+            }
+        }
+        StoreWavePatch<uint8_t, C>(p, x0, y0 + g, lane, q);
+    }
 }
 
 // 8-bit bilinear at horizontal scales up to 2. The cost of the wave-patch form there is the number
@@ -1869,6 +2067,14 @@ __global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs 
     ResizeWavePatch<T, C, INTERP, false>(p, blockIdx.x * kPatchTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 4);
 }
 
+// 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows).
+template<int C>
+__global__ __launch_bounds__(256) void ResizeCubicStripU8Kernel(const ResizeArgs a)
+{
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizeCubicStripU8<C>(p, blockIdx.x * kPatchTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kCubicStripRows);
+}
+
 template<class T, int C, int INTERP>
 __global__ __launch_bounds__(256) void ResizePatchVarShapeKernel(const ResizeArgs a, const VarTiles tiles)
 {
@@ -2059,11 +2265,6 @@ __device__ __forceinline__ void AreaFixedRows(int n, const uint8_t *row, int src
     {
         AreaFixedRowsOf<C, K, false>(n, row, srcRow, lastRowIn, at, shift, rowBytes, w01, w23, wy, start, out);
     }
-}
-
-__device__ __forceinline__ float ReadLane(float v, int lane)
-{
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
 // The tile of 64 columns x 16 rows whose top left pixel is (x0, y0), both wave-uniform (y0 even).
@@ -2385,6 +2586,19 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             dim3 agrid(DivUp(a.dstW, kAreaTileW), DivUp(a.dstH, kAreaTileH), N);
             hipLaunchKernelGGL((ResizeAreaFixedTensorKernel<C>), agrid, dim3(256), 0, stream, a);
             CheckLaunch("ResizeAreaFixedTensorKernel");
+            return;
+        }
+    }
+    if constexpr (INTERP == NVCV_INTERP_CUBIC && std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4))
+    {
+        // strips of 16 rows per wave where consecutive windows overlap (vertical scales up to 2) and the launch
+        // still has 8 waves and more per CU
+        const int64_t strips = (int64_t)DivUp(a.dstW, kPatchTileW) * DivUp(a.dstH, kCubicStripRows) * N;
+        if (a.srcH <= 2 * (int64_t)a.dstH && strips >= 8 * 256 && a.srcW >= 4 && a.srcW * C >= (C == 1 ? 8 : 16))
+        {
+            dim3 sgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, 4 * kCubicStripRows), N);
+            hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C>), sgrid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeCubicStripU8Kernel");
             return;
         }
     }
