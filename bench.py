@@ -698,7 +698,7 @@ class Streaming:
         "resize-linear-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
                                   "ResizeLinearQuadsU8Kernel<3>", "i32", "Resize LINEAR 1280x720 -> 1920x1080"),
         "resize-cubic-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
-                              "ResizeCubicStripU8Kernel<3>", "i32", "Resize CUBIC 1920x1080 -> 1280x720"),
+                              "ResizeCubicStripU8Kernel<3,4>", "i32", "Resize CUBIC 1920x1080 -> 1280x720"),
         "resize-area-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
                              "ResizeAreaFixedTensorKernel<3>", "i32", "Resize AREA 1920x1080 -> 1280x720"),
         "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t,false>>", "f32",

@@ -14,8 +14,8 @@
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
 //  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows (4 x 8 when enlarging by 1.5 or
 //    more) and fetches each source row once for all its columns, lane pairs swap a pixel pair each;
-//  * 8-bit bicubic tensors at vertical scales up to 2, large launches: a wave owns 64 columns x 16 rows and forms
-//    every source row's sums once, adding them to the output rows in flight;
+//  * 8-bit bicubic tensors of 3 and 4 channels at vertical scales of 1/2 to 2, large launches: a wave owns 64 columns
+//    x 16 rows and forms every source row's sums once, adding them to the output rows in flight;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
 //  * AREA of 8-bit pixels at reductions of up to 3: fixed-point row sums, a wave owns 64 columns x 16 rows and
 //    produces vertically adjacent rows in pairs from the source rows they share;
@@ -1357,22 +1357,27 @@ __device__ __forceinline__ void CubicRowSumsQ14(const RawQuadWindow<C> &w, uint3
 }
 
 // One wave resizes 64 columns x 16 rows whose top left pixel is (x0, y0), both wave-uniform; lane l owns column
-// x0 + l. The windows of consecutive output rows overlap (at scale 1.5 they advance by 1 or 2 source rows), so the
-// strip walks down the source rows once: a row's sums are formed once and added, times the row's weight in each,
-// to the output pixels whose windows hold it - the current output row and the three after it, which is all of them
-// while windows advance by at least one row. The four running pixels live in fixed registers (output row r in slot
-// r mod 4, four steps unrolled); a row outside a pixel's window is added with weight 0, which changes nothing, so
-// the instruction stream does not depend on the scale. An output row is finished when the last row of its window
-// has been added, its slot then starts the pixel four rows down. Every pixel adds its four row sums in ascending
-// order (the first to a zero, which gives the product), as CubicRowsQ14 does: the same result bit for bit. Per
-// output pixel 1.5 row sums at scale 1.5 where the patch form takes 2.75, and the column terms once per 16 rows.
-// The one or two rows a step adds are requested a step ahead, both always (no test in front of a load).
-// A strip takes this form when its windows advance by 1 or 2 rows from each output row to the next and stay clear
-// of the image's last row; others (the image's top and bottom, other scales) go one output row at a time with
-// guarded loads. The launch requires sources wide enough for the window loads (16 bytes a row, 8 for one channel).
-template<int C>
+// x0 + l. The windows of consecutive output rows overlap (reducing by 1.5 they advance by 1 or 2 source rows,
+// enlarging by 0 or 1), so the strip walks down the source rows once: a row's sums are formed once and added, times
+// the row's weight in each, to the output pixels whose windows can hold it - the current output row and the S - 1
+// after it. S = 4 when reducing (all of them while windows advance by at least one row), S = 8 when enlarging (all
+// of them while the window 8 rows down starts 4 or more source rows later: enlargements up to 2). The S running
+// pixels live in fixed registers (output row r in slot r mod S, S steps unrolled); a row outside a pixel's window
+// is added with weight 0, which changes nothing, so the instruction stream does not depend on the scale. An output
+// row is finished when the last row of its window has been added, its slot then starts the pixel S rows down.
+// Every pixel adds its four row sums in ascending order (the first to a zero, which gives the product), as
+// CubicRowsQ14 does: the same result bit for bit. Per output pixel 1.5 row sums when reducing by 1.5 where the patch
+// form takes 2.75, 0.67 when enlarging by 1.5 where it takes 2.25, and the column terms once per 16 rows.
+// The rows a step can add (reducing: two, enlarging: one) are requested two steps ahead, needed or not (no test in
+// front of a load).
+// A strip takes this form when its windows advance as said from each output row to the next and stay clear of the
+// image's last row; others (the image's top and bottom, other scales) go one output row at a time with guarded
+// loads. The launch requires sources wide enough for the window loads (16 bytes a row, 8 for one channel).
+template<int C, int S>
 __device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y0)
 {
+    static_assert(S == 4 || S == 8);
+    constexpr bool kReducing = S == 4;
     if (x0 >= p.dstW || y0 >= p.dstH)
     {
         return;
@@ -1387,7 +1392,13 @@ __device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y
     const int   t     = lane & 3;
     const float wLane = (t == 0 ? rows.w[0] : t == 1 ? rows.w[1] : t == 2 ? rows.w[2] : rows.w[3]) * (1.f / 16384.f);
     const int   apartLane = __shfl_down(rows.s, 4) - rows.s;
-    const bool  regular   = lane >= 4 * (R - 1) || (apartLane >= 1 && apartLane <= 2);
+    bool        regular   = lane >= 4 * (R - 1) || (apartLane >= (kReducing ? 1 : 0) && apartLane <= (kReducing ? 2 : 1));
+    if constexpr (!kReducing)
+    {
+        // (every lane takes part in the exchange: a lane that has left reads as 0)
+        const int farLane = __shfl_down(rows.s, 4 * S) - rows.s;
+        regular           = regular & ((lane >= 4 * (R - S)) | (farLane >= 4));
+    }
     const CubicColumnQ14 cq = CubicColumn<C>(col);
     auto second = [&](int r) { return __builtin_amdgcn_readlane(rows.s, 4 * min(r, R - 1)); }; // the row of output row r's second tap
     if (y0 + R > p.dstH || __builtin_amdgcn_ballot_w64(!regular) != 0 || second(R - 1) + 2 >= p.srcH - 1) // wave-uniform
@@ -1411,12 +1422,12 @@ __device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y
     }
     auto request = [&](int row) { return RequestQuadWindow<C>(p.src + (int64_t)row * p.srcRow, cq.at); };
 
-    float acc[4][C] = {};
+    float acc[S][C] = {};
     // The weight of source row j in output row r, whose second tap is row sr: tap j - (sr - 1) where that is 0 .. 3,
     // else 0. Output rows past the strip (r >= 16, terms of row 15) collect sums that are never stored. The lane is
     // read either way (no branch; the instruction takes the lane number modulo 64) and the choice is written as scalar
     // instructions, which the compiler otherwise turns into a move and a select on the vector unit per weight.
-    // always: the tap is known to be one of the four (windows advance by 1 or 2 rows), nothing to choose.
+    // always: the tap is known to be one of the four, nothing to choose.
     auto weight = [&](int j, int sr, int r, bool always)
     {
         const int tap = j - sr + 1;
@@ -1430,13 +1441,13 @@ __device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y
         return __int_as_float(chosen);
     };
     // Source row j, whose window is w, into the output rows r .. r + outputs - 1 (slots K .. ; K is a constant once
-    // unrolled), whose second taps are rows sr[0 .. 3]; the first `sure` of them hold the row for certain.
-    auto add = [&](int K, const RawQuadWindow<C> &w, int j, int r, const int (&sr)[4], int outputs, int sure)
+    // unrolled), whose second taps are rows sr[0 ..]; the first `sure` of them hold the row for certain.
+    auto add = [&](int K, const RawQuadWindow<C> &w, int j, int r, const int (&sr)[S], int outputs, int sure)
     {
         float h[C];
         CubicRowSumsQ14<C>(w, cq.shift, cq.w01, cq.w23, h);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < S; ++i)
         {
             if (i >= outputs)
             {
@@ -1446,52 +1457,86 @@ __device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
-                acc[(K + i) & 3][c] = fmaf(h[c], wi, acc[(K + i) & 3][c]);
+                acc[(K + i) & (S - 1)][c] = fmaf(h[c], wi, acc[(K + i) & (S - 1)][c]);
             }
         }
     };
-    int sr[4] = {second(0), second(1), second(2), second(3)};
+    int sr[S];
+#pragma unroll
+    for (int i = 0; i < S; ++i)
+    {
+        sr[i] = second(i);
+    }
     // output row 0's window but for its last row
     {
         const RawQuadWindow<C> w0 = request(sr[0] - 1), w1 = request(sr[0]), w2 = request(sr[0] + 1);
-        add(0, w0, sr[0] - 1, 0, sr, 4, 1);
-        add(0, w1, sr[0], 0, sr, 4, 1);
-        add(0, w2, sr[0] + 1, 0, sr, 4, 1);
+        add(0, w0, sr[0] - 1, 0, sr, S, 1);
+        add(0, w1, sr[0], 0, sr, S, 1);
+        add(0, w2, sr[0] + 1, 0, sr, S, 1);
     }
-    // the step to output row r adds rows sr + 1 (if the window advanced by 2) and sr + 2; they are requested two
-    // steps ahead (even steps use one pair of registers, odd steps the other)
-    RawQuadWindow<C> ahead[2][2] = {{request(sr[0] + 1), request(sr[0] + 2)}, {request(sr[1] + 1), request(sr[1] + 2)}};
-    int              apart       = 1; // row sr[0] + 1 is in already
+    // The step to output row r adds row sr + 2 if the window advanced, and before it row sr + 1 if it advanced by 2.
+    // They are requested two steps ahead (even steps use one set of registers, odd steps the other).
+    constexpr int    M = kReducing ? 2 : 1;
+    RawQuadWindow<C> ahead[2][M];
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+    {
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+        {
+            ahead[e][m] = request(sr[e] + 2 - (M - 1 - m));
+        }
+    }
+    int apart = 1; // the rows before sr[0] + 2 are in already
 #pragma unroll 1
-    for (int g = 0; g < R; g += 4)
+    for (int g = 0; g < R; g += S)
     {
         uint32_t q[1][4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
+        for (int k = 0; k < S; ++k)
         {
-            const int              r  = g + k;
-            const RawQuadWindow<C> c0 = ahead[k & 1][0], c1 = ahead[k & 1][1];
-            ahead[k & 1][0] = request(sr[2] + 1);
-            ahead[k & 1][1] = request(sr[2] + 2);
-            if (apart == 2)
+            const int        r = g + k;
+            RawQuadWindow<C> now[M];
+#pragma unroll
+            for (int m = 0; m < M; ++m)
             {
-                add(k, c0, sr[0] + 1, r, sr, 3, 2); // the row above the window's last is in none of output row r + 3's
+                now[m]           = ahead[k & 1][m];
+                ahead[k & 1][m] = request(sr[2] + 2 - (M - 1 - m));
             }
-            add(k, c1, sr[0] + 2, r, sr, 4, 2);
+            if constexpr (kReducing)
+            {
+                if (apart == 2)
+                {
+                    add(k, now[0], sr[0] + 1, r, sr, 3, 2); // the row above the window's last is in none of output row r + 3's
+                }
+                add(k, now[1], sr[0] + 2, r, sr, 4, 2);
+            }
+            else
+            {
+                if (apart == 1)
+                {
+                    add(k, now[0], sr[0] + 2, r, sr, S, 1);
+                }
+            }
             apart = sr[1] - sr[0];
-            sr[0] = sr[1];
-            sr[1] = sr[2];
-            sr[2] = sr[3];
-            sr[3] = second(r + 4);
-            q[0][k] = 0;
+#pragma unroll
+            for (int i = 0; i + 1 < S; ++i)
+            {
+                sr[i] = sr[i + 1];
+            }
+            sr[S - 1] = second(r + S);
+            q[0][k & 3] = 0;
 #pragma unroll
             for (int c = 0; c < C; ++c)
             {
-                q[0][k]   = __builtin_amdgcn_cvt_pk_u8_f32(fabsf(acc[k][c]), c, q[0][k]);
-                acc[k][c] = 0.f;
+                q[0][k & 3] = __builtin_amdgcn_cvt_pk_u8_f32(fabsf(acc[k][c]), c, q[0][k & 3]);
+                acc[k][c]   = 0.f;
+            }
+            if ((k & 3) == 3)
+            {
+                StoreWavePatch<uint8_t, C>(p, x0, y0 + r - 3, lane, q);
             }
         }
-        StoreWavePatch<uint8_t, C>(p, x0, y0 + g, lane, q);
     }
 }
 
@@ -2029,13 +2074,26 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArg
     ResizeLinearPairsU8<C, false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
 }
 
-constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x kStripRows rows, stacked
+constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x kQuadsRows rows, stacked
+
+// Rows per wave of the four-column form: strips for 1 and 3 channels; 4-byte pixels stay with two rows (their strip
+// holds 9 windows of 4 dwords and 32 tap pairs per source row: 16 x 720p -> 1080p 59.5 us against 43.7 us).
+template<int C>
+constexpr int kQuadsRows = C == 4 ? 2 : kStripRows;
 
 template<int C>
 __global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeLinearQuadStripU8<C>(p, blockIdx.x * kQuadsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * kStripRows);
+    const int y0 = (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * kQuadsRows<C>;
+    if constexpr (kQuadsRows<C> == kStripRows)
+    {
+        ResizeLinearQuadStripU8<C>(p, blockIdx.x * kQuadsTileW, y0);
+    }
+    else
+    {
+        ResizeLinearQuadsU8<C>(p, blockIdx.x * kQuadsTileW, y0);
+    }
 }
 
 // Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
@@ -2068,11 +2126,11 @@ __global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs 
 }
 
 // 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows).
-template<int C>
+template<int C, int S>
 __global__ __launch_bounds__(256) void ResizeCubicStripU8Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeCubicStripU8<C>(p, blockIdx.x * kPatchTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kCubicStripRows);
+    ResizeCubicStripU8<C, S>(p, blockIdx.x * kPatchTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kCubicStripRows);
 }
 
 template<class T, int C, int INTERP>
@@ -2566,7 +2624,7 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     {
         if (a.srcW >= 4 && 3 * (int64_t)a.srcW <= 2 * (int64_t)a.dstW)
         {
-            dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, 4 * kStripRows), N);
+            dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, 4 * kQuadsRows<C>), N);
             hipLaunchKernelGGL((ResizeLinearQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
             CheckLaunch("ResizeLinearQuadsU8Kernel");
             return;
@@ -2589,17 +2647,27 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             return;
         }
     }
-    if constexpr (INTERP == NVCV_INTERP_CUBIC && std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4))
+    if constexpr (INTERP == NVCV_INTERP_CUBIC && std::is_same_v<T, uint8_t> && (C == 3 || C == 4))
     {
-        // strips of 16 rows per wave where consecutive windows overlap (vertical scales up to 2) and the launch
-        // still has 8 waves and more per CU
+        // strips of 16 rows per wave where consecutive windows overlap (vertical scales of 1/2 to 2) and the launch
+        // still has 8 waves and more per CU; one channel is as fast or faster as wave patches (16 x 720p -> 1080p
+        // 46.6 us against 50.9 as strips, 1080p -> 720p 27.2 against 28.1)
         const int64_t strips = (int64_t)DivUp(a.dstW, kPatchTileW) * DivUp(a.dstH, kCubicStripRows) * N;
-        if (a.srcH <= 2 * (int64_t)a.dstH && strips >= 8 * 256 && a.srcW >= 4 && a.srcW * C >= (C == 1 ? 8 : 16))
+        if (strips >= 8 * 256 && a.srcW >= 4 && a.srcW * C >= (C == 1 ? 8 : 16))
         {
             dim3 sgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, 4 * kCubicStripRows), N);
-            hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C>), sgrid, dim3(256), 0, stream, a);
-            CheckLaunch("ResizeCubicStripU8Kernel");
-            return;
+            if (a.srcH >= a.dstH && a.srcH <= 2 * (int64_t)a.dstH)
+            {
+                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 4>), sgrid, dim3(256), 0, stream, a);
+                CheckLaunch("ResizeCubicStripU8Kernel");
+                return;
+            }
+            if (a.srcH < a.dstH && 2 * (int64_t)a.srcH >= a.dstH)
+            {
+                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 8>), sgrid, dim3(256), 0, stream, a);
+                CheckLaunch("ResizeCubicStripU8Kernel");
+                return;
+            }
         }
     }
     if constexpr (kPatchForm<T, C, INTERP>)

@@ -83,13 +83,17 @@ def test_tensor_cubic_reduction(cv, orc, gpu, row):
     test_tensor_table(cv, orc, gpu, row)
 
 
-# 8-bit bicubic at vertical scales up to 2 runs as strips of 16 rows per wave once the launch has 2048 strips: the
+# 8-bit bicubic at vertical scales of 1/2 to 2 runs as strips of 16 rows per wave once the launch has 2048 strips: the
 # benchmark's shape, ragged widths and heights, scale 2 exactly (every window advances by 2), 1.25, an enlargement
-# (windows that do not advance: every strip takes the row-by-row path), horizontal enlargement with vertical reduction
+# beyond 2 vertically (every strip takes the row-by-row path), horizontal enlargement with vertical reduction
 STRIPS = [(sw, sh, dw, dh, CUBIC, n, np.uint8, c)
-          for c in (3, 1, 4)
+          for c in (3, 4, 1)  # (one channel stays with wave patches at these sizes too)
           for (sw, sh, dw, dh, n) in [(1920, 1080, 1280, 720, 3), (1917, 1083, 1283, 719, 3), (1024, 1408, 512, 704, 8),
-                                      (1600, 900, 1280, 720, 3), (640, 360, 1000, 1100, 2), (300, 1080, 700, 720, 6)]]
+                                      (1600, 900, 1280, 720, 3), (640, 360, 1000, 1100, 2), (300, 1080, 700, 720, 6),
+                                      # enlargements: by 1.5, by 2 exactly (the limit of the enlarging strips), by 1.2 with
+                                      # ragged sizes, and equal heights (every window advances by 1)
+                                      (1280, 720, 1920, 1080, 2), (640, 360, 1280, 720, 3), (1003, 601, 1201, 721, 3),
+                                      (1920, 720, 1280, 720, 3)]]
 
 
 @pytest.mark.parametrize("row", STRIPS, ids=lambda r: "%dx%d-%dx%d-i%d-n%d-%s%d" % (r[:6] + (np.dtype(r[6]).name, r[7])))
