@@ -12,8 +12,9 @@
 // Six kernel shapes, all with streaming stores, var-shape batches on a packed tile grid:
 //  * pixels of up to 8 bytes: wave patches (64 columns x 4 rows per wave; adjacent taps in one load,
 //    row terms computed once per wave, 4x4 lane transposes so that every lane stores whole dwords);
-//  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 2 rows (4 x 8 when enlarging by 1.5 or
-//    more) and fetches each source row once for all its columns, lane pairs swap a pixel pair each;
+//  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 4 rows (image batches x 2; 4 x 8 when
+//    enlarging by 1.5 or more) and fetches each source row once for all its columns and rows, lane pairs swap a
+//    pixel pair each;
 //  * 8-bit bicubic tensors of 3 and 4 channels at vertical scales of 1/2 to 2, large launches: a wave owns 64 columns
 //    x 16 rows and forms every source row's sums once, adding them to the output rows in flight;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
@@ -1923,13 +1924,43 @@ __device__ __forceinline__ void ResizeLinearQuadsU8(const Plane &p, int x0, int 
     }
 }
 
+// The windows of rows 0 .. last (wave-uniform, under 9) from `at` on, a lane's own column offset included: only those
+// that are needed, and all of them requested before the first is touched - taken into place inside its test, each
+// load would be waited for before the next goes out (nine round trips one after the other: 62 us instead of 51 for
+// the two-column strips). The empty statement uses every raw window, so the loads can neither sink below it nor
+// the funnel shifts rise above it. That all windows are in before a strip's row loop starts also keeps waits for
+// them out of the loop: stores and loads share one counter of outstanding operations here, and such a wait, after
+// rows have been stored, would be a wait for those stores to reach memory as well.
+template<int C>
+__device__ __forceinline__ void RequestStripWindows(const uint8_t *at, int rowStride, int last, TapWindow<C> (&win)[9])
+{
+    RawTapWindow<C> raw[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k)
+    {
+        if (k <= last)
+        {
+            raw[k] = RequestTapWindow<C>(at + (int64_t)k * rowStride);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::"v"(raw[0].d[0]), "v"(raw[1].d[0]), "v"(raw[2].d[0]), "v"(raw[3].d[0]), "v"(raw[4].d[0]), "v"(raw[5].d[0]),
+                 "v"(raw[6].d[0]), "v"(raw[7].d[0]), "v"(raw[8].d[0]));
+#pragma unroll
+    for (int k = 0; k < 9; ++k)
+    {
+        win[k] = FinishTapWindow<C>(raw[k]);
+    }
+}
+
 // The four-column form over a strip of kStripRows output rows per wave. When not reducing vertically those rows
-// lie between at most kStripRows + 1 consecutive source rows. All their windows are requested up front (rows past
-// the last one needed repeat it), a source row's tap pairs are formed once for every output row that uses it as
+// lie between at most kStripRows + 1 consecutive source rows. All their windows are requested up front, a source
+// row's tap pairs are formed once for every output row that uses it as
 // its upper or its lower row, and the column terms are paid once per 8 rows instead of once per 2. The blend per
 // output pixel is BilinearQ15 as everywhere. A wave that reaches the image's last source row, reduces vertically
 // (more source rows than fit) or has a lane whose columns do not fit its window runs as four two-row steps.
 constexpr int kStripRows = 8, kStripWindows = kStripRows + 1;
+static_assert(kStripWindows == 9);
 
 template<int C>
 __device__ __forceinline__ void ResizeLinearQuadStripU8(const Plane &p, int x0, int y0)
@@ -1962,11 +1993,7 @@ __device__ __forceinline__ void ResizeLinearQuadStripU8(const Plane &p, int x0, 
     }
     TapWindow<C>   win[kStripWindows];
     const uint8_t *at = p.src + (int64_t)yFirst * p.srcRow + col[0].s * C;
-#pragma unroll
-    for (int k = 0; k < kStripWindows; ++k)
-    {
-        win[k] = LoadTapWindowAt<C>(at + (int64_t)min(k, yLast - yFirst) * p.srcRow);
-    }
+    RequestStripWindows<C>(at, p.srcRow, yLast - yFirst, win);
     // lanes past the last column stay (the row terms are read from lanes 0 .. 7 below); they store nothing
     uint32_t ax[4];
     int      d[4];
@@ -2051,6 +2078,142 @@ __device__ __forceinline__ void ResizeLinearQuadStripU8(const Plane &p, int x0, 
     }
 }
 
+// The two-column form over strips of kPairStripRows output rows per wave (128 columns x 4 rows). At vertical scales
+// up to 2 those rows lie between at most 9 consecutive source rows: the windows are requested up front, a source row
+// is taken apart into its (first tap | second tap) pairs once for every output row that uses it as its upper or its
+// lower row, and the column terms are paid once per 4 rows instead of once per 2. Every output row is finished on its
+// own: a lane rounds the channels of its 2 pixels straight into the bytes they have in the row, the lanes of a pair
+// swap them, and the even lane stores the 4 pixels as whole dwords. The blend per output pixel is BilinearQ15 as
+// everywhere. A wave that reaches the image's last source row or reduces vertically by more than 2 runs as two
+// two-row steps.
+constexpr int kPairStripRows = 4, kPairStripWindows = 2 * kPairStripRows + 1;
+static_assert(kPairStripWindows == 9);
+
+template<int C>
+__device__ __forceinline__ void ResizeLinearPairStripU8(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    constexpr int R    = kPairStripRows;
+    const int     lane = threadIdx.x & 63;
+    const int     dx0  = x0 + 2 * lane;
+    // columns and rows past the output compute a duplicate of the last one: every lane takes part in the swap
+    const auto colA  = Axis<NVCV_INTERP_LINEAR>(p.scaleX, min(dx0, p.dstW - 1), p.srcW);
+    const auto colB  = Axis<NVCV_INTERP_LINEAR>(p.scaleX, min(dx0 + 1, p.dstW - 1), p.srcW);
+    const int  delta = colB.s - colA.s; // 0 .. 2 at scales up to 2
+    // lane r holds the terms of output row y0 + r
+    const auto     rows   = Axis<NVCV_INTERP_LINEAR>(p.scaleY, min(y0 + (lane & (R - 1)), p.dstH - 1), p.srcH);
+    const uint32_t ayLane = FractionQ15(rows.w[0]);
+    const int      yFirst = __builtin_amdgcn_readlane(rows.s, 0), yLast = __builtin_amdgcn_readlane(rows.s, R - 1) + 1;
+    if (yLast >= p.srcH - 1 || yLast - yFirst >= kPairStripWindows) // wave-uniform
+    {
+        ResizeLinearPairsU8<C, false>(p, x0, y0);
+        ResizeLinearPairsU8<C, false>(p, x0, y0 + 2);
+        return;
+    }
+    TapWindow<C>   win[kPairStripWindows];
+    const uint8_t *at = p.src + (int64_t)yFirst * p.srcRow + colA.s * C;
+    RequestStripWindows<C>(at, p.srcRow, yLast - yFirst, win);
+    const uint32_t axA = FractionQ15(colA.w[0]), axB = FractionQ15(colB.w[0]);
+    // (first tap | second tap << 16) of both columns and every channel of a source row
+    auto pairs = [&](const TapWindow<C> &w, uint32_t (&t)[2][C])
+    {
+        const uint32_t k0 = WindowPixel<C>(w, 0), k1 = WindowPixel<C>(w, 1), k2 = WindowPixel<C>(w, 2), k3 = WindowPixel<C>(w, 3);
+        const uint32_t first = delta == 0 ? k0 : (delta == 1 ? k1 : k2), second = delta == 0 ? k1 : (delta == 1 ? k2 : k3);
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+        {
+            t[0][c] = ChannelPair(k0, k1, c);
+            t[1][c] = ChannelPair(first, second, c);
+        }
+    };
+    const int  nRows = min(R, p.dstH - y0);
+    const bool even  = (lane & 1) == 0;
+    int        r     = 0;
+    uint8_t   *to    = p.dst + (int64_t)y0 * p.dstRow + (int64_t)dx0 * C; // (used by even lanes: 4 pixels from their first)
+    uint32_t   top[2][C], bot[2][C];
+    pairs(win[0], bot);
+#pragma unroll
+    for (int k = 0; k + 1 < kPairStripWindows; ++k)
+    {
+        if (r < nRows) // wave-uniform
+        {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+            {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    top[j][c] = bot[j][c];
+                }
+            }
+            pairs(win[k + 1], bot);
+            // the output rows between source rows yFirst + k and the next one
+            while (r < nRows && __builtin_amdgcn_readlane(rows.s, r) == yFirst + k)
+            {
+                const uint32_t ay = __builtin_amdgcn_readlane(ayLane, r);
+                // the lane's 2 pixels as the 2 C bytes they are in the row
+                uint32_t mine[2] = {0, 0};
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                {
+                    uint32_t wt, wb;
+                    WeightPairsQ15(j == 0 ? axA : axB, ay, wt, wb);
+#pragma unroll
+                    for (int c = 0; c < C; ++c)
+                    {
+                        const int at8 = j * C + c;
+                        mine[at8 >> 2] = BlendQ15(top[j][c], bot[j][c], wt, wb, at8 & 3, mine[at8 >> 2]);
+                    }
+                }
+                // the even lane takes its neighbour's and stores 4 pixels
+                uint32_t w[C];
+                if constexpr (C == 4)
+                {
+                    w[0] = mine[0];
+                    w[1] = mine[1];
+                    w[2] = FromLaneXor1(mine[0]);
+                    w[3] = FromLaneXor1(mine[1]);
+                }
+                else if constexpr (C == 3)
+                {
+                    const uint32_t lo = FromLaneXor1(mine[0]), hi = FromLaneXor1(mine[1]);
+                    w[0] = mine[0];
+                    w[1] = mine[1] | (lo << 16);
+                    w[2] = __builtin_amdgcn_alignbit(hi, lo, 16);
+                }
+                else
+                {
+                    static_assert(C == 1);
+                    w[0] = mine[0] | (FromLaneXor1(mine[0]) << 16);
+                }
+                if (even && dx0 < p.dstW)
+                {
+                    if (dx0 + 4 <= p.dstW)
+                    {
+                        StoreDwordsNT<C>(to, w);
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int i = 0; i < 3 * C; ++i)
+                        {
+                            if (dx0 + i / C < p.dstW)
+                            {
+                                to[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+                            }
+                        }
+                    }
+                }
+                to += p.dstRow;
+                ++r;
+            }
+        }
+    }
+}
+
 // Which (type, channels, interpolation) take the two-columns-per-lane form. The code is written for 1, 3
 // and 4 channels; with 1 and 4 it measured slower than the wave patches (u8x1 43 -> 58 us, u8x4 91 -> 104 us
 // on 1080p -> 720p: the column terms of two columns are amortised over 2 rows only), so 3 it is.
@@ -2067,11 +2230,12 @@ __host__ __device__ __forceinline__ bool PairsFormScale(int srcW, int dstW)
 
 constexpr int kPairsTileW = 128, kPairsTileH = 8; // block = 4 waves of 128 columns x 2 rows, stacked
 
+// Tensors: strips of 4 rows per wave, a block = 4 waves stacked (128 columns x 16 rows).
 template<int C>
 __global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeLinearPairsU8<C, false>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 2);
+    ResizeLinearPairStripU8<C>(p, blockIdx.x * kPairsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * kPairStripRows);
 }
 
 constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x kQuadsRows rows, stacked
@@ -2631,7 +2795,7 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         }
         if (PairsFormScale<C>(a.srcW, a.dstW))
         {
-            dim3 pgrid(DivUp(a.dstW, kPairsTileW), DivUp(a.dstH, kPairsTileH), N);
+            dim3 pgrid(DivUp(a.dstW, kPairsTileW), DivUp(a.dstH, 4 * kPairStripRows), N);
             hipLaunchKernelGGL((ResizeLinearPairsU8Kernel<C>), pgrid, dim3(256), 0, stream, a);
             CheckLaunch("ResizeLinearPairsU8Kernel");
             return;
