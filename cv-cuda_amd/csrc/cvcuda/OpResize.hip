@@ -15,6 +15,7 @@
 //  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 4 rows (image batches x 2; 4 x 8 when
 //    enlarging by 1.5 or more) and fetches each source row once for all its columns and rows, lane pairs swap a
 //    pixel pair each;
+//    nearest neighbour of 1 and 3 channels takes the same strips when enlarging by 1.5 or more;
 //  * 8-bit bicubic tensors of 3 and 4 channels at vertical scales of 1/2 to 2, large launches: a wave owns 64 columns
 //    x 16 rows and forms every source row's sums once, adding them to the output rows in flight;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
@@ -2078,6 +2079,89 @@ __device__ __forceinline__ void ResizeLinearQuadStripU8(const Plane &p, int x0, 
     }
 }
 
+// Nearest neighbour when enlarging by 1.5 or more (3 * srcW <= 2 * dstW), in the shape of the four-column strips:
+// the source pixels of four neighbouring output columns lie within 3 source pixels, so a lane owns 4 columns x 8
+// rows, takes them from one window per source row and stores every output row that maps to that source row from
+// the same registers. The wave patches spend one 3-byte load per output pixel there (8 x 720p -> 1080p u8x3: 19.0 us,
+// the bilinear strips 22.9; as strips 16.7). Indices are those of Axis<NEAREST>; waves that reach the image's last row,
+// reduce vertically or have a lane whose columns do not fit its window run as wave patches.
+template<int C>
+__device__ __forceinline__ void ResizeNearestQuadStripU8(const Plane &p, int x0, int y0)
+{
+    if (x0 >= p.dstW || y0 >= p.dstH)
+    {
+        return;
+    }
+    const int lane = threadIdx.x & 63;
+    const int dx0  = x0 + 4 * lane;
+    int       s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        s[j] = Axis<NVCV_INTERP_NEAREST>(p.scaleX, min(dx0 + j, p.dstW - 1), p.srcW).s;
+    }
+    // lane r holds the source row of output row y0 + r
+    const int  rowLane = Axis<NVCV_INTERP_NEAREST>(p.scaleY, min(y0 + (lane & (kStripRows - 1)), p.dstH - 1), p.srcH).s;
+    const int  yFirst = __builtin_amdgcn_readlane(rowLane, 0), yLast = __builtin_amdgcn_readlane(rowLane, kStripRows - 1);
+    const bool narrow = s[3] - s[0] <= 3;
+    if (yLast >= p.srcH - 1 || yLast - yFirst >= kStripWindows || __builtin_amdgcn_ballot_w64(!narrow) != 0) // wave-uniform
+    {
+#pragma unroll 1
+        for (int i = 0; i < 8; ++i)
+        {
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_NEAREST, false>(p, x0 + 64 * (i & 3), y0 + 4 * (i >> 2));
+        }
+        return;
+    }
+    TapWindow<C>   win[kStripWindows];
+    const uint8_t *at = p.src + (int64_t)yFirst * p.srcRow + s[0] * C;
+    RequestStripWindows<C>(at, p.srcRow, yLast - yFirst, win);
+    const int nRows = min(kStripRows, p.dstH - y0);
+    int       r     = 0;
+    uint8_t  *to    = p.dst + (int64_t)y0 * p.dstRow + (int64_t)dx0 * C;
+#pragma unroll
+    for (int k = 0; k < kStripWindows; ++k)
+    {
+        if (r < nRows) // wave-uniform
+        {
+            // the lane's 4 pixels of source row yFirst + k, packed as they are stored
+            const uint32_t mask  = C == 4 ? 0xffffffffu : (1u << (8 * C)) - 1u;
+            const uint32_t k0 = WindowPixel<C>(win[k], 0) & mask, k1 = WindowPixel<C>(win[k], 1) & mask,
+                           k2 = WindowPixel<C>(win[k], 2) & mask, k3 = WindowPixel<C>(win[k], 3) & mask;
+            uint32_t       q[1][4];
+            q[0][0] = k0;
+#pragma unroll
+            for (int j = 1; j < 4; ++j)
+            {
+                const int d = s[j] - s[0];
+                q[0][j]     = d == 0 ? k0 : (d == 1 ? k1 : (d == 2 ? k2 : k3));
+            }
+            uint32_t w[C];
+            PackQuad<C>(q, w);
+            while (r < nRows && __builtin_amdgcn_readlane(rowLane, r) == yFirst + k)
+            {
+                if (dx0 + 4 <= p.dstW)
+                {
+                    StoreDwordsNT<C>(to, w);
+                }
+                else
+                {
+#pragma unroll
+                    for (int i = 0; i < 3 * C; ++i)
+                    {
+                        if (dx0 + i / C < p.dstW)
+                        {
+                            to[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+                        }
+                    }
+                }
+                to += p.dstRow;
+                ++r;
+            }
+        }
+    }
+}
+
 // The two-column form over strips of kPairStripRows output rows per wave (128 columns x 4 rows). At vertical scales
 // up to 2 those rows lie between at most 9 consecutive source rows: the windows are requested up front, a source row
 // is taken apart into its (first tap | second tap) pairs once for every output row that uses it as its upper or its
@@ -2258,6 +2342,13 @@ __global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArg
     {
         ResizeLinearQuadsU8<C>(p, blockIdx.x * kQuadsTileW, y0);
     }
+}
+
+template<int C>
+__global__ __launch_bounds__(256) void ResizeNearestQuadsU8Kernel(const ResizeArgs a)
+{
+    const Plane p = GetPlanes<false>(a, blockIdx.z);
+    ResizeNearestQuadStripU8<C>(p, blockIdx.x * kQuadsTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * kStripRows);
 }
 
 // Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
@@ -2781,6 +2872,21 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         {
             hipLaunchKernelGGL((ResizeCubicStagedKernel<T, C>), grid, dim3(256), 0, stream, a);
             CheckLaunch("ResizeCubicStagedKernel");
+            return;
+        }
+    }
+    // (4-byte pixels are faster as wave patches: 8 x 720p -> 1080p 21.2 us against 36.1 as strips; 1 channel 12.4 ->
+    // 8.4 us, 3 channels 19.0 -> 16.7 us)
+    if constexpr (std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_NEAREST && (C == 1 || C == 3))
+    {
+        const int64_t strips = (int64_t)DivUp(a.dstW, kQuadsTileW) * DivUp(a.dstH, kStripRows) * N;
+        // (a window may start at a row's last pixel and, with the bytes a load takes along, runs up to 13 bytes into
+        // the next row: sources of 8 columns and more)
+        if (a.srcW >= 8 && 3 * (int64_t)a.srcW <= 2 * (int64_t)a.dstW && a.srcH <= a.dstH && strips >= 8 * 256)
+        {
+            dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, 4 * kStripRows), N);
+            hipLaunchKernelGGL((ResizeNearestQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
+            CheckLaunch("ResizeNearestQuadsU8Kernel");
             return;
         }
     }

@@ -101,6 +101,20 @@ def test_tensor_cubic_u8_strips(cv, orc, gpu, row):
     test_tensor_table(cv, orc, gpu, row)
 
 
+# 8-bit nearest neighbour enlarging by 1.5 or more horizontally (and not reducing vertically) runs as strips once the
+# launch has 2048 of them: 1.5, 2 and 3 times, ragged sizes, mixed scales (2.5 across, 1 down: every source row once),
+# and a vertical reduction with the same widths (wave patches)
+NN_STRIPS = [(sw, sh, dw, dh, NEAREST, n, np.uint8, c)
+             for c in (3, 1, 4)
+             for (sw, sh, dw, dh, n) in [(1280, 720, 1920, 1080, 2), (640, 360, 1280, 720, 6), (427, 241, 1283, 725, 6),
+                                         (512, 720, 1280, 720, 6), (512, 720, 1280, 700, 6), (9, 2000, 30, 2100, 8)]]
+
+
+@pytest.mark.parametrize("row", NN_STRIPS, ids=lambda r: "%dx%d-%dx%d-i%d-n%d-%s%d" % (r[:6] + (np.dtype(r[6]).name, r[7])))
+def test_tensor_nearest_u8_strips(cv, orc, gpu, row):
+    test_tensor_table(cv, orc, gpu, row)
+
+
 # 8-bit bilinear at horizontal scales up to 2 takes the kernel in which a lane owns two columns: both
 # directions, the scale limit itself, ragged widths (1 - 3 columns left over), odd heights, tiny outputs
 PAIRS = [(sw, sh, dw, dh, LINEAR, n, np.uint8, c)
