@@ -115,6 +115,34 @@ def test_tensor_nearest_u8_strips(cv, orc, gpu, row):
     test_tensor_table(cv, orc, gpu, row)
 
 
+# the strip kernels on views that start at an odd byte and have an odd row pitch (their window loads take the aligned
+# dwords around a pixel: nothing may be assumed of where a row starts), output bytes outside the rows untouched
+@pytest.mark.parametrize("c", [3, 1, 4])
+@pytest.mark.parametrize("shape", [(1531, 700, 1021, 467, LINEAR), (701, 500, 1283, 915, LINEAR), (1531, 700, 1021, 467, CUBIC),
+                                   (701, 500, 1283, 915, CUBIC), (701, 500, 1283, 915, NEAREST)],
+                         ids=lambda sh: "%dx%d-%dx%d-i%d" % sh)
+def test_strips_on_odd_bases_and_pitches(cv, orc, gpu, shape, c):
+    sw, sh, dw, dh, interp = shape
+    n = 6
+    src = make_input(orc, (n, sh, sw, c), np.uint8, 0xBEEF + sw + c)
+
+    def view(w, h, fill):
+        pitch, plane = w * c + 3, (w * c + 3) * h + 7
+        buf = torch.full((n * plane + 64,), fill, dtype=torch.uint8, device="cuda")
+        t = cv.Tensor.wrap(buf.data_ptr() + 1, [n, h, w, c], [plane, pitch, c, 1], np.uint8, "NHWC", keep=buf)
+        return buf, t, torch.as_strided(buf[1:], (n, h, w, c), (plane, pitch, c, 1)), (plane, pitch)
+
+    big_in, tin, in_view, _ = view(sw, sh, 0)
+    in_view.copy_(torch.from_numpy(src).cuda())
+    big_out, tout, out_view, (plane, pitch) = view(dw, dh, 0xCD)
+    cv.Resize()(None, tin, tout, interp)
+    torch.cuda.synchronize()
+    check(out_view.cpu().numpy(), src, (dh, dw), interp, orc)
+    mask = torch.ones_like(big_out, dtype=torch.bool)
+    torch.as_strided(mask[1:], (n, dh, dw * c), (plane, pitch, 1)).fill_(False)
+    assert bool((big_out[mask] == 0xCD).all())
+
+
 # 8-bit bilinear at horizontal scales up to 2 takes the kernel in which a lane owns two columns: both
 # directions, the scale limit itself, ragged widths (1 - 3 columns left over), odd heights, tiny outputs
 PAIRS = [(sw, sh, dw, dh, LINEAR, n, np.uint8, c)
