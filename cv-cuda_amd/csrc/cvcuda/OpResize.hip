@@ -2370,6 +2370,68 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8VarShapeKernel(const R
     }
 }
 
+// Large image-batch launches resize each image in the tensor kernels' strips. WIDE (most of the launch is enlarged by
+// 1.5 or more; 1 and 3 channels): a 256 x 32 tile per block - four columns per lane where the image is enlarged so
+// (a wave takes 8 rows), else two columns per lane at horizontal scales up to 2 (16 strips of 128 x 4, four per wave),
+// else 32 wave patches. Otherwise a 128 x 16 tile: a two-column strip per wave, or two wave patches.
+template<bool WIDE>
+constexpr int kStripsTileW = WIDE ? 256 : 128;
+template<bool WIDE>
+constexpr int kStripsTileH = WIDE ? 32 : 16;
+
+template<int C>
+__host__ __device__ __forceinline__ bool QuadStripScale(int srcW, int dstW)
+{
+    return kQuadsRows<C> == kStripRows && srcW >= 4 && 3 * (int64_t)srcW <= 2 * (int64_t)dstW;
+}
+
+template<int C, bool WIDE>
+__global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc   = LocateTile(tiles, blockIdx.x);
+    const Plane     p    = GetPlanes<true>(a, tc.image);
+    const int       wave = threadIdx.x >> 6;
+    const int       x0 = tc.tx * kStripsTileW<WIDE>, y0 = tc.ty * kStripsTileH<WIDE>;
+    if constexpr (WIDE)
+    {
+        if (QuadStripScale<C>(p.srcW, p.dstW))
+        {
+            if constexpr (kQuadsRows<C> == kStripRows)
+            {
+                ResizeLinearQuadStripU8<C>(p, x0, y0 + wave * kStripRows);
+            }
+        }
+        else if (PairsFormScale<C>(p.srcW, p.dstW))
+        {
+#pragma unroll 1
+            for (int i = wave; i < 16; i += 4)
+            {
+                ResizeLinearPairStripU8<C>(p, x0 + (i & 1) * kPairsTileW, y0 + (i >> 1) * kPairStripRows);
+            }
+        }
+        else
+        {
+#pragma unroll 1
+            for (int i = wave; i < 32; i += 4)
+            {
+                ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + (i & 3) * 64, y0 + (i >> 2) * 4);
+            }
+        }
+    }
+    else
+    {
+        if (PairsFormScale<C>(p.srcW, p.dstW))
+        {
+            ResizeLinearPairStripU8<C>(p, x0, y0 + wave * kPairStripRows);
+        }
+        else
+        {
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0, y0 + wave * 4);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + 64, y0 + wave * 4);
+        }
+    }
+}
+
 constexpr int kPatchTileW = 64, kPatchTileH = 16; // block = 4 waves stacked vertically
 
 template<class T, int C, int INTERP>
@@ -2956,7 +3018,8 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
 }
 
 template<class T, int C, int INTERP>
-void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, int N, hipStream_t stream)
+void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, const NVCVImageBufferStrided *dstHost, int N,
+                    hipStream_t stream)
 {
     for (int first = 0; first < N; first += kMaxTileImages)
     {
@@ -2964,7 +3027,30 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, 
         const int count = std::min(kMaxTileImages, N - first);
         if constexpr (kPairsForm<T, C, INTERP>)
         {
-            int total = BuildVarTiles(tiles, dstHost, first, count, kPairsTileW, kPairsTileH);
+            // strips when that still gives every CU 8 blocks: the wide tile where most output pixels belong to images
+            // that take four columns per lane
+            int64_t quadPixels = 0, allPixels = 0;
+            for (int i = first; i < first + count; ++i)
+            {
+                const int64_t px = (int64_t)dstHost[i].planes[0].width * dstHost[i].planes[0].height;
+                allPixels += px;
+                quadPixels += QuadStripScale<C>(srcHost[i].planes[0].width, dstHost[i].planes[0].width) ? px : 0;
+            }
+            int total = 2 * quadPixels > allPixels ? BuildVarTiles(tiles, dstHost, first, count, kStripsTileW<true>, kStripsTileH<true>) : 0;
+            if (total >= 8 * 256)
+            {
+                hipLaunchKernelGGL((ResizeLinearStripsU8VarShapeKernel<C, true>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeLinearStripsU8VarShapeKernel");
+                continue;
+            }
+            total = BuildVarTiles(tiles, dstHost, first, count, kStripsTileW<false>, kStripsTileH<false>);
+            if (total >= 8 * 256)
+            {
+                hipLaunchKernelGGL((ResizeLinearStripsU8VarShapeKernel<C, false>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeLinearStripsU8VarShapeKernel");
+                continue;
+            }
+            total = BuildVarTiles(tiles, dstHost, first, count, kPairsTileW, kPairsTileH);
             if (total > 0)
             {
                 hipLaunchKernelGGL((ResizeLinearPairsU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
@@ -3003,25 +3089,26 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, 
 }
 
 template<class T, int C>
-void DispatchInterp(bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, int N, int interp,
+void DispatchInterp(bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *srcHost,
+                    const NVCVImageBufferStrided *dstHost, int N, int interp,
                     hipStream_t stream)
 {
     switch (interp)
     {
     case NVCV_INTERP_NEAREST:
-        varshape ? LaunchVarShape<T, C, NVCV_INTERP_NEAREST>(a, dstHost, N, stream)
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_NEAREST>(a, srcHost, dstHost, N, stream)
                  : LaunchTensor<T, C, NVCV_INTERP_NEAREST>(a, N, stream);
         break;
     case NVCV_INTERP_LINEAR:
-        varshape ? LaunchVarShape<T, C, NVCV_INTERP_LINEAR>(a, dstHost, N, stream)
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_LINEAR>(a, srcHost, dstHost, N, stream)
                  : LaunchTensor<T, C, NVCV_INTERP_LINEAR>(a, N, stream);
         break;
     case NVCV_INTERP_CUBIC:
-        varshape ? LaunchVarShape<T, C, NVCV_INTERP_CUBIC>(a, dstHost, N, stream)
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_CUBIC>(a, srcHost, dstHost, N, stream)
                  : LaunchTensor<T, C, NVCV_INTERP_CUBIC>(a, N, stream);
         break;
     case NVCV_INTERP_AREA:
-        varshape ? LaunchVarShape<T, C, NVCV_INTERP_AREA>(a, dstHost, N, stream)
+        varshape ? LaunchVarShape<T, C, NVCV_INTERP_AREA>(a, srcHost, dstHost, N, stream)
                  : LaunchTensor<T, C, NVCV_INTERP_AREA>(a, N, stream);
         break;
     default:
@@ -3030,26 +3117,27 @@ void DispatchInterp(bool varshape, const ResizeArgs &a, const NVCVImageBufferStr
 }
 
 template<class T>
-void DispatchChannels(int channels, bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *dstHost, int N,
+void DispatchChannels(int channels, bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *srcHost,
+                      const NVCVImageBufferStrided *dstHost, int N,
                       int interp, hipStream_t stream)
 {
     switch (channels)
     {
     case 1:
-        DispatchInterp<T, 1>(varshape, a, dstHost, N, interp, stream);
+        DispatchInterp<T, 1>(varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     case 3:
-        DispatchInterp<T, 3>(varshape, a, dstHost, N, interp, stream);
+        DispatchInterp<T, 3>(varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     case 4:
-        DispatchInterp<T, 4>(varshape, a, dstHost, N, interp, stream);
+        DispatchInterp<T, 4>(varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     default:
         throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input data type");
     }
 }
 
-void DispatchType(ElemType elem, int channels, bool varshape, const ResizeArgs &a,
+void DispatchType(ElemType elem, int channels, bool varshape, const ResizeArgs &a, const NVCVImageBufferStrided *srcHost,
                   const NVCVImageBufferStrided *dstHost, int N, int interp, hipStream_t stream)
 {
     if (N == 0)
@@ -3059,16 +3147,16 @@ void DispatchType(ElemType elem, int channels, bool varshape, const ResizeArgs &
     switch (elem)
     {
     case kU8:
-        DispatchChannels<uint8_t>(channels, varshape, a, dstHost, N, interp, stream);
+        DispatchChannels<uint8_t>(channels, varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     case kU16:
-        DispatchChannels<uint16_t>(channels, varshape, a, dstHost, N, interp, stream);
+        DispatchChannels<uint16_t>(channels, varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     case kS16:
-        DispatchChannels<int16_t>(channels, varshape, a, dstHost, N, interp, stream);
+        DispatchChannels<int16_t>(channels, varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     case kF32:
-        DispatchChannels<float>(channels, varshape, a, dstHost, N, interp, stream);
+        DispatchChannels<float>(channels, varshape, a, srcHost, dstHost, N, interp, stream);
         break;
     default:
         throw OpError(NVCV_ERROR_INVALID_ARGUMENT, "Invalid input data type");
@@ -3131,7 +3219,7 @@ public:
         }
         a.scaleX = static_cast<float>(in.W) / out.W; // IEEE float32 division, as the kernels would do it
         a.scaleY = static_cast<float>(in.H) / out.H;
-        DispatchType(in.elem, in.C, false, a, nullptr, in.N, interp, stream);
+        DispatchType(in.elem, in.C, false, a, nullptr, nullptr, in.N, interp, stream);
     }
 
     void submit(hipStream_t stream, NVCVImageBatchHandle hin, NVCVImageBatchHandle hout,
@@ -3156,7 +3244,7 @@ public:
         ResizeArgs a = {};
         a.srcList    = in.data.buffer.varShapeStrided.imageList;
         a.dstList    = out.data.buffer.varShapeStrided.imageList;
-        DispatchType(fi.elem, fi.channels, true, a, out.hostList, in.N, interp, stream);
+        DispatchType(fi.elem, fi.channels, true, a, in.hostList, out.hostList, in.N, interp, stream);
     }
 };
 

@@ -255,6 +255,37 @@ def test_varshape(cv, K, orc, gpu, interp, dt, c):
         check(res, a[None], (h, w), interp, orc, varshape=True)
 
 
+# large image batches of 8-bit bilinear resizes run in the tensor kernels' strips: mostly enlarged by 1.5 or more (wide
+# tiles, with a reduced and a strongly reduced image among them), mostly reduced or slightly enlarged (narrow tiles)
+@pytest.mark.parametrize("c", [3, 1, 4])
+@pytest.mark.parametrize("mix", ["enlarging", "reducing"])
+def test_varshape_linear_u8_strips(cv, K, orc, gpu, mix, c):
+    rng = np.random.default_rng(23 + c)
+    fmt = _format_for(cv, K, np.uint8, c)
+    n = 16  # (2048 tiles and more of 256 x 32, respectively 128 x 16)
+    bin_, bout, hosts, outs = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], []
+    for i in range(n):
+        if mix == "enlarging":
+            sw, sh = int(rng.integers(700, 900)), int(rng.integers(500, 650))
+            f = [1.5, 1.9, 2.0, 3.1][i % 4] if i < n - 2 else [0.7, 0.3][i - (n - 2)]
+        else:
+            sw, sh = int(rng.integers(900, 1300)), int(rng.integers(500, 800))
+            f = [1 / 1.5, 0.5, 0.9, 1.2, 1 / 1.51][i % 5] if i < n - 2 else [0.31, 1.6][i - (n - 2)]
+        dw, dh = max(1, int(sw * f) + int(rng.integers(0, 3))), max(1, int(sh * f) + int(rng.integers(0, 3)))
+        a = make_input(orc, (sh, sw, c), np.uint8, 500 + i)
+        hosts.append(a)
+        bin_.push_back(cv.Image.from_numpy(a, fmt))
+        o = cv.Image.alloc((dw, dh), fmt)
+        outs.append(o)
+        bout.push_back(o)
+    cv.Resize()(None, bin_, bout, LINEAR)
+    torch.cuda.synchronize()
+    for a, o in zip(hosts, outs):
+        w, h = o.size
+        res = o.plane_view(0, np.uint8, c).cpu().numpy()[None]
+        check(res, a[None], (h, w), LINEAR, orc, varshape=True)
+
+
 AREA = 3
 AREA_ROWS = [(44, 40, 22, 20, 2, np.uint8, 4), (30, 30, 20, 20, 2, np.uint8, 4), (30, 30, 60, 60, 4, np.uint8, 4),
              (1440, 2560, 1080, 1920, 1, np.uint8, 4), (720, 1280, 360, 640, 1, np.uint8, 4),
