@@ -2442,6 +2442,44 @@ __global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs 
     ResizeWavePatch<T, C, INTERP, false>(p, blockIdx.x * kPatchTileW, (blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 4);
 }
 
+// Which of the bicubic strip forms an image takes by its vertical scale and row length: 4 (reducing by up to 2), 8
+// (enlarging by up to 2) or 0 (none: wave patches).
+template<int C>
+__host__ __device__ __forceinline__ int CubicStripForm(int srcW, int srcH, int dstH)
+{
+    if (!(C == 3 || C == 4) || srcW < 4 || srcW * C < 16)
+    {
+        return 0;
+    }
+    return (srcH >= dstH && srcH <= 2 * (int64_t)dstH) ? 4 : ((srcH < dstH && 2 * (int64_t)srcH >= dstH) ? 8 : 0);
+}
+
+// Large image batches: a 64 x 64 tile per block, a strip per wave where the image's scale allows, else four patches.
+template<int C>
+__global__ __launch_bounds__(256) void ResizeCubicStripU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc   = LocateTile(tiles, blockIdx.x);
+    const Plane     p    = GetPlanes<true>(a, tc.image);
+    const int       x0 = tc.tx * kPatchTileW, y0 = tc.ty * 4 * kCubicStripRows + (threadIdx.x >> 6) * kCubicStripRows;
+    const int       form = CubicStripForm<C>(p.srcW, p.srcH, p.dstH);
+    if (form == 4)
+    {
+        ResizeCubicStripU8<C, 4>(p, x0, y0);
+    }
+    else if (form == 8)
+    {
+        ResizeCubicStripU8<C, 8>(p, x0, y0);
+    }
+    else
+    {
+#pragma unroll 1
+        for (int g = 0; g < kCubicStripRows; g += 4)
+        {
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_CUBIC, true>(p, x0, y0 + g);
+        }
+    }
+}
+
 // 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows).
 template<int C, int S>
 __global__ __launch_bounds__(256) void ResizeCubicStripU8Kernel(const ResizeArgs a)
@@ -2985,21 +3023,20 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         // still has 8 waves and more per CU; one channel is as fast or faster as wave patches (16 x 720p -> 1080p
         // 46.6 us against 50.9 as strips, 1080p -> 720p 27.2 against 28.1)
         const int64_t strips = (int64_t)DivUp(a.dstW, kPatchTileW) * DivUp(a.dstH, kCubicStripRows) * N;
-        if (strips >= 8 * 256 && a.srcW >= 4 && a.srcW * C >= (C == 1 ? 8 : 16))
+        const int     form   = CubicStripForm<C>(a.srcW, a.srcH, a.dstH);
+        if (strips >= 8 * 256 && form != 0)
         {
             dim3 sgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, 4 * kCubicStripRows), N);
-            if (a.srcH >= a.dstH && a.srcH <= 2 * (int64_t)a.dstH)
+            if (form == 4)
             {
                 hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 4>), sgrid, dim3(256), 0, stream, a);
-                CheckLaunch("ResizeCubicStripU8Kernel");
-                return;
             }
-            if (a.srcH < a.dstH && 2 * (int64_t)a.srcH >= a.dstH)
+            else
             {
                 hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 8>), sgrid, dim3(256), 0, stream, a);
-                CheckLaunch("ResizeCubicStripU8Kernel");
-                return;
             }
+            CheckLaunch("ResizeCubicStripU8Kernel");
+            return;
         }
     }
     if constexpr (kPatchForm<T, C, INTERP>)
@@ -3067,6 +3104,24 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
                 CheckLaunch("ResizeAreaVarShapeKernel");
             }
             continue;
+        }
+        if constexpr (INTERP == NVCV_INTERP_CUBIC && std::is_same_v<T, uint8_t> && (C == 3 || C == 4))
+        {
+            // strips where most output pixels belong to images that can take them and every CU still gets 8 blocks
+            int64_t stripPixels = 0, allPixels = 0;
+            for (int i = first; i < first + count; ++i)
+            {
+                const int64_t px = (int64_t)dstHost[i].planes[0].width * dstHost[i].planes[0].height;
+                allPixels += px;
+                stripPixels += CubicStripForm<C>(srcHost[i].planes[0].width, srcHost[i].planes[0].height, dstHost[i].planes[0].height) != 0 ? px : 0;
+            }
+            int total = 2 * stripPixels > allPixels ? BuildVarTiles(tiles, dstHost, first, count, kPatchTileW, 4 * kCubicStripRows) : 0;
+            if (total >= 8 * 256)
+            {
+                hipLaunchKernelGGL((ResizeCubicStripU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeCubicStripU8VarShapeKernel");
+                continue;
+            }
         }
         if constexpr (kPatchForm<T, C, INTERP>)
         {

@@ -286,6 +286,32 @@ def test_varshape_linear_u8_strips(cv, K, orc, gpu, mix, c):
         check(res, a[None], (h, w), LINEAR, orc, varshape=True)
 
 
+# large image batches of 8-bit bicubic resizes of 3 and 4 channels run in the tensor kernels' strips (64 x 64 tiles,
+# 2048 and more): reductions up to 2, enlargements up to 2, and a few images outside both among them
+@pytest.mark.parametrize("c", [3, 4])
+def test_varshape_cubic_u8_strips(cv, K, orc, gpu, c):
+    rng = np.random.default_rng(41 + c)
+    fmt = _format_for(cv, K, np.uint8, c)
+    n = 16
+    bin_, bout, hosts, outs = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], []
+    for i in range(n):
+        sw, sh = int(rng.integers(600, 900)), int(rng.integers(400, 650))
+        f = [1 / 1.5, 1.5, 2.0, 0.5, 1.0, 1.25][i % 6] if i < n - 2 else [0.3, 2.6][i - (n - 2)]
+        dw, dh = max(1, int(sw * f) + int(rng.integers(0, 3))), max(1, int(sh * f) + int(rng.integers(0, 3)))
+        a = make_input(orc, (sh, sw, c), np.uint8, 700 + i)
+        hosts.append(a)
+        bin_.push_back(cv.Image.from_numpy(a, fmt))
+        o = cv.Image.alloc((dw, dh), fmt)
+        outs.append(o)
+        bout.push_back(o)
+    cv.Resize()(None, bin_, bout, CUBIC)
+    torch.cuda.synchronize()
+    for a, o in zip(hosts, outs):
+        w, h = o.size
+        res = o.plane_view(0, np.uint8, c).cpu().numpy()[None]
+        check(res, a[None], (h, w), CUBIC, orc, varshape=True)
+
+
 AREA = 3
 AREA_ROWS = [(44, 40, 22, 20, 2, np.uint8, 4), (30, 30, 20, 20, 2, np.uint8, 4), (30, 30, 60, 60, 4, np.uint8, 4),
              (1440, 2560, 1080, 1920, 1, np.uint8, 4), (720, 1280, 360, 640, 1, np.uint8, 4),
