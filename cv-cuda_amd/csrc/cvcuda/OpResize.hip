@@ -2432,6 +2432,37 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
     }
 }
 
+// Nearest neighbour: whether an image takes the four-column strips (enlarged by 1.5 or more across, not reduced down;
+// 1 and 3 channels; a window may start at a row's last pixel and, with the bytes a load takes along, runs up to 13
+// bytes into the next row: sources of 8 columns and more).
+template<int C>
+__host__ __device__ __forceinline__ bool NearestStripScale(int srcW, int srcH, int dstW, int dstH)
+{
+    return (C == 1 || C == 3) && srcW >= 8 && 3 * (int64_t)srcW <= 2 * (int64_t)dstW && srcH <= dstH;
+}
+
+// Large image batches that are mostly such images: a 256 x 32 tile per block, a strip per wave or eight patches.
+template<int C>
+__global__ __launch_bounds__(256) void ResizeNearestStripsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+{
+    const TileCoord tc   = LocateTile(tiles, blockIdx.x);
+    const Plane     p    = GetPlanes<true>(a, tc.image);
+    const int       wave = threadIdx.x >> 6;
+    const int       x0 = tc.tx * kStripsTileW<true>, y0 = tc.ty * kStripsTileH<true>;
+    if (NearestStripScale<C>(p.srcW, p.srcH, p.dstW, p.dstH))
+    {
+        ResizeNearestQuadStripU8<C>(p, x0, y0 + wave * kStripRows);
+    }
+    else
+    {
+#pragma unroll 1
+        for (int i = wave; i < 32; i += 4)
+        {
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_NEAREST, true>(p, x0 + (i & 3) * 64, y0 + (i >> 2) * 4);
+        }
+    }
+}
+
 constexpr int kPatchTileW = 64, kPatchTileH = 16; // block = 4 waves stacked vertically
 
 template<class T, int C, int INTERP>
@@ -2980,9 +3011,7 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     if constexpr (std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_NEAREST && (C == 1 || C == 3))
     {
         const int64_t strips = (int64_t)DivUp(a.dstW, kQuadsTileW) * DivUp(a.dstH, kStripRows) * N;
-        // (a window may start at a row's last pixel and, with the bytes a load takes along, runs up to 13 bytes into
-        // the next row: sources of 8 columns and more)
-        if (a.srcW >= 8 && 3 * (int64_t)a.srcW <= 2 * (int64_t)a.dstW && a.srcH <= a.dstH && strips >= 8 * 256)
+        if (NearestStripScale<C>(a.srcW, a.srcH, a.dstW, a.dstH) && strips >= 8 * 256)
         {
             dim3 qgrid(DivUp(a.dstW, kQuadsTileW), DivUp(a.dstH, 4 * kStripRows), N);
             hipLaunchKernelGGL((ResizeNearestQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
@@ -3104,6 +3133,24 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
                 CheckLaunch("ResizeAreaVarShapeKernel");
             }
             continue;
+        }
+        if constexpr (INTERP == NVCV_INTERP_NEAREST && std::is_same_v<T, uint8_t> && (C == 1 || C == 3))
+        {
+            int64_t stripPixels = 0, allPixels = 0;
+            for (int i = first; i < first + count; ++i)
+            {
+                const NVCVImagePlaneStrided &sp = srcHost[i].planes[0], &dp = dstHost[i].planes[0];
+                const int64_t                px = (int64_t)dp.width * dp.height;
+                allPixels += px;
+                stripPixels += NearestStripScale<C>(sp.width, sp.height, dp.width, dp.height) ? px : 0;
+            }
+            int total = 2 * stripPixels > allPixels ? BuildVarTiles(tiles, dstHost, first, count, kStripsTileW<true>, kStripsTileH<true>) : 0;
+            if (total >= 8 * 256)
+            {
+                hipLaunchKernelGGL((ResizeNearestStripsU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
+                CheckLaunch("ResizeNearestStripsU8VarShapeKernel");
+                continue;
+            }
         }
         if constexpr (INTERP == NVCV_INTERP_CUBIC && std::is_same_v<T, uint8_t> && (C == 3 || C == 4))
         {

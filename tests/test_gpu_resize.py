@@ -286,6 +286,32 @@ def test_varshape_linear_u8_strips(cv, K, orc, gpu, mix, c):
         check(res, a[None], (h, w), LINEAR, orc, varshape=True)
 
 
+# large image batches of 8-bit nearest-neighbour enlargements of 1 and 3 channels run in the tensor kernel's strips
+# (256 x 32 tiles, 2048 and more), images of other scales among them as patches
+@pytest.mark.parametrize("c", [3, 1])
+def test_varshape_nearest_u8_strips(cv, K, orc, gpu, c):
+    rng = np.random.default_rng(61 + c)
+    fmt = _format_for(cv, K, np.uint8, c)
+    n = 16
+    bin_, bout, hosts, outs = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], []
+    for i in range(n):
+        sw, sh = int(rng.integers(700, 900)), int(rng.integers(500, 650))
+        f = [1.5, 1.9, 2.0, 3.1][i % 4] if i < n - 2 else [0.7, 1.2][i - (n - 2)]
+        dw, dh = max(1, int(sw * f) + int(rng.integers(0, 3))), max(1, int(sh * f) + int(rng.integers(0, 3)))
+        a = make_input(orc, (sh, sw, c), np.uint8, 900 + i)
+        hosts.append(a)
+        bin_.push_back(cv.Image.from_numpy(a, fmt))
+        o = cv.Image.alloc((dw, dh), fmt)
+        outs.append(o)
+        bout.push_back(o)
+    cv.Resize()(None, bin_, bout, NEAREST)
+    torch.cuda.synchronize()
+    for a, o in zip(hosts, outs):
+        w, h = o.size
+        res = o.plane_view(0, np.uint8, c).cpu().numpy()[None]
+        check(res, a[None], (h, w), NEAREST, orc, varshape=True)
+
+
 # large image batches of 8-bit bicubic resizes of 3 and 4 channels run in the tensor kernels' strips (64 x 64 tiles,
 # 2048 and more): reductions up to 2, enlargements up to 2, and a few images outside both among them
 @pytest.mark.parametrize("c", [3, 4])
