@@ -699,6 +699,10 @@ class Streaming:
                                   "ResizeLinearQuadsU8Kernel<3>", "i32", "Resize LINEAR 1280x720 -> 1920x1080"),
         "resize-cubic-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
                               "ResizeCubicStripU8Kernel<3,4>", "i32", "Resize CUBIC 1920x1080 -> 1280x720"),
+        "resize-cubic-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
+                                 "ResizeCubicStripU8Kernel<3,8>", "i32", "Resize CUBIC 1280x720 -> 1920x1080"),
+        "resize-nearest-upscale": ("Resize", 32, ("uint8", 3, 720, 1280), ("uint8", 3, "NHWC", 1080, 1920),
+                                   "ResizeNearestQuadsU8Kernel<3>", "f32", "Resize NEAREST 1280x720 -> 1920x1080"),
         "resize-area-720p": ("Resize", 32, ("uint8", 3), ("uint8", 3, "NHWC", 720, 1280),
                              "ResizeAreaFixedTensorKernel<3>", "i32", "Resize AREA 1920x1080 -> 1280x720"),
         "cvtcolor-bgr2hsv": ("CvtColor", 32, ("uint8", 3), ("uint8", 3, "NHWC"), "MapTensor<HsvFromBgr<uint8_t,false>>", "f32",
@@ -711,7 +715,8 @@ class Streaming:
     # what differs from the operator's default call above: colour code by name, interpolation
     CODES = {"cvtcolor-bgr2rgb": "COLOR_BGR2RGB", "cvtcolor-bgr2gray": "COLOR_BGR2GRAY", "cvtcolor-bgr2hsv": "COLOR_BGR2HSV",
              "cvtcolor-bgr2nv12": "COLOR_BGR2YUV_NV12", "cvtcolor-yuy2-bgr": "COLOR_YUV2BGR_YUY2"}
-    INTERP = {"resize-area-720p": AREA, "resize-cubic-720p": CUBIC}
+    INTERP = {"resize-area-720p": AREA, "resize-cubic-720p": CUBIC, "resize-cubic-upscale": CUBIC,
+              "resize-nearest-upscale": NEAREST}
 
     def __init__(self, cv, orc, np, torch, key):
         self.cv, self.orc, self.np, self.torch, self.key = cv, orc, np, torch, key
@@ -838,7 +843,7 @@ WORKLOADS.update({k: (lambda *a, k=k: StreamMix(*a, k)) for k in StreamMix.SPECS
 BOUNDS = {"warp-affine-varshape": "valu-issue", "warp-affine-tensor-linear": "valu-issue",
           "warp-affine-tensor-cubic": "valu-issue", "warp-affine-tensor-nearest": "vmem-issue",
           "resize-area-720p": "valu-issue", "resize-cubic-720p": "valu-issue", "cvtcolor-bgr2hsv": "valu-issue",
-          "resize-linear-720p": "vmem-issue", "resize-linear-upscale": "valu-issue",
+          "resize-linear-720p": "valu-issue", "resize-linear-upscale": "valu-issue", "resize-cubic-upscale": "valu-issue",
           "resize-nearest": "launch-latency", "resize-linear": "launch-latency", "empty-launch": "launch-latency"}
 
 # The other BASELINE configurations, timed after the headline when no --workload is given.
