@@ -1455,6 +1455,12 @@ __device__ __forceinline__ void ResizeCubicStripU8(const Plane &p, int x0, int y
             {
                 break;
             }
+            // taps fall with i: from the first pixel whose window starts below the row on, nothing is added (tested
+            // where it pays: once for pixels 4 - 5 and once for 6 - 7 of the enlarging form; wave-uniform)
+            if ((i == 4 || i == 6) && j - sr[i] + 1 < 0)
+            {
+                break;
+            }
             const float wi = weight(j, sr[i], r + i, i < sure);
 #pragma unroll
             for (int c = 0; c < C; ++c)
