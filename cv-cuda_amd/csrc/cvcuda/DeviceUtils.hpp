@@ -128,6 +128,16 @@ __device__ __forceinline__ uint64_t LoadU64Unaligned(const uint8_t *p)
 template<int N>
 __device__ __forceinline__ void StoreDwordsNT(uint8_t *p, const uint32_t (&w)[N])
 {
+    if constexpr (N == 4)
+    {
+        // as one 16-byte value: left to merge four dword stores the compiler sometimes settles for 12 + 4 or
+        // 4 + 8 + 4 bytes, i.e. two or three partial writes of every 16 bytes
+        typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+        typedef U32x4    UnalignedU32x4 __attribute__((aligned(1)));
+        const U32x4      v = {w[0], w[1], w[2], w[3]};
+        __builtin_nontemporal_store(v, reinterpret_cast<UnalignedU32x4 *>(p));
+        return;
+    }
     UnalignedU32 *o = reinterpret_cast<UnalignedU32 *>(p);
 #pragma unroll
     for (int i = 0; i < N; ++i)

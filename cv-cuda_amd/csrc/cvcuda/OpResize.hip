@@ -15,7 +15,7 @@
 //  * 8-bit bilinear at horizontal scales up to 2: a lane owns 2 columns x 4 rows (image batches x 2; 4 x 8 when
 //    enlarging by 1.5 or more) and fetches each source row once for all its columns and rows, lane pairs swap a
 //    pixel pair each;
-//    nearest neighbour of 1 and 3 channels takes the same strips when enlarging by 1.5 or more;
+//    nearest neighbour takes the same strips when enlarging by 1.5 or more;
 //  * 8-bit bicubic tensors of 3 and 4 channels at vertical scales of 1/2 to 2, large launches: a wave owns 64 columns
 //    x 16 rows and forms every source row's sums once, adding them to the output rows in flight;
 //  * bicubic reductions >= 2x of 12/16-byte pixels: tap-major loads exchanged through LDS;
@@ -1931,13 +1931,17 @@ __device__ __forceinline__ void ResizeLinearQuadsU8(const Plane &p, int x0, int 
     }
 }
 
-// The windows of rows 0 .. last (wave-uniform, under 9) from `at` on, a lane's own column offset included: only those
-// that are needed, and all of them requested before the first is touched - taken into place inside its test, each
-// load would be waited for before the next goes out (nine round trips one after the other: 62 us instead of 51 for
-// the two-column strips). The empty statement uses every raw window, so the loads can neither sink below it nor
-// the funnel shifts rise above it. That all windows are in before a strip's row loop starts also keeps waits for
-// them out of the loop: stores and loads share one counter of outstanding operations here, and such a wait, after
-// rows have been stored, would be a wait for those stores to reach memory as well.
+// The windows of rows 0 .. last (wave-uniform, under 9) from `at` on, a lane's own column offset included, all of them
+// requested before the first is touched: taken into place inside a test on `last`, each load would be waited for
+// before the next goes out (nine round trips one after the other: 62 us instead of 51 for the two-column strips).
+// The empty statement uses every raw window, so the loads can neither sink below it nor the funnel shifts rise
+// above it. That all windows are in before a strip's row loop starts also keeps waits for them out of the loop:
+// stores and loads share one counter of outstanding operations here, and such a wait, after rows have been stored,
+// would be a wait for those stores to reach memory as well.
+// 1 and 3 channels request only the windows that are needed. With 4-byte pixels the compiler joins a window that exists
+// on one side of the test only to the statement through a register move, which waits for its load, so those request
+// all nine (rows past `last` repeat it: an L1 hit, but a load instruction; 16 x 720p -> 900p u8x3 36.8 us against
+// 31.3). Two whole variants, 5 windows or 9, were slower for every pixel size (65 us for the two-column strips).
 template<int C>
 __device__ __forceinline__ void RequestStripWindows(const uint8_t *at, int rowStride, int last, TapWindow<C> (&win)[9])
 {
@@ -1945,9 +1949,16 @@ __device__ __forceinline__ void RequestStripWindows(const uint8_t *at, int rowSt
 #pragma unroll
     for (int k = 0; k < 9; ++k)
     {
-        if (k <= last)
+        if constexpr (C == 4)
         {
-            raw[k] = RequestTapWindow<C>(at + (int64_t)k * rowStride);
+            raw[k] = RequestTapWindow<C>(at + (int64_t)min(k, last) * rowStride);
+        }
+        else
+        {
+            if (k <= last)
+            {
+                raw[k] = RequestTapWindow<C>(at + (int64_t)k * rowStride);
+            }
         }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -2330,10 +2341,10 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArg
 
 constexpr int kQuadsTileW = 256; // block = 4 waves of 256 columns x kQuadsRows rows, stacked
 
-// Rows per wave of the four-column form: strips for 1 and 3 channels; 4-byte pixels stay with two rows (their strip
-// holds 9 windows of 4 dwords and 32 tap pairs per source row: 16 x 720p -> 1080p 59.5 us against 43.7 us).
+// Rows per wave of the four-column form (strips for every pixel size; with 16-byte stores that the compiler had
+// split into 12 + 4 bytes, 4-byte pixels were faster in two-row steps: 16 x 720p -> 1080p 43.7 us, now 37.7 as strips).
 template<int C>
-constexpr int kQuadsRows = C == 4 ? 2 : kStripRows;
+constexpr int kQuadsRows = kStripRows;
 
 template<int C>
 __global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArgs a)
@@ -2377,7 +2388,7 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8VarShapeKernel(const R
 }
 
 // Large image-batch launches resize each image in the tensor kernels' strips. WIDE (most of the launch is enlarged by
-// 1.5 or more; 1 and 3 channels): a 256 x 32 tile per block - four columns per lane where the image is enlarged so
+// 1.5 or more): a 256 x 32 tile per block - four columns per lane where the image is enlarged so
 // (a wave takes 8 rows), else two columns per lane at horizontal scales up to 2 (16 strips of 128 x 4, four per wave),
 // else 32 wave patches. Otherwise a 128 x 16 tile: a two-column strip per wave, or two wave patches.
 template<bool WIDE>
@@ -2439,12 +2450,12 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
 }
 
 // Nearest neighbour: whether an image takes the four-column strips (enlarged by 1.5 or more across, not reduced down;
-// 1 and 3 channels; a window may start at a row's last pixel and, with the bytes a load takes along, runs up to 13
+// a window may start at a row's last pixel and, with the bytes a load takes along, runs up to 13
 // bytes into the next row: sources of 8 columns and more).
 template<int C>
 __host__ __device__ __forceinline__ bool NearestStripScale(int srcW, int srcH, int dstW, int dstH)
 {
-    return (C == 1 || C == 3) && srcW >= 8 && 3 * (int64_t)srcW <= 2 * (int64_t)dstW && srcH <= dstH;
+    return srcW >= 8 && 3 * (int64_t)srcW <= 2 * (int64_t)dstW && srcH <= dstH;
 }
 
 // Large image batches that are mostly such images: a 256 x 32 tile per block, a strip per wave or eight patches.
@@ -3012,9 +3023,8 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             return;
         }
     }
-    // (4-byte pixels are faster as wave patches: 8 x 720p -> 1080p 21.2 us against 36.1 as strips; 1 channel 12.4 ->
-    // 8.4 us, 3 channels 19.0 -> 16.7 us)
-    if constexpr (std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_NEAREST && (C == 1 || C == 3))
+    // (8 x 720p -> 1080p: 1 channel 12.4 -> 8.4 us, 3 channels 19.0 -> 16.7 us, 4 channels 21.2 -> 18.7 us)
+    if constexpr (std::is_same_v<T, uint8_t> && INTERP == NVCV_INTERP_NEAREST && (C == 1 || C == 3 || C == 4))
     {
         const int64_t strips = (int64_t)DivUp(a.dstW, kQuadsTileW) * DivUp(a.dstH, kStripRows) * N;
         if (NearestStripScale<C>(a.srcW, a.srcH, a.dstW, a.dstH) && strips >= 8 * 256)
@@ -3140,7 +3150,7 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
             }
             continue;
         }
-        if constexpr (INTERP == NVCV_INTERP_NEAREST && std::is_same_v<T, uint8_t> && (C == 1 || C == 3))
+        if constexpr (INTERP == NVCV_INTERP_NEAREST && std::is_same_v<T, uint8_t> && (C == 1 || C == 3 || C == 4))
         {
             int64_t stripPixels = 0, allPixels = 0;
             for (int i = first; i < first + count; ++i)
