@@ -88,9 +88,14 @@ __device__ __forceinline__ void StorePixel(const FusedArgs &a, DstT *rowOut, int
             __builtin_memcpy(w, mine + lane * 4, 4);
             StoreDwordsNT<1>(to + lane * 4, w);
         }
-        if (lane < (total & 3)) // the row's last 1-3 bytes
+        // the row's last 1-3 bytes, all from lane 0: only the lanes of columns inside the output are here, and a
+        // wave that holds the row's last column alone has 3 bytes to store
+        if (lane == 0)
         {
-            __builtin_nontemporal_store(mine[dwords * 4 + lane], to + dwords * 4 + lane);
+            for (int i = dwords * 4; i < total; ++i)
+            {
+                __builtin_nontemporal_store(mine[i], to + i);
+            }
         }
         WaveExchangeFence(); // the next row reuses the staging area
     }

@@ -5,6 +5,8 @@ sizes, resize targets, crops, interpolation, scale/offset, srcCast, layouts) wit
 input recipe (x+y+c)&255 (:198-221), plus seeded random inputs and the benchmark configuration.
 Tolerances: nearest bit-exact; u8 output <= 1 LSB; f32 output |d| <= 1e-5*max(1,|ref|).
 """
+import itertools
+
 import numpy as np
 import pytest
 import torch
@@ -71,6 +73,11 @@ ROWS = [
     (1, 1, 2, 2, 0, 0, 2, 2, 2, LINEAR, np.float32, True, 0, 1.0, 0.0, False),   # images smaller than one 8-byte load
     (2, 1, 5, 3, 1, 0, 3, 3, 1, LINEAR, np.uint8, False, 1, 1.0, 0.0, True),
     (3, 1, 7, 2, 0, 0, 7, 2, 1, LINEAR, np.float32, False, 0, 1.0, 0.0, False),  # exactly 9 bytes: shifted tail load
+    # interleaved 8-bit outputs whose last wave holds one column (width = 1 mod 64): its 3 bytes are a row's tail
+    (130, 40, 65, 20, 0, 0, 65, 20, 2, LINEAR, np.uint8, False, 0, 1.0, 0.0, True),
+    (130, 40, 140, 30, 11, 3, 129, 20, 1, NEAREST, np.uint8, False, 1, 1.0, 0.0, False),
+    (6, 61, 12, 150, 8, 59, 1, 67, 1, NEAREST, np.uint8, False, 0, 2.0, -100.0, False),
+    (6, 61, 12, 150, 8, 59, 1, 67, 2, LINEAR, np.uint8, False, 1, 0.5, 3.0, False),
 ]
 
 
@@ -228,21 +235,23 @@ def test_pitched_unaligned_source_view(cv, orc, gpu):
 def test_varshape(cv, K, orc, gpu):
     rng = np.random.default_rng(3)
     sizes = [(int(rng.integers(60, 140)), int(rng.integers(50, 120))) for _ in range(5)]
-    for interp, odt, planar in ((LINEAR, np.float32, True), (NEAREST, np.uint8, False), (LINEAR, np.uint8, True)):
+    # (65 columns: an interleaved 8-bit row whose second wave holds the last column alone)
+    for (interp, odt, planar), ow in itertools.product(((LINEAR, np.float32, True), (NEAREST, np.uint8, False),
+                                                        (LINEAR, np.uint8, True), (LINEAR, np.uint8, False)), (40, 65)):
         batch = cv.ImageBatchVarShape(8)
         hosts = []
         for i, (w, h) in enumerate(sizes):
             a = orc.fill_u8((h, w, 3), 1000 + i)
             hosts.append(a)
             batch.push_back(cv.Image.from_numpy(a, K.IMAGE_FORMAT_RGB8))
-        shape, layout = ([5, 3, 32, 40], "NCHW") if planar else ([5, 32, 40, 3], "NHWC")
+        shape, layout = ([5, 3, 32, ow], "NCHW") if planar else ([5, 32, ow, 3], "NHWC")
         tout = cv.Tensor.alloc(shape, odt, layout)
         op = cv.ResizeCropConvertReformat()
-        op(None, batch, tout, (48, 40), interp, (4, 3), 1, 0.5, 1.0, False)
+        op(None, batch, tout, (ow + 8, 40), interp, (4, 3), 1, 0.5, 1.0, False)
         torch.cuda.synchronize()
         res = tout.numpy()
         for i, a in enumerate(hosts):
-            ref = orc.fused_rccr(a[None], (32, 40), (48, 40), (4, 3), interp, odt, planar, 1, 0.5, 1.0, False)
+            ref = orc.fused_rccr(a[None], (32, ow), (ow + 8, 40), (4, 3), interp, odt, planar, 1, 0.5, 1.0, False)
             compare(res[i:i + 1], ref, interp, odt)
 
 

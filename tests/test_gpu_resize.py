@@ -426,6 +426,83 @@ def test_area_varshape(cv, K, orc, gpu, dt, c):
             assert bad.mean() <= (0.0 if (sw, sh, dw, dh) in sizes[:3] else 0.02), (sw, sh, dw, dh, bad.mean())
 
 
+# seeded random cases: 8-bit pixels of 1, 3 and 4 channels, every interpolation, scales of 0.42 to 2.4 per axis (now
+# and then equal, or exactly 1/2, 2/3, 1, 1.5, 2), small and 1080p-sized images, batches below and above the sizes
+# at which the strip kernels take over, as packed tensors, as views with odd leads and pitches (bytes outside the
+# rows must stay untouched) and as image batches of mixed sizes
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_shapes_scales_and_pitches(cv, K, orc, gpu, seed):
+    rng = np.random.default_rng(seed)
+    for it in range(36):
+        c = int(rng.choice([3, 3, 4, 1]))
+        interp = int(rng.choice([NEAREST, LINEAR, LINEAR, CUBIC, CUBIC, AREA]))
+        kind = str(rng.choice(["tensor", "view", "varshape"]))
+        fx, fy = (float(np.exp(rng.uniform(np.log(0.42), np.log(2.4)))) for _ in range(2))
+        if rng.random() < 0.2:
+            fy = fx
+        if rng.random() < 0.1:
+            fx = float(rng.choice([0.5, 1.0, 1.5, 2.0, 2 / 3]))
+        if rng.random() < 0.4:
+            sw, sh = int(rng.integers(600, 2300)), int(rng.integers(400, 1300))
+        else:
+            sw, sh = int(rng.integers(4, 700)), int(rng.integers(4, 500))
+        dw, dh = max(1, int(round(sw * fx))), max(1, int(round(sh * fy)))
+        n = int(np.clip(rng.choice([1, 2, 2048 * 64 * 16 // (dw * dh) + 1, 2048 * 256 * 8 // (dw * dh) + 1]), 1, 16))
+        n = min(n, max(1, int(60e6 / ((sw * sh + dw * dh) * c))))
+        case = "seed %d case %d: %s u8x%d interp %d %dx%d -> %dx%d n %d" % (seed, it, kind, c, interp, sw, sh, dw, dh, n)
+
+        def compare(res, src, out_hw, varshape):
+            if interp == AREA:  # (the golden's box filter parts ways with the device expression on enlargements)
+                np.testing.assert_array_equal(res, orc.resize_shipped(src, out_hw, AREA, varshape), err_msg=case)
+            else:
+                check(res, src, out_hw, interp, orc, varshape)
+
+        try:
+            if kind == "varshape":
+                fmt = _format_for(cv, K, np.uint8, c)
+                bin_, bout, hosts, outs = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], []
+                for i in range(n):
+                    w, h = max(8, sw + int(rng.integers(-30, 30))), max(8, sh + int(rng.integers(-30, 30)))
+                    gx, gy = (fx, fy) if rng.random() < 0.8 else (float(rng.uniform(0.3, 3)), float(rng.uniform(0.3, 3)))
+                    hosts.append(make_input(orc, (h, w, c), np.uint8, 1000 * it + i + seed))
+                    bin_.push_back(cv.Image.from_numpy(hosts[-1], fmt))
+                    outs.append(cv.Image.alloc((max(1, int(w * gx)), max(1, int(h * gy))), fmt))
+                    bout.push_back(outs[-1])
+                cv.Resize()(None, bin_, bout, interp)
+                torch.cuda.synchronize()
+                for a, o in zip(hosts, outs):
+                    w, h = o.size
+                    compare(o.plane_view(0, np.uint8, c).cpu().numpy()[None], a[None], (h, w), True)
+                continue
+            src = make_input(orc, (n, sh, sw, c), np.uint8, 77 * it + seed)
+            if kind == "tensor":
+                tout = cv.Tensor.alloc([n, dh, dw, c], np.uint8, "NHWC")
+                cv.Resize()(None, cv.Tensor.from_numpy(src, "NHWC"), tout, interp)
+                torch.cuda.synchronize()
+                compare(tout.numpy(), src, (dh, dw), False)
+                continue
+
+            def view(w, h, fill):
+                pad, lead = int(rng.integers(0, 9)), int(rng.integers(0, 5))
+                pitch = w * c + pad
+                plane = pitch * h + int(rng.integers(0, 9))
+                buf = torch.full((n * plane + 64,), fill, dtype=torch.uint8, device="cuda")
+                t = cv.Tensor.wrap(buf.data_ptr() + lead, [n, h, w, c], [plane, pitch, c, 1], np.uint8, "NHWC", keep=buf)
+                return buf, t, lead, plane, pitch
+
+            _, tin, lead, plane, pitch = view(sw, sh, 0)
+            torch.as_strided(_[lead:], (n, sh, sw, c), (plane, pitch, c, 1)).copy_(torch.from_numpy(src).cuda())
+            big_out, tout, lead, plane, pitch = view(dw, dh, 0xCD)
+            cv.Resize()(None, tin, tout, interp)
+            torch.cuda.synchronize()
+            compare(torch.as_strided(big_out[lead:], (n, dh, dw, c), (plane, pitch, c, 1)).cpu().numpy(), src, (dh, dw), False)
+            mask = torch.ones_like(big_out, dtype=torch.bool)
+            torch.as_strided(mask[lead:], (n, dh, dw * c), (plane, pitch, 1)).fill_(False)
+            assert bool((big_out[mask] == 0xCD).all()), "bytes outside the rows written"
+        except AssertionError as e:
+            raise AssertionError(case + ": " + str(e)) from e
+
+
 def test_negative_cases(cv, gpu):
     a = cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC")
     op = cv.Resize()
