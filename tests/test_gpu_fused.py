@@ -255,6 +255,69 @@ def test_varshape(cv, K, orc, gpu):
             compare(res[i:i + 1], ref, interp, odt)
 
 
+# seeded random cases: sizes from 1 pixel to 1080p-sized, resize factors 0.1 to 3, any crop of the resized image
+# (1-pixel-wide outputs included), both interpolations, output types and layouts, channel order, scale / offset, the
+# cast before scaling; as tensors, as views with odd leads and pitches whose last row ends the allocation, and as
+# image batches. Exact against the device-order restatement; against the golden order within one unit of |scale|
+# where the cast's rounding can tie, 1 LSB for 8-bit outputs and 1e-3 * max(1, |scale|) otherwise (a float32 sum in
+# another order, scaled, before an offset that may cancel it).
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_cases(cv, K, orc, gpu, seed):
+    rng = np.random.default_rng(seed)
+    op = cv.ResizeCropConvertReformat()
+    for it in range(120):
+        if rng.random() < 0.25:
+            sw, sh = int(rng.integers(500, 2000)), int(rng.integers(300, 1200))
+        else:
+            sw, sh = int(rng.integers(1, 300)), int(rng.integers(1, 200))
+        f = float(np.exp(rng.uniform(np.log(0.1), np.log(3))))
+        nw = max(2, min(1500, int(sw * f * rng.uniform(0.8, 1.25))))
+        nh = max(2, min(1000, int(sh * f * rng.uniform(0.8, 1.25))))
+        ow, oh = int(rng.integers(1, nw + 1)), int(rng.integers(1, nh + 1))
+        cx, cy = int(rng.integers(0, nw - ow + 1)), int(rng.integers(0, nh - oh + 1))
+        n = int(rng.integers(1, 5))
+        interp, odt = int(rng.integers(0, 2)), [np.uint8, np.float32][int(rng.integers(0, 2))]
+        planar, manip, cast = bool(rng.integers(0, 2)), int(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        scale, offset = [(1.0, 0.0), (1 / 127.5, -1.0), (0.5, 3.25), (-1.0, 255.0), (2.0, -100.0)][int(rng.integers(0, 5))]
+        kind = str(rng.choice(["tensor", "view", "varshape"]))
+        case = "seed %d case %d: %s %dx%d -> %dx%d crop (%d,%d) %dx%d n %d interp %d %s planar %d manip %d scale %g cast %d" % (
+            seed, it, kind, sw, sh, nw, nh, cx, cy, ow, oh, n, interp, np.dtype(odt).name, planar, manip, scale, cast)
+        tout = cv.Tensor.alloc([n, 3, oh, ow] if planar else [n, oh, ow, 3], odt, "NCHW" if planar else "NHWC")
+        args = ((nw, nh), interp, (cx, cy), manip, scale, offset, cast)
+
+        def exact(res, a):
+            dev = orc.fused_rccr(a, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast, order=1)
+            gold = orc.fused_rccr(a, (oh, ow), (nw, nh), (cx, cy), interp, odt, planar, manip, scale, offset, cast, order=0)
+            np.testing.assert_array_equal(res, dev, err_msg=case)
+            bar = 0.0 if interp == NEAREST else max(1.0, abs(scale)) * (1.0 if cast or odt == np.uint8 else 1e-3)
+            assert np.abs(res.astype(np.float64) - gold.astype(np.float64)).max() <= bar, case
+
+        if kind == "varshape":
+            batch, hosts = cv.ImageBatchVarShape(n), []
+            for i in range(n):
+                w, h = max(1, sw + int(rng.integers(-20, 20))), max(1, sh + int(rng.integers(-20, 20)))
+                hosts.append(orc.fill_u8((h, w, 3), 1000 * it + i + seed))
+                batch.push_back(cv.Image.from_numpy(hosts[-1], K.IMAGE_FORMAT_RGB8))
+            op(None, batch, tout, *args)
+            torch.cuda.synchronize()
+            res = tout.numpy()
+            for i, a in enumerate(hosts):
+                exact(res[i:i + 1], a[None])
+            continue
+        src = orc.fill_u8((n, sh, sw, 3), 31 * it + seed)
+        if kind == "view":
+            pad, lead = int(rng.integers(0, 9)), int(rng.integers(0, 5))
+            pitch = sw * 3 + pad
+            buf = torch.zeros((lead + (n * sh - 1) * pitch + sw * 3,), dtype=torch.uint8, device="cuda")
+            torch.as_strided(buf[lead:], (n, sh, sw, 3), (pitch * sh, pitch, 3, 1)).copy_(torch.from_numpy(src).cuda())
+            tin = cv.Tensor.wrap(buf.data_ptr() + lead, [n, sh, sw, 3], [pitch * sh, pitch, 3, 1], np.uint8, "NHWC", keep=buf)
+        else:
+            tin = cv.Tensor.from_numpy(src, "NHWC")
+        op(None, tin, tout, *args)
+        torch.cuda.synchronize()
+        exact(tout.numpy(), src)
+
+
 def test_benchmark_config_full_size(cv, orc, gpu):
     # BASELINE config 2 at full size: batch 64 of 1080p, every image different (one random image rolled by
     # 7 * n columns and n rows, so an image index that aliases would show), the oracle on all 64.

@@ -239,6 +239,81 @@ def test_warp_perspective(cv, K, orc, gpu):
         np.testing.assert_array_equal(outs[i].plane_view(0, np.uint8, 3).cpu().numpy(), ref[i])
 
 
+# seeded random cases: every element type and channel count, interpolation and border mode; sources and outputs from 1
+# pixel to 1400 x 900; rotations by any angle with independent axis scales of 0.4 to 2.5 and a shear, mapped near the
+# source's centre or far outside it; affine and perspective; tensors and image batches of mixed sizes. Inverse maps
+# are given, so device and oracle start from the same float32 matrix: exact for integers, 1e-3 for float32.
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_cases(cv, K, orc, gpu, seed):
+    rng = np.random.default_rng(seed)
+    fmts = {(np.uint8, 1): "U8", (np.uint8, 3): "RGB8", (np.uint8, 4): "RGBA8", (np.float32, 1): "F32", (np.float32, 3): "RGBf32"}
+    types = [(np.uint8, 3), (np.uint8, 3), (np.uint8, 1), (np.uint8, 4), (np.uint16, 3), (np.int16, 1), (np.float32, 3),
+             (np.float32, 4), (np.float32, 1)]
+    for it in range(150):
+        dt, c = types[int(rng.integers(0, len(types)))]
+        interp, border, n = int(rng.integers(0, 3)), int(rng.integers(0, 5)), int(rng.integers(1, 4))
+        persp = rng.random() < 0.3
+        varshape = (dt, c) in fmts and rng.random() < 0.5
+        big = rng.random() < 0.2
+        bval = tuple(float(v) for v in rng.integers(0, 255, 4))
+
+        def size():
+            if big:
+                return int(rng.integers(300, 1400)), int(rng.integers(200, 900))
+            return int(rng.integers(1, 200)), int(rng.integers(1, 150))
+
+        def matrix(sw, sh, dw, dh):
+            t = np.deg2rad(float(rng.uniform(-180, 180)) if rng.random() < 0.8 else float(rng.choice([0, 90, 180, 45])))
+            sx, sy = float(np.exp(rng.uniform(-0.9, 0.9))), float(np.exp(rng.uniform(-0.9, 0.9)))
+            a, b, d, e = sx * np.cos(t), -sy * np.sin(t) + float(rng.uniform(-0.2, 0.2)), sx * np.sin(t), sy * np.cos(t)
+            off = float(rng.uniform(-0.3, 0.3)) if rng.random() < 0.85 else float(rng.uniform(-3, 3))
+            cx, cy = (sw - 1) / 2 + off * sw, (sh - 1) / 2 + off * sh
+            m = [a, b, cx - a * (dw - 1) / 2 - b * (dh - 1) / 2, d, e, cy - d * (dw - 1) / 2 - e * (dh - 1) / 2]
+            if persp:
+                m += [float(rng.uniform(-2e-4, 2e-4)), float(rng.uniform(-2e-4, 2e-4)), 1.0]
+            return np.asarray(m, np.float32)
+
+        def image(h, w, s):
+            if dt == np.float32:
+                return orc.fill_f32((h, w, c), s) * 255
+            return orc.fill_u8((h, w, c, np.dtype(dt).itemsize), s).view(dt).reshape(h, w, c)
+
+        def compare(res, src, hw, m, what):
+            dev = orc.warp(src, hw, m, interp, border, bval, perspective=persp, variant=device_variant(interp, dt))
+            case = "seed %d case %d %s: %s x%d interp %d border %d persp %d %s -> %s m %s" % (
+                seed, it, what, np.dtype(dt).name, c, interp, border, persp, src.shape, hw, m.tolist())
+            if dt == np.float32:
+                assert np.abs(res - dev).max() <= 1e-3, case
+            else:
+                np.testing.assert_array_equal(res, dev, err_msg=case)
+
+        op = (cv.WarpPerspective if persp else cv.WarpAffine)(8)
+        if varshape:
+            fmt = getattr(K, "IMAGE_FORMAT_" + fmts[(dt, c)])
+            bi, bo, hosts, outs, mats = cv.ImageBatchVarShape(n), cv.ImageBatchVarShape(n), [], [], []
+            for i in range(n):
+                (sw, sh), (dw, dh) = size(), size()
+                hosts.append(image(sh, sw, 100 * it + i + seed))
+                bi.push_back(cv.Image.from_numpy(hosts[-1], fmt))
+                outs.append(cv.Image.alloc((dw, dh), fmt))
+                bo.push_back(outs[-1])
+                mats.append(matrix(sw, sh, dw, dh))
+            mats = np.asarray(mats, np.float32)
+            op(None, bi, bo, cv.Tensor.from_numpy(mats, "NW"), interp | INVERSE_MAP, border, bval)
+            torch.cuda.synchronize()
+            for i in range(n):
+                w, h = outs[i].size
+                compare(outs[i].plane_view(0, dt, c).cpu().numpy()[None], hosts[i][None], (h, w), mats[i], "image %d" % i)
+        else:
+            (sw, sh), (dw, dh) = size(), size()
+            src = np.stack([image(sh, sw, 100 * it + i + seed) for i in range(n)])
+            m = matrix(sw, sh, dw, dh)
+            tout = cv.Tensor.alloc([n, dh, dw, c], dt, "NHWC")
+            op(None, cv.Tensor.from_numpy(src, "NHWC"), tout, m.tolist(), interp | INVERSE_MAP, border, bval)
+            torch.cuda.synchronize()
+            compare(tout.numpy(), src, (dh, dw), m, "tensor")
+
+
 def test_tensor_negative(cv, gpu):
     op = cv.WarpAffine(0)
     a = cv.Tensor.alloc([2, 8, 8, 3], np.uint8, "NHWC")
