@@ -2574,12 +2574,21 @@ __global__ __launch_bounds__(256) void ResizeCubicStripU8VarShapeKernel(const Re
     }
 }
 
-// 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows).
+// 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows) when enlarging, side by side when
+// reducing (measured on one machine, 32 x u8x3: 1080p -> 720p 78.7 us stacked, 76.0 us side by side; 720p -> 1080p
+// 120.9 us stacked, 125.8 us side by side).
 template<int C, int S>
 __global__ __launch_bounds__(256) void ResizeCubicStripU8Kernel(const ResizeArgs a)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeCubicStripU8<C, S>(p, blockIdx.x * kPatchTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kCubicStripRows);
+    if constexpr (S == 4) // reducing: a block's waves side by side (256 columns x 16 rows)
+    {
+        ResizeCubicStripU8<C, S>(p, (blockIdx.x * 4 + (threadIdx.x >> 6)) * kPatchTileW, blockIdx.y * kCubicStripRows);
+    }
+    else
+    {
+        ResizeCubicStripU8<C, S>(p, blockIdx.x * kPatchTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kCubicStripRows);
+    }
 }
 
 template<class T, int C, int INTERP>
@@ -2587,7 +2596,7 @@ __global__ __launch_bounds__(256) void ResizePatchVarShapeKernel(const ResizeArg
 {
     const TileCoord tc = LocateTile(tiles, blockIdx.x);
     const Plane     p  = GetPlanes<true>(a, tc.image);
-    ResizeWavePatch<T, C, INTERP, true>(p, tc.tx * kPatchTileW, tc.ty * kPatchTileH + (threadIdx.x >> 6) * 4);
+    ResizeWavePatch<T, C, INTERP, true>(p, (tc.tx * 4 + (threadIdx.x >> 6)) * kPatchTileW, tc.ty * 4);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -3120,7 +3129,8 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
             dim3 sgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, 4 * kCubicStripRows), N);
             if (form == 4)
             {
-                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 4>), sgrid, dim3(256), 0, stream, a);
+                dim3 flat(DivUp(a.dstW, 4 * kPatchTileW), DivUp(a.dstH, kCubicStripRows), N);
+                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 4>), flat, dim3(256), 0, stream, a);
             }
             else
             {
@@ -3240,7 +3250,7 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
         }
         if constexpr (kPatchForm<T, C, INTERP>)
         {
-            int total = BuildVarTiles(tiles, dstHost, first, count, kPatchTileW, kPatchTileH);
+            int total = BuildVarTiles(tiles, dstHost, first, count, 4 * kPatchTileW, 4);
             if (total > 0)
             {
                 hipLaunchKernelGGL((ResizePatchVarShapeKernel<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a,
