@@ -37,7 +37,7 @@ NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
 # write parts are in the summary files named below. The counters sit between the L2s and the fabric:
 # a batch that fits the memory-side cache (warp-affine-varshape) has part of those reads served there.
 MEASURED_TRAFFIC_BYTES = {"fused": 122963923, "resize-cubic-4k": 1474458644, "resize-nearest": 12249763,
-                          "resize-linear": 23286608, "nv12-to-rgb": 298655003, "warp-affine-varshape": 298562951}
+                          "resize-linear": 23286608, "nv12-to-rgb": 298659855, "warp-affine-varshape": 298562951}
 # The rocprofv3 counter summary each figure above is the "total" line of (a CPU test compares them).
 TRAFFIC_PROFILES = {"fused": "FusedBilinear_batch64_1080p_to_224",
                     "resize-cubic-4k": "ResizeCubicStagedKernel_f32x4_batch16_4k_to_640x360",

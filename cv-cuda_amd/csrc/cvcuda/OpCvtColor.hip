@@ -28,8 +28,8 @@ namespace {
 // ---------------------------------------------------------------------------------------------------
 // YUV 4:2:0 -> RGB
 constexpr int kYuvBlockW = 8;               // pixels per lane and row (a lane converts a kYuvBlockW x 2 block)
-constexpr int kYuvTileW  = 64 * kYuvBlockW; // pixels per block row
-constexpr int kYuvTileH  = 8;               // rows per block: 4 waves x 2 rows
+constexpr int kYuvTileW  = 64 * kYuvBlockW; // pixels per wave and row
+constexpr int kYuvTileH  = 8;               // image batches: rows per block, 4 waves x 2 rows (tensors: 4 waves side by side)
 
 struct YuvArgs
 {
@@ -255,8 +255,10 @@ __device__ __forceinline__ void ConvertLaneBlock(const uint8_t *src, int srcRow,
 template<int DCN, bool SEMIPLANAR>
 __global__ __launch_bounds__(256) void Yuv420ToRgbTensor(const YuvArgs a)
 {
-    const int x = (blockIdx.x * 64 + (threadIdx.x & 63)) * kYuvBlockW;
-    const int y = (blockIdx.y * 4 + (threadIdx.x >> 6)) * 2;
+    // a block's four waves side by side on one pair of rows (2048 columns): 32 x 1080p 51.5 -> 50.8 us against the
+    // block of 512 columns x 8 rows, on one machine
+    const int x = (blockIdx.x * 256 + threadIdx.x) * kYuvBlockW;
+    const int y = blockIdx.y * 2;
     if (x >= a.W || y >= a.H)
     {
         return;
@@ -590,7 +592,7 @@ void LaunchYuv(const YuvArgs &a, int N, const NVCVImageBufferStrided *dstHost, h
 {
     if (dstHost == nullptr)
     {
-        dim3 grid(DivUp(a.W, kYuvTileW), DivUp(a.H, kYuvTileH), N);
+        dim3 grid(DivUp(a.W, 4 * kYuvTileW), DivUp(a.H, 2), N);
         hipLaunchKernelGGL((Yuv420ToRgbTensor<DCN, SEMIPLANAR>), grid, dim3(256), 0, stream, a);
         CheckLaunch("Yuv420ToRgbTensor");
         return;

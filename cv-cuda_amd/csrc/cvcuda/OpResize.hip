@@ -2434,13 +2434,15 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8VarShapeKernel(const R
 }
 
 // Large image-batch launches resize each image in the tensor kernels' strips. WIDE (most of the launch is enlarged by
-// 1.5 or more): a 256 x 32 tile per block - four columns per lane where the image is enlarged so
-// (a wave takes 8 rows), else two columns per lane at horizontal scales up to 2 (16 strips of 128 x 4, four per wave),
-// else 32 wave patches. Otherwise a 128 x 16 tile: a two-column strip per wave, or two wave patches.
+// 1.5 or more): a 1024 x 8 tile per block - four columns per lane where the image is enlarged so
+// (the block's waves side by side, 256 columns x 8 rows each), else two columns per lane at horizontal scales up to 2
+// (16 strips of 128 x 4, four per wave), else 32 wave patches. Otherwise a 512 x 4 tile: a two-column strip per wave, or
+// two wave patches. (As 256 x 32 and 128 x 16 tiles of stacked waves, on one machine: u8x4 nearest neighbour enlarging
+// by 1.5 57.4 against 51.4 us, u8x1 bilinear enlarging by 1.2 38.3 against 36.5 us, the rest within 2 %.)
 template<bool WIDE>
-constexpr int kStripsTileW = WIDE ? 256 : 128;
+constexpr int kStripsTileW = WIDE ? 1024 : 512;
 template<bool WIDE>
-constexpr int kStripsTileH = WIDE ? 32 : 16;
+constexpr int kStripsTileH = WIDE ? 8 : 4;
 
 template<int C>
 __host__ __device__ __forceinline__ bool QuadStripScale(int srcW, int dstW)
@@ -2461,7 +2463,7 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
         {
             if constexpr (kQuadsRows<C> == kStripRows)
             {
-                ResizeLinearQuadStripU8<C>(p, x0, y0 + wave * kStripRows);
+                ResizeLinearQuadStripU8<C>(p, x0 + wave * kQuadsTileW, y0);
             }
         }
         else if (PairsFormScale<C>(p.srcW, p.dstW))
@@ -2469,7 +2471,7 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
 #pragma unroll 1
             for (int i = wave; i < 16; i += 4)
             {
-                ResizeLinearPairStripU8<C>(p, x0 + (i & 1) * kPairsTileW, y0 + (i >> 1) * kPairStripRows);
+                ResizeLinearPairStripU8<C>(p, x0 + (i & 7) * kPairsTileW, y0 + (i >> 3) * kPairStripRows);
             }
         }
         else
@@ -2477,7 +2479,7 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
 #pragma unroll 1
             for (int i = wave; i < 32; i += 4)
             {
-                ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + (i & 3) * 64, y0 + (i >> 2) * 4);
+                ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + (i & 15) * 64, y0 + (i >> 4) * 4);
             }
         }
     }
@@ -2485,12 +2487,12 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
     {
         if (PairsFormScale<C>(p.srcW, p.dstW))
         {
-            ResizeLinearPairStripU8<C>(p, x0, y0 + wave * kPairStripRows);
+            ResizeLinearPairStripU8<C>(p, x0 + wave * kPairsTileW, y0);
         }
         else
         {
-            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0, y0 + wave * 4);
-            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + 64, y0 + wave * 4);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + wave * 128, y0);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + wave * 128 + 64, y0);
         }
     }
 }
@@ -2514,14 +2516,14 @@ __global__ __launch_bounds__(256) void ResizeNearestStripsU8VarShapeKernel(const
     const int       x0 = tc.tx * kStripsTileW<true>, y0 = tc.ty * kStripsTileH<true>;
     if (NearestStripScale<C>(p.srcW, p.srcH, p.dstW, p.dstH))
     {
-        ResizeNearestQuadStripU8<C>(p, x0, y0 + wave * kStripRows);
+        ResizeNearestQuadStripU8<C>(p, x0 + wave * kQuadsTileW, y0);
     }
     else
     {
 #pragma unroll 1
         for (int i = wave; i < 32; i += 4)
         {
-            ResizeWavePatch<uint8_t, C, NVCV_INTERP_NEAREST, true>(p, x0 + (i & 3) * 64, y0 + (i >> 2) * 4);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_NEAREST, true>(p, x0 + (i & 15) * 64, y0 + (i >> 4) * 4);
         }
     }
 }
