@@ -17,11 +17,11 @@ namespace cvamd {
 // 7 / 6 / 4 of 8 gave 23.7 / 25.9 / 28.8 us).
 constexpr int kRowsPerWave  = 1;
 constexpr int kWavesPerBlk  = 4;
-// Waves of a workgroup side by side on an output row, the others stacked. One: a workgroup is 64 columns x 4
-// rows. With all four on ONE row (a workgroup then reads two contiguous source spans of 2.8 KB and writes 896
-// contiguous bytes per plane) the same launch took 22.46 us against 22.57 us: within the noise of the memory
-// system, not shipped.
-constexpr int kWavesAcross = 1;
+// Waves of a workgroup side by side on an output row, the others stacked. With all four on ONE row a workgroup
+// reads two contiguous source spans of 2.8 KB and writes 896 contiguous bytes per plane. Against 64 columns x 4 rows
+// (kWavesAcross = 1), alternating on one machine, three times each: 22.58 -> 22.48 us for the batch of 64 tensors
+// images, 22.21 -> 22.03 us for the image batch; two waves across: no change.
+constexpr int kWavesAcross = 4;
 constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlk / kWavesAcross;
 constexpr int kColsPerBlock = 64 * kWavesAcross;
 
