@@ -36,7 +36,7 @@ NEAREST, LINEAR, CUBIC, AREA = 0, 1, 2, 3
 # kernel and the workload, not of a run, so it is recorded here rather than re-measured; read and
 # write parts are in the summary files named below. The counters sit between the L2s and the fabric:
 # a batch that fits the memory-side cache (warp-affine-varshape) has part of those reads served there.
-MEASURED_TRAFFIC_BYTES = {"fused": 122963923, "resize-cubic-4k": 1474458644, "resize-nearest": 12249763,
+MEASURED_TRAFFIC_BYTES = {"fused": 122963893, "resize-cubic-4k": 1474458644, "resize-nearest": 12249763,
                           "resize-linear": 23286608, "nv12-to-rgb": 298659855, "warp-affine-varshape": 298562951}
 # The rocprofv3 counter summary each figure above is the "total" line of (a CPU test compares them).
 TRAFFIC_PROFILES = {"fused": "FusedBilinear_batch64_1080p_to_224",
