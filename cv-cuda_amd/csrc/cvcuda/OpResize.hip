@@ -2373,16 +2373,44 @@ __host__ __device__ __forceinline__ bool PairsFormScale(int srcW, int dstW)
 
 constexpr int kPairsTileW = 128, kPairsTileH = 8; // image batches: block = 4 waves of 128 columns x 2 rows, stacked
 
-// Tensors: strips of 4 rows per wave, a block = 4 waves side by side (512 columns x 4 rows). The strip kernels of
-// tensors all place a block's waves side by side: a block then writes 4 rows of 1.5 to 3 KB each instead of 16 or 32
-// rows of a quarter of that, and the launches whose time is the memory's got shorter by 3 to 8 % (32 x u8x3: 1080p ->
-// 720p 51.2 -> 49.8 us, 720p -> 1080p bilinear 66.6 -> 61.4 us, nearest 58.2 -> 55.0 us, AREA 60.9 -> 59.2 us). The
-// bicubic strips, whose time is the vector ALU's, did not gain (enlarging they lost 5 %) and stay stacked.
+// The tile (in units of a wave's tile) of this wave in a launch of the tensor kernels below: a block's waves lie side by
+// side (flat) or are stacked. Flat, a block writes few long row pieces instead of many short ones, which the memory
+// likes better when the launch is bound by it (32 x u8x3, the two shapes alternating on one machine: 720p -> 1080p
+// bilinear 67.3 -> 65.1 us, nearest 58.0 -> 55.4 us; 1080p -> 720p box filter 61.5 -> 59.6 us, bicubic 79.0 -> 77.3 us,
+// bilinear 51.4 -> 51.2 us; bicubic enlarging 120.9 -> 125.8 us, which stays stacked). Rows much shorter than a flat
+// block's span leave most of its waves without columns, and on small images the rows of a stacked block share source
+// rows in the L1 (256 x 448 x 448 -> 300 x 300 u8x3 bicubic: 72.6 us stacked, 91.8 us flat), so the host chooses flat
+// blocks for rows of 1024 pixels and more that fill their blocks to 80 % (FlatBlocks).
+struct WaveTile
+{
+    int x, y;
+};
+
+__device__ __forceinline__ WaveTile WaveTileOf(int flat)
+{
+    const int waves = blockDim.x >> 6, wave = threadIdx.x >> 6;
+    return flat ? WaveTile{(int)blockIdx.x * waves + wave, (int)blockIdx.y} : WaveTile{(int)blockIdx.x, (int)blockIdx.y * waves + wave};
+}
+
+static inline bool FlatBlocks(int dstW, int waveW)
+{
+    const int64_t span = 4 * (int64_t)waveW;
+    return dstW >= 1024 && DivUp(dstW, (int)span) * span * 4 <= (int64_t)dstW * 5;
+}
+
+// Grid of a launch of four-wave blocks whose waves own tiles of waveW x waveH.
+static inline dim3 WaveTileGrid(int dstW, int dstH, int N, int waveW, int waveH, bool flat, int waves = 4)
+{
+    return flat ? dim3(DivUp(dstW, waves * waveW), DivUp(dstH, waveH), N) : dim3(DivUp(dstW, waveW), DivUp(dstH, waves * waveH), N);
+}
+
+// Tensors: strips of 4 rows per wave.
 template<int C>
-__global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArgs a)
+__global__ __launch_bounds__(256) void ResizeLinearPairsU8Kernel(const ResizeArgs a, const int flat)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeLinearPairStripU8<C>(p, (blockIdx.x * 4 + (threadIdx.x >> 6)) * kPairsTileW, blockIdx.y * kPairStripRows);
+    const WaveTile t = WaveTileOf(flat);
+    ResizeLinearPairStripU8<C>(p, t.x * kPairsTileW, t.y * kPairStripRows);
 }
 
 constexpr int kQuadsTileW = 256; // a wave's columns; tensors: block = 4 waves side by side (1024 columns x kQuadsRows rows)
@@ -2393,25 +2421,19 @@ template<int C>
 constexpr int kQuadsRows = kStripRows;
 
 template<int C>
-__global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArgs a)
+__global__ __launch_bounds__(256) void ResizeLinearQuadsU8Kernel(const ResizeArgs a, const int flat)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    const int y0 = blockIdx.y * kQuadsRows<C>;
-    if constexpr (kQuadsRows<C> == kStripRows)
-    {
-        ResizeLinearQuadStripU8<C>(p, (blockIdx.x * 4 + (threadIdx.x >> 6)) * kQuadsTileW, y0);
-    }
-    else
-    {
-        ResizeLinearQuadsU8<C>(p, blockIdx.x * kQuadsTileW, y0);
-    }
+    const WaveTile t = WaveTileOf(flat);
+    ResizeLinearQuadStripU8<C>(p, t.x * kQuadsTileW, t.y * kStripRows);
 }
 
 template<int C>
-__global__ __launch_bounds__(256) void ResizeNearestQuadsU8Kernel(const ResizeArgs a)
+__global__ __launch_bounds__(256) void ResizeNearestQuadsU8Kernel(const ResizeArgs a, const int flat)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeNearestQuadStripU8<C>(p, (blockIdx.x * 4 + (threadIdx.x >> 6)) * kQuadsTileW, blockIdx.y * kStripRows);
+    const WaveTile t = WaveTileOf(flat);
+    ResizeNearestQuadStripU8<C>(p, t.x * kQuadsTileW, t.y * kStripRows);
 }
 
 // Image batches: the same 128 x 8 tile per block for every image; an image whose horizontal scale is
@@ -2433,16 +2455,22 @@ __global__ __launch_bounds__(256) void ResizeLinearPairsU8VarShapeKernel(const R
     }
 }
 
-// Large image-batch launches resize each image in the tensor kernels' strips. WIDE (most of the launch is enlarged by
-// 1.5 or more): a 1024 x 8 tile per block - four columns per lane where the image is enlarged so
-// (the block's waves side by side, 256 columns x 8 rows each), else two columns per lane at horizontal scales up to 2
-// (16 strips of 128 x 4, four per wave), else 32 wave patches. Otherwise a 512 x 4 tile: a two-column strip per wave, or
-// two wave patches. (As 256 x 32 and 128 x 16 tiles of stacked waves, on one machine: u8x4 nearest neighbour enlarging
-// by 1.5 57.4 against 51.4 us, u8x1 bilinear enlarging by 1.2 38.3 against 36.5 us, the rest within 2 %.)
+// Large image-batch launches resize each image in the tensor kernels' strips; a wave owns a tile of 256 x 8 (WIDE: most of
+// the launch is enlarged by 1.5 or more) or 128 x 4 output pixels, a block four of them, side by side or stacked as
+// in the tensor kernels (WaveTileOf; the host chooses by the images' widths). WIDE: four columns per lane where the
+// image is enlarged so, else two columns per lane at horizontal scales up to 2 (4 strips of 128 x 4), else 8 wave
+// patches. Otherwise a two-column strip, or two wave patches.
 template<bool WIDE>
-constexpr int kStripsTileW = WIDE ? 1024 : 512;
+constexpr int kStripsWaveW = WIDE ? kQuadsTileW : kPairsTileW;
 template<bool WIDE>
-constexpr int kStripsTileH = WIDE ? 8 : 4;
+constexpr int kStripsWaveH = WIDE ? kStripRows : kPairStripRows;
+
+// The tile (in units of a wave's tile) of this wave in an image-batch block whose tile is 4 wave tiles wide (flat) or high.
+__device__ __forceinline__ WaveTile VarWaveTileOf(const TileCoord &tc, int flat)
+{
+    const int wave = threadIdx.x >> 6;
+    return flat ? WaveTile{tc.tx * 4 + wave, tc.ty} : WaveTile{tc.tx, tc.ty * 4 + wave};
+}
 
 template<int C>
 __host__ __device__ __forceinline__ bool QuadStripScale(int srcW, int dstW)
@@ -2451,35 +2479,32 @@ __host__ __device__ __forceinline__ bool QuadStripScale(int srcW, int dstW)
 }
 
 template<int C, bool WIDE>
-__global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+__global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles, const int flat)
 {
-    const TileCoord tc   = LocateTile(tiles, blockIdx.x);
-    const Plane     p    = GetPlanes<true>(a, tc.image);
-    const int       wave = threadIdx.x >> 6;
-    const int       x0 = tc.tx * kStripsTileW<WIDE>, y0 = tc.ty * kStripsTileH<WIDE>;
+    const TileCoord tc = LocateTile(tiles, blockIdx.x);
+    const Plane     p  = GetPlanes<true>(a, tc.image);
+    const WaveTile  t  = VarWaveTileOf(tc, flat);
+    const int       x0 = t.x * kStripsWaveW<WIDE>, y0 = t.y * kStripsWaveH<WIDE>;
     if constexpr (WIDE)
     {
         if (QuadStripScale<C>(p.srcW, p.dstW))
         {
-            if constexpr (kQuadsRows<C> == kStripRows)
-            {
-                ResizeLinearQuadStripU8<C>(p, x0 + wave * kQuadsTileW, y0);
-            }
+            ResizeLinearQuadStripU8<C>(p, x0, y0);
         }
         else if (PairsFormScale<C>(p.srcW, p.dstW))
         {
 #pragma unroll 1
-            for (int i = wave; i < 16; i += 4)
+            for (int i = 0; i < 4; ++i)
             {
-                ResizeLinearPairStripU8<C>(p, x0 + (i & 7) * kPairsTileW, y0 + (i >> 3) * kPairStripRows);
+                ResizeLinearPairStripU8<C>(p, x0 + (i & 1) * kPairsTileW, y0 + (i >> 1) * kPairStripRows);
             }
         }
         else
         {
 #pragma unroll 1
-            for (int i = wave; i < 32; i += 4)
+            for (int i = 0; i < 8; ++i)
             {
-                ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + (i & 15) * 64, y0 + (i >> 4) * 4);
+                ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + (i & 3) * 64, y0 + (i >> 2) * 4);
             }
         }
     }
@@ -2487,12 +2512,12 @@ __global__ __launch_bounds__(256) void ResizeLinearStripsU8VarShapeKernel(const 
     {
         if (PairsFormScale<C>(p.srcW, p.dstW))
         {
-            ResizeLinearPairStripU8<C>(p, x0 + wave * kPairsTileW, y0);
+            ResizeLinearPairStripU8<C>(p, x0, y0);
         }
         else
         {
-            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + wave * 128, y0);
-            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + wave * 128 + 64, y0);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0, y0);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_LINEAR, true>(p, x0 + 64, y0);
         }
     }
 }
@@ -2506,24 +2531,24 @@ __host__ __device__ __forceinline__ bool NearestStripScale(int srcW, int srcH, i
     return srcW >= 8 && 3 * (int64_t)srcW <= 2 * (int64_t)dstW && srcH <= dstH;
 }
 
-// Large image batches that are mostly such images: a 256 x 32 tile per block, a strip per wave or eight patches.
+// Large image batches that are mostly such images: a 256 x 8 tile per wave, a strip or eight patches.
 template<int C>
-__global__ __launch_bounds__(256) void ResizeNearestStripsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+__global__ __launch_bounds__(256) void ResizeNearestStripsU8VarShapeKernel(const ResizeArgs a, const VarTiles tiles, const int flat)
 {
-    const TileCoord tc   = LocateTile(tiles, blockIdx.x);
-    const Plane     p    = GetPlanes<true>(a, tc.image);
-    const int       wave = threadIdx.x >> 6;
-    const int       x0 = tc.tx * kStripsTileW<true>, y0 = tc.ty * kStripsTileH<true>;
+    const TileCoord tc = LocateTile(tiles, blockIdx.x);
+    const Plane     p  = GetPlanes<true>(a, tc.image);
+    const WaveTile  t  = VarWaveTileOf(tc, flat);
+    const int       x0 = t.x * kStripsWaveW<true>, y0 = t.y * kStripsWaveH<true>;
     if (NearestStripScale<C>(p.srcW, p.srcH, p.dstW, p.dstH))
     {
-        ResizeNearestQuadStripU8<C>(p, x0 + wave * kQuadsTileW, y0);
+        ResizeNearestQuadStripU8<C>(p, x0, y0);
     }
     else
     {
 #pragma unroll 1
-        for (int i = wave; i < 32; i += 4)
+        for (int i = 0; i < 8; ++i)
         {
-            ResizeWavePatch<uint8_t, C, NVCV_INTERP_NEAREST, true>(p, x0 + (i & 15) * 64, y0 + (i >> 4) * 4);
+            ResizeWavePatch<uint8_t, C, NVCV_INTERP_NEAREST, true>(p, x0 + (i & 3) * 64, y0 + (i >> 2) * 4);
         }
     }
 }
@@ -2531,11 +2556,12 @@ __global__ __launch_bounds__(256) void ResizeNearestStripsU8VarShapeKernel(const
 constexpr int kPatchTileW = 64, kPatchTileH = 16; // block = 4 waves stacked vertically
 
 template<class T, int C, int INTERP>
-__global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs a)
+__global__ __launch_bounds__(256) void ResizePatchTensorKernel(const ResizeArgs a, const int flat)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    // blocks are 4 waves side by side, or single waves when the whole launch is small
-    ResizeWavePatch<T, C, INTERP, false>(p, (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * kPatchTileW, blockIdx.y * 4);
+    // blocks are 4 waves, or single waves when the whole launch is small
+    const WaveTile t = WaveTileOf(flat);
+    ResizeWavePatch<T, C, INTERP, false>(p, t.x * kPatchTileW, t.y * 4);
 }
 
 // Which of the bicubic strip forms an image takes by its vertical scale and row length: 4 (reducing by up to 2), 8
@@ -2576,29 +2602,22 @@ __global__ __launch_bounds__(256) void ResizeCubicStripU8VarShapeKernel(const Re
     }
 }
 
-// 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows) when enlarging, side by side when
-// reducing (measured on one machine, 32 x u8x3: 1080p -> 720p 78.7 us stacked, 76.0 us side by side; 720p -> 1080p
-// 120.9 us stacked, 125.8 us side by side).
+// 8-bit bicubic strips: block = 4 waves stacked vertically (64 columns x 64 rows) or, reducing wide images, side by side.
 template<int C, int S>
-__global__ __launch_bounds__(256) void ResizeCubicStripU8Kernel(const ResizeArgs a)
+__global__ __launch_bounds__(256) void ResizeCubicStripU8Kernel(const ResizeArgs a, const int flat)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    if constexpr (S == 4) // reducing: a block's waves side by side (256 columns x 16 rows)
-    {
-        ResizeCubicStripU8<C, S>(p, (blockIdx.x * 4 + (threadIdx.x >> 6)) * kPatchTileW, blockIdx.y * kCubicStripRows);
-    }
-    else
-    {
-        ResizeCubicStripU8<C, S>(p, blockIdx.x * kPatchTileW, (blockIdx.y * 4 + (threadIdx.x >> 6)) * kCubicStripRows);
-    }
+    const WaveTile t = WaveTileOf(flat);
+    ResizeCubicStripU8<C, S>(p, t.x * kPatchTileW, t.y * kCubicStripRows);
 }
 
 template<class T, int C, int INTERP>
-__global__ __launch_bounds__(256) void ResizePatchVarShapeKernel(const ResizeArgs a, const VarTiles tiles)
+__global__ __launch_bounds__(256) void ResizePatchVarShapeKernel(const ResizeArgs a, const VarTiles tiles, const int flat)
 {
     const TileCoord tc = LocateTile(tiles, blockIdx.x);
     const Plane     p  = GetPlanes<true>(a, tc.image);
-    ResizeWavePatch<T, C, INTERP, true>(p, (tc.tx * 4 + (threadIdx.x >> 6)) * kPatchTileW, tc.ty * 4);
+    const WaveTile  t  = VarWaveTileOf(tc, flat);
+    ResizeWavePatch<T, C, INTERP, true>(p, t.x * kPatchTileW, t.y * 4);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2920,10 +2939,11 @@ __device__ __forceinline__ void ResizeAreaPlainWaveTile(const Plane &p, int x0, 
 }
 
 template<int C>
-__global__ __launch_bounds__(256) void ResizeAreaFixedTensorKernel(const ResizeArgs a)
+__global__ __launch_bounds__(256) void ResizeAreaFixedTensorKernel(const ResizeArgs a, const int flat)
 {
     const Plane p = GetPlanes<false>(a, blockIdx.z);
-    ResizeAreaFixedWaveTile<C>(p, (blockIdx.x * 4 + (threadIdx.x >> 6)) * kAreaTileW, blockIdx.y * kAreaRowsPerWave);
+    const WaveTile t = WaveTileOf(flat);
+    ResizeAreaFixedWaveTile<C>(p, t.x * kAreaTileW, t.y * kAreaRowsPerWave);
 }
 
 template<int C>
@@ -3086,8 +3106,9 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         const int64_t strips = (int64_t)DivUp(a.dstW, kQuadsTileW) * DivUp(a.dstH, kStripRows) * N;
         if (NearestStripScale<C>(a.srcW, a.srcH, a.dstW, a.dstH) && strips >= 8 * 256)
         {
-            dim3 qgrid(DivUp(a.dstW, 4 * kQuadsTileW), DivUp(a.dstH, kStripRows), N);
-            hipLaunchKernelGGL((ResizeNearestQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
+            const bool flat = FlatBlocks(a.dstW, kQuadsTileW);
+            hipLaunchKernelGGL((ResizeNearestQuadsU8Kernel<C>), WaveTileGrid(a.dstW, a.dstH, N, kQuadsTileW, kStripRows, flat), dim3(256), 0,
+                               stream, a, (int)flat);
             CheckLaunch("ResizeNearestQuadsU8Kernel");
             return;
         }
@@ -3096,15 +3117,17 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     {
         if (a.srcW >= 4 && 3 * (int64_t)a.srcW <= 2 * (int64_t)a.dstW)
         {
-            dim3 qgrid(DivUp(a.dstW, 4 * kQuadsTileW), DivUp(a.dstH, kQuadsRows<C>), N);
-            hipLaunchKernelGGL((ResizeLinearQuadsU8Kernel<C>), qgrid, dim3(256), 0, stream, a);
+            const bool flat = FlatBlocks(a.dstW, kQuadsTileW);
+            hipLaunchKernelGGL((ResizeLinearQuadsU8Kernel<C>), WaveTileGrid(a.dstW, a.dstH, N, kQuadsTileW, kStripRows, flat), dim3(256), 0,
+                               stream, a, (int)flat);
             CheckLaunch("ResizeLinearQuadsU8Kernel");
             return;
         }
         if (PairsFormScale<C>(a.srcW, a.dstW))
         {
-            dim3 pgrid(DivUp(a.dstW, 4 * kPairsTileW), DivUp(a.dstH, kPairStripRows), N);
-            hipLaunchKernelGGL((ResizeLinearPairsU8Kernel<C>), pgrid, dim3(256), 0, stream, a);
+            const bool flat = FlatBlocks(a.dstW, kPairsTileW);
+            hipLaunchKernelGGL((ResizeLinearPairsU8Kernel<C>), WaveTileGrid(a.dstW, a.dstH, N, kPairsTileW, kPairStripRows, flat), dim3(256),
+                               0, stream, a, (int)flat);
             CheckLaunch("ResizeLinearPairsU8Kernel");
             return;
         }
@@ -3113,8 +3136,9 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     {
         if (AreaFixedDomain(a.scaleX, a.scaleY, a.srcW * C, a.srcH))
         {
-            dim3 agrid(DivUp(a.dstW, 4 * kAreaTileW), DivUp(a.dstH, kAreaRowsPerWave), N);
-            hipLaunchKernelGGL((ResizeAreaFixedTensorKernel<C>), agrid, dim3(256), 0, stream, a);
+            const bool flat = FlatBlocks(a.dstW, kAreaTileW);
+            hipLaunchKernelGGL((ResizeAreaFixedTensorKernel<C>), WaveTileGrid(a.dstW, a.dstH, N, kAreaTileW, kAreaRowsPerWave, flat),
+                               dim3(256), 0, stream, a, (int)flat);
             CheckLaunch("ResizeAreaFixedTensorKernel");
             return;
         }
@@ -3128,15 +3152,15 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         const int     form   = CubicStripForm<C>(a.srcW, a.srcH, a.dstH);
         if (strips >= 8 * 256 && form != 0)
         {
-            dim3 sgrid(DivUp(a.dstW, kPatchTileW), DivUp(a.dstH, 4 * kCubicStripRows), N);
+            const bool flat = form == 4 && FlatBlocks(a.dstW, kPatchTileW); // (enlarging: stacked, see WaveTileOf)
+            const dim3 sgrid = WaveTileGrid(a.dstW, a.dstH, N, kPatchTileW, kCubicStripRows, flat);
             if (form == 4)
             {
-                dim3 flat(DivUp(a.dstW, 4 * kPatchTileW), DivUp(a.dstH, kCubicStripRows), N);
-                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 4>), flat, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 4>), sgrid, dim3(256), 0, stream, a, (int)flat);
             }
             else
             {
-                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 8>), sgrid, dim3(256), 0, stream, a);
+                hipLaunchKernelGGL((ResizeCubicStripU8Kernel<C, 8>), sgrid, dim3(256), 0, stream, a, (int)flat);
             }
             CheckLaunch("ResizeCubicStripU8Kernel");
             return;
@@ -3148,8 +3172,9 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
         // and finishes sooner the more CUs take part
         const int64_t blocks = (int64_t)DivUp(a.dstW, kPatchTileW) * DivUp(a.dstH, kPatchTileH) * N;
         const int     waves  = blocks < 8 * 256 ? 1 : 4;
-        dim3          pgrid(DivUp(a.dstW, kPatchTileW * waves), DivUp(a.dstH, 4), N);
-        hipLaunchKernelGGL((ResizePatchTensorKernel<T, C, INTERP>), pgrid, dim3(64 * waves), 0, stream, a);
+        const bool    flat   = waves == 4 && FlatBlocks(a.dstW, kPatchTileW);
+        hipLaunchKernelGGL((ResizePatchTensorKernel<T, C, INTERP>), WaveTileGrid(a.dstW, a.dstH, N, kPatchTileW, 4, flat, waves),
+                           dim3(64 * waves), 0, stream, a, (int)flat);
         CheckLaunch("ResizePatchTensorKernel");
         return;
     }
@@ -3157,7 +3182,7 @@ void LaunchTensor(const ResizeArgs &a, int N, hipStream_t stream)
     // f32x3 bilinear 56.4 -> 45.5 us, f32x4 68.1 -> 56.3 us); reducing, it is the reads, and the four rows of the
     // 64 x 4 block share source rows (1080p -> 720p f32x3 bilinear 41.1 us against 49.3 us flat).
     // (bicubic keeps the 64 x 4 block: its time is the arithmetic's and did not change with the block)
-    const int flat = INTERP != NVCV_INTERP_CUBIC && (int64_t)a.dstW * a.dstH > (int64_t)a.srcW * a.srcH;
+    const int flat = INTERP != NVCV_INTERP_CUBIC && (int64_t)a.dstW * a.dstH > (int64_t)a.srcW * a.srcH && FlatBlocks(a.dstW, kTileW);
     hipLaunchKernelGGL((ResizeTensorKernel<T, C, INTERP>), flat ? dim3(DivUp(a.dstW, kTileW * kTileH), a.dstH, N) : grid, dim3(256), 0, stream,
                        a, flat);
     CheckLaunch("ResizeTensorKernel");
@@ -3171,6 +3196,21 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
     {
         VarTiles  tiles;
         const int count = std::min(kMaxTileImages, N - first);
+        // whether most output pixels of this launch lie in images for which a block of four waves side by side pays
+        // (FlatBlocks), given a wave's tile; and the block's tile either way
+        auto flatFor = [&](int waveW)
+        {
+            int64_t flatPixels = 0, allPixels = 0;
+            for (int i = first; i < first + count; ++i)
+            {
+                const int64_t px = (int64_t)dstHost[i].planes[0].width * dstHost[i].planes[0].height;
+                allPixels += px;
+                flatPixels += FlatBlocks(dstHost[i].planes[0].width, waveW) ? px : 0;
+            }
+            return 2 * flatPixels > allPixels;
+        };
+        auto buildTiles = [&](int waveW, int waveH, bool flat)
+        { return BuildVarTiles(tiles, dstHost, first, count, flat ? 4 * waveW : waveW, flat ? waveH : 4 * waveH); };
         if constexpr (kPairsForm<T, C, INTERP>)
         {
             // strips when that still gives every CU 8 blocks: the wide tile where most output pixels belong to images
@@ -3182,17 +3222,19 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
                 allPixels += px;
                 quadPixels += QuadStripScale<C>(srcHost[i].planes[0].width, dstHost[i].planes[0].width) ? px : 0;
             }
-            int total = 2 * quadPixels > allPixels ? BuildVarTiles(tiles, dstHost, first, count, kStripsTileW<true>, kStripsTileH<true>) : 0;
+            bool flat  = flatFor(kStripsWaveW<true>);
+            int  total = 2 * quadPixels > allPixels ? buildTiles(kStripsWaveW<true>, kStripsWaveH<true>, flat) : 0;
             if (total >= 8 * 256)
             {
-                hipLaunchKernelGGL((ResizeLinearStripsU8VarShapeKernel<C, true>), dim3(total), dim3(256), 0, stream, a, tiles);
+                hipLaunchKernelGGL((ResizeLinearStripsU8VarShapeKernel<C, true>), dim3(total), dim3(256), 0, stream, a, tiles, (int)flat);
                 CheckLaunch("ResizeLinearStripsU8VarShapeKernel");
                 continue;
             }
-            total = BuildVarTiles(tiles, dstHost, first, count, kStripsTileW<false>, kStripsTileH<false>);
+            flat  = flatFor(kStripsWaveW<false>);
+            total = buildTiles(kStripsWaveW<false>, kStripsWaveH<false>, flat);
             if (total >= 8 * 256)
             {
-                hipLaunchKernelGGL((ResizeLinearStripsU8VarShapeKernel<C, false>), dim3(total), dim3(256), 0, stream, a, tiles);
+                hipLaunchKernelGGL((ResizeLinearStripsU8VarShapeKernel<C, false>), dim3(total), dim3(256), 0, stream, a, tiles, (int)flat);
                 CheckLaunch("ResizeLinearStripsU8VarShapeKernel");
                 continue;
             }
@@ -3224,10 +3266,11 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
                 allPixels += px;
                 stripPixels += NearestStripScale<C>(sp.width, sp.height, dp.width, dp.height) ? px : 0;
             }
-            int total = 2 * stripPixels > allPixels ? BuildVarTiles(tiles, dstHost, first, count, kStripsTileW<true>, kStripsTileH<true>) : 0;
+            const bool flat  = flatFor(kStripsWaveW<true>);
+            int        total = 2 * stripPixels > allPixels ? buildTiles(kStripsWaveW<true>, kStripsWaveH<true>, flat) : 0;
             if (total >= 8 * 256)
             {
-                hipLaunchKernelGGL((ResizeNearestStripsU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles);
+                hipLaunchKernelGGL((ResizeNearestStripsU8VarShapeKernel<C>), dim3(total), dim3(256), 0, stream, a, tiles, (int)flat);
                 CheckLaunch("ResizeNearestStripsU8VarShapeKernel");
                 continue;
             }
@@ -3252,11 +3295,12 @@ void LaunchVarShape(const ResizeArgs &a, const NVCVImageBufferStrided *srcHost, 
         }
         if constexpr (kPatchForm<T, C, INTERP>)
         {
-            int total = BuildVarTiles(tiles, dstHost, first, count, 4 * kPatchTileW, 4);
+            const bool flat  = flatFor(kPatchTileW);
+            int        total = buildTiles(kPatchTileW, 4, flat);
             if (total > 0)
             {
                 hipLaunchKernelGGL((ResizePatchVarShapeKernel<T, C, INTERP>), dim3(total), dim3(256), 0, stream, a,
-                                   tiles);
+                                   tiles, (int)flat);
                 CheckLaunch("ResizePatchVarShapeKernel");
             }
             continue;
