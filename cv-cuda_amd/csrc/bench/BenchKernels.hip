@@ -19,8 +19,8 @@ __global__ __launch_bounds__(256) void FusedCopyBound(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
     const int     n    = tp.n;
-    const int     dx   = FusedColumnOf(tp.tx);
-    const int     dy0  = FusedFirstRowOf(tp.ty);
+    const int     dx   = FusedColumnOf(tp.tx, a.wavesAcross);
+    const int     dy0  = FusedFirstRowOf(tp.ty, a.wavesAcross);
     if (dx >= a.dstW)
     {
         return;
@@ -168,7 +168,7 @@ extern "C" __attribute__((visibility("default"))) int cvamdBenchFusedCopyBound(
     a.cropY  = cropY;
     a.scaleX = static_cast<float>(srcW) / newW;
     a.scaleY = static_cast<float>(srcH) / newH;
-    if (N > kFusedImagesPerLaunch || (dstH + kRowsPerBlock - 1) / kRowsPerBlock / (int)kXcdCount >= 65535)
+    if (N > kFusedImagesPerLaunch || dstH / (int)kXcdCount >= 65535)
     {
         return (int)hipErrorInvalidValue;
     }

@@ -17,23 +17,41 @@ namespace cvamd {
 // 7 / 6 / 4 of 8 gave 23.7 / 25.9 / 28.8 us).
 constexpr int kRowsPerWave  = 1;
 constexpr int kWavesPerBlk  = 4;
-// Waves of a workgroup side by side on an output row, the others stacked. With all four on ONE row a workgroup
-// reads two contiguous source spans of 2.8 KB and writes 896 contiguous bytes per plane. Against 64 columns x 4 rows
-// (kWavesAcross = 1), alternating on one machine, three times each: 22.58 -> 22.48 us for the batch of 64 tensors
-// images, 22.21 -> 22.03 us for the image batch; two waves across: no change.
-constexpr int kWavesAcross = 4;
-constexpr int kRowsPerBlock = kRowsPerWave * kWavesPerBlk / kWavesAcross;
-constexpr int kColsPerBlock = 64 * kWavesAcross;
-
-// Output column of this lane and first output row of its wave within tile (tx, ty).
-__device__ __forceinline__ int FusedColumnOf(int tx)
+// Waves of a workgroup side by side on an output row (the others stacked): 1 or 4, chosen per launch
+// (FusedArgs::wavesAcross). With all four on ONE row a workgroup reads two contiguous source spans of 2.8 KB and
+// writes 896 contiguous bytes per plane; against 64 columns x 4 rows, alternating on one machine, three times each:
+// 22.58 -> 22.48 us for the batch of 64 tensor images, 22.21 -> 22.03 us for the image batch (two waves across: no
+// change). Other row lengths keep 64 x 4 (FusedWavesAcross).
+__host__ __device__ __forceinline__ int FusedColsPerBlock(int wavesAcross)
 {
-    return tx * kColsPerBlock + (int)(threadIdx.x & (kColsPerBlock - 1));
+    return 64 * wavesAcross;
 }
 
-__device__ __forceinline__ int FusedFirstRowOf(int ty)
+__host__ __device__ __forceinline__ int FusedRowsPerBlock(int wavesAcross)
 {
-    return ty * kRowsPerBlock + (int)(threadIdx.x / kColsPerBlock) * kRowsPerWave;
+    return kRowsPerWave * kWavesPerBlk / wavesAcross;
+}
+
+inline int FusedWavesAcross(int dstW)
+{
+    // one workgroup per output row where the row fills it to 80 % (205 .. 256 columns: the 224 of the usual network
+    // input). Wider rows measured no gain for planar outputs and a loss for interleaved 8-bit ones (64 x 1280 x 720 ->
+    // 640 x 360: 47.9 -> 51.6 us), narrower ones leave waves without columns.
+    const int span = FusedColsPerBlock(kWavesPerBlk);
+    return dstW <= span && (int64_t)dstW * 5 >= (int64_t)span * 4 ? kWavesPerBlk : 1;
+}
+
+// Output column of this lane and first output row of its wave within tile (tx, ty).
+__device__ __forceinline__ int FusedColumnOf(int tx, int wavesAcross)
+{
+    const int cols = FusedColsPerBlock(wavesAcross);
+    return tx * cols + (int)(threadIdx.x & (cols - 1));
+}
+
+__device__ __forceinline__ int FusedFirstRowOf(int ty, int wavesAcross)
+{
+    // (1 wave across: the workgroup's waves are its rows; 4 across: one row)
+    return wavesAcross == 1 ? ty * (kRowsPerWave * kWavesPerBlk) + (int)(threadIdx.x >> 6) * kRowsPerWave : ty * kRowsPerWave;
 }
 
 struct FusedArgs
@@ -59,6 +77,7 @@ struct FusedArgs
     int32_t srcCast;
     // launch shape: column tiles and row tiles per image, first image of this launch
     uint32_t tilesX, tilesY;
+    int32_t  wavesAcross; // 1 or 4: the workgroup is 64 columns x 4 rows or 256 columns x 1 row (set by SetFusedGrid)
     uint32_t firstImage;
     // per-channel normalisation of the extension entry points, indexed by source channel:
     // ((scale*v + offset) - normBase) * normMul * normGlobal + normShift
@@ -99,8 +118,9 @@ constexpr int kFusedImagesPerLaunch = 65535;
 // images (at most kFusedImagesPerLaunch) starting at a.firstImage.
 inline dim3 SetFusedGrid(FusedArgs &a, int images)
 {
-    a.tilesX = (uint32_t)((a.dstW + kColsPerBlock - 1) / kColsPerBlock);
-    a.tilesY = (uint32_t)((a.dstH + kRowsPerBlock - 1) / kRowsPerBlock);
+    a.wavesAcross = FusedWavesAcross(a.dstW);
+    a.tilesX      = (uint32_t)((a.dstW + FusedColsPerBlock(a.wavesAcross) - 1) / FusedColsPerBlock(a.wavesAcross));
+    a.tilesY      = (uint32_t)((a.dstH + FusedRowsPerBlock(a.wavesAcross) - 1) / FusedRowsPerBlock(a.wavesAcross));
     return dim3(a.tilesX * kXcdCount, (a.tilesY + kXcdCount - 1) / kXcdCount, (uint32_t)images);
 }
 

@@ -253,12 +253,12 @@ __device__ __forceinline__ void ConvertLaneBlock(const uint8_t *src, int srcRow,
 }
 
 template<int DCN, bool SEMIPLANAR>
-__global__ __launch_bounds__(256) void Yuv420ToRgbTensor(const YuvArgs a)
+__global__ __launch_bounds__(256) void Yuv420ToRgbTensor(const YuvArgs a, const int flat)
 {
-    // a block's four waves side by side on one pair of rows (2048 columns): 32 x 1080p 51.5 -> 50.8 us against the
-    // block of 512 columns x 8 rows, on one machine
-    const int x = (blockIdx.x * 256 + threadIdx.x) * kYuvBlockW;
-    const int y = blockIdx.y * 2;
+    // flat: a block's four waves side by side on one pair of rows (2048 columns) instead of 512 columns x 8 rows: 32 x
+    // 1080p 51.5 -> 50.8 us, the two alternating on one machine. The host asks for it where rows fill such blocks to 80 %.
+    const int x = (flat ? blockIdx.x * 256 + threadIdx.x : blockIdx.x * 64 + (threadIdx.x & 63)) * kYuvBlockW;
+    const int y = (flat ? blockIdx.y : blockIdx.y * 4 + (threadIdx.x >> 6)) * 2;
     if (x >= a.W || y >= a.H)
     {
         return;
@@ -592,8 +592,10 @@ void LaunchYuv(const YuvArgs &a, int N, const NVCVImageBufferStrided *dstHost, h
 {
     if (dstHost == nullptr)
     {
-        dim3 grid(DivUp(a.W, 4 * kYuvTileW), DivUp(a.H, 2), N);
-        hipLaunchKernelGGL((Yuv420ToRgbTensor<DCN, SEMIPLANAR>), grid, dim3(256), 0, stream, a);
+        const int64_t span = 4 * kYuvTileW;
+        const bool    flat = DivUp(a.W, (int)span) * span * 4 <= (int64_t)a.W * 5;
+        dim3          grid(DivUp(a.W, flat ? 4 * kYuvTileW : kYuvTileW), DivUp(a.H, flat ? 2 : kYuvTileH), N);
+        hipLaunchKernelGGL((Yuv420ToRgbTensor<DCN, SEMIPLANAR>), grid, dim3(256), 0, stream, a, (int)flat);
         CheckLaunch("Yuv420ToRgbTensor");
         return;
     }

@@ -106,8 +106,8 @@ __global__ __launch_bounds__(256) void FusedNearest(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
     const int     n    = tp.n;
-    const int     dx   = FusedColumnOf(tp.tx);
-    const int     dy0  = FusedFirstRowOf(tp.ty);
+    const int     dx   = FusedColumnOf(tp.tx, a.wavesAcross);
+    const int     dy0  = FusedFirstRowOf(tp.ty, a.wavesAcross);
     if (dx >= a.dstW)
     {
         return;
@@ -141,8 +141,8 @@ __global__ __launch_bounds__(256) void FusedBilinear(const FusedArgs a)
 {
     const TilePos tp   = LocateFusedTile(a);
     const int     n    = tp.n;
-    const int     dx   = FusedColumnOf(tp.tx);
-    const int     dy0  = FusedFirstRowOf(tp.ty);
+    const int     dx   = FusedColumnOf(tp.tx, a.wavesAcross);
+    const int     dy0  = FusedFirstRowOf(tp.ty, a.wavesAcross);
     if (dx >= a.dstW)
     {
         return;
@@ -205,7 +205,7 @@ void LaunchKernels(FusedArgs a, int N, NVCVInterpolationType interp, bool tinyIm
     {
         return;
     }
-    if ((a.dstW + kColsPerBlock - 1) / kColsPerBlock > (INT32_MAX / (int)kXcdCount) || (a.dstH + kRowsPerBlock - 1) / kRowsPerBlock / (int)kXcdCount >= 65535)
+    if ((a.dstW + 63) / 64 > (INT32_MAX / (int)kXcdCount) || a.dstH / (int)kXcdCount >= 65535)
     {
         throw OpError(NVCV_ERROR_OVERFLOW, "Output of %d x %d needs too many tiles for one launch", a.dstW, a.dstH);
     }
