@@ -257,8 +257,10 @@ __global__ __launch_bounds__(256) void Yuv420ToRgbTensor(const YuvArgs a, const 
 {
     // flat: a block's four waves side by side on one pair of rows (2048 columns) instead of 512 columns x 8 rows: 32 x
     // 1080p 51.5 -> 50.8 us, the two alternating on one machine. The host asks for it where rows fill such blocks to 80 %.
-    const int x = (flat ? blockIdx.x * 256 + threadIdx.x : blockIdx.x * 64 + (threadIdx.x & 63)) * kYuvBlockW;
-    const int y = (flat ? blockIdx.y : blockIdx.y * 4 + (threadIdx.x >> 6)) * 2;
+    // (arithmetic rather than a branch on `flat`, so that the other arguments are loaded at once)
+    const int f = flat != 0;
+    const int x = (int)(blockIdx.x * (64u << (2 * f)) + (threadIdx.x & (63u | (192u * f)))) * kYuvBlockW;
+    const int y = (int)(blockIdx.y * (4 - 3 * f) + (threadIdx.x >> 6) * (1 - f)) * 2;
     if (x >= a.W || y >= a.H)
     {
         return;
