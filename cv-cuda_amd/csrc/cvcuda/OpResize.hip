@@ -2391,7 +2391,8 @@ __device__ __forceinline__ WaveTile WaveTileOf(int flat)
     // (arithmetic, not a branch: behind a branch on `flat` the compiler loads the kernel's other arguments only after
     // that test, one more round trip to memory before a wave's first pixel load, 0.3 us on the 4 - 6 us launches of small
     // batches)
-    const int waves = blockDim.x >> 6, wave = threadIdx.x >> 6, f = flat != 0;
+    // (the wave's number as a scalar: tile origins, row terms and loop counters then stay on the scalar unit)
+    const int waves = blockDim.x >> 6, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), f = flat != 0;
     const int across = f * (waves - 1) + 1, down = waves + 1 - across; // flat: waves, 1; stacked: 1, waves
     return WaveTile{(int)blockIdx.x * across + wave * f, (int)blockIdx.y * down + wave * (1 - f)};
 }
@@ -2472,7 +2473,7 @@ constexpr int kStripsWaveH = WIDE ? kStripRows : kPairStripRows;
 // The tile (in units of a wave's tile) of this wave in an image-batch block whose tile is 4 wave tiles wide (flat) or high.
 __device__ __forceinline__ WaveTile VarWaveTileOf(const TileCoord &tc, int flat)
 {
-    const int wave = threadIdx.x >> 6, f = flat != 0;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), f = flat != 0;
     return WaveTile{tc.tx * (3 * f + 1) + wave * f, tc.ty * (4 - 3 * f) + wave * (1 - f)};
 }
 
